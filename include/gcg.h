@@ -1,0 +1,119 @@
+/*
+ * gcg.h -- C ABI of the MI355X (gfx950) gated chunked causal convolution
+ *
+ *     u = B * x ;  y2[b,t,c] = sum_k h[c/dg, k] * u[b, t-(hl-1)+k, c] ;  y = C * y2
+ *
+ * and its backward (dx, dB, dC, dh).  This is the boundary a replacement for
+ * savanna's `gcg_two_pass` path binds to: every entry point takes plain device
+ * pointers, sizes and a HIP stream, returns 0 or a negative error code, never
+ * throws, never synchronises the host and never allocates device memory.
+ *
+ * Tensors x, B, C, y, y2, bx, dy, dx, dB, dC are (bs, L, g, dg), contiguous,
+ * channel fastest (d = g*dg); h and dh are (g, 1, hl), contiguous.  All share
+ * one element type `dtype`.  Cross-correlation convention: tap hl-1 multiplies
+ * the current sample and samples before t = 0 are zero
+ * (savanna/kernels/triton_src/cgcg/ref_fwd.py:41,109-129).
+ */
+#ifndef GCG_H
+#define GCG_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define GCG_API __attribute__((visibility("default")))
+#else
+#define GCG_API
+#endif
+
+/* Element types (the reference's `cgcg_dtype`, savanna/arguments/global_config.py:404). */
+enum { GCG_F32 = 0, GCG_BF16 = 1, GCG_F16 = 2 };
+
+/* Kernel families.  GCG_ALGO_AUTO picks by (dtype, hl, dg); the others force one
+ * family and fail with GCG_ERR_UNSUPPORTED when the shape does not fit it. */
+enum {
+    GCG_ALGO_AUTO   = 0,
+    GCG_ALGO_DIRECT = 1, /* LDS-tiled sliding window on the vector ALUs, any hl/dg/dtype */
+    GCG_ALGO_WINDOW = 2, /* register sliding window, hl <= 8 (Hyena-SE)                   */
+    GCG_ALGO_MFMA   = 3  /* banded Toeplitz GEMM on MFMA, bf16/f16, hl <= 128, dg % 16 == 0 (Hyena-MR) */
+};
+
+/* Error codes. */
+enum {
+    GCG_OK              = 0,
+    GCG_ERR_BAD_ARG     = -1, /* null pointer, non-positive size, unknown dtype/algo */
+    GCG_ERR_UNSUPPORTED = -2, /* shape outside what the forced algo handles          */
+    GCG_ERR_WORKSPACE   = -3, /* workspace missing or smaller than *_workspace_bytes */
+    GCG_ERR_LAUNCH      = -4, /* hipLaunchKernel / stream error; see gcg_last_hip_error */
+    GCG_ERR_DEVICE      = -5  /* current device is not gfx950                        */
+};
+
+/* Human-readable text for a code above. */
+GCG_API const char *gcg_strerror(int code);
+
+/* hipError_t of the last failed HIP call made by this library on the calling
+ * thread (0 when none). */
+GCG_API int gcg_last_hip_error(void);
+
+/* Library version, e.g. 100 for 0.1.0. */
+GCG_API int gcg_version(void);
+
+/*
+ * Forward.
+ * Replaces two_pass_fwd_grouped(x, B, C, h, return_bx=, return_y2=)
+ * (savanna/kernels/triton_src/cgcg/src/fwd.py:13-233), which launches
+ * _two_pass_fwd_refactor_kernel (src/fwd_kernels.py:585-750).
+ *
+ *   y            out, required
+ *   y2_or_null   out, optional: the convolution before the post-gate (fwd.py `return_y2`)
+ *   bx_or_null   out, optional: the pre-gate product B*x             (fwd.py `return_bx`)
+ *   stream       hipStream_t to enqueue on (NULL = the null stream)
+ */
+GCG_API int gcg_fwd(const void *x, const void *B, const void *C, const void *h,
+            void *y, void *y2_or_null, void *bx_or_null,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, int32_t algo, void *stream);
+
+/*
+ * Workspace the backward needs for the deterministic filter-gradient reduction
+ * (per-workgroup partial sums of dh).  Depends on the sizes, dtype and algo only.
+ * Returns 0 on invalid arguments.
+ */
+GCG_API size_t gcg_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                               int32_t dtype, int32_t algo);
+
+/*
+ * Backward.
+ * Replaces two_pass_bwd_refactor(dy, Bx, y2, x, B, C, h, bs, seqlen, g, dg, ...)
+ * (savanna/kernels/triton_src/cgcg/src/bwd.py:347-474: pre_conv_kernel,
+ * conv1d_input, conv1d_weight, group sum, post_conv_kernel).  The saved
+ * activations Bx and y2 of the reference are not needed: both are recomputed
+ * on chip from x, B, h.
+ *
+ *   dx, dB, dC   out, (bs, L, g, dg), element type `dtype`
+ *   dh           out, (g, 1, hl), element type `dtype`, overwritten (not accumulated)
+ *   workspace    device scratch of at least gcg_bwd_workspace_bytes(...) bytes,
+ *                256-byte aligned; contents on entry are ignored
+ */
+GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C, const void *h,
+            void *dx, void *dB, void *dC, void *dh,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, int32_t algo, void *stream);
+
+/*
+ * Name of the kernel family GCG_ALGO_AUTO resolves to for these sizes
+ * (GCG_ALGO_DIRECT / _WINDOW / _MFMA), or a negative error code.
+ * `backward` selects the rule for gcg_bwd.
+ */
+GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                    int32_t dtype, int32_t backward);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GCG_H */

@@ -1,0 +1,149 @@
+"""ctypes binding of libgcg_hip.so (C ABI: include/gcg.h).
+
+There is no CPU or PyTorch fallback: if the library is missing, or a call fails,
+an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import threading
+
+import torch
+
+_CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB_PATH = os.path.join(_CSRC, "libgcg_hip.so")
+
+GCG_F32, GCG_BF16, GCG_F16 = 0, 1, 2
+ALGO_AUTO, ALGO_DIRECT, ALGO_WINDOW, ALGO_MFMA = 0, 1, 2, 3
+ALGO_NAMES = {"auto": ALGO_AUTO, "direct": ALGO_DIRECT, "window": ALGO_WINDOW, "mfma": ALGO_MFMA}
+
+_DTYPES = {torch.float32: GCG_F32, torch.bfloat16: GCG_BF16, torch.float16: GCG_F16}
+
+# every symbol include/gcg.h declares
+EXPORTS = (
+    "gcg_strerror", "gcg_last_hip_error", "gcg_version", "gcg_fwd",
+    "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_select_algo",
+)
+
+_lock = threading.Lock()
+_lib = None
+
+
+class GcgError(RuntimeError):
+    """A gcg_* entry point returned a negative code."""
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library built in-tree (``make -C savanna_amd/csrc``)."""
+    global _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise ImportError(
+                f"{LIB_PATH} is not built; run `python -c 'import __graft_entry__ as g; g.build()'` "
+                "or `make -C savanna_amd/csrc`. There is no fallback path."
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        vp, i64, i32, sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, ctypes.c_size_t
+        lib.gcg_strerror.argtypes = [ctypes.c_int]
+        lib.gcg_strerror.restype = ctypes.c_char_p
+        lib.gcg_last_hip_error.argtypes = []
+        lib.gcg_last_hip_error.restype = ctypes.c_int
+        lib.gcg_version.argtypes = []
+        lib.gcg_version.restype = ctypes.c_int
+        lib.gcg_fwd.argtypes = [vp] * 7 + [i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_fwd.restype = ctypes.c_int
+        lib.gcg_bwd_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32, i32]
+        lib.gcg_bwd_workspace_bytes.restype = sz
+        lib.gcg_bwd.argtypes = [vp] * 10 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_bwd.restype = ctypes.c_int
+        lib.gcg_select_algo.argtypes = [i64, i64, i32, i32, i32, i32, i32]
+        lib.gcg_select_algo.restype = ctypes.c_int
+        _lib = lib
+        return lib
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dtype}; expected float32, bfloat16 or float16") from None
+
+
+def algo_code(algo) -> int:
+    if isinstance(algo, str):
+        return ALGO_NAMES[algo]
+    return int(algo)
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        lib = load()
+        msg = lib.gcg_strerror(rc).decode()
+        raise GcgError(f"{what}: {msg} (code {rc}, hipError {lib.gcg_last_hip_error()})")
+
+
+def _require_gpu(t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            "savanna_amd runs on an MI355X (gfx950) device only; got a tensor on "
+            f"{t.device}. There is no CPU path."
+        )
+
+
+def fwd(x, B, C, h, return_bx=False, return_y2=False, algo=ALGO_AUTO):
+    """y (and optionally bx, y2) for contiguous (bs, L, g, dg) inputs and (g, 1, hl) filter."""
+    lib = load()
+    _require_gpu(x)
+    bs, L, g, dg = x.shape
+    hl = h.shape[-1]
+    y = torch.empty_like(x)
+    y2 = torch.empty_like(x) if return_y2 else None
+    bx = torch.empty_like(x) if return_bx else None
+    if x.numel() == 0:
+        return bx, y2, y
+    with torch.cuda.device(x.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_fwd(
+            x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), y.data_ptr(),
+            y2.data_ptr() if y2 is not None else None,
+            bx.data_ptr() if bx is not None else None,
+            bs, L, g, dg, hl, dtype_code(x.dtype), algo_code(algo), st,
+        )
+    check(rc, "gcg_fwd")
+    return bx, y2, y
+
+
+def bwd(dy, x, B, C, h, algo=ALGO_AUTO):
+    """(dx, dB, dC, dh) for contiguous inputs; dh has h's shape and dtype."""
+    lib = load()
+    _require_gpu(x)
+    bs, L, g, dg = x.shape
+    hl = h.shape[-1]
+    dx, dB, dC = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    dh = torch.empty_like(h)
+    if x.numel() == 0:
+        return dx, dB, dC, dh.zero_()
+    code, a = dtype_code(x.dtype), algo_code(algo)
+    nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, a)
+    if nbytes == 0:
+        raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")
+    with torch.cuda.device(x.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_bwd(
+            dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(),
+            dx.data_ptr(), dB.data_ptr(), dC.data_ptr(), dh.data_ptr(),
+            ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, a, st,
+        )
+    check(rc, "gcg_bwd")
+    return dx, dB, dC, dh
+
+
+def select_algo(bs, L, g, dg, hl, dtype: torch.dtype, backward=False) -> str:
+    rc = load().gcg_select_algo(bs, L, g, dg, hl, dtype_code(dtype), int(backward))
+    if rc < 0:
+        check(rc, "gcg_select_algo")
+    return {v: k for k, v in ALGO_NAMES.items()}[rc]

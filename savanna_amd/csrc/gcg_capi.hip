@@ -1,0 +1,151 @@
+// C ABI (include/gcg.h): argument checks, kernel-family selection, launch.
+#include "gcg_common.h"
+
+#include <mutex>
+
+namespace {
+
+thread_local int tls_hip_error = 0;
+
+// gfx950 check, cached per device ordinal.
+int check_device()
+{
+    static std::mutex mu;
+    static int ok[64];  // 0 unknown, 1 yes, -1 no
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { tls_hip_error = (int)e; return GCG_ERR_LAUNCH; }
+    if (dev < 0 || dev >= 64) return GCG_OK;
+    std::lock_guard<std::mutex> lk(mu);
+    if (ok[dev] == 0) {
+        hipDeviceProp_t p;
+        e = hipGetDeviceProperties(&p, dev);
+        if (e != hipSuccess) { tls_hip_error = (int)e; return GCG_ERR_LAUNCH; }
+        ok[dev] = (__builtin_strncmp(p.gcnArchName, "gfx950", 6) == 0) ? 1 : -1;
+    }
+    return ok[dev] == 1 ? GCG_OK : GCG_ERR_DEVICE;
+}
+
+int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, gcg::Dims *dm)
+{
+    if (bs <= 0 || L <= 0 || g <= 0 || dg <= 0 || hl <= 0) return GCG_ERR_BAD_ARG;
+    if (dtype != GCG_F32 && dtype != GCG_BF16 && dtype != GCG_F16) return GCG_ERR_BAD_ARG;
+    dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg;
+    return GCG_OK;
+}
+
+int resolve_algo(int algo, int dtype, const gcg::Dims &dm, bool backward)
+{
+    (void)backward;
+    switch (algo) {
+    case GCG_ALGO_AUTO:
+        if (gcg::window_supported(dm)) return GCG_ALGO_WINDOW;
+        if (gcg::mfma_supported(dtype, dm)) return GCG_ALGO_MFMA;
+        return GCG_ALGO_DIRECT;
+    case GCG_ALGO_DIRECT: return GCG_ALGO_DIRECT;
+    case GCG_ALGO_WINDOW: return gcg::window_supported(dm) ? GCG_ALGO_WINDOW : GCG_ERR_UNSUPPORTED;
+    case GCG_ALGO_MFMA:   return gcg::mfma_supported(dtype, dm) ? GCG_ALGO_MFMA : GCG_ERR_UNSUPPORTED;
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
+int finish(int hip_rc)
+{
+    if (hip_rc == 0) return GCG_OK;
+    tls_hip_error = hip_rc;
+    return GCG_ERR_LAUNCH;
+}
+
+} // namespace
+
+extern "C" {
+
+GCG_API const char *gcg_strerror(int code)
+{
+    switch (code) {
+    case GCG_OK:              return "ok";
+    case GCG_ERR_BAD_ARG:     return "bad argument (null pointer, non-positive size, unknown dtype or algo)";
+    case GCG_ERR_UNSUPPORTED: return "shape not supported by the requested kernel family";
+    case GCG_ERR_WORKSPACE:   return "workspace missing, misaligned or too small";
+    case GCG_ERR_LAUNCH:      return "HIP launch failed (see gcg_last_hip_error)";
+    case GCG_ERR_DEVICE:      return "current device is not gfx950";
+    }
+    return "unknown error";
+}
+
+GCG_API int gcg_last_hip_error(void) { return tls_hip_error; }
+
+GCG_API int gcg_version(void) { return 100; }
+
+GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t backward)
+{
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    return resolve_algo(GCG_ALGO_AUTO, dtype, dm, backward != 0);
+}
+
+GCG_API int gcg_fwd(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t algo,
+            void *stream)
+{
+    if (!x || !B || !C || !h || !y) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    const int a = resolve_algo(algo, dtype, dm, false);
+    if (a < 0) return a;
+    rc = check_device();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (a) {
+    case GCG_ALGO_DIRECT: return finish(gcg::direct_fwd_launch(dtype, x, B, C, h, y, y2, bx, dm, st));
+    case GCG_ALGO_WINDOW: return finish(gcg::window_fwd_launch(dtype, x, B, C, h, y, y2, bx, dm, st));
+    case GCG_ALGO_MFMA:   return finish(gcg::mfma_fwd_launch(dtype, x, B, C, h, y, y2, bx, dm, st));
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
+GCG_API size_t gcg_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype,
+                               int32_t algo)
+{
+    gcg::Dims dm;
+    if (make_dims(bs, L, g, dg, hl, dtype, &dm)) return 0;
+    const int a = resolve_algo(algo, dtype, dm, true);
+    size_t n = 0;
+    switch (a) {
+    case GCG_ALGO_DIRECT: n = gcg::direct_bwd_workspace(dm); break;
+    case GCG_ALGO_WINDOW: n = gcg::window_bwd_workspace(dm); break;
+    case GCG_ALGO_MFMA:   n = gcg::mfma_bwd_workspace(dm); break;
+    default: return 0;
+    }
+    return (n + 255) & ~(size_t)255;
+}
+
+GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
+            void *dC, void *dh, void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g,
+            int32_t dg, int32_t hl, int32_t dtype, int32_t algo, void *stream)
+{
+    if (!dy || !x || !B || !C || !h || !dx || !dB || !dC || !dh) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    const int a = resolve_algo(algo, dtype, dm, true);
+    if (a < 0) return a;
+    const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (a) {
+    case GCG_ALGO_DIRECT:
+        return finish(gcg::direct_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    case GCG_ALGO_WINDOW:
+        return finish(gcg::window_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    case GCG_ALGO_MFMA:
+        return finish(gcg::mfma_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
+} // extern "C"

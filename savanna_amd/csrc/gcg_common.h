@@ -1,0 +1,90 @@
+// Shared device helpers for the gated chunked causal convolution kernels (gfx950).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/gcg.h"
+
+namespace gcg {
+
+// ---- element types -------------------------------------------------------------------
+// bf16 and f16 travel as raw 16-bit patterns; arithmetic is always fp32.
+struct bf16_t { uint16_t v; };
+struct f16_t  { uint16_t v; };
+
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t lo16)
+{
+    return __uint_as_float(lo16 << 16);
+}
+
+// round-to-nearest-even fp32 -> bf16 bit pattern (NaN kept quiet)
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static __device__ __forceinline__ float load(const float *p) { return *p; }
+    static __device__ __forceinline__ void store(float *p, float v) { *p = v; }
+};
+template <> struct Elem<bf16_t> {
+    static __device__ __forceinline__ float load(const bf16_t *p) { return bf16_bits_to_float(p->v); }
+    static __device__ __forceinline__ void store(bf16_t *p, float v) { p->v = (uint16_t)float_to_bf16_bits(v); }
+};
+template <> struct Elem<f16_t> {
+    static __device__ __forceinline__ float load(const f16_t *p)
+    {
+        _Float16 hv;
+        __builtin_memcpy(&hv, &p->v, 2);
+        return (float)hv;
+    }
+    static __device__ __forceinline__ void store(f16_t *p, float v)
+    {
+        _Float16 hv = (_Float16)v;
+        __builtin_memcpy(&p->v, &hv, 2);
+    }
+};
+
+// ---- launch descriptors shared by host dispatch and kernels --------------------------
+struct Dims {
+    int64_t bs, L;
+    int32_t g, dg, hl;
+    int64_t d; // g * dg
+};
+
+constexpr int kWave = 64;
+
+} // namespace gcg
+
+// Host-side launchers, one translation unit per kernel family.  Each returns a
+// hipError_t as int; none of them allocates or synchronises.
+namespace gcg {
+
+int direct_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h,
+                      void *y, void *y2, void *bx, const Dims &dm, hipStream_t st);
+size_t direct_bwd_workspace(const Dims &dm);
+int direct_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C,
+                      const void *h, void *dx, void *dB, void *dC, void *dh, void *ws,
+                      const Dims &dm, hipStream_t st);
+
+bool window_supported(const Dims &dm);
+int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h,
+                      void *y, void *y2, void *bx, const Dims &dm, hipStream_t st);
+size_t window_bwd_workspace(const Dims &dm);
+int window_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C,
+                      const void *h, void *dx, void *dB, void *dC, void *dh, void *ws,
+                      const Dims &dm, hipStream_t st);
+
+bool mfma_supported(int dtype, const Dims &dm);
+int mfma_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h,
+                    void *y, void *y2, void *bx, const Dims &dm, hipStream_t st);
+size_t mfma_bwd_workspace(const Dims &dm);
+int mfma_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C,
+                    const void *h, void *dx, void *dB, void *dC, void *dh, void *ws,
+                    const Dims &dm, hipStream_t st);
+
+} // namespace gcg

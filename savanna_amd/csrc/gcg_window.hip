@@ -1,0 +1,399 @@
+// Register sliding-window kernels for short filters (hl <= 8, Hyena-SE).
+//
+// At 7 taps the operator moves 8 bytes per output for 14 flops, far below the
+// machine balance, so there is nothing for the matrix cores to do: each lane owns
+// V adjacent channels (one vector load per row) and walks a run of time rows,
+// keeping the last 8 rows of the pre-gate product (and, in the backward, of the
+// gated upstream gradient and the raw x / B rows) in a register ring whose slot
+// indices are compile-time after unrolling by 8.  Adjacent lanes take adjacent
+// channel vectors, so every row access of a wave is one contiguous segment.
+#include "gcg_common.h"
+
+namespace gcg {
+namespace {
+
+constexpr int RING = 8;
+
+template <typename T, int V> struct Vec;
+template <> struct Vec<float, 4> { typedef float4 raw; };
+template <> struct Vec<bf16_t, 4> { typedef uint2 raw; };
+template <> struct Vec<f16_t, 4> { typedef uint2 raw; };
+
+template <typename T> __device__ __forceinline__ void unpack4(const typename Vec<T, 4>::raw &r, float (&f)[4]);
+template <> __device__ __forceinline__ void unpack4<float>(const float4 &r, float (&f)[4])
+{
+    f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w;
+}
+template <> __device__ __forceinline__ void unpack4<bf16_t>(const uint2 &r, float (&f)[4])
+{
+    f[0] = __uint_as_float(r.x << 16); f[1] = __uint_as_float(r.x & 0xffff0000u);
+    f[2] = __uint_as_float(r.y << 16); f[3] = __uint_as_float(r.y & 0xffff0000u);
+}
+template <> __device__ __forceinline__ void unpack4<f16_t>(const uint2 &r, float (&f)[4])
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 a, b;
+    __builtin_memcpy(&a, &r.x, 4);
+    __builtin_memcpy(&b, &r.y, 4);
+    f[0] = (float)a[0]; f[1] = (float)a[1]; f[2] = (float)b[0]; f[3] = (float)b[1];
+}
+
+template <typename T> __device__ __forceinline__ typename Vec<T, 4>::raw pack4(const float (&f)[4]);
+template <> __device__ __forceinline__ float4 pack4<float>(const float (&f)[4])
+{
+    return make_float4(f[0], f[1], f[2], f[3]);
+}
+template <> __device__ __forceinline__ uint2 pack4<bf16_t>(const float (&f)[4])
+{
+    uint2 r;
+    r.x = float_to_bf16_bits(f[0]) | (float_to_bf16_bits(f[1]) << 16);
+    r.y = float_to_bf16_bits(f[2]) | (float_to_bf16_bits(f[3]) << 16);
+    return r;
+}
+template <> __device__ __forceinline__ uint2 pack4<f16_t>(const float (&f)[4])
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 a = {(_Float16)f[0], (_Float16)f[1]}, b = {(_Float16)f[2], (_Float16)f[3]};
+    uint2 r;
+    __builtin_memcpy(&r.x, &a, 4);
+    __builtin_memcpy(&r.y, &b, 4);
+    return r;
+}
+
+template <typename T> __device__ __forceinline__ typename Vec<T, 4>::raw zero_raw();
+template <> __device__ __forceinline__ float4 zero_raw<float>() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+template <> __device__ __forceinline__ uint2 zero_raw<bf16_t>() { return make_uint2(0u, 0u); }
+template <> __device__ __forceinline__ uint2 zero_raw<f16_t>() { return make_uint2(0u, 0u); }
+
+struct WinPlan { int nvec, nseg, ts; int64_t nthreads; };
+
+constexpr int V = 4;
+
+// ---------------------------------------------------------------------------- forward
+template <typename T, int HL>
+__global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x, const T *__restrict__ B,
+                                                         const T *__restrict__ C, const T *__restrict__ h,
+                                                         T *__restrict__ y, T *__restrict__ y2,
+                                                         T *__restrict__ bx, Dims dm, WinPlan pl)
+{
+    typedef typename Vec<T, V>::raw raw_t;
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= pl.nthreads) return;
+    const int cv = (int)(gid % pl.nvec);
+    const int seg = (int)((gid / pl.nvec) % pl.nseg);
+    const int64_t b = gid / ((int64_t)pl.nvec * pl.nseg);
+    const int64_t L = dm.L, d = dm.d;
+    const int64_t c = (int64_t)cv * V;
+    const int hl = dm.hl;
+    const T *hg = h + (c / dm.dg) * hl;
+
+    float hr[HL];  // hr[j] multiplies the sample j rows in the past
+#pragma unroll
+    for (int j = 0; j < HL; ++j) hr[j] = (j < hl) ? Elem<T>::load(hg + hl - 1 - j) : 0.f;
+
+    const int64_t t_start = (int64_t)seg * pl.ts;
+    const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
+    const int64_t base = b * L * d + c;
+
+    float ring[RING][V];
+#pragma unroll
+    for (int s = 0; s < RING; ++s)
+#pragma unroll
+        for (int v = 0; v < V; ++v) ring[s][v] = 0.f;
+    // halo: rows t_start-(HL-1) .. t_start-1 go to slots (t & 7); t_start is a multiple of 8
+#pragma unroll
+    for (int i = 1; i < HL; ++i) {
+        const int64_t t = t_start - i;
+        if (t >= 0) {
+            float xf[V], Bf[V];
+            unpack4<T>(*(const raw_t *)(x + base + t * d), xf);
+            unpack4<T>(*(const raw_t *)(B + base + t * d), Bf);
+#pragma unroll
+            for (int v = 0; v < V; ++v) ring[RING - i][v] = xf[v] * Bf[v];
+        }
+    }
+
+    for (int64_t tb = t_start; tb < t_end; tb += RING) {
+        raw_t xr[RING], Br[RING], Cr[RING];
+#pragma unroll
+        for (int k = 0; k < RING; ++k) {
+            const int64_t t = tb + k;
+            if (t < t_end) {
+                xr[k] = *(const raw_t *)(x + base + t * d);
+                Br[k] = *(const raw_t *)(B + base + t * d);
+                Cr[k] = *(const raw_t *)(C + base + t * d);
+            } else {
+                xr[k] = zero_raw<T>(); Br[k] = zero_raw<T>(); Cr[k] = zero_raw<T>();
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < RING; ++k) {
+            const int64_t t = tb + k;
+            float xf[V], Bf[V], Cf[V], acc[V], out[V];
+            unpack4<T>(xr[k], xf);
+            unpack4<T>(Br[k], Bf);
+            unpack4<T>(Cr[k], Cf);
+#pragma unroll
+            for (int v = 0; v < V; ++v) { ring[k][v] = xf[v] * Bf[v]; acc[v] = 0.f; }
+#pragma unroll
+            for (int j = HL - 1; j >= 0; --j)
+#pragma unroll
+                for (int v = 0; v < V; ++v) acc[v] = fmaf(hr[j], ring[(k - j) & (RING - 1)][v], acc[v]);
+            if (t < t_end) {
+                if (y2) *(raw_t *)(y2 + base + t * d) = pack4<T>(acc);
+                if (bx) *(raw_t *)(bx + base + t * d) = pack4<T>(ring[k]);
+#pragma unroll
+                for (int v = 0; v < V; ++v) out[v] = Cf[v] * acc[v];
+                *(raw_t *)(y + base + t * d) = pack4<T>(out);
+            }
+        }
+    }
+}
+
+// --------------------------------------------------------------------------- backward
+// Per lane: rows [t_start, t_end).  Row r is loaded at step r; dC[r] and the dh terms
+// of row r are produced at once (they look back), du[r-(HL-1)] is produced at step r
+// (it looks forward), so the walk runs HL-1 rows past t_end reading only dy and C.
+template <typename T, int HL>
+__global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x,
+                                                         const T *__restrict__ B, const T *__restrict__ C,
+                                                         const T *__restrict__ h, T *__restrict__ dx,
+                                                         T *__restrict__ dB, T *__restrict__ dC,
+                                                         float *__restrict__ ws, Dims dm, WinPlan pl)
+{
+    typedef typename Vec<T, V>::raw raw_t;
+    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (gid >= pl.nthreads) return;
+    const int cv = (int)(gid % pl.nvec);
+    const int seg = (int)((gid / pl.nvec) % pl.nseg);
+    const int64_t b = gid / ((int64_t)pl.nvec * pl.nseg);
+    const int64_t L = dm.L, d = dm.d;
+    const int64_t c = (int64_t)cv * V;
+    const int hl = dm.hl;
+    const T *hg = h + (c / dm.dg) * hl;
+
+    float hr[HL];
+#pragma unroll
+    for (int j = 0; j < HL; ++j) hr[j] = (j < hl) ? Elem<T>::load(hg + hl - 1 - j) : 0.f;
+
+    const int64_t t_start = (int64_t)seg * pl.ts;
+    const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
+    const int64_t base = b * L * d + c;
+
+    float ur[RING][V], gr[RING][V], dha[HL];
+    raw_t xs[RING], Bs[RING];
+#pragma unroll
+    for (int s = 0; s < RING; ++s) {
+        xs[s] = zero_raw<T>(); Bs[s] = zero_raw<T>();
+#pragma unroll
+        for (int v = 0; v < V; ++v) { ur[s][v] = 0.f; gr[s][v] = 0.f; }
+    }
+#pragma unroll
+    for (int j = 0; j < HL; ++j) dha[j] = 0.f;
+#pragma unroll
+    for (int i = 1; i < HL; ++i) {
+        const int64_t t = t_start - i;
+        if (t >= 0) {
+            float xf[V], Bf[V];
+            unpack4<T>(*(const raw_t *)(x + base + t * d), xf);
+            unpack4<T>(*(const raw_t *)(B + base + t * d), Bf);
+#pragma unroll
+            for (int v = 0; v < V; ++v) ur[RING - i][v] = xf[v] * Bf[v];
+        }
+    }
+
+    const int64_t t_stop = t_end + (HL - 1);  // exclusive bound of the walk
+    for (int64_t tb = t_start; tb < t_stop; tb += RING) {
+        raw_t dyr[RING], Cr[RING];
+#pragma unroll
+        for (int k = 0; k < RING; ++k) {
+            const int64_t t = tb + k;
+            if (t < t_end) {
+                xs[k] = *(const raw_t *)(x + base + t * d);
+                Bs[k] = *(const raw_t *)(B + base + t * d);
+            }
+            if (t < L && t < t_stop) {
+                dyr[k] = *(const raw_t *)(dy + base + t * d);
+                Cr[k] = *(const raw_t *)(C + base + t * d);
+            } else {
+                dyr[k] = zero_raw<T>(); Cr[k] = zero_raw<T>();
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < RING; ++k) {
+            const int64_t t = tb + k;
+            float dyf[V], Cf[V];
+            unpack4<T>(dyr[k], dyf);
+            unpack4<T>(Cr[k], Cf);
+#pragma unroll
+            for (int v = 0; v < V; ++v) gr[k][v] = dyf[v] * Cf[v];
+            if (t < t_end) {
+                float xf[V], Bf[V], y2v[V], o[V];
+                unpack4<T>(xs[k], xf);
+                unpack4<T>(Bs[k], Bf);
+#pragma unroll
+                for (int v = 0; v < V; ++v) { ur[k][v] = xf[v] * Bf[v]; y2v[v] = 0.f; }
+#pragma unroll
+                for (int j = HL - 1; j >= 0; --j) {
+                    float s = 0.f;
+#pragma unroll
+                    for (int v = 0; v < V; ++v) {
+                        const float u = ur[(k - j) & (RING - 1)][v];
+                        y2v[v] = fmaf(hr[j], u, y2v[v]);
+                        s = fmaf(gr[k][v], u, s);
+                    }
+                    dha[j] += s;
+                }
+#pragma unroll
+                for (int v = 0; v < V; ++v) o[v] = dyf[v] * y2v[v];
+                *(raw_t *)(dC + base + t * d) = pack4<T>(o);
+            }
+            // du for row t-(HL-1): sum_j hr[j] * g2[row + j]
+            const int64_t orow = t - (HL - 1);
+            if (orow >= t_start && orow < t_end) {
+                float du[V], xf[V], Bf[V], o[V];
+#pragma unroll
+                for (int v = 0; v < V; ++v) du[v] = 0.f;
+#pragma unroll
+                for (int j = 0; j < HL; ++j)
+#pragma unroll
+                    for (int v = 0; v < V; ++v)
+                        du[v] = fmaf(hr[j], gr[(k - (HL - 1) + j) & (RING - 1)][v], du[v]);
+                unpack4<T>(xs[(k - (HL - 1)) & (RING - 1)], xf);
+                unpack4<T>(Bs[(k - (HL - 1)) & (RING - 1)], Bf);
+#pragma unroll
+                for (int v = 0; v < V; ++v) o[v] = du[v] * Bf[v];
+                *(raw_t *)(dx + base + orow * d) = pack4<T>(o);
+#pragma unroll
+                for (int v = 0; v < V; ++v) o[v] = du[v] * xf[v];
+                *(raw_t *)(dB + base + orow * d) = pack4<T>(o);
+            }
+        }
+    }
+    // per-lane filter-gradient partials, tap-major so the reducer reads rows
+    float *slot = ws + gid;
+#pragma unroll
+    for (int j = 0; j < HL; ++j)
+        if (j < hl) slot[(size_t)(hl - 1 - j) * pl.nthreads] = dha[j];
+}
+
+// One workgroup per (group, tap): fixed-order strided sums, then a fixed LDS tree.
+template <typename T>
+__global__ __launch_bounds__(256) void window_dh_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dh,
+                                                               Dims dm, WinPlan pl)
+{
+    __shared__ float red[256];
+    const int grp = blockIdx.x / dm.hl, k = blockIdx.x % dm.hl;
+    const int lpg = dm.dg / V;                       // lanes (channel vectors) per group
+    const int64_t nrow = dm.bs * pl.nseg;            // (batch, segment) pairs
+    const int64_t nterm = nrow * lpg;
+    const float *src = ws + (size_t)k * pl.nthreads;
+    float s = 0.f;
+    for (int64_t i = threadIdx.x; i < nterm; i += 256) {
+        const int64_t row = i / lpg, l = i % lpg;
+        s += src[row * pl.nvec + (int64_t)grp * lpg + l];
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int w = 128; w > 0; w >>= 1) {
+        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) Elem<T>::store(dh + (size_t)grp * dm.hl + k, red[0]);
+}
+
+WinPlan plan(const Dims &dm)
+{
+    WinPlan p;
+    p.nvec = (int)(dm.d / V);
+    p.ts = 128;
+    // shorter runs when the problem is too small to fill the chip with 128-row runs
+    while (p.ts > 16 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 256 * 1024) p.ts >>= 1;
+    p.nseg = (int)((dm.L + p.ts - 1) / p.ts);
+    p.nthreads = dm.bs * p.nseg * p.nvec;
+    return p;
+}
+
+template <typename T, int HL>
+int fwd_t(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
+          const Dims &dm, hipStream_t st)
+{
+    const WinPlan p = plan(dm);
+    const int64_t nwg = (p.nthreads + 255) / 256;
+    if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((window_fwd_kernel<T, HL>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)x,
+                       (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+    return (int)hipGetLastError();
+}
+
+template <typename T, int HL>
+int bwd_t(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
+          void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
+{
+    const WinPlan p = plan(dm);
+    const int64_t nwg = (p.nthreads + 255) / 256;
+    if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((window_bwd_kernel<T, HL>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)dy,
+                       (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
+                       (float *)ws, dm, p);
+    int e = (int)hipGetLastError();
+    if (e) return e;
+    hipLaunchKernelGGL(window_dh_reduce_kernel<T>, dim3((unsigned)(dm.g * dm.hl)), dim3(256), 0, st,
+                       (const float *)ws, (T *)dh, dm, p);
+    return (int)hipGetLastError();
+}
+
+template <typename T>
+int fwd_hl(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
+           const Dims &dm, hipStream_t st)
+{
+    if (dm.hl <= 4) return fwd_t<T, 4>(x, B, C, h, y, y2, bx, dm, st);
+    if (dm.hl <= 7) return fwd_t<T, 7>(x, B, C, h, y, y2, bx, dm, st);
+    return fwd_t<T, 8>(x, B, C, h, y, y2, bx, dm, st);
+}
+
+template <typename T>
+int bwd_hl(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
+           void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
+{
+    if (dm.hl <= 4) return bwd_t<T, 4>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    if (dm.hl <= 7) return bwd_t<T, 7>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    return bwd_t<T, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+}
+
+} // namespace
+
+bool window_supported(const Dims &dm)
+{
+    return dm.hl <= RING && dm.dg % V == 0 && (int64_t)dm.g * dm.hl <= 0x7fffffffLL;
+}
+
+int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h, void *y,
+                      void *y2, void *bx, const Dims &dm, hipStream_t st)
+{
+    switch (dtype) {
+    case GCG_F32:  return fwd_hl<float>(x, B, C, h, y, y2, bx, dm, st);
+    case GCG_BF16: return fwd_hl<bf16_t>(x, B, C, h, y, y2, bx, dm, st);
+    case GCG_F16:  return fwd_hl<f16_t>(x, B, C, h, y, y2, bx, dm, st);
+    }
+    return (int)hipErrorInvalidValue;
+}
+
+size_t window_bwd_workspace(const Dims &dm)
+{
+    const WinPlan p = plan(dm);
+    return (size_t)p.nthreads * dm.hl * sizeof(float);
+}
+
+int window_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C, const void *h,
+                      void *dx, void *dB, void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
+{
+    switch (dtype) {
+    case GCG_F32:  return bwd_hl<float>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    case GCG_BF16: return bwd_hl<bf16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    case GCG_F16:  return bwd_hl<f16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    }
+    return (int)hipErrorInvalidValue;
+}
+
+} // namespace gcg

@@ -1,0 +1,125 @@
+"""Synthetic workloads: the five benchmark configurations and their input recipe.
+
+Naming: the workload descriptions speak of q, k (pre-gate pair) and v (post-gate);
+the kernel arguments are B = q, x = k, C = v  (y = v * conv(q * k, h)).
+
+Inputs are drawn on the CPU from ``torch.Generator().manual_seed(seed)`` in fp32 in the
+fixed order q, k, v, filter noise w, filter decay a, dy, then cast and copied, so a
+CPU checker and the GPU see bit-identical values.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class Workload:
+    name: str
+    bs: int
+    L: int
+    g: int
+    dg: int
+    filters: Tuple[int, ...]      # filter lengths of the ops applied in sequence
+    dtype: torch.dtype
+    backward: bool
+    about: str
+
+    @property
+    def d(self) -> int:
+        return self.g * self.dg
+
+    @property
+    def tokens(self) -> int:
+        return self.bs * self.L
+
+    @property
+    def elem_bytes(self) -> int:
+        return torch.empty((), dtype=self.dtype).element_size()
+
+    def algorithmic_bytes(self) -> int:
+        """Compulsory HBM traffic of one pass: forward reads q, k, v and writes y (4
+        tensors); forward+backward adds reads of dy, q, k, v and writes of dq, dk, dv
+        (11 tensors).  Filter and filter-gradient traffic (<= 256 KB) is not counted."""
+        per_op = 11 if self.backward else 4
+        return per_op * self.bs * self.L * self.d * self.elem_bytes * len(self.filters)
+
+    def algorithmic_flops(self) -> int:
+        """2*bs*L*hl*d per convolution pass, three passes for forward+backward
+        (savanna/mfu.py:423-431, :113-124)."""
+        passes = 3 if self.backward else 1
+        return sum(2 * self.bs * self.L * hl * self.d * passes for hl in self.filters)
+
+
+WORKLOADS = {
+    "se_fwd_fp32": Workload("se_fwd_fp32", 1, 2048, 16, 16, (7,), torch.float32, False,
+                            "Hyena-SE forward, fp32, B=1 L=2048 D=256 G=16 hl=7"),
+    "mr_fwd_7b": Workload("mr_fwd_7b", 2, 8192, 256, 16, (128,), torch.bfloat16, False,
+                          "Hyena-MR forward, bf16, Evo2-7B layer shape B=2 L=8192 D=4096 G=256 hl=128"),
+    "mr_fwdbwd_7b": Workload("mr_fwdbwd_7b", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
+                             "Hyena-MR forward+backward, bf16, Evo2-7B layer shape B=2 L=8192 D=4096 G=256 hl=128"),
+    "se_mr_fwdbwd_40b": Workload("se_mr_fwdbwd_40b", 1, 32768, 512, 16, (7, 128), torch.bfloat16, True,
+                                 "Hyena-SE then Hyena-MR forward+backward, bf16, B=1 L=32768 D=8192 G=512"),
+    "mr_fwd_1m": Workload("mr_fwd_1m", 1, 1048576, 256, 16, (128,), torch.bfloat16, False,
+                          "Hyena-MR forward, bf16, B=1 L=1048576 D=4096 G=256 hl=128"),
+}
+# order of BASELINE.json's `configs`
+WORKLOAD_ORDER = ("se_fwd_fp32", "mr_fwd_7b", "mr_fwdbwd_7b", "se_mr_fwdbwd_40b", "mr_fwd_1m")
+
+
+def se_filter(g: int, hl: int, gen: torch.Generator) -> torch.Tensor:
+    """Short explicit filter: h ~ N(0, 1/hl), shape (g, 1, hl), fp32."""
+    return torch.randn(g, 1, hl, generator=gen) / math.sqrt(hl)
+
+
+def mr_filter(g: int, hl: int, gen: torch.Generator) -> torch.Tensor:
+    """Medium explicit filter with exponential decay: h[g,t] = w[g,t] * exp(-a_g * t),
+    w ~ N(0, 1/hl), a_g log-uniform in [1e-3, 1e-1]; shape (g, 1, hl), fp32.
+    Same family as ExplicitSingleDecayFilter
+    (savanna/model/operators/hyena/parametrization/explicit.py:40-75)."""
+    w = torch.randn(g, hl, generator=gen) / math.sqrt(hl)
+    lo, hi = math.log(1e-3), math.log(1e-1)
+    a = torch.exp(lo + (hi - lo) * torch.rand(g, generator=gen))
+    t = torch.arange(hl, dtype=torch.float32)
+    return (w * torch.exp(-a[:, None] * t[None, :])).unsqueeze(1)
+
+
+def make_inputs(bs: int, L: int, g: int, dg: int, hl: int, dtype: torch.dtype, seed: int = 0,
+                decay: Optional[bool] = None, device="cpu", with_dy: bool = True):
+    """Returns dict(q, k, v, h, dy) of tensors in ``dtype`` on ``device``.
+
+    ``decay``: True = mr_filter, False = se_filter, None = by length (hl > 8 decays).
+    """
+    gen = torch.Generator().manual_seed(seed)
+    shape = (bs, L, g, dg)
+    q = torch.randn(shape, generator=gen)
+    k = torch.randn(shape, generator=gen)
+    v = torch.randn(shape, generator=gen)
+    use_decay = (hl > 8) if decay is None else decay
+    h = mr_filter(g, hl, gen) if use_decay else se_filter(g, hl, gen)
+    out = {"q": q, "k": k, "v": v, "h": h}
+    if with_dy:
+        out["dy"] = torch.randn(shape, generator=gen)
+    return {n: t.to(dtype).to(device) for n, t in out.items()}
+
+
+def make_inputs_device(bs: int, L: int, g: int, dg: int, hl: int, dtype: torch.dtype, device,
+                       seed: int = 0, with_dy: bool = True, slab_rows: int = 65536):
+    """Same distributions generated on the device in time slabs, for shapes too large
+    to stage through host memory (the 2^32-element case).  Values differ from
+    make_inputs; a slab is reproducible from (seed, slab index)."""
+    names = ["q", "k", "v"] + (["dy"] if with_dy else [])
+    out = {n: torch.empty((bs, L, g, dg), dtype=dtype, device=device) for n in names}
+    gen = torch.Generator(device=device)
+    for i, n in enumerate(names):
+        for s, t0 in enumerate(range(0, L, slab_rows)):
+            t1 = min(L, t0 + slab_rows)
+            gen.manual_seed(seed * 1000003 + i * 10007 + s)
+            out[n][:, t0:t1].normal_(generator=gen)
+    hgen = torch.Generator().manual_seed(seed)
+    h = mr_filter(g, hl, hgen) if hl > 8 else se_filter(g, hl, hgen)
+    out["h"] = h.to(dtype).to(device)
+    return out

@@ -1,0 +1,102 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C ABI (ctypes binding in
+savanna_amd/_lib.py).  Modelled on the reference's tests/test_fwd_refactor.py:53-114 and
+tests/test_bwd_refactor.py:70-143: same quantities (Bx, y2, y; dx, dB, dC, dh), same
+parameter grid style, seeded CPU inputs so checker and kernel see identical values.
+"""
+import pytest
+import torch
+
+from helpers import TOL, TOL_DH, assert_close, inputs, oracle_bwd, oracle_fwd
+from savanna_amd import _lib
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def algos_for(hl, dg, dtype):
+    out = ["direct"]
+    if hl <= 8 and dg % 4 == 0:
+        out.append("window")
+    if hl <= 128 and dg % 16 == 0 and dtype != torch.float32:
+        out.append("mfma")
+    return out
+
+
+# (bs, L, g, dg, hl): ragged lengths, partial channel tiles, one-tap and full-length filters
+SMALL = [
+    (1, 32, 1, 16, 4),
+    (2, 32, 2, 32, 4),       # the reference's debug configs (tests/test_fwd_refactor.py:33-36)
+    (2, 128, 2, 16, 128),
+    (1, 256, 4, 16, 128),
+    (2, 300, 3, 16, 128),    # L not a multiple of the chunk
+    (1, 1000, 5, 16, 100),   # filter shorter than the chunk, d = 80 (partial 64-channel tile)
+    (1, 513, 2, 48, 33),
+    (2, 200, 4, 16, 7),
+    (1, 77, 8, 4, 7),        # dg below the matrix-core width
+    (3, 130, 2, 20, 3),
+    (1, 64, 6, 1, 5),        # one channel per filter
+    (1, 70, 2, 24, 1),       # single tap
+    (1, 400, 1, 64, 8),
+    (1, 700, 2, 16, 200),    # filter longer than a chunk (direct kernel only)
+]
+
+
+def _cases():
+    for shape in SMALL:
+        bs, L, g, dg, hl = shape
+        for dtype in DTYPES:
+            for algo in algos_for(hl, dg, dtype):
+                yield pytest.param(*shape, dtype, algo, id=f"{bs}x{L}x{g}x{dg}-hl{hl}-{str(dtype)[6:]}-{algo}")
+
+
+@pytest.mark.parametrize("bs,L,g,dg,hl,dtype,algo", list(_cases()))
+def test_fwd_small(gcg_lib, bs, L, g, dg, hl, dtype, algo):
+    x, B, C, h, _ = inputs(bs, L, g, dg, hl, dtype)
+    bx_ref, y2_ref, y_ref = oracle_fwd(x, B, C, h)
+    bx, y2, y = _lib.fwd(x.to(DEV), B.to(DEV), C.to(DEV), h.to(DEV), return_bx=True, return_y2=True, algo=algo)
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and y.shape == (bs, L, g, dg)
+    assert_close(bx, bx_ref, TOL[dtype], "Bx")
+    assert_close(y2, y2_ref, TOL[dtype], "y2")
+    assert_close(y, y_ref, TOL[dtype], "y")
+    # outputs that were not requested must not be needed
+    _, _, y_only = _lib.fwd(x.to(DEV), B.to(DEV), C.to(DEV), h.to(DEV), algo=algo)
+    assert torch.equal(y_only, y)
+
+
+@pytest.mark.parametrize("bs,L,g,dg,hl,dtype,algo", list(_cases()))
+def test_bwd_small(gcg_lib, bs, L, g, dg, hl, dtype, algo):
+    x, B, C, h, dy = inputs(bs, L, g, dg, hl, dtype, seed=1, dy_scale=0.1)  # dy = 0.1*randn as in test_bwd_refactor.py:98
+    ref = oracle_bwd(dy, x, B, C, h)
+    got = _lib.bwd(dy.to(DEV), x.to(DEV), B.to(DEV), C.to(DEV), h.to(DEV), algo=algo)
+    torch.cuda.synchronize()
+    for o, r, n in zip(got, ref, ("dx", "dB", "dC", "dh")):
+        assert o.dtype == dtype
+        assert_close(o, r, TOL_DH[dtype] if n == "dh" else TOL[dtype], n)
+
+
+@pytest.mark.parametrize("algo", ["direct", "window"])
+def test_bwd_is_deterministic(gcg_lib, algo):
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(2, 512, 4, 16, 7, torch.float32, seed=3))
+    a = _lib.bwd(dy, x, B, C, h, algo=algo)
+    b = _lib.bwd(dy, x, B, C, h, algo=algo)
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)
+
+
+def test_error_codes(gcg_lib):
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(1, 64, 2, 16, 200, torch.bfloat16))
+    with pytest.raises(_lib.GcgError, match="not supported"):
+        _lib.fwd(x, B, C, h, algo="mfma")        # hl > 128
+    with pytest.raises(_lib.GcgError, match="not supported"):
+        _lib.fwd(x, B, C, h, algo="window")      # hl > 8
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        _lib.fwd(x.cpu(), B.cpu(), C.cpu(), h.cpu())
+    lib = _lib.load()
+    assert lib.gcg_fwd(None, B.data_ptr(), C.data_ptr(), h.data_ptr(), x.data_ptr(), None, None,
+                       1, 64, 2, 16, 200, 1, 0, None) == -1
+    assert lib.gcg_bwd(dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(),
+                       x.data_ptr(), x.data_ptr(), x.data_ptr(), h.data_ptr(), None, 0,
+                       1, 64, 2, 16, 200, 1, 0, None) == -3
