@@ -17,13 +17,34 @@ __device__ __forceinline__ float bf16_bits_to_float(uint32_t lo16)
     return __uint_as_float(lo16 << 16);
 }
 
-// round-to-nearest-even fp32 -> bf16 bit pattern (NaN kept quiet)
+// fp32 -> bf16, round to nearest even; gfx950 has a packed hardware conversion
+// (v_cvt_pk_bf16_f32) that the compiler selects for these casts.
 __device__ __forceinline__ uint32_t float_to_bf16_bits(float f)
 {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+    const __bf16 b = (__bf16)f;
+    uint16_t u;
+    __builtin_memcpy(&u, &b, 2);
+    return u;
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi)
+{
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 r;
+    r[0] = (__bf16)lo;
+    r[1] = (__bf16)hi;
+    uint32_t u;
+    __builtin_memcpy(&u, &r, 4);
+    return u;
+}
+
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 r = {(_Float16)lo, (_Float16)hi};
+    uint32_t u;
+    __builtin_memcpy(&u, &r, 4);
+    return u;
 }
 
 template <typename T> struct Elem;

@@ -46,8 +46,8 @@ template <> __device__ __forceinline__ float4 pack4<float>(const float (&f)[4])
 template <> __device__ __forceinline__ uint2 pack4<bf16_t>(const float (&f)[4])
 {
     uint2 r;
-    r.x = float_to_bf16_bits(f[0]) | (float_to_bf16_bits(f[1]) << 16);
-    r.y = float_to_bf16_bits(f[2]) | (float_to_bf16_bits(f[3]) << 16);
+    r.x = pack_bf16x2(f[0], f[1]);
+    r.y = pack_bf16x2(f[2], f[3]);
     return r;
 }
 template <> __device__ __forceinline__ uint2 pack4<f16_t>(const float (&f)[4])
@@ -204,13 +204,17 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 
     const int64_t t_stop = t_end + (HL - 1);  // exclusive bound of the walk
     for (int64_t tb = t_start; tb < t_stop; tb += RING) {
-        raw_t dyr[RING], Cr[RING];
+        // rows are fetched eight at a time into staging registers; the x / B rings are
+        // only overwritten slot by slot below, after the delayed du row has read them
+        raw_t dyr[RING], Cr[RING], xr[RING], Br[RING];
 #pragma unroll
         for (int k = 0; k < RING; ++k) {
             const int64_t t = tb + k;
             if (t < t_end) {
-                xs[k] = *(const raw_t *)(x + base + t * d);
-                Bs[k] = *(const raw_t *)(B + base + t * d);
+                xr[k] = *(const raw_t *)(x + base + t * d);
+                Br[k] = *(const raw_t *)(B + base + t * d);
+            } else {
+                xr[k] = zero_raw<T>(); Br[k] = zero_raw<T>();
             }
             if (t < L && t < t_stop) {
                 dyr[k] = *(const raw_t *)(dy + base + t * d);
@@ -227,6 +231,8 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
             unpack4<T>(Cr[k], Cf);
 #pragma unroll
             for (int v = 0; v < V; ++v) gr[k][v] = dyf[v] * Cf[v];
+            xs[k] = xr[k];
+            Bs[k] = Br[k];
             if (t < t_end) {
                 float xf[V], Bf[V], y2v[V], o[V];
                 unpack4<T>(xs[k], xf);
