@@ -1,6 +1,7 @@
 // C ABI (include/gcg.h): argument checks, kernel-family selection, launch.
 #include "gcg_common.h"
 
+#include <initializer_list>
 #include <mutex>
 
 namespace {
@@ -34,19 +35,30 @@ int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t 
     return GCG_OK;
 }
 
-int resolve_algo(int algo, int dtype, const gcg::Dims &dm, bool backward)
+// The window and MFMA kernels move 8- and 16-byte vectors and need 16-byte aligned
+// tensors; the direct kernels load element by element and take any alignment.
+int resolve_algo(int algo, int dtype, const gcg::Dims &dm, bool backward, bool aligned16 = true)
 {
-    (void)backward;
+    const bool mfma_ok = aligned16 && gcg::mfma_supported(dtype, dm) && (!backward || gcg::mfma_bwd_available());
     switch (algo) {
     case GCG_ALGO_AUTO:
-        if (gcg::window_supported(dm)) return GCG_ALGO_WINDOW;
-        if (gcg::mfma_supported(dtype, dm)) return GCG_ALGO_MFMA;
+        if (aligned16 && gcg::window_supported(dm)) return GCG_ALGO_WINDOW;
+        if (mfma_ok) return GCG_ALGO_MFMA;
         return GCG_ALGO_DIRECT;
     case GCG_ALGO_DIRECT: return GCG_ALGO_DIRECT;
-    case GCG_ALGO_WINDOW: return gcg::window_supported(dm) ? GCG_ALGO_WINDOW : GCG_ERR_UNSUPPORTED;
-    case GCG_ALGO_MFMA:   return gcg::mfma_supported(dtype, dm) ? GCG_ALGO_MFMA : GCG_ERR_UNSUPPORTED;
+    case GCG_ALGO_WINDOW:
+        return (aligned16 && gcg::window_supported(dm)) ? GCG_ALGO_WINDOW : GCG_ERR_UNSUPPORTED;
+    case GCG_ALGO_MFMA:
+        return mfma_ok ? GCG_ALGO_MFMA : GCG_ERR_UNSUPPORTED;
     }
     return GCG_ERR_BAD_ARG;
+}
+
+bool all_aligned16(std::initializer_list<const void *> ps)
+{
+    for (const void *p : ps)
+        if (p && ((uintptr_t)p & 15)) return false;
+    return true;
 }
 
 int finish(int hip_rc)
@@ -93,7 +105,7 @@ GCG_API int gcg_fwd(const void *x, const void *B, const void *C, const void *h, 
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
     if (rc) return rc;
-    const int a = resolve_algo(algo, dtype, dm, false);
+    const int a = resolve_algo(algo, dtype, dm, false, all_aligned16({x, B, C, y, y2, bx}));
     if (a < 0) return a;
     rc = check_device();
     if (rc) return rc;
@@ -119,6 +131,8 @@ GCG_API size_t gcg_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t
     case GCG_ALGO_MFMA:   n = gcg::mfma_bwd_workspace(dm); break;
     default: return 0;
     }
+    // under AUTO a misaligned tensor reroutes to the direct kernels: size for both
+    if (algo == GCG_ALGO_AUTO && gcg::direct_bwd_workspace(dm) > n) n = gcg::direct_bwd_workspace(dm);
     return (n + 255) & ~(size_t)255;
 }
 
@@ -130,7 +144,7 @@ GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C,
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
     if (rc) return rc;
-    const int a = resolve_algo(algo, dtype, dm, true);
+    const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, x, B, C, dx, dB, dC}));
     if (a < 0) return a;
     const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;

@@ -101,6 +101,7 @@ int window_bwd_launch(int dtype, const void *dy, const void *x, const void *B, c
                       const Dims &dm, hipStream_t st);
 
 bool mfma_supported(int dtype, const Dims &dm);
+bool mfma_bwd_available();
 int mfma_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h,
                     void *y, void *y2, void *bx, const Dims &dm, hipStream_t st);
 size_t mfma_bwd_workspace(const Dims &dm);

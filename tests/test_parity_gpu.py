@@ -13,6 +13,7 @@ pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+MFMA_BWD = False   # the matrix-core backward kernel is not in yet
 
 
 def algos_for(hl, dg, dtype):
@@ -43,11 +44,13 @@ SMALL = [
 ]
 
 
-def _cases():
+def _cases(backward=False):
     for shape in SMALL:
         bs, L, g, dg, hl = shape
         for dtype in DTYPES:
             for algo in algos_for(hl, dg, dtype):
+                if backward and algo == "mfma" and not MFMA_BWD:
+                    continue
                 yield pytest.param(*shape, dtype, algo, id=f"{bs}x{L}x{g}x{dg}-hl{hl}-{str(dtype)[6:]}-{algo}")
 
 
@@ -66,7 +69,7 @@ def test_fwd_small(gcg_lib, bs, L, g, dg, hl, dtype, algo):
     assert torch.equal(y_only, y)
 
 
-@pytest.mark.parametrize("bs,L,g,dg,hl,dtype,algo", list(_cases()))
+@pytest.mark.parametrize("bs,L,g,dg,hl,dtype,algo", list(_cases(backward=True)))
 def test_bwd_small(gcg_lib, bs, L, g, dg, hl, dtype, algo):
     x, B, C, h, dy = inputs(bs, L, g, dg, hl, dtype, seed=1, dy_scale=0.1)  # dy = 0.1*randn as in test_bwd_refactor.py:98
     ref = oracle_bwd(dy, x, B, C, h)
