@@ -1,0 +1,216 @@
+#!/usr/bin/env python3
+"""Benchmark of the gated chunked causal convolution on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+
+A step is one pass of the hot path over one batch of synthetic input that is already
+resident in HBM: forward, plus backward for the forward+backward workloads.  The default
+workload is the one the headline metric is quoted on (Hyena-MR forward+backward at the
+Evo2-7B layer shape).  One JSON line is printed; it carries the whole-job throughput in
+tokens/s, the roofline position of the dominant kernel (algorithmic bytes over the HIP-event
+duration of that launch) and a CPU baseline timed on the host cores in the same run.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+from savanna_amd import _lib  # noqa: E402
+from savanna_amd.synthetic import WORKLOAD_ORDER, WORKLOADS, make_inputs, make_inputs_device  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
+
+
+class Op:
+    """One convolution of a workload with its resident inputs (rotated over `nsets` copies
+    when a single copy would sit in the 256 MB last-level cache)."""
+
+    def __init__(self, wl, hl, device, rotate_bytes=512 << 20):
+        n_in = 5 if wl.backward else 3
+        set_bytes = n_in * wl.bs * wl.L * wl.d * wl.elem_bytes
+        self.nsets = int(max(1, min(64, -(-rotate_bytes // set_bytes))))
+        self.sets = []
+        big = wl.bs * wl.L * wl.d >= (1 << 31)
+        for i in range(self.nsets):
+            if big:
+                t = make_inputs_device(wl.bs, wl.L, wl.g, wl.dg, hl, wl.dtype, device, seed=i,
+                                       with_dy=wl.backward)
+            else:
+                t = make_inputs(wl.bs, wl.L, wl.g, wl.dg, hl, wl.dtype, seed=i, device=device,
+                                with_dy=wl.backward)
+            self.sets.append(t)
+        self.hl = hl
+        self.backward = wl.backward
+        self.i = 0
+        n = wl.bs * wl.L * wl.d * wl.elem_bytes
+        self.fwd_bytes, self.bwd_bytes = 4 * n, 7 * n
+
+    def run(self, ev=None):
+        t = self.sets[self.i % self.nsets]
+        self.i += 1
+        # kernel names: B = q, x = k, C = v
+        if ev is not None and not self.backward:
+            ev[0].record()
+        _, _, y = _lib.fwd(t["k"], t["q"], t["v"], t["h"])
+        if ev is not None and not self.backward:
+            ev[1].record()
+        if self.backward:
+            if ev is not None:
+                ev[0].record()
+            _lib.bwd(t["dy"], t["k"], t["q"], t["v"], t["h"])
+            if ev is not None:
+                ev[1].record()
+        return y
+
+
+def time_workload(wl, device, steps, warmup):
+    ops = [Op(wl, hl, device) for hl in wl.filters]
+    dom = max(range(len(ops)), key=lambda i: ops[i].hl)     # dominant launch: longest filter
+    for _ in range(warmup):
+        for op in ops:
+            op.run()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(steps):
+        for i, op in enumerate(ops):
+            op.run(events[k] if i == dom else None)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / steps
+    kern_ms = sum(a.elapsed_time(b) for a, b in events) / steps
+    op = ops[dom]
+    kern_bytes = op.bwd_bytes if op.backward else op.fwd_bytes
+    kern_name = ("gcg_bwd" if op.backward else "gcg_fwd") + f" hl={op.hl} " + _lib.select_algo(
+        wl.bs, wl.L, wl.g, wl.dg, op.hl, wl.dtype, op.backward)
+    achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
+    res = {
+        "workload": wl.name,
+        "ms_per_step": ms_per_step,
+        "tokens_per_s": wl.tokens / (ms_per_step * 1e-3),
+        "step_gbs": wl.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9,
+        "step_hbm_frac": wl.algorithmic_bytes() / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "step_tflops": wl.algorithmic_flops() / (ms_per_step * 1e-3) / 1e12,
+        "kernel": kern_name,
+        "kernel_ms": kern_ms,
+        "kernel_bytes": kern_bytes,
+        "kernel_gbs": achieved,
+        "kernel_hbm_frac": achieved / HBM_PEAK_GBS,
+        "input_sets": [o.nsets for o in ops],
+    }
+    del ops
+    torch.cuda.empty_cache()
+    return res
+
+
+def cpu_baseline(wl, budget_s=20.0):
+    """The CPU port (oracle/: depthwise F.conv1d formulation + autograd, fp32) timed on this
+    host's cores on a bounded sample of the workload: one batch row and as many whole filter
+    groups as fit the time budget, scaled to full width (the cost is linear in channels)."""
+    import oracle  # the checker, timed here only as the reported baseline
+
+    threads = torch.get_num_threads()
+    hl = max(wl.filters)
+    L = min(wl.L, 8192)
+    g_s = min(wl.g, 32)
+
+    def once(g_use):
+        t = make_inputs(1, L, g_use, wl.dg, hl, torch.float32, seed=0, with_dy=wl.backward)
+        t0 = time.perf_counter()
+        if wl.backward:
+            oracle.gcg_bwd_ref_torch(t["dy"], t["k"], t["q"], t["v"], t["h"], dtype=torch.float32)
+        else:
+            oracle.gcg_fwd_ref_torch(t["k"], t["q"], t["v"], t["h"])
+        return time.perf_counter() - t0
+
+    once(g_s)                                   # warm-up (thread pool, mkldnn primitives)
+    dt = once(g_s)
+    # grow the sample towards the budget, keep at least two timed runs
+    while g_s * 2 <= wl.g and dt * 2 * 3 < budget_s:
+        g_s *= 2
+        dt = once(g_s)
+    dt = min(dt, once(g_s))
+    tokens_per_s = L / dt * (g_s / wl.g) / len(wl.filters)
+    return {
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"1 batch row x {L} tokens x {g_s * wl.dg} of {wl.d} channels, hl={hl}, fp32, "
+                  f"{'fwd+bwd' if wl.backward else 'fwd'}; best of 2; scaled linearly to {wl.d} channels"
+                  + (f" and {len(wl.filters)} ops" if len(wl.filters) > 1 else ""),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="mr_fwdbwd_7b", choices=list(WORKLOADS))
+    ap.add_argument("--all", action="store_true", help="also time the other four configurations")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build is single-GPU; the path has no collective or sharded variant, "
+              "so --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the kernels have no CPU path", file=sys.stderr)
+        sys.exit(3)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    _lib.load()
+
+    wl = WORKLOADS[args.workload]
+    res = time_workload(wl, device, args.steps, args.warmup)
+    line = {
+        "metric": "Hyena-MR fwd+bwd tokens/s and HBM GB/s (% roofline) at 1 MI355X",
+        "value": res["tokens_per_s"],
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": str(wl.dtype).replace("torch.", "").replace("bfloat16", "bf16").replace("float32", "f32"),
+        "data": "synthetic",
+        "config": {"workload": wl.name, "about": wl.about, "bs": wl.bs, "L": wl.L, "d": wl.d, "g": wl.g,
+                   "filters": list(wl.filters), "backward": wl.backward,
+                   "step_algorithmic_bytes": wl.algorithmic_bytes(), "step_gbs": res["step_gbs"],
+                   "step_hbm_frac": res["step_hbm_frac"], "step_tflops": res["step_tflops"],
+                   "step_mfma_frac": res["step_tflops"] / MFMA_BF16_PEAK_TFLOPS},
+        "roofline": {"bound": "hbm", "kernel": res["kernel"], "achieved": res["kernel_gbs"],
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": res["kernel_hbm_frac"],
+                     "kernel_ms": res["kernel_ms"], "algorithmic_bytes": res["kernel_bytes"],
+                     "traffic": None},
+    }
+    if args.all:
+        others = {}
+        for name in WORKLOAD_ORDER:
+            if name == wl.name:
+                continue
+            w = WORKLOADS[name]
+            k = args.steps if w.bs * w.L * w.d < (1 << 30) else max(3, args.steps // 10)
+            others[name] = time_workload(w, device, k, max(2, args.warmup // 2))
+        line["all_configs"] = others
+    if not args.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

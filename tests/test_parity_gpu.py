@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
 DTYPES = [torch.float32, torch.bfloat16, torch.float16]
-MFMA_BWD = False   # the matrix-core backward kernel is not in yet
+MFMA_BWD = True
 
 
 def algos_for(hl, dg, dtype):
