@@ -161,6 +161,9 @@ def main():
     ap.add_argument("--workload", default="mr_fwdbwd_7b", choices=list(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also time the other four configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy three times, so a counter profile of this "
+                         "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build is single-GPU; the path has no collective or sharded variant, "
@@ -207,6 +210,13 @@ def main():
             k = args.steps if w.bs * w.L * w.d < (1 << 30) else max(3, args.steps // 10)
             others[name] = time_workload(w, device, k, max(2, args.warmup // 2))
         line["all_configs"] = others
+    if args.copy_calibration:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device=device)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        line["copy_calibration"] = {"bytes_read": src.numel(), "bytes_written": dst.numel(), "launches": 3}
     if not args.no_cpu:
         line["cpu_baseline"] = cpu_baseline(wl)
     print(json.dumps(line), flush=True)

@@ -91,6 +91,31 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char *p)
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p);
 }
 
+// Streaming accesses: every tensor element is touched once, so loads and stores carry the
+// nontemporal hint (GCG_MFMA_NT=0 at build time turns it off for comparison).
+#ifndef GCG_MFMA_NT
+#define GCG_MFMA_NT 3
+#endif
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <typename T> __device__ __forceinline__ uint4 ldg16(const T *p)
+{
+#if GCG_MFMA_NT & 1
+    const u32x4 v = __builtin_nontemporal_load((const u32x4 *)p);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+#else
+    return *(const uint4 *)p;
+#endif
+}
+template <typename T> __device__ __forceinline__ void stg16(T *p, const uint4 &v)
+{
+#if GCG_MFMA_NT & 2
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (u32x4 *)p);
+#else
+    *(uint4 *)p = v;
+#endif
+}
+
 struct MfmaPlan { int ncb, nseg, steps_per_seg, nw; int64_t nsteps, nwg; };
 
 // Operand tile of the banded Toeplitz matrix at row offset doff = (out time) - (in time) of
@@ -177,9 +202,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
         xo = zero4; Bo = zero4; Co = zero4;
         if (cvalid && t < L) {
             const int64_t o = col + t * d;
-            xo = *(const uint4 *)(x + o);
-            Bo = *(const uint4 *)(B + o);
-            if (s >= s_lo) Co = *(const uint4 *)(C + o);
+            xo = ldg16(x + o);
+            Bo = ldg16(B + o);
+            if (s >= s_lo) Co = ldg16(C + o);
         }
     };
     fetch(s_first, xr, Br, Cr);
@@ -202,7 +227,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                 *(uint4 *)u_wr = up;
                 const int64_t t = s * STEP + row_in_step;
                 const bool store_ok = main_step && cvalid && t < L;
-                if (bxo && store_ok) *(uint4 *)(bxo + col + t * d) = up;
+                if (bxo && store_ok) stg16(bxo + col + t * d, up);
                 __syncthreads();
                 {
                     const s16x4 lo = lds_read_tr(u_rd);
@@ -229,8 +254,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                     unpack8<T>(Cr, Cf);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) yf[e] = Cf[e] * y2f[e];
-                    *(uint4 *)(y + col + t * d) = pack8<T>(yf);
-                    if (y2o) *(uint4 *)(y2o + col + t * d) = pack8<T>(y2f);
+                    stg16(y + col + t * d, pack8<T>(yf));
+                    if (y2o) stg16(y2o + col + t * d, pack8<T>(y2f));
                 }
                 xr = xn; Br = Bn; Cr = Cn;
                 ++s;
@@ -349,13 +374,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         if (cvalid) {
             const int64_t t = sg * STEP + r;
             if (t >= 0 && t < L) {
-                xo = *(const uint4 *)(x + col + t * d);
-                Bo = *(const uint4 *)(B + col + t * d);
+                xo = ldg16(x + col + t * d);
+                Bo = ldg16(B + col + t * d);
             }
             const int64_t t2 = t + (NK - 1) * STEP;
             if (t2 >= 0 && t2 < L) {
-                dyo = *(const uint4 *)(dy + col + t2 * d);
-                Co = *(const uint4 *)(C + col + t2 * d);
+                dyo = ldg16(dy + col + t2 * d);
+                Co = ldg16(C + col + t2 * d);
             }
         }
     };
@@ -439,7 +464,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         unpack8<T>(dyq[ph], dyf);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = dyf[e] * y2f[e];
-                        *(uint4 *)(dC + o) = pack8<T>(of);
+                        stg16(dC + o, pack8<T>(of));
                     }
                     {
                         const f32x4 p0 = *(const f32x4 *)d_rd;
@@ -448,10 +473,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         float of[8];
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * Bf[e];
-                        *(uint4 *)(dx + o) = pack8<T>(of);
+                        stg16(dx + o, pack8<T>(of));
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * xf[e];
-                        *(uint4 *)(dB + o) = pack8<T>(of);
+                        stg16(dB + o, pack8<T>(of));
                     }
                 }
                 xr = xn; Br = Bn; dyr = dyn; Cr = Cn;
