@@ -1,0 +1,173 @@
+"""Operator dispatch for the gated convolution: the callers of the kernel boundary.
+
+Counterparts of the ``use_cgcg`` branches of savanna's hyena operators, calling the HIP
+kernels directly:
+
+* ``HyenaMROperator``  <- ParallelHyenaOperator.forward, medium-cgcg branch
+  (savanna/model/operators/hyena/hyena.py:483-535; config built at :270-293)
+* ``HyenaSEOperator``  <- ParallelShortHyenaOperator.forward, cgcg short / mlp branch
+  (hyena.py:795-844; config built at :657-697)
+
+What is reproduced: the argument mapping (x1 -> C post-gate, x2 -> B, v -> x), the round trip
+through ``cgcg_dtype``, the filter shapes ((g, L_cache) explicit decayed filter cut to
+``hyena_mr_len``; (g, 1, hl) short filter), the kernel-config records, and the output reshape
+to (b, l, g*dg).  As in the reference's cgcg branch the convolution is a cross-correlation
+without the ``conv_bias`` skip term (the non-cgcg branches differ, hyena.py:477-478, 544-555).
+Everything model-parallel, context-parallel or FFT-based in those classes is outside this
+path and absent here.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from ..kernels.cgcg.interface import two_pass_chunked_gate_conv_gate
+from ..kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
+
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
+
+
+def get_groups_and_group_sizes(hidden_size: int, num_groups: int, world_size: int = 1, expand_factor: float = 1):
+    """(width per rank, groups per rank, channels per group) as hyena.py:184-188; world_size is
+    1 on this single-GPU path."""
+    assert hidden_size % world_size == 0 and num_groups % world_size == 0
+    width = hidden_size // world_size
+    groups = int(num_groups // world_size * expand_factor)
+    return width, groups, width // groups
+
+
+@dataclass
+class CgcgConfig:
+    """The flags of savanna/arguments/global_config.py that reach this path (:389-523),
+    with the reference's defaults."""
+    cgcg_dtype: str = "float32"                 # global_config.py:404; the 7B configs set "bfloat16"
+    cgcg_fwd_chunk_size: int = 128              # :417-440 (medium) / :445-468 (short): Triton tile knobs
+    cgcg_fwd_block_d: int = 128
+    cgcg_fwd_chunk_tiles_per_program: int = 1
+    cgcg_fwd_threadblock_swizzle: str = "row"
+    cgcg_fwd_num_warps: int = 4
+    cgcg_fwd_num_stages: int = 3
+    cgcg_bwd_autotune: bool = True              # :473
+    cgcg_fused_bwd: bool = True                 # :478
+    cgcg_bwd_pre_conv_block_x: int = 128        # :485-520
+    cgcg_bwd_pre_conv_block_y: int = 128
+    cgcg_bwd_pre_conv_num_warps: int = 8
+    cgcg_bwd_post_conv_block_x: int = 32
+    cgcg_bwd_post_conv_block_y: int = 128
+    cgcg_bwd_post_conv_num_warps: int = 4
+
+    def torch_dtype(self) -> torch.dtype:
+        return _DTYPES[self.cgcg_dtype]
+
+    def fwd_kernel_cfg(self, group_dim: int) -> FwdKernelConfigRefactor:
+        # BLOCK_D = min(group_dim, configured) as hyena.py:279, :664
+        return FwdKernelConfigRefactor(
+            CHUNK_SIZE=self.cgcg_fwd_chunk_size,
+            BLOCK_D=min(group_dim, self.cgcg_fwd_block_d),
+            CHUNK_TILES_PER_PROGRAM=self.cgcg_fwd_chunk_tiles_per_program,
+            THREADBLOCK_SWIZZLE=self.cgcg_fwd_threadblock_swizzle,
+            num_warps=self.cgcg_fwd_num_warps,
+            num_stages=self.cgcg_fwd_num_stages,
+        )
+
+    def bwd_kernel_cfg(self) -> BwdKernelConfigRefactor:
+        return BwdKernelConfigRefactor(
+            pre_conv_BLOCK_X=self.cgcg_bwd_pre_conv_block_x,
+            pre_conv_BLOCK_Y=self.cgcg_bwd_pre_conv_block_y,
+            pre_conv_num_warps=self.cgcg_bwd_pre_conv_num_warps,
+            post_conv_BLOCK_X=self.cgcg_bwd_post_conv_block_x,
+            post_conv_BLOCK_Y=self.cgcg_bwd_post_conv_block_y,
+            post_conv_num_warps=self.cgcg_bwd_post_conv_num_warps,
+        )
+
+
+class ExplicitSingleDecayFilter(nn.Module):
+    """h[g, t] = w[g, t] * exp(-r_g * t / (L_cache - 1)), r_g log-spaced over the groups
+    (savanna/model/operators/hyena/parametrization/explicit.py:15-75, single rank)."""
+
+    PRESETS = {"strong": (0, 2), "normal": (-1, 2), "weak": (-2, 2)}
+
+    def __init__(self, d_model: int, L_cache: int, decay_preset: str = "strong", small_init: bool = True,
+                 unit_passthrough: bool = False, device=None):
+        super().__init__()
+        assert decay_preset in self.PRESETS
+        log_r_min, log_r_max = self.PRESETS[decay_preset]
+        w = torch.randn(d_model, L_cache, device=device) / math.sqrt(L_cache)
+        if small_init:
+            w = w * 1e-5
+        if unit_passthrough:
+            w[:, :1] = 1.0
+        self.h = nn.Parameter(w)
+        t = torch.linspace(0, 1, L_cache, device=device)[None]
+        rates = torch.logspace(log_r_min, log_r_max, d_model, device=device)[:, None]
+        self.register_buffer("decay", torch.exp(-rates * t))
+
+    def forward(self, L: int) -> torch.Tensor:
+        return self.h[:, :L] * self.decay[:, :L]
+
+
+class _CgcgOperatorBase(nn.Module):
+    def __init__(self, hidden_size: int, num_groups: int, cfg: Optional[CgcgConfig]):
+        super().__init__()
+        self.cfg = cfg or CgcgConfig()
+        self.hidden_size, self.num_groups, self.group_dim = get_groups_and_group_sizes(hidden_size, num_groups)
+        self.cgcg_dtype = self.cfg.torch_dtype()
+        self.cgcg_fn = two_pass_chunked_gate_conv_gate
+        self.cgcg_fwd_config = self.cfg.fwd_kernel_cfg(self.group_dim)
+        self.cgcg_bwd_config = self.cfg.bwd_kernel_cfg()
+
+    def _filter(self, L: int) -> torch.Tensor:          # (g, 1, hl)
+        raise NotImplementedError
+
+    def forward(self, x1: torch.Tensor, x2: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+        """x1 (post-gate), x2, v (pre-gate pair): (b, l, g, dg) -> z: (b, l, g*dg)."""
+        dtype = x1.dtype
+        h = self._filter(x1.shape[1])
+        if self.cgcg_dtype != dtype:
+            x, B, C, h = (t.to(self.cgcg_dtype) for t in (v, x2, x1, h))
+        else:
+            x, B, C = v, x2, x1
+        bs, seqlen, g, dg = x.shape
+        z = self.cgcg_fn(
+            x=x, B=B, C=C, h=h, bs=bs, seqlen=seqlen, g=g, dg=dg,
+            fwd_autotune=False,
+            bwd_autotune=self.cfg.cgcg_bwd_autotune,
+            fused_bwd=self.cfg.cgcg_fused_bwd,
+            fwd_kernel_cfg=self.cgcg_fwd_config,
+            bwd_kernel_cfg=None if self.cfg.cgcg_bwd_autotune else self.cgcg_bwd_config,
+        )
+        z = z.reshape(bs, seqlen, g * dg)
+        return z.to(dtype) if self.cgcg_dtype != dtype else z
+
+
+class HyenaMROperator(_CgcgOperatorBase):
+    """Hyena-MR: explicit decayed filter of length ``hyena_mr_len`` (128 in the 7B configs)."""
+
+    def __init__(self, hidden_size: int, num_groups: int, hyena_mr_len: int = 128, cfg: Optional[CgcgConfig] = None,
+                 decay_preset: str = "strong", small_init: bool = True, device=None):
+        super().__init__(hidden_size, num_groups, cfg)
+        self.hyena_mr_len = hyena_mr_len
+        self.filter = ExplicitSingleDecayFilter(self.num_groups, hyena_mr_len, decay_preset=decay_preset,
+                                                small_init=small_init, device=device)
+
+    def _filter(self, L: int) -> torch.Tensor:
+        return self.filter(min(self.hyena_mr_len, L))[:, None]      # hyena.py:440-441, :503
+
+
+class HyenaSEOperator(_CgcgOperatorBase):
+    """Hyena-SE: short explicit filter (g, 1, hl), hl = ``hyena_se_len`` (7 in the 7B configs);
+    initialised uniform(+-sqrt(1/hl)) like short_conv_weight (hyena.py:120-130)."""
+
+    def __init__(self, hidden_size: int, num_groups: int, hyena_se_len: int = 7, cfg: Optional[CgcgConfig] = None,
+                 device=None):
+        super().__init__(hidden_size, num_groups, cfg)
+        bound = math.sqrt(1.0 / hyena_se_len)
+        self.short_conv_weight = nn.Parameter(
+            torch.empty(self.num_groups, 1, hyena_se_len, device=device).uniform_(-bound, bound))
+
+    def _filter(self, L: int) -> torch.Tensor:
+        return self.short_conv_weight

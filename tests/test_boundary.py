@@ -1,0 +1,166 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports exactly what
+include/gcg.h declares, argument errors are reported before anything touches a device, and
+the Python mirrors keep the reference's preconditions (interface.py:148-159, :48-49;
+kernel_utils.py:289-294)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+
+from savanna_amd import _lib, two_pass_chunked_gate_conv_gate
+from savanna_amd.kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
+from savanna_amd.operators import hyena
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "gcg.h")).read()
+    return sorted(set(re.findall(r"GCG_API[^;(]*?\b(gcg_\w+)\s*\(", text)))
+
+
+def test_header_and_library_agree(gcg_lib):
+    want = declared_symbols()
+    assert want == sorted(_lib.EXPORTS), "binding list and header differ"
+    for name in want:
+        assert hasattr(gcg_lib, name), f"{name} not exported"
+    out = subprocess.check_output(["nm", "-D", "--defined-only", _lib.LIB_PATH], text=True)
+    exported = sorted(re.findall(r" T (gcg_\w+)", out))
+    assert exported == want, "library exports symbols the header does not declare (or misses some)"
+
+
+def test_version_and_error_text(gcg_lib):
+    assert gcg_lib.gcg_version() >= 100
+    assert gcg_lib.gcg_strerror(0) == b"ok"
+    for code in (-1, -2, -3, -4, -5):
+        assert len(gcg_lib.gcg_strerror(code)) > 5
+    assert gcg_lib.gcg_strerror(-99) == b"unknown error"
+
+
+def test_argument_errors_need_no_device(gcg_lib):
+    p = ctypes.c_void_p(4096)   # never dereferenced: the calls fail on the checks before any launch
+    # null pointer
+    assert gcg_lib.gcg_fwd(None, p, p, p, p, None, None, 1, 64, 2, 16, 7, 0, 0, None) == -1
+    # non-positive size, unknown dtype, unknown algo
+    assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 0, 2, 16, 7, 0, 0, None) == -1
+    assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 7, 9, 0, None) == -1
+    assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 7, 0, 9, None) == -1
+    # forced family that cannot take the shape
+    assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 200, 1, 3, None) == -2   # mfma, hl > 128
+    assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 128, 0, 3, None) == -2   # mfma, fp32
+    assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 9, 0, 2, None) == -2     # window, hl > 8
+    assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 8, 64, 1, 3, None) == -2     # mfma, dg % 16
+    # backward without workspace
+    assert gcg_lib.gcg_bwd(p, p, p, p, p, p, p, p, p, None, 0, 1, 64, 2, 16, 7, 0, 0, None) == -3
+    assert gcg_lib.gcg_bwd_workspace_bytes(1, 64, 2, 16, 7, 0, 0) > 0
+    assert gcg_lib.gcg_bwd_workspace_bytes(1, 64, 2, 16, 7, 0, 0) % 256 == 0
+    assert gcg_lib.gcg_bwd_workspace_bytes(0, 64, 2, 16, 7, 0, 0) == 0
+
+
+def test_algo_selection(gcg_lib):
+    bf, f32 = torch.bfloat16, torch.float32
+    assert _lib.select_algo(2, 8192, 256, 16, 128, bf) == "mfma"          # Hyena-MR, bf16
+    assert _lib.select_algo(2, 8192, 256, 16, 128, bf, backward=True) == "mfma"
+    assert _lib.select_algo(1, 32768, 512, 16, 7, bf) == "window"         # Hyena-SE
+    assert _lib.select_algo(1, 2048, 16, 16, 7, f32) == "window"          # fp32 SE config
+    assert _lib.select_algo(2, 8192, 256, 16, 128, f32) == "direct"       # fp32 keeps full precision on the VALU
+    assert _lib.select_algo(1, 512, 4, 16, 300, bf) == "direct"           # filter longer than a chunk
+    assert _lib.select_algo(1, 512, 64, 1, 64, bf) == "direct"            # one channel per filter
+
+
+def test_no_cpu_path():
+    x = torch.randn(1, 8, 1, 16)
+    h = torch.randn(1, 1, 3)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        _lib.fwd(x, x, x, h)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        _lib.bwd(x, x, x, x, h)
+    with pytest.raises(TypeError):
+        _lib.dtype_code(torch.float64)
+
+
+def test_interface_preconditions():
+    x = torch.randn(1, 8, 1, 16)
+    h = torch.randn(1, 1, 3)
+    cfg = FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row")
+    with pytest.raises(AssertionError, match="fwd_kernel_cfg"):
+        two_pass_chunked_gate_conv_gate(x, x, x, h, 1, 8, 1, 16)
+    with pytest.raises(AssertionError, match="bwd_kernel_cfg"):
+        two_pass_chunked_gate_conv_gate(x, x, x, h, 1, 8, 1, 16, fwd_kernel_cfg=cfg, bwd_autotune=False)
+    with pytest.raises(AssertionError):   # declared shape must match the tensors
+        two_pass_chunked_gate_conv_gate(x, x, x, h, 1, 9, 1, 16, fwd_kernel_cfg=cfg)
+    with pytest.raises(AssertionError):   # B of another shape
+        two_pass_chunked_gate_conv_gate(x, x[:, :4], x, h, 1, 8, 1, 16, fwd_kernel_cfg=cfg)
+    with pytest.warns(UserWarning, match="Both autotune and fwd_kernel_cfg"):
+        with pytest.raises(RuntimeError, match="no CPU path"):
+            two_pass_chunked_gate_conv_gate(x, x, x, h, 1, 8, 1, 16, fwd_autotune=True, fwd_kernel_cfg=cfg)
+
+
+def test_kernel_config_records():
+    cfg = FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row")
+    assert cfg.schedule == "default" and cfg.RETURN_BX and cfg.RETURN_Y2 and cfg.version == "refactor"
+    assert cfg == FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row")
+    assert hash(cfg) == hash(FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row"))
+    assert "CHUNK_SIZE=128" in str(cfg)
+    with pytest.raises(AssertionError):
+        FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="diag")
+    with pytest.raises(AssertionError):
+        FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row", schedule="streamk")
+    with pytest.raises(AssertionError):
+        FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row", NUM_PIPELINE_STAGES=2)
+    b = BwdKernelConfigRefactor()
+    assert (b.pre_conv_BLOCK_X, b.post_conv_BLOCK_Y, b.name) == (128, 128, "bwd-refactor")
+
+
+class _Spy:
+    """Stands in for the kernel entry point to record how the operator calls it."""
+
+    def __init__(self):
+        self.kw = None
+
+    def __call__(self, **kw):
+        self.kw = kw
+        return torch.zeros_like(kw["x"])
+
+
+def test_operator_argument_mapping():
+    """x1 -> C (post-gate), x2 -> B, v -> x; tensors and filter go through cgcg_dtype and the
+    result comes back in the activation dtype as (b, l, g*dg) (hyena.py:494-534, :807-843)."""
+    b, l, g, dg = 2, 16, 4, 16
+    x1, x2, v = (torch.randn(b, l, g, dg, dtype=torch.bfloat16) for _ in range(3))
+    for op in (hyena.HyenaMROperator(g * dg, g, hyena_mr_len=8, cfg=hyena.CgcgConfig(cgcg_dtype="float32")),
+               hyena.HyenaSEOperator(g * dg, g, hyena_se_len=7, cfg=hyena.CgcgConfig(cgcg_dtype="float32"))):
+        spy = _Spy()
+        op.cgcg_fn = spy
+        z = op(x1, x2, v)
+        kw = spy.kw
+        assert torch.equal(kw["x"], v.float()) and torch.equal(kw["B"], x2.float()) and torch.equal(kw["C"], x1.float())
+        assert kw["h"].dtype == torch.float32 and kw["h"].shape[:2] == (g, 1)
+        assert (kw["bs"], kw["seqlen"], kw["g"], kw["dg"]) == (b, l, g, dg)
+        assert kw["fwd_autotune"] is False and kw["fwd_kernel_cfg"].BLOCK_D == dg
+        assert kw["bwd_kernel_cfg"] is None and kw["bwd_autotune"] is True and kw["fused_bwd"] is True
+        assert z.shape == (b, l, g * dg) and z.dtype == torch.bfloat16
+    # no cast when the activation dtype already is cgcg_dtype
+    op = hyena.HyenaSEOperator(g * dg, g, cfg=hyena.CgcgConfig(cgcg_dtype="bfloat16", cgcg_bwd_autotune=False))
+    op = op.to(torch.bfloat16)
+    spy = _Spy()
+    op.cgcg_fn = spy
+    op(x1, x2, v)
+    assert spy.kw["x"] is v and spy.kw["C"] is x1 and spy.kw["bwd_kernel_cfg"] is not None
+
+
+def test_explicit_filter_recipe():
+    f = hyena.ExplicitSingleDecayFilter(8, 128, decay_preset="strong", small_init=False)
+    h = f(128)
+    assert h.shape == (8, 128)
+    # decay = exp(-r_g * t), t in [0, 1], r_g = logspace(0, 2): first column undamped,
+    # last column damped by exp(-r_g)
+    torch.testing.assert_close(h[:, 0], f.h[:, 0])
+    rates = torch.logspace(0, 2, 8)
+    torch.testing.assert_close(h[:, -1], f.h[:, -1] * torch.exp(-rates))
+    assert f(64).shape == (8, 64)
+    assert hyena.get_groups_and_group_sizes(4096, 256) == (4096, 256, 16)
+    assert hyena.get_groups_and_group_sizes(8192, 512, world_size=8) == (1024, 64, 16)

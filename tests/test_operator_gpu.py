@@ -1,0 +1,80 @@
+"""The drop-in path end to end on the GPU: operator module -> autograd function -> C ABI.
+Mirrors tests/test_bwd_refactor.py:270-369 of the reference (the full
+two_pass_chunked_gate_conv_gate autograd path against autograd of the F.conv1d form)."""
+import pytest
+import torch
+
+import oracle
+from helpers import TOL, TOL_DH, assert_close
+from savanna_amd import two_pass_chunked_gate_conv_gate
+from savanna_amd.kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
+from savanna_amd.operators import hyena
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("hl", [4, 7, 128])
+@pytest.mark.parametrize("fused", [True, False])
+def test_autograd_path(gcg_lib, hl, dtype, fused):
+    bs, L, g, dg = 2, 1024, 8, 16
+    gen = torch.Generator().manual_seed(hl)
+    x, B, C = (torch.randn(bs, L, g, dg, generator=gen).to(dtype) for _ in range(3))
+    h = (torch.randn(g, 1, hl, generator=gen) / hl ** 0.5).to(dtype)
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen)).to(dtype)
+    dev = [t.to(DEV).requires_grad_(True) for t in (x, B, C, h)]
+    cfg = FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row", num_warps=4, num_stages=3)
+    y = two_pass_chunked_gate_conv_gate(*dev, bs, L, g, dg, fwd_autotune=False, bwd_autotune=not fused,
+                                        fused_bwd=fused, fwd_kernel_cfg=cfg,
+                                        bwd_kernel_cfg=BwdKernelConfigRefactor() if fused else None)
+    assert y.shape == (bs, L, g, dg) and y.dtype == dtype
+    y.backward(dy.to(DEV))
+    y_ref = oracle.gcg_fwd_ref_torch(x.double(), B.double(), C.double(), h.double())
+    grads_ref = oracle.gcg_bwd_ref_torch(dy, x, B, C, h)
+    assert_close(y, y_ref, TOL[dtype], "y")
+    for t, r, n in zip(dev, grads_ref, ("dx", "dB", "dC", "dh")):
+        assert t.grad.shape == t.shape and t.grad.dtype == dtype
+        assert_close(t.grad, r, TOL_DH[dtype] if n == "dh" else TOL[dtype], n)
+
+
+def test_non_contiguous_inputs_are_accepted(gcg_lib):
+    """The block hands the operator stride-3 views of the projected features
+    (savanna/model/block.py:886-888); the boundary copies them (interface.py:51-54)."""
+    bs, L, g, dg = 1, 256, 4, 16
+    feats = torch.randn(bs, L, g, 3, dg, device=DEV, dtype=torch.bfloat16)
+    x1, x2, v = feats.unbind(3)
+    assert not x1.is_contiguous()
+    h = torch.randn(g, 1, 7, device=DEV, dtype=torch.bfloat16) * 0.3
+    cfg = FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row")
+    y = two_pass_chunked_gate_conv_gate(v, x2, x1, h, bs, L, g, dg, fwd_kernel_cfg=cfg)
+    ref = oracle.gcg_fwd_oracle(v.float().cpu(), x2.float().cpu(), x1.float().cpu(), h.float().cpu())
+    assert_close(y, ref, 1e-2, "y")
+
+
+@pytest.mark.parametrize("kind", ["mr", "se"])
+def test_operator_modules(gcg_lib, kind):
+    b, l, g, dg = 2, 512, 8, 16
+    gen = torch.Generator().manual_seed(1)
+    x1, x2, v = (torch.randn(b, l, g, dg, generator=gen).to(torch.bfloat16).to(DEV) for _ in range(3))
+    cfg = hyena.CgcgConfig(cgcg_dtype="bfloat16")
+    if kind == "mr":
+        op = hyena.HyenaMROperator(g * dg, g, hyena_mr_len=128, cfg=cfg, small_init=False)
+    else:
+        op = hyena.HyenaSEOperator(g * dg, g, hyena_se_len=7, cfg=cfg)
+    op = op.to(DEV).to(torch.bfloat16)
+    z = op(x1, x2, v)
+    assert z.shape == (b, l, g * dg) and z.dtype == torch.bfloat16
+    h = op._filter(l).detach()
+    ref = oracle.gcg_fwd_oracle(v.float().cpu(), x2.float().cpu(), x1.float().cpu(), h.float().cpu())
+    assert_close(z.reshape(b, l, g, dg), ref, 1e-2, "z")
+    # the pre-gate pair is symmetric: swapping x2 and v changes nothing
+    assert_close(op(x1, v, x2), z.float(), 2e-3, "swap")
+    # gradients reach the filter parameters
+    z.float().square().mean().backward()
+    p = op.filter.h if kind == "mr" else op.short_conv_weight
+    assert p.grad is not None and torch.isfinite(p.grad).all() and p.grad.abs().max() > 0
+    # fp32 kernel dtype under bf16 activations: cast in, cast out (hyena.py:499-503, 533-534)
+    op32 = hyena.HyenaSEOperator(g * dg, g, hyena_se_len=7, cfg=hyena.CgcgConfig(cgcg_dtype="float32")).to(DEV)
+    z32 = op32(x1, x2, v)
+    assert z32.dtype == torch.bfloat16
