@@ -12,7 +12,8 @@ import threading
 import torch
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
-LIB_PATH = os.path.join(_CSRC, "libgcg_hip.so")
+# GCG_HIP_LIB points at another build of the same library (e.g. a tuning variant)
+LIB_PATH = os.environ.get("GCG_HIP_LIB") or os.path.join(_CSRC, "libgcg_hip.so")
 
 GCG_F32, GCG_BF16, GCG_F16 = 0, 1, 2
 ALGO_AUTO, ALGO_DIRECT, ALGO_WINDOW, ALGO_MFMA = 0, 1, 2, 3
