@@ -30,6 +30,14 @@ from savanna_amd.synthetic import WORKLOAD_ORDER, WORKLOADS, make_inputs, make_i
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this script scaled by a 256 MiB copy in the same run (profiles/mr_fwdbwd_7b_hbm_traffic.md).
+# Counters cannot be read from inside the process; configurations without a profile report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("mr_fwdbwd_7b", "gcg_bwd hl=128 mfma"): 935785 * 1024,
+    ("mr_fwd_7b", "gcg_fwd hl=128 mfma"): 537018 * 1024,
+}
+
 
 class Op:
     """One convolution of a workload with its resident inputs (rotated over `nsets` copies
@@ -199,7 +207,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": res["kernel"], "achieved": res["kernel_gbs"],
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": res["kernel_hbm_frac"],
                      "kernel_ms": res["kernel_ms"], "algorithmic_bytes": res["kernel_bytes"],
-                     "traffic": None},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get((wl.name, res["kernel"]))},
     }
     if args.all:
         others = {}

@@ -1,0 +1,121 @@
+// Access-pattern ceilings for the convolution kernels: the same reads and writes, no arithmetic.
+//
+//   ./membench            (built by `make -C savanna_amd/csrc membench`)
+//
+// Prints the HBM rate of (a) flat streams with R reads and W writes per element, plain and
+// nontemporal, and (b) the tile walk the MFMA kernels perform -- a workgroup owns ROWB bytes of
+// every row of a (bs, L, d) bf16 tensor set and walks a run of 32-row steps with a one-step
+// prefetch -- for several row widths, read/write mixes and row strides.  These are the rates the
+// memory system gives the kernels' access pattern; the kernels are compared with them, not
+// only with the 8 TB/s nominal peak.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+
+#define CK(x) do { hipError_t e_ = (x); if (e_ != hipSuccess) { printf("HIP error %s at line %d\n", hipGetErrorString(e_), __LINE__); exit(1); } } while (0)
+
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+
+template <int NT> __device__ __forceinline__ u4 ld(const u4 *p) { return NT ? __builtin_nontemporal_load(p) : *p; }
+template <int NT> __device__ __forceinline__ void st(u4 *p, u4 v) { if (NT) __builtin_nontemporal_store(v, p); else *p = v; }
+
+template <int R, int W, int NT>
+__global__ __launch_bounds__(256) void flat_kernel(const u4 *a, const u4 *b, const u4 *c, const u4 *e, u4 *y, u4 *z, u4 *w, int64_t n)
+{
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        u4 v = ld<NT>(a + i);
+        if (R > 1) v ^= ld<NT>(b + i);
+        if (R > 2) v ^= ld<NT>(c + i);
+        if (R > 3) v ^= ld<NT>(e + i);
+        if (W > 0) st<NT>(y + i, v); else if (v.x == 0x12345678u) y[0] = v;
+        if (W > 1) st<NT>(z + i, v);
+        if (W > 2) st<NT>(w + i, v);
+    }
+}
+
+// THREADS lanes cover (THREADS*16/ROWB) rows of ROWB bytes per step
+template <int THREADS, int ROWB, int R, int W>
+__global__ __launch_bounds__(THREADS) void tile_kernel(const char *a, const char *b, const char *c, const char *e, char *y, char *z, char *w,
+                                                       int64_t L, int64_t rowbytes, int ncb, int nseg, int steps)
+{
+    int64_t id = blockIdx.x;
+    const int cb = id % ncb; id /= ncb;
+    const int seg = id % nseg;
+    const int64_t bb = id / nseg;
+    constexpr int LPR = ROWB / 16, RPS = THREADS / LPR;
+    const int r = threadIdx.x / LPR, l = threadIdx.x % LPR;
+    int64_t o = bb * L * rowbytes + (int64_t)cb * ROWB + l * 16 + ((int64_t)seg * steps * RPS + r) * rowbytes;
+    u4 v0 = ld<1>((const u4 *)(a + o)), v1 = v0, v2 = v0, v3 = v0;
+    if (R > 1) v1 = ld<1>((const u4 *)(b + o));
+    if (R > 2) v2 = ld<1>((const u4 *)(c + o));
+    if (R > 3) v3 = ld<1>((const u4 *)(e + o));
+    for (int s = 0; s < steps; ++s) {
+        const int64_t on = o + (int64_t)RPS * rowbytes;
+        u4 n0 = v0, n1 = v1, n2 = v2, n3 = v3;
+        if (s + 1 < steps) {
+            n0 = ld<1>((const u4 *)(a + on));
+            if (R > 1) n1 = ld<1>((const u4 *)(b + on));
+            if (R > 2) n2 = ld<1>((const u4 *)(c + on));
+            if (R > 3) n3 = ld<1>((const u4 *)(e + on));
+        }
+        const u4 t = v0 ^ v1 ^ v2 ^ v3;
+        st<1>((u4 *)(y + o), t);
+        if (W > 1) st<1>((u4 *)(z + o), t ^ v1);
+        if (W > 2) st<1>((u4 *)(w + o), t ^ v2);
+        v0 = n0; v1 = n1; v2 = n2; v3 = n3; o = on;
+    }
+}
+
+static hipEvent_t e0, e1;
+template <typename F> static void timeit(const char *name, double bytes, F launch)
+{
+    for (int i = 0; i < 3; ++i) launch();
+    CK(hipDeviceSynchronize());
+    float best = 1e9f, tot = 0.f;
+    const int K = 20;
+    for (int i = 0; i < K; ++i) {
+        CK(hipEventRecord(e0)); launch(); CK(hipEventRecord(e1)); CK(hipEventSynchronize(e1));
+        float ms; CK(hipEventElapsedTime(&ms, e0, e1));
+        tot += ms; if (ms < best) best = ms;
+    }
+    printf("%-58s avg %7.1f us  %5.0f GB/s  (best %5.0f)\n", name, tot / K * 1e3, bytes / (tot / K) / 1e6, bytes / best / 1e6);
+    fflush(stdout);
+}
+
+int main()
+{
+    const int64_t bs = 2, L = 8192, d = 4096;            // the Evo2-7B layer shape, bf16
+    CK(hipEventCreate(&e0)); CK(hipEventCreate(&e1));
+    for (int pad = 0; pad < 2; ++pad) {
+        const int64_t rowbytes = d * 2 + (pad ? 256 : 0); // pad = 1: row stride no longer a power of two
+        const int64_t bytes = bs * L * rowbytes;
+        char *p[7];
+        for (int i = 0; i < 7; ++i) { CK(hipMalloc(&p[i], bytes)); CK(hipMemset(p[i], i + 1, bytes)); }
+        const double n1 = (double)bs * L * d * 2;
+        char nm[128];
+        if (!pad) {
+            const int64_t n16 = bytes / 16;
+            u4 **q = (u4 **)p;
+            timeit("flat 1R0W", 1 * n1, [&] { flat_kernel<1, 0, 0><<<8192, 256>>>(q[0], q[1], q[2], q[3], q[4], q[5], q[6], n16); });
+            timeit("flat 1R1W", 2 * n1, [&] { flat_kernel<1, 1, 0><<<8192, 256>>>(q[0], q[1], q[2], q[3], q[4], q[5], q[6], n16); });
+            timeit("flat 1R1W nontemporal", 2 * n1, [&] { flat_kernel<1, 1, 1><<<8192, 256>>>(q[0], q[1], q[2], q[3], q[4], q[5], q[6], n16); });
+            timeit("flat 3R1W", 4 * n1, [&] { flat_kernel<3, 1, 0><<<8192, 256>>>(q[0], q[1], q[2], q[3], q[4], q[5], q[6], n16); });
+            timeit("flat 3R1W nontemporal", 4 * n1, [&] { flat_kernel<3, 1, 1><<<8192, 256>>>(q[0], q[1], q[2], q[3], q[4], q[5], q[6], n16); });
+            timeit("flat 4R3W nontemporal", 7 * n1, [&] { flat_kernel<4, 3, 1><<<8192, 256>>>(q[0], q[1], q[2], q[3], q[4], q[5], q[6], n16); });
+        }
+        auto tile = [&](auto kern, int threads, int rowb, int rd, int wr, int steps) {
+            const int ncb = (int)(d * 2 / rowb), rps = threads * 16 / rowb, nseg = (int)(L / rps / steps);
+            snprintf(nm, sizeof nm, "tile %dR%dW rows of %3d B, %4d threads, %3d steps, stride %lld", rd, wr, rowb, threads, steps, (long long)rowbytes);
+            timeit(nm, (rd + wr) * n1, [&] { kern<<<(unsigned)(bs * nseg * ncb), threads>>>(p[0], p[1], p[2], p[3], p[4], p[5], p[6], L, rowbytes, ncb, nseg, steps); });
+        };
+        tile(tile_kernel<256, 128, 3, 1>, 256, 128, 3, 1, 128);
+        tile(tile_kernel<512, 256, 3, 1>, 512, 256, 3, 1, 64);
+        tile(tile_kernel<1024, 512, 3, 1>, 1024, 512, 3, 1, 32);
+        tile(tile_kernel<256, 128, 4, 3>, 256, 128, 4, 3, 128);
+        tile(tile_kernel<512, 256, 4, 3>, 512, 256, 4, 3, 64);
+        tile(tile_kernel<1024, 512, 4, 3>, 1024, 512, 4, 3, 32);
+        for (int i = 0; i < 7; ++i) CK(hipFree(p[i]));
+    }
+    return 0;
+}
