@@ -13,59 +13,63 @@ namespace gcg {
 namespace {
 
 constexpr int RING = 8;
+constexpr int BATCH = 4;   // rows fetched together
+
+typedef float f32v4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32v2 __attribute__((ext_vector_type(2)));
 
 template <typename T, int V> struct Vec;
-template <> struct Vec<float, 4> { typedef float4 raw; };
-template <> struct Vec<bf16_t, 4> { typedef uint2 raw; };
-template <> struct Vec<f16_t, 4> { typedef uint2 raw; };
+template <> struct Vec<float, 4> { typedef f32v4 raw; };
+template <> struct Vec<bf16_t, 4> { typedef u32v2 raw; };
+template <> struct Vec<f16_t, 4> { typedef u32v2 raw; };
+
+// every row is read once and written once: stream past the caches
+template <typename R> __device__ __forceinline__ R ldg(const void *p) { return __builtin_nontemporal_load((const R *)p); }
+template <typename R> __device__ __forceinline__ void stg(void *p, const R &v) { __builtin_nontemporal_store(v, (R *)p); }
 
 template <typename T> __device__ __forceinline__ void unpack4(const typename Vec<T, 4>::raw &r, float (&f)[4]);
-template <> __device__ __forceinline__ void unpack4<float>(const float4 &r, float (&f)[4])
+template <> __device__ __forceinline__ void unpack4<float>(const f32v4 &r, float (&f)[4])
 {
-    f[0] = r.x; f[1] = r.y; f[2] = r.z; f[3] = r.w;
+    f[0] = r[0]; f[1] = r[1]; f[2] = r[2]; f[3] = r[3];
 }
-template <> __device__ __forceinline__ void unpack4<bf16_t>(const uint2 &r, float (&f)[4])
+template <> __device__ __forceinline__ void unpack4<bf16_t>(const u32v2 &r, float (&f)[4])
 {
-    f[0] = __uint_as_float(r.x << 16); f[1] = __uint_as_float(r.x & 0xffff0000u);
-    f[2] = __uint_as_float(r.y << 16); f[3] = __uint_as_float(r.y & 0xffff0000u);
+    f[0] = __uint_as_float(r[0] << 16); f[1] = __uint_as_float(r[0] & 0xffff0000u);
+    f[2] = __uint_as_float(r[1] << 16); f[3] = __uint_as_float(r[1] & 0xffff0000u);
 }
-template <> __device__ __forceinline__ void unpack4<f16_t>(const uint2 &r, float (&f)[4])
+template <> __device__ __forceinline__ void unpack4<f16_t>(const u32v2 &r, float (&f)[4])
 {
     typedef _Float16 h2 __attribute__((ext_vector_type(2)));
     h2 a, b;
-    __builtin_memcpy(&a, &r.x, 4);
-    __builtin_memcpy(&b, &r.y, 4);
+    const uint32_t r0 = r[0], r1 = r[1];
+    __builtin_memcpy(&a, &r0, 4);
+    __builtin_memcpy(&b, &r1, 4);
     f[0] = (float)a[0]; f[1] = (float)a[1]; f[2] = (float)b[0]; f[3] = (float)b[1];
 }
 
 template <typename T> __device__ __forceinline__ typename Vec<T, 4>::raw pack4(const float (&f)[4]);
-template <> __device__ __forceinline__ float4 pack4<float>(const float (&f)[4])
+template <> __device__ __forceinline__ f32v4 pack4<float>(const float (&f)[4])
 {
-    return make_float4(f[0], f[1], f[2], f[3]);
+    return f32v4{f[0], f[1], f[2], f[3]};
 }
-template <> __device__ __forceinline__ uint2 pack4<bf16_t>(const float (&f)[4])
+template <> __device__ __forceinline__ u32v2 pack4<bf16_t>(const float (&f)[4])
 {
-    uint2 r;
-    r.x = pack_bf16x2(f[0], f[1]);
-    r.y = pack_bf16x2(f[2], f[3]);
+    u32v2 r;
+    r[0] = pack_bf16x2(f[0], f[1]);
+    r[1] = pack_bf16x2(f[2], f[3]);
     return r;
 }
-template <> __device__ __forceinline__ uint2 pack4<f16_t>(const float (&f)[4])
+template <> __device__ __forceinline__ u32v2 pack4<f16_t>(const float (&f)[4])
 {
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    h2 a = {(_Float16)f[0], (_Float16)f[1]}, b = {(_Float16)f[2], (_Float16)f[3]};
-    uint2 r;
-    __builtin_memcpy(&r.x, &a, 4);
-    __builtin_memcpy(&r.y, &b, 4);
-    return r;
+    return u32v2{pack_f16x2(f[0], f[1]), pack_f16x2(f[2], f[3])};
 }
 
 template <typename T> __device__ __forceinline__ typename Vec<T, 4>::raw zero_raw();
-template <> __device__ __forceinline__ float4 zero_raw<float>() { return make_float4(0.f, 0.f, 0.f, 0.f); }
-template <> __device__ __forceinline__ uint2 zero_raw<bf16_t>() { return make_uint2(0u, 0u); }
-template <> __device__ __forceinline__ uint2 zero_raw<f16_t>() { return make_uint2(0u, 0u); }
+template <> __device__ __forceinline__ f32v4 zero_raw<float>() { return f32v4{0.f, 0.f, 0.f, 0.f}; }
+template <> __device__ __forceinline__ u32v2 zero_raw<bf16_t>() { return u32v2{0u, 0u}; }
+template <> __device__ __forceinline__ u32v2 zero_raw<f16_t>() { return u32v2{0u, 0u}; }
 
-struct WinPlan { int nvec, nseg, ts; int64_t nthreads; };
+struct WinPlan { int nvec, nseg, ts, ncvb; int64_t nthreads, nwg; };
 
 constexpr int V = 4;
 
@@ -77,11 +81,16 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
                                                          T *__restrict__ bx, Dims dm, WinPlan pl)
 {
     typedef typename Vec<T, V>::raw raw_t;
-    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (gid >= pl.nthreads) return;
-    const int cv = (int)(gid % pl.nvec);
-    const int seg = (int)((gid / pl.nvec) % pl.nseg);
-    const int64_t b = gid / ((int64_t)pl.nvec * pl.nseg);
+    // (batch, run, block of 256 channel vectors) come from the workgroup index, so row addresses
+    // are wave-uniform and only the channel offset is per lane
+    int64_t wg = blockIdx.x;
+    const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
+    const int seg = (int)(wg % pl.nseg);
+    const int64_t b = wg / pl.nseg;
+    const int cv = cvb * 256 + (int)threadIdx.x;
+    if (cv >= pl.nvec) return;
+    const int64_t gid = (b * pl.nseg + seg) * pl.nvec + cv;     // index of this lane's workspace slot
+    (void)gid;
     const int64_t L = dm.L, d = dm.d;
     const int64_t c = (int64_t)cv * V;
     const int hl = dm.hl;
@@ -93,7 +102,7 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
-    const int64_t base = b * L * d + c;
+    const int64_t base = b * L * d + c;   // (b*L + t)*d is uniform, c per lane
 
     float ring[RING][V];
 #pragma unroll
@@ -106,45 +115,51 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
         const int64_t t = t_start - i;
         if (t >= 0) {
             float xf[V], Bf[V];
-            unpack4<T>(*(const raw_t *)(x + base + t * d), xf);
-            unpack4<T>(*(const raw_t *)(B + base + t * d), Bf);
+            unpack4<T>(ldg<raw_t>(x + base + t * d), xf);
+            unpack4<T>(ldg<raw_t>(B + base + t * d), Bf);
 #pragma unroll
             for (int v = 0; v < V; ++v) ring[RING - i][v] = xf[v] * Bf[v];
         }
     }
 
     for (int64_t tb = t_start; tb < t_end; tb += RING) {
-        raw_t xr[RING], Br[RING], Cr[RING];
 #pragma unroll
-        for (int k = 0; k < RING; ++k) {
-            const int64_t t = tb + k;
-            if (t < t_end) {
-                xr[k] = *(const raw_t *)(x + base + t * d);
-                Br[k] = *(const raw_t *)(B + base + t * d);
-                Cr[k] = *(const raw_t *)(C + base + t * d);
-            } else {
-                xr[k] = zero_raw<T>(); Br[k] = zero_raw<T>(); Cr[k] = zero_raw<T>();
+        for (int half = 0; half < RING / BATCH; ++half) {
+            // rows are fetched BATCH at a time: enough loads in flight per lane without
+            // pushing the register count past four waves per SIMD
+            raw_t xr[BATCH], Br[BATCH], Cr[BATCH];
+#pragma unroll
+            for (int kk = 0; kk < BATCH; ++kk) {
+                const int64_t t = tb + half * BATCH + kk;
+                if (t < t_end) {
+                    xr[kk] = ldg<raw_t>(x + base + t * d);
+                    Br[kk] = ldg<raw_t>(B + base + t * d);
+                    Cr[kk] = ldg<raw_t>(C + base + t * d);
+                } else {
+                    xr[kk] = zero_raw<T>(); Br[kk] = zero_raw<T>(); Cr[kk] = zero_raw<T>();
+                }
             }
-        }
 #pragma unroll
-        for (int k = 0; k < RING; ++k) {
-            const int64_t t = tb + k;
-            float xf[V], Bf[V], Cf[V], acc[V], out[V];
-            unpack4<T>(xr[k], xf);
-            unpack4<T>(Br[k], Bf);
-            unpack4<T>(Cr[k], Cf);
+            for (int kk = 0; kk < BATCH; ++kk) {
+                const int k = half * BATCH + kk;
+                const int64_t t = tb + k;
+                float xf[V], Bf[V], Cf[V], acc[V], out[V];
+                unpack4<T>(xr[kk], xf);
+                unpack4<T>(Br[kk], Bf);
+                unpack4<T>(Cr[kk], Cf);
 #pragma unroll
-            for (int v = 0; v < V; ++v) { ring[k][v] = xf[v] * Bf[v]; acc[v] = 0.f; }
+                for (int v = 0; v < V; ++v) { ring[k][v] = xf[v] * Bf[v]; acc[v] = 0.f; }
 #pragma unroll
-            for (int j = HL - 1; j >= 0; --j)
+                for (int j = HL - 1; j >= 0; --j)
 #pragma unroll
-                for (int v = 0; v < V; ++v) acc[v] = fmaf(hr[j], ring[(k - j) & (RING - 1)][v], acc[v]);
-            if (t < t_end) {
-                if (y2) *(raw_t *)(y2 + base + t * d) = pack4<T>(acc);
-                if (bx) *(raw_t *)(bx + base + t * d) = pack4<T>(ring[k]);
+                    for (int v = 0; v < V; ++v) acc[v] = fmaf(hr[j], ring[(k - j) & (RING - 1)][v], acc[v]);
+                if (t < t_end) {
+                    if (y2) stg<raw_t>(y2 + base + t * d, pack4<T>(acc));
+                    if (bx) stg<raw_t>(bx + base + t * d, pack4<T>(ring[k]));
 #pragma unroll
-                for (int v = 0; v < V; ++v) out[v] = Cf[v] * acc[v];
-                *(raw_t *)(y + base + t * d) = pack4<T>(out);
+                    for (int v = 0; v < V; ++v) out[v] = Cf[v] * acc[v];
+                    stg<raw_t>(y + base + t * d, pack4<T>(out));
+                }
             }
         }
     }
@@ -162,11 +177,16 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                                                          float *__restrict__ ws, Dims dm, WinPlan pl)
 {
     typedef typename Vec<T, V>::raw raw_t;
-    const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (gid >= pl.nthreads) return;
-    const int cv = (int)(gid % pl.nvec);
-    const int seg = (int)((gid / pl.nvec) % pl.nseg);
-    const int64_t b = gid / ((int64_t)pl.nvec * pl.nseg);
+    // (batch, run, block of 256 channel vectors) come from the workgroup index, so row addresses
+    // are wave-uniform and only the channel offset is per lane
+    int64_t wg = blockIdx.x;
+    const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
+    const int seg = (int)(wg % pl.nseg);
+    const int64_t b = wg / pl.nseg;
+    const int cv = cvb * 256 + (int)threadIdx.x;
+    if (cv >= pl.nvec) return;
+    const int64_t gid = (b * pl.nseg + seg) * pl.nvec + cv;     // index of this lane's workspace slot
+    (void)gid;
     const int64_t L = dm.L, d = dm.d;
     const int64_t c = (int64_t)cv * V;
     const int hl = dm.hl;
@@ -178,7 +198,7 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
-    const int64_t base = b * L * d + c;
+    const int64_t base = b * L * d + c;   // (b*L + t)*d is uniform, c per lane
 
     float ur[RING][V], gr[RING][V], dha[HL];
     raw_t xs[RING], Bs[RING];
@@ -195,8 +215,8 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
         const int64_t t = t_start - i;
         if (t >= 0) {
             float xf[V], Bf[V];
-            unpack4<T>(*(const raw_t *)(x + base + t * d), xf);
-            unpack4<T>(*(const raw_t *)(B + base + t * d), Bf);
+            unpack4<T>(ldg<raw_t>(x + base + t * d), xf);
+            unpack4<T>(ldg<raw_t>(B + base + t * d), Bf);
 #pragma unroll
             for (int v = 0; v < V; ++v) ur[RING - i][v] = xf[v] * Bf[v];
         }
@@ -204,75 +224,79 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 
     const int64_t t_stop = t_end + (HL - 1);  // exclusive bound of the walk
     for (int64_t tb = t_start; tb < t_stop; tb += RING) {
-        // rows are fetched eight at a time into staging registers; the x / B rings are
-        // only overwritten slot by slot below, after the delayed du row has read them
-        raw_t dyr[RING], Cr[RING], xr[RING], Br[RING];
 #pragma unroll
-        for (int k = 0; k < RING; ++k) {
-            const int64_t t = tb + k;
-            if (t < t_end) {
-                xr[k] = *(const raw_t *)(x + base + t * d);
-                Br[k] = *(const raw_t *)(B + base + t * d);
-            } else {
-                xr[k] = zero_raw<T>(); Br[k] = zero_raw<T>();
-            }
-            if (t < L && t < t_stop) {
-                dyr[k] = *(const raw_t *)(dy + base + t * d);
-                Cr[k] = *(const raw_t *)(C + base + t * d);
-            } else {
-                dyr[k] = zero_raw<T>(); Cr[k] = zero_raw<T>();
-            }
-        }
+        for (int half = 0; half < RING / BATCH; ++half) {
+            // rows are fetched BATCH at a time into staging registers; the x / B rings are only
+            // overwritten slot by slot below, after the delayed du row has read them
+            raw_t dyr[BATCH], Cr[BATCH], xr[BATCH], Br[BATCH];
 #pragma unroll
-        for (int k = 0; k < RING; ++k) {
-            const int64_t t = tb + k;
-            float dyf[V], Cf[V];
-            unpack4<T>(dyr[k], dyf);
-            unpack4<T>(Cr[k], Cf);
-#pragma unroll
-            for (int v = 0; v < V; ++v) gr[k][v] = dyf[v] * Cf[v];
-            xs[k] = xr[k];
-            Bs[k] = Br[k];
-            if (t < t_end) {
-                float xf[V], Bf[V], y2v[V], o[V];
-                unpack4<T>(xs[k], xf);
-                unpack4<T>(Bs[k], Bf);
-#pragma unroll
-                for (int v = 0; v < V; ++v) { ur[k][v] = xf[v] * Bf[v]; y2v[v] = 0.f; }
-#pragma unroll
-                for (int j = HL - 1; j >= 0; --j) {
-                    float s = 0.f;
-#pragma unroll
-                    for (int v = 0; v < V; ++v) {
-                        const float u = ur[(k - j) & (RING - 1)][v];
-                        y2v[v] = fmaf(hr[j], u, y2v[v]);
-                        s = fmaf(gr[k][v], u, s);
-                    }
-                    dha[j] += s;
+            for (int kk = 0; kk < BATCH; ++kk) {
+                const int64_t t = tb + half * BATCH + kk;
+                if (t < t_end) {
+                    xr[kk] = ldg<raw_t>(x + base + t * d);
+                    Br[kk] = ldg<raw_t>(B + base + t * d);
+                } else {
+                    xr[kk] = zero_raw<T>(); Br[kk] = zero_raw<T>();
                 }
-#pragma unroll
-                for (int v = 0; v < V; ++v) o[v] = dyf[v] * y2v[v];
-                *(raw_t *)(dC + base + t * d) = pack4<T>(o);
+                if (t < L && t < t_stop) {
+                    dyr[kk] = ldg<raw_t>(dy + base + t * d);
+                    Cr[kk] = ldg<raw_t>(C + base + t * d);
+                } else {
+                    dyr[kk] = zero_raw<T>(); Cr[kk] = zero_raw<T>();
+                }
             }
-            // du for row t-(HL-1): sum_j hr[j] * g2[row + j]
-            const int64_t orow = t - (HL - 1);
-            if (orow >= t_start && orow < t_end) {
-                float du[V], xf[V], Bf[V], o[V];
 #pragma unroll
-                for (int v = 0; v < V; ++v) du[v] = 0.f;
+            for (int kk = 0; kk < BATCH; ++kk) {
+                const int k = half * BATCH + kk;
+                const int64_t t = tb + k;
+                float dyf[V], Cf[V];
+                unpack4<T>(dyr[kk], dyf);
+                unpack4<T>(Cr[kk], Cf);
 #pragma unroll
-                for (int j = 0; j < HL; ++j)
+                for (int v = 0; v < V; ++v) gr[k][v] = dyf[v] * Cf[v];
+                xs[k] = xr[kk];
+                Bs[k] = Br[kk];
+                if (t < t_end) {
+                    float xf[V], Bf[V], y2v[V], o[V];
+                    unpack4<T>(xs[k], xf);
+                    unpack4<T>(Bs[k], Bf);
 #pragma unroll
-                    for (int v = 0; v < V; ++v)
-                        du[v] = fmaf(hr[j], gr[(k - (HL - 1) + j) & (RING - 1)][v], du[v]);
-                unpack4<T>(xs[(k - (HL - 1)) & (RING - 1)], xf);
-                unpack4<T>(Bs[(k - (HL - 1)) & (RING - 1)], Bf);
+                    for (int v = 0; v < V; ++v) { ur[k][v] = xf[v] * Bf[v]; y2v[v] = 0.f; }
 #pragma unroll
-                for (int v = 0; v < V; ++v) o[v] = du[v] * Bf[v];
-                *(raw_t *)(dx + base + orow * d) = pack4<T>(o);
+                    for (int j = HL - 1; j >= 0; --j) {
+                        float sacc = 0.f;
 #pragma unroll
-                for (int v = 0; v < V; ++v) o[v] = du[v] * xf[v];
-                *(raw_t *)(dB + base + orow * d) = pack4<T>(o);
+                        for (int v = 0; v < V; ++v) {
+                            const float u = ur[(k - j) & (RING - 1)][v];
+                            y2v[v] = fmaf(hr[j], u, y2v[v]);
+                            sacc = fmaf(gr[k][v], u, sacc);
+                        }
+                        dha[j] += sacc;
+                    }
+#pragma unroll
+                    for (int v = 0; v < V; ++v) o[v] = dyf[v] * y2v[v];
+                    stg<raw_t>(dC + base + t * d, pack4<T>(o));
+                }
+                // du for row t-(HL-1): sum_j hr[j] * g2[row + j]
+                const int64_t orow = t - (HL - 1);
+                if (orow >= t_start && orow < t_end) {
+                    float du[V], xf[V], Bf[V], o[V];
+#pragma unroll
+                    for (int v = 0; v < V; ++v) du[v] = 0.f;
+#pragma unroll
+                    for (int j = 0; j < HL; ++j)
+#pragma unroll
+                        for (int v = 0; v < V; ++v)
+                            du[v] = fmaf(hr[j], gr[(k - (HL - 1) + j) & (RING - 1)][v], du[v]);
+                    unpack4<T>(xs[(k - (HL - 1)) & (RING - 1)], xf);
+                    unpack4<T>(Bs[(k - (HL - 1)) & (RING - 1)], Bf);
+#pragma unroll
+                    for (int v = 0; v < V; ++v) o[v] = du[v] * Bf[v];
+                    stg<raw_t>(dx + base + orow * d, pack4<T>(o));
+#pragma unroll
+                    for (int v = 0; v < V; ++v) o[v] = du[v] * xf[v];
+                    stg<raw_t>(dB + base + orow * d, pack4<T>(o));
+                }
             }
         }
     }
@@ -316,7 +340,9 @@ WinPlan plan(const Dims &dm)
     // shorter runs when the problem is too small to fill the chip with 128-row runs
     while (p.ts > 16 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 256 * 1024) p.ts >>= 1;
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);
-    p.nthreads = dm.bs * p.nseg * p.nvec;
+    p.nthreads = dm.bs * p.nseg * p.nvec;       // workspace slots (one per lane with work)
+    p.ncvb = (p.nvec + 255) / 256;
+    p.nwg = dm.bs * p.nseg * p.ncvb;
     return p;
 }
 
@@ -325,7 +351,7 @@ int fwd_t(const void *x, const void *B, const void *C, const void *h, void *y, v
           const Dims &dm, hipStream_t st)
 {
     const WinPlan p = plan(dm);
-    const int64_t nwg = (p.nthreads + 255) / 256;
+    const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((window_fwd_kernel<T, HL>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)x,
                        (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
@@ -337,7 +363,7 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
           void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
     const WinPlan p = plan(dm);
-    const int64_t nwg = (p.nthreads + 255) / 256;
+    const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((window_bwd_kernel<T, HL>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
