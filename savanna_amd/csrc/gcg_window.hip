@@ -15,66 +15,77 @@ namespace {
 constexpr int RING = 8;
 constexpr int BATCH = 4;   // rows fetched together
 
-typedef float f32v4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32v2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32v4 __attribute__((ext_vector_type(4)));
 
-template <typename T, int V> struct Vec;
-template <> struct Vec<float, 4> { typedef f32v4 raw; };
-template <> struct Vec<bf16_t, 4> { typedef u32v2 raw; };
-template <> struct Vec<f16_t, 4> { typedef u32v2 raw; };
+// A lane's row vector: VV channels as raw 32-bit words (fp32: one channel per word;
+// bf16 / f16: two).  VV = 4 everywhere, or 8 for the 16-bit types (16-byte accesses).
+template <typename T, int VV> struct Vec;
+template <> struct Vec<float, 4> { typedef u32v4 raw; static constexpr int W = 4; };
+template <> struct Vec<bf16_t, 4> { typedef u32v2 raw; static constexpr int W = 2; };
+template <> struct Vec<f16_t, 4> { typedef u32v2 raw; static constexpr int W = 2; };
+template <> struct Vec<bf16_t, 8> { typedef u32v4 raw; static constexpr int W = 4; };
+template <> struct Vec<f16_t, 8> { typedef u32v4 raw; static constexpr int W = 4; };
 
 // every row is read once and written once: stream past the caches
 template <typename R> __device__ __forceinline__ R ldg(const void *p) { return __builtin_nontemporal_load((const R *)p); }
 template <typename R> __device__ __forceinline__ void stg(void *p, const R &v) { __builtin_nontemporal_store(v, (R *)p); }
 
-template <typename T> __device__ __forceinline__ void unpack4(const typename Vec<T, 4>::raw &r, float (&f)[4]);
-template <> __device__ __forceinline__ void unpack4<float>(const f32v4 &r, float (&f)[4])
-{
-    f[0] = r[0]; f[1] = r[1]; f[2] = r[2]; f[3] = r[3];
-}
-template <> __device__ __forceinline__ void unpack4<bf16_t>(const u32v2 &r, float (&f)[4])
-{
-    f[0] = __uint_as_float(r[0] << 16); f[1] = __uint_as_float(r[0] & 0xffff0000u);
-    f[2] = __uint_as_float(r[1] << 16); f[3] = __uint_as_float(r[1] & 0xffff0000u);
-}
-template <> __device__ __forceinline__ void unpack4<f16_t>(const u32v2 &r, float (&f)[4])
-{
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    h2 a, b;
-    const uint32_t r0 = r[0], r1 = r[1];
-    __builtin_memcpy(&a, &r0, 4);
-    __builtin_memcpy(&b, &r1, 4);
-    f[0] = (float)a[0]; f[1] = (float)a[1]; f[2] = (float)b[0]; f[3] = (float)b[1];
-}
+template <typename T> struct Word;   // conversions of one 32-bit word
+template <> struct Word<float> {
+    static constexpr int N = 1;
+    static __device__ __forceinline__ void unpack(uint32_t w, float *f) { f[0] = __uint_as_float(w); }
+    static __device__ __forceinline__ uint32_t pack(const float *f) { return __float_as_uint(f[0]); }
+};
+template <> struct Word<bf16_t> {
+    static constexpr int N = 2;
+    static __device__ __forceinline__ void unpack(uint32_t w, float *f)
+    {
+        f[0] = __uint_as_float(w << 16);
+        f[1] = __uint_as_float(w & 0xffff0000u);
+    }
+    static __device__ __forceinline__ uint32_t pack(const float *f) { return pack_bf16x2(f[0], f[1]); }
+};
+template <> struct Word<f16_t> {
+    static constexpr int N = 2;
+    static __device__ __forceinline__ void unpack(uint32_t w, float *f)
+    {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 a;
+        __builtin_memcpy(&a, &w, 4);
+        f[0] = (float)a[0];
+        f[1] = (float)a[1];
+    }
+    static __device__ __forceinline__ uint32_t pack(const float *f) { return pack_f16x2(f[0], f[1]); }
+};
 
-template <typename T> __device__ __forceinline__ typename Vec<T, 4>::raw pack4(const float (&f)[4]);
-template <> __device__ __forceinline__ f32v4 pack4<float>(const float (&f)[4])
+template <typename T, int VV>
+__device__ __forceinline__ void unpackv(const typename Vec<T, VV>::raw &r, float (&f)[VV])
 {
-    return f32v4{f[0], f[1], f[2], f[3]};
+#pragma unroll
+    for (int i = 0; i < Vec<T, VV>::W; ++i) Word<T>::unpack(r[i], &f[i * Word<T>::N]);
 }
-template <> __device__ __forceinline__ u32v2 pack4<bf16_t>(const float (&f)[4])
+template <typename T, int VV>
+__device__ __forceinline__ typename Vec<T, VV>::raw packv(const float (&f)[VV])
 {
-    u32v2 r;
-    r[0] = pack_bf16x2(f[0], f[1]);
-    r[1] = pack_bf16x2(f[2], f[3]);
+    typename Vec<T, VV>::raw r;
+#pragma unroll
+    for (int i = 0; i < Vec<T, VV>::W; ++i) r[i] = Word<T>::pack(&f[i * Word<T>::N]);
     return r;
 }
-template <> __device__ __forceinline__ u32v2 pack4<f16_t>(const float (&f)[4])
+template <typename T, int VV> __device__ __forceinline__ typename Vec<T, VV>::raw zero_raw()
 {
-    return u32v2{pack_f16x2(f[0], f[1]), pack_f16x2(f[2], f[3])};
+    typename Vec<T, VV>::raw r;
+#pragma unroll
+    for (int i = 0; i < Vec<T, VV>::W; ++i) r[i] = 0u;
+    return r;
 }
 
-template <typename T> __device__ __forceinline__ typename Vec<T, 4>::raw zero_raw();
-template <> __device__ __forceinline__ f32v4 zero_raw<float>() { return f32v4{0.f, 0.f, 0.f, 0.f}; }
-template <> __device__ __forceinline__ u32v2 zero_raw<bf16_t>() { return u32v2{0u, 0u}; }
-template <> __device__ __forceinline__ u32v2 zero_raw<f16_t>() { return u32v2{0u, 0u}; }
+struct WinPlan { int v, nvec, nseg, ts, ncvb; int64_t nthreads, nwg; };
 
-struct WinPlan { int nvec, nseg, ts, ncvb; int64_t nthreads, nwg; };
-
-constexpr int V = 4;
 
 // ---------------------------------------------------------------------------- forward
-template <typename T, int HL>
+template <typename T, int HL, int V>
 __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x, const T *__restrict__ B,
                                                          const T *__restrict__ C, const T *__restrict__ h,
                                                          T *__restrict__ y, T *__restrict__ y2,
@@ -115,8 +126,8 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
         const int64_t t = t_start - i;
         if (t >= 0) {
             float xf[V], Bf[V];
-            unpack4<T>(ldg<raw_t>(x + base + t * d), xf);
-            unpack4<T>(ldg<raw_t>(B + base + t * d), Bf);
+            unpackv<T, V>(ldg<raw_t>(x + base + t * d), xf);
+            unpackv<T, V>(ldg<raw_t>(B + base + t * d), Bf);
 #pragma unroll
             for (int v = 0; v < V; ++v) ring[RING - i][v] = xf[v] * Bf[v];
         }
@@ -136,7 +147,7 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
                     Br[kk] = ldg<raw_t>(B + base + t * d);
                     Cr[kk] = ldg<raw_t>(C + base + t * d);
                 } else {
-                    xr[kk] = zero_raw<T>(); Br[kk] = zero_raw<T>(); Cr[kk] = zero_raw<T>();
+                    xr[kk] = zero_raw<T, V>(); Br[kk] = zero_raw<T, V>(); Cr[kk] = zero_raw<T, V>();
                 }
             }
 #pragma unroll
@@ -144,9 +155,9 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
                 const int k = half * BATCH + kk;
                 const int64_t t = tb + k;
                 float xf[V], Bf[V], Cf[V], acc[V], out[V];
-                unpack4<T>(xr[kk], xf);
-                unpack4<T>(Br[kk], Bf);
-                unpack4<T>(Cr[kk], Cf);
+                unpackv<T, V>(xr[kk], xf);
+                unpackv<T, V>(Br[kk], Bf);
+                unpackv<T, V>(Cr[kk], Cf);
 #pragma unroll
                 for (int v = 0; v < V; ++v) { ring[k][v] = xf[v] * Bf[v]; acc[v] = 0.f; }
 #pragma unroll
@@ -154,11 +165,11 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
 #pragma unroll
                     for (int v = 0; v < V; ++v) acc[v] = fmaf(hr[j], ring[(k - j) & (RING - 1)][v], acc[v]);
                 if (t < t_end) {
-                    if (y2) stg<raw_t>(y2 + base + t * d, pack4<T>(acc));
-                    if (bx) stg<raw_t>(bx + base + t * d, pack4<T>(ring[k]));
+                    if (y2) stg<raw_t>(y2 + base + t * d, packv<T, V>(acc));
+                    if (bx) stg<raw_t>(bx + base + t * d, packv<T, V>(ring[k]));
 #pragma unroll
                     for (int v = 0; v < V; ++v) out[v] = Cf[v] * acc[v];
-                    stg<raw_t>(y + base + t * d, pack4<T>(out));
+                    stg<raw_t>(y + base + t * d, packv<T, V>(out));
                 }
             }
         }
@@ -169,7 +180,7 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
 // Per lane: rows [t_start, t_end).  Row r is loaded at step r; dC[r] and the dh terms
 // of row r are produced at once (they look back), du[r-(HL-1)] is produced at step r
 // (it looks forward), so the walk runs HL-1 rows past t_end reading only dy and C.
-template <typename T, int HL>
+template <typename T, int HL, int V>
 __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                          const T *__restrict__ B, const T *__restrict__ C,
                                                          const T *__restrict__ h, T *__restrict__ dx,
@@ -204,7 +215,7 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
     raw_t xs[RING], Bs[RING];
 #pragma unroll
     for (int s = 0; s < RING; ++s) {
-        xs[s] = zero_raw<T>(); Bs[s] = zero_raw<T>();
+        xs[s] = zero_raw<T, V>(); Bs[s] = zero_raw<T, V>();
 #pragma unroll
         for (int v = 0; v < V; ++v) { ur[s][v] = 0.f; gr[s][v] = 0.f; }
     }
@@ -215,8 +226,8 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
         const int64_t t = t_start - i;
         if (t >= 0) {
             float xf[V], Bf[V];
-            unpack4<T>(ldg<raw_t>(x + base + t * d), xf);
-            unpack4<T>(ldg<raw_t>(B + base + t * d), Bf);
+            unpackv<T, V>(ldg<raw_t>(x + base + t * d), xf);
+            unpackv<T, V>(ldg<raw_t>(B + base + t * d), Bf);
 #pragma unroll
             for (int v = 0; v < V; ++v) ur[RING - i][v] = xf[v] * Bf[v];
         }
@@ -236,13 +247,13 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                     xr[kk] = ldg<raw_t>(x + base + t * d);
                     Br[kk] = ldg<raw_t>(B + base + t * d);
                 } else {
-                    xr[kk] = zero_raw<T>(); Br[kk] = zero_raw<T>();
+                    xr[kk] = zero_raw<T, V>(); Br[kk] = zero_raw<T, V>();
                 }
                 if (t < L && t < t_stop) {
                     dyr[kk] = ldg<raw_t>(dy + base + t * d);
                     Cr[kk] = ldg<raw_t>(C + base + t * d);
                 } else {
-                    dyr[kk] = zero_raw<T>(); Cr[kk] = zero_raw<T>();
+                    dyr[kk] = zero_raw<T, V>(); Cr[kk] = zero_raw<T, V>();
                 }
             }
 #pragma unroll
@@ -250,16 +261,16 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                 const int k = half * BATCH + kk;
                 const int64_t t = tb + k;
                 float dyf[V], Cf[V];
-                unpack4<T>(dyr[kk], dyf);
-                unpack4<T>(Cr[kk], Cf);
+                unpackv<T, V>(dyr[kk], dyf);
+                unpackv<T, V>(Cr[kk], Cf);
 #pragma unroll
                 for (int v = 0; v < V; ++v) gr[k][v] = dyf[v] * Cf[v];
                 xs[k] = xr[kk];
                 Bs[k] = Br[kk];
                 if (t < t_end) {
                     float xf[V], Bf[V], y2v[V], o[V];
-                    unpack4<T>(xs[k], xf);
-                    unpack4<T>(Bs[k], Bf);
+                    unpackv<T, V>(xs[k], xf);
+                    unpackv<T, V>(Bs[k], Bf);
 #pragma unroll
                     for (int v = 0; v < V; ++v) { ur[k][v] = xf[v] * Bf[v]; y2v[v] = 0.f; }
 #pragma unroll
@@ -275,7 +286,7 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                     }
 #pragma unroll
                     for (int v = 0; v < V; ++v) o[v] = dyf[v] * y2v[v];
-                    stg<raw_t>(dC + base + t * d, pack4<T>(o));
+                    stg<raw_t>(dC + base + t * d, packv<T, V>(o));
                 }
                 // du for row t-(HL-1): sum_j hr[j] * g2[row + j]
                 const int64_t orow = t - (HL - 1);
@@ -288,14 +299,14 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 #pragma unroll
                         for (int v = 0; v < V; ++v)
                             du[v] = fmaf(hr[j], gr[(k - (HL - 1) + j) & (RING - 1)][v], du[v]);
-                    unpack4<T>(xs[(k - (HL - 1)) & (RING - 1)], xf);
-                    unpack4<T>(Bs[(k - (HL - 1)) & (RING - 1)], Bf);
+                    unpackv<T, V>(xs[(k - (HL - 1)) & (RING - 1)], xf);
+                    unpackv<T, V>(Bs[(k - (HL - 1)) & (RING - 1)], Bf);
 #pragma unroll
                     for (int v = 0; v < V; ++v) o[v] = du[v] * Bf[v];
-                    stg<raw_t>(dx + base + orow * d, pack4<T>(o));
+                    stg<raw_t>(dx + base + orow * d, packv<T, V>(o));
 #pragma unroll
                     for (int v = 0; v < V; ++v) o[v] = du[v] * xf[v];
-                    stg<raw_t>(dB + base + orow * d, pack4<T>(o));
+                    stg<raw_t>(dB + base + orow * d, packv<T, V>(o));
                 }
             }
         }
@@ -314,7 +325,7 @@ __global__ __launch_bounds__(256) void window_dh_reduce_kernel(const float *__re
 {
     __shared__ float red[256];
     const int grp = blockIdx.x / dm.hl, k = blockIdx.x % dm.hl;
-    const int lpg = dm.dg / V;                       // lanes (channel vectors) per group
+    const int lpg = dm.dg / pl.v;                    // lanes (channel vectors) per group
     const int64_t nrow = dm.bs * pl.nseg;            // (batch, segment) pairs
     const int64_t nterm = nrow * lpg;
     const float *src = ws + (size_t)k * pl.nthreads;
@@ -332,10 +343,11 @@ __global__ __launch_bounds__(256) void window_dh_reduce_kernel(const float *__re
     if (threadIdx.x == 0) Elem<T>::store(dh + (size_t)grp * dm.hl + k, red[0]);
 }
 
-WinPlan plan(const Dims &dm)
+WinPlan plan(const Dims &dm, int v)
 {
     WinPlan p;
-    p.nvec = (int)(dm.d / V);
+    p.v = v;
+    p.nvec = (int)(dm.d / v);
     p.ts = 128;
     // shorter runs when the problem is too small to fill the chip with 128-row runs
     while (p.ts > 16 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 256 * 1024) p.ts >>= 1;
@@ -346,14 +358,16 @@ WinPlan plan(const Dims &dm)
     return p;
 }
 
-template <typename T, int HL>
-int fwd_t(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
+constexpr int BWD_V = 4;   // the backward keeps four rings per lane: 4 channels is what fits
+
+template <typename T, int HL, int V>
+int fwd_v(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
           const Dims &dm, hipStream_t st)
 {
-    const WinPlan p = plan(dm);
+    const WinPlan p = plan(dm, V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((window_fwd_kernel<T, HL>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)x,
+    hipLaunchKernelGGL((window_fwd_kernel<T, HL, V>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)x,
                        (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     return (int)hipGetLastError();
 }
@@ -362,10 +376,10 @@ template <typename T, int HL>
 int bwd_t(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
           void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    const WinPlan p = plan(dm);
+    const WinPlan p = plan(dm, BWD_V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((window_bwd_kernel<T, HL>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)dy,
+    hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
                        (float *)ws, dm, p);
     int e = (int)hipGetLastError();
@@ -373,6 +387,15 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
     hipLaunchKernelGGL(window_dh_reduce_kernel<T>, dim3((unsigned)(dm.g * dm.hl)), dim3(256), 0, st,
                        (const float *)ws, (T *)dh, dm, p);
     return (int)hipGetLastError();
+}
+
+// Four channels per lane in both directions.  Eight (16-byte vectors for the 16-bit types) was
+// measured slower at the 40B shape: half as many lanes in flight outweighs the wider access.
+template <typename T, int HL>
+int fwd_t(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
+          const Dims &dm, hipStream_t st)
+{
+    return fwd_v<T, HL, 4>(x, B, C, h, y, y2, bx, dm, st);
 }
 
 template <typename T>
@@ -397,7 +420,7 @@ int bwd_hl(const void *dy, const void *x, const void *B, const void *C, const vo
 
 bool window_supported(const Dims &dm)
 {
-    return dm.hl <= RING && dm.dg % V == 0 && (int64_t)dm.g * dm.hl <= 0x7fffffffLL;
+    return dm.hl <= RING && dm.dg % 4 == 0 && (int64_t)dm.g * dm.hl <= 0x7fffffffLL;
 }
 
 int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h, void *y,
@@ -413,7 +436,7 @@ int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, co
 
 size_t window_bwd_workspace(const Dims &dm)
 {
-    const WinPlan p = plan(dm);
+    const WinPlan p = plan(dm, BWD_V);
     return (size_t)p.nthreads * dm.hl * sizeof(float);
 }
 
