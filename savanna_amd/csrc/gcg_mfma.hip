@@ -93,6 +93,9 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char *p)
 
 // Streaming accesses: every tensor element is touched once, so loads and stores carry the
 // nontemporal hint (GCG_MFMA_NT=0 at build time turns it off for comparison).
+#ifndef GCG_XCD_SWIZZLE
+#define GCG_XCD_SWIZZLE 1
+#endif
 #ifndef GCG_MFMA_NT
 #define GCG_MFMA_NT 3
 #endif
@@ -114,6 +117,17 @@ template <typename T> __device__ __forceinline__ void stg16(T *p, const uint4 &v
 #else
     *(uint4 *)p = v;
 #endif
+}
+
+// Workgroups are dealt to the 8 XCDs round-robin by index.  Re-labelling them so that each XCD
+// receives a contiguous run of (batch, segment, channel-block) triples makes the workgroups of
+// one XCD cover whole tensor rows between them, which its L2 and the memory channels prefer.
+__device__ __forceinline__ int64_t xcd_contiguous_id(int64_t id, int64_t n)
+{
+#if GCG_XCD_SWIZZLE
+    if ((n & 7) == 0) return (id & 7) * (n >> 3) + (id >> 3);
+#endif
+    return id;
 }
 
 struct MfmaPlan { int ncb, nseg, steps_per_seg, nw; int64_t nsteps, nwg; };
@@ -145,7 +159,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     __shared__ __attribute__((aligned(16))) unsigned char y_st[STEP * YROW];
     __shared__ uint16_t htab[NW][HTAB];
 
-    int64_t wg = blockIdx.x;
+    int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
     const int seg = (int)(wg % pl.nseg);
     const int64_t b = wg / pl.nseg;
@@ -306,7 +320,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     unsigned char *u_rm = smem + OFF_U, *g_rm = smem + OFF_G, *y_st = smem + OFF_Y, *d_st = smem + OFF_D;
     uint16_t *htab = (uint16_t *)(smem + OFF_H);
 
-    int64_t wg = blockIdx.x;
+    int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
     const int seg = (int)(wg % pl.nseg);
     const int64_t b = wg / pl.nseg;
@@ -494,7 +508,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         for (int v = 0; v < 4; ++v) pt[dl * 256 + (4 * q + v) * 16 + j] = P[dl][v];
     __syncthreads();
     if (wave_valid) {
-        float *out = ws + ((size_t)blockIdx.x * NW + w) * 128;
+        float *out = ws + ((size_t)xcd_contiguous_id(blockIdx.x, gridDim.x) * NW + w) * 128;
         for (int lag = l; lag < 128; lag += 64) {
             const int d0 = lag >> 4, rr = lag & 15;
             float sum = 0.f;
