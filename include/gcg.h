@@ -39,7 +39,7 @@ enum {
     GCG_ALGO_AUTO   = 0,
     GCG_ALGO_DIRECT = 1, /* LDS-tiled sliding window on the vector ALUs, any hl/dg/dtype */
     GCG_ALGO_WINDOW = 2, /* register sliding window, hl <= 8 (Hyena-SE)                   */
-    GCG_ALGO_MFMA   = 3  /* banded Toeplitz GEMM on MFMA, bf16/f16, hl <= 128, dg % 16 == 0 (Hyena-MR) */
+    GCG_ALGO_MFMA   = 3  /* banded Toeplitz GEMM on MFMA, any dtype, hl <= 128, dg % 16 == 0 (Hyena-MR) */
 };
 
 /* Error codes. */

@@ -128,7 +128,7 @@ GCG_API size_t gcg_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t
     switch (a) {
     case GCG_ALGO_DIRECT: n = gcg::direct_bwd_workspace(dm); break;
     case GCG_ALGO_WINDOW: n = gcg::window_bwd_workspace(dm); break;
-    case GCG_ALGO_MFMA:   n = gcg::mfma_bwd_workspace(dm); break;
+    case GCG_ALGO_MFMA:   n = gcg::mfma_bwd_workspace(dtype, dm); break;
     default: return 0;
     }
     // under AUTO a misaligned tensor reroutes to the direct kernels: size for both

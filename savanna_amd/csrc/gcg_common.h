@@ -104,7 +104,7 @@ bool mfma_supported(int dtype, const Dims &dm);
 bool mfma_bwd_available();
 int mfma_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h,
                     void *y, void *y2, void *bx, const Dims &dm, hipStream_t st);
-size_t mfma_bwd_workspace(const Dims &dm);
+size_t mfma_bwd_workspace(int dtype, const Dims &dm);
 int mfma_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C,
                     const void *h, void *dx, void *dB, void *dC, void *dh, void *ws,
                     const Dims &dm, hipStream_t st);

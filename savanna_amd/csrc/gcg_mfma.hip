@@ -1,20 +1,25 @@
-// Banded Toeplitz GEMM on the matrix cores (bf16 / f16 I/O, fp32 accumulate, hl <= 128).
+// Banded Toeplitz GEMM on the matrix cores (bf16 / f16 / fp32 I/O, fp32 accumulate, hl <= 128).
 //
-// Streaming form of the two-pass chunked convolution.  A workgroup of four waves owns 64
+// Streaming form of the two-pass chunked convolution.  A workgroup of NW waves owns 16*NW
 // adjacent channels of one batch row and walks a run of time steps of 32 rows.  Wave w owns
 // the 16 channels [16w, 16w+16) -- one filter -- and computes, per step, the transposed
 // output tile  Y2^T (16 channels x 32 times) = sum_i  U_{s-i}^T (16 x 32)  *  W_i (32 x 32)
-// with v_mfma_f32_16x16x32, where U_{s-i} is the pre-gate product of step s-i and W_i the
-// slice of the banded Toeplitz matrix of the filter at time offset 32*i.  The NK = 5 slices
-// (10 operand tiles of 16 output times) live in registers for the whole walk, and the last
-// NK operand tiles of U are carried in registers, so the "carry from the previous chunk" of
-// the two-pass form never goes back to memory: q, k, v are read once and y written once.
+// on the matrix cores, where U_{s-i} is the pre-gate product of step s-i and W_i the slice of
+// the banded Toeplitz matrix of the filter at time offset 32*i.  The NK = 5 slices (10 operand
+// tiles of 16 output times) live in registers for the whole walk, and the last NK operand
+// tiles of U are carried in registers, so the "carry from the previous chunk" of the two-pass
+// form never goes back to memory: q, k, v are read once and y written once.
 //
-// Memory side: the four waves load each 32 x 64 tile with full 128-byte rows, form
-// u = bf16(x*B) in registers, park it row-major in LDS, and every wave fetches its matrix
-// operand from there with the transposing LDS read (ds_read_b64_tr_b16), which hands a lane
-// four consecutive time samples of one channel.  The fp32 result tile returns through LDS to
-// the row layout, is gated with C in fp32 and stored with full 128-byte rows.
+// Memory side: the waves load each 32-row tile with full rows (32*NW bytes at 16 bits), form
+// u = x*B in registers, park it row-major in LDS, and every wave fetches its matrix operand
+// from there.  The fp32 result tile returns through LDS to the row layout, is gated with C in
+// fp32 and stored with full rows.
+//
+// Element types.  bf16 / f16: v_mfma_f32_16x16x32; the operand (8 consecutive time samples of
+// one channel per lane) comes from the transposing LDS read ds_read_b64_tr_b16.  fp32: the
+// same 32-deep product is eight v_mfma_f32_16x16x4_f32 (exact fp32 multiply-add, so the fp32
+// path keeps fp32 accuracy); a lane's eight operand values are time samples q, q+4, ... of one
+// channel, read straight from the row-major tile.
 #include "gcg_common.h"
 
 #include <cstdlib>
@@ -27,22 +32,73 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int STEP = 32;          // time rows per step (K of one MFMA)
-// A workgroup of NW waves owns CB = 16*NW adjacent channels; its LDS rows are padded so that
-// consecutive time rows start 8 (u, 2-byte elements) or 4 (y2, fp32) banks apart.
-template <int NW> struct Geo {
-    static constexpr int CB = 16 * NW;          // channels per workgroup
-    static constexpr int LPR = CB / 8;          // lanes per row in the row layout (8 channels each)
-    static constexpr int UROW = CB * 2 + 32;    // bytes per LDS row of u
-    static constexpr int YROW = CB * 4 + 16;    // bytes per LDS row of y2
-    static constexpr int NT = 64 * NW;          // threads
-};
+constexpr int STEP = 32;          // time rows per step (contraction depth of one product)
 constexpr int HPAD = 32;          // filter table holds lags [-32, 160)
 constexpr int HTAB = 192;
 
+// Transposing LDS read: within each block of 16 lanes, lane i receives element (i % 4) of
+// the 8-byte rows addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4 of that block.
+__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char *p)
+{
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p);
+}
+
+// Per element type: the matrix operand, how it is fetched from a row-major LDS tile of
+// `urow` bytes per time row, and the 32-deep product.  Operand element e of the lane in
+// quad q stands for contraction index kmap(q, e); both factors of a product use the same map.
 template <typename T> struct MT;
-template <> struct MT<bf16_t> {
-    typedef bf16x8 op_t;
+
+template <typename OP> struct MT16 {
+    static constexpr int ES = 2;                 // bytes per element
+    static constexpr int RW = 1;                 // 16-byte words per 8-channel row vector
+    static constexpr int UPAD = 32;              // row padding: consecutive rows start 8 banks apart
+    typedef OP op_t;
+    typedef uint16_t hraw_t;
+    static __device__ __forceinline__ int kmap(int q, int e) { return 8 * q + e; }
+    static __device__ __forceinline__ op_t zero_op()
+    {
+        op_t r;
+        const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+        __builtin_memcpy(&r, &z, 16);
+        return r;
+    }
+    // time samples kmap(q, .) of channel 16w+j from rows row0 .. row0+31 (reversed: 31-k)
+    static __device__ __forceinline__ op_t load_operand(const unsigned char *tile, int urow, int w, int j, int q,
+                                                        bool reversed)
+    {
+        const int col = (16 * w + 4 * (j & 3)) * 2;
+        const int r0 = reversed ? 31 - 8 * q - (j >> 2) : 8 * q + (j >> 2);
+        const int r1 = reversed ? r0 - 4 : r0 + 4;
+        const s16x4 lo = lds_read_tr(tile + r0 * urow + col);
+        const s16x4 hi = lds_read_tr(tile + r1 * urow + col);
+        const short v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        op_t r;
+        __builtin_memcpy(&r, v, 16);
+        return r;
+    }
+    // natural-layout operand of the filter-gradient product: 8 channels of one of two rows;
+    // lane quad q takes row half q>>1 and channels 8*(q&1)..+7 of the wave's 16
+    static __device__ __forceinline__ op_t load_natural(const unsigned char *row_half0,
+                                                        const unsigned char *row_half1, int w, int q)
+    {
+        const unsigned char *p = ((q >> 1) ? row_half1 : row_half0) + (16 * w + 8 * (q & 1)) * 2;
+        const uint4 t4 = *(const uint4 *)p;
+        op_t r;
+        __builtin_memcpy(&r, &t4, 16);
+        return r;
+    }
+    static __device__ __forceinline__ op_t toeplitz(const hraw_t *htab, int doff, int j, int q)
+    {
+        uint16_t v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = htab[doff + j - kmap(q, e) + HPAD];
+        op_t r;
+        __builtin_memcpy(&r, v, 16);
+        return r;
+    }
+};
+
+template <> struct MT<bf16_t> : MT16<bf16x8> {
     static __device__ __forceinline__ f32x4 mfma(op_t a, op_t b, f32x4 c)
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -54,8 +110,7 @@ template <> struct MT<bf16_t> {
     }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 };
-template <> struct MT<f16_t> {
-    typedef f16x8 op_t;
+template <> struct MT<f16_t> : MT16<f16x8> {
     static __device__ __forceinline__ f32x4 mfma(op_t a, op_t b, f32x4 c)
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -71,24 +126,110 @@ template <> struct MT<f16_t> {
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
 };
 
-template <typename T> __device__ __forceinline__ void unpack8(const uint4 &r, float (&f)[8])
-{
-    MT<T>::unpack2(r.x, f[0], f[1]);
-    MT<T>::unpack2(r.y, f[2], f[3]);
-    MT<T>::unpack2(r.z, f[4], f[5]);
-    MT<T>::unpack2(r.w, f[6], f[7]);
-}
-template <typename T> __device__ __forceinline__ uint4 pack8(const float (&f)[8])
-{
-    return make_uint4(MT<T>::pack2(f[0], f[1]), MT<T>::pack2(f[2], f[3]), MT<T>::pack2(f[4], f[5]),
-                      MT<T>::pack2(f[6], f[7]));
-}
+struct F32x8 { float v[8]; };
+template <> struct MT<float> {
+    static constexpr int ES = 4;
+    static constexpr int RW = 2;
+    static constexpr int UPAD = 64;              // consecutive rows start 16 banks apart
+    typedef F32x8 op_t;
+    typedef float hraw_t;
+    // instruction e of the eight contracts time samples 4e .. 4e+3, one per lane quad
+    static __device__ __forceinline__ int kmap(int q, int e) { return 4 * e + q; }
+    static __device__ __forceinline__ op_t zero_op()
+    {
+        op_t r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r.v[e] = 0.f;
+        return r;
+    }
+    static __device__ __forceinline__ op_t load_operand(const unsigned char *tile, int urow, int w, int j, int q,
+                                                        bool reversed)
+    {
+        op_t r;
+        const int col = (16 * w + j) * 4;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int k = kmap(q, e);
+            r.v[e] = *(const float *)(tile + (reversed ? 31 - k : k) * urow + col);
+        }
+        return r;
+    }
+    // element e: row half e>>2, channel 4q + (e&3) of the wave's 16
+    static __device__ __forceinline__ op_t load_natural(const unsigned char *row_half0,
+                                                        const unsigned char *row_half1, int w, int q)
+    {
+        const int col = (16 * w + 4 * q) * 4;
+        const f32x4 a = *(const f32x4 *)(row_half0 + col), b = *(const f32x4 *)(row_half1 + col);
+        op_t r;
+        r.v[0] = a[0]; r.v[1] = a[1]; r.v[2] = a[2]; r.v[3] = a[3];
+        r.v[4] = b[0]; r.v[5] = b[1]; r.v[6] = b[2]; r.v[7] = b[3];
+        return r;
+    }
+    static __device__ __forceinline__ op_t toeplitz(const hraw_t *htab, int doff, int j, int q)
+    {
+        op_t r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r.v[e] = htab[doff + j - kmap(q, e) + HPAD];
+        return r;
+    }
+    static __device__ __forceinline__ f32x4 mfma(const op_t &a, const op_t &b, f32x4 c)
+    {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[e], b.v[e], c, 0, 0, 0);
+        return c;
+    }
+};
 
-// Transposing LDS read: within each block of 16 lanes, lane i receives element (i % 4) of
-// the 8-byte rows addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4 of that block.
-__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char *p)
+// A workgroup of NW waves owns CB = 16*NW adjacent channels; LDS rows are padded (see UPAD;
+// the fp32 result tile: consecutive rows start 4 banks apart).
+template <typename T, int NW> struct Geo {
+    static constexpr int CB = 16 * NW;                          // channels per workgroup
+    static constexpr int LPR = CB / 8;                          // lanes per row in the row layout (8 channels each)
+    static constexpr int UROW = CB * MT<T>::ES + MT<T>::UPAD;   // bytes per LDS row of u / g2
+    static constexpr int YROW = CB * 4 + 16;                    // bytes per LDS row of y2 / du
+    static constexpr int NT = 64 * NW;                          // threads
+};
+
+// A lane's 8 channels of one row: RW 16-byte words.
+template <typename T> struct Row { uint4 w[MT<T>::RW]; };
+
+template <typename T> __device__ __forceinline__ void unpack8(const Row<T> &r, float (&f)[8])
 {
-    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p);
+    if constexpr (MT<T>::ES == 4) {
+        f[0] = __uint_as_float(r.w[0].x); f[1] = __uint_as_float(r.w[0].y);
+        f[2] = __uint_as_float(r.w[0].z); f[3] = __uint_as_float(r.w[0].w);
+        f[4] = __uint_as_float(r.w[1].x); f[5] = __uint_as_float(r.w[1].y);
+        f[6] = __uint_as_float(r.w[1].z); f[7] = __uint_as_float(r.w[1].w);
+    } else {
+        MT<T>::unpack2(r.w[0].x, f[0], f[1]);
+        MT<T>::unpack2(r.w[0].y, f[2], f[3]);
+        MT<T>::unpack2(r.w[0].z, f[4], f[5]);
+        MT<T>::unpack2(r.w[0].w, f[6], f[7]);
+    }
+}
+template <typename T> __device__ __forceinline__ Row<T> pack8(const float (&f)[8])
+{
+    Row<T> r;
+    if constexpr (MT<T>::ES == 4) {
+        r.w[0] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+        r.w[1] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]), __float_as_uint(f[6]), __float_as_uint(f[7]));
+    } else {
+        r.w[0] = make_uint4(MT<T>::pack2(f[0], f[1]), MT<T>::pack2(f[2], f[3]), MT<T>::pack2(f[4], f[5]),
+                            MT<T>::pack2(f[6], f[7]));
+    }
+    return r;
+}
+template <typename T> __device__ __forceinline__ Row<T> zero_row()
+{
+    Row<T> r;
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) r.w[i] = make_uint4(0u, 0u, 0u, 0u);
+    return r;
+}
+template <typename T> __device__ __forceinline__ void lds_store_row(unsigned char *p, const Row<T> &r)
+{
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) *(uint4 *)(p + 16 * i) = r.w[i];
 }
 
 // Streaming accesses: every tensor element is touched once, so loads and stores carry the
@@ -100,6 +241,20 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char *p)
 #define GCG_MFMA_NT 3
 #endif
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <typename T> __device__ __forceinline__ uint4 ldg16(const T *p);
+template <typename T> __device__ __forceinline__ void stg16(T *p, const uint4 &v);
+template <typename T> __device__ __forceinline__ Row<T> ldg_row(const T *p)
+{
+    Row<T> r;
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) r.w[i] = ldg16((const unsigned char *)p + 16 * i);
+    return r;
+}
+template <typename T> __device__ __forceinline__ void stg_row(T *p, const Row<T> &r)
+{
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) stg16((unsigned char *)p + 16 * i, r.w[i]);
+}
 template <typename T> __device__ __forceinline__ uint4 ldg16(const T *p)
 {
 #if GCG_MFMA_NT & 1
@@ -132,18 +287,8 @@ __device__ __forceinline__ int64_t xcd_contiguous_id(int64_t id, int64_t n)
 
 struct MfmaPlan { int ncb, nseg, steps_per_seg, nw; int64_t nsteps, nwg; };
 
-// Operand tile of the banded Toeplitz matrix at row offset doff = (out time) - (in time) of
-// the tile origins: element e of lane (j, q) is the tap for lag doff + j - 8q - e.
-template <typename T>
-__device__ __forceinline__ typename MT<T>::op_t toeplitz_operand(const uint16_t *htab, int doff, int j, int q)
-{
-    uint16_t v[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e) v[e] = htab[doff + j - 8 * q - e + HPAD];
-    typename MT<T>::op_t r;
-    __builtin_memcpy(&r, v, 16);
-    return r;
-}
+// Operand tile of the banded Toeplitz matrix at row offset doff = (out time) - (in time) of the
+// tile origins: element e of lane (j, q) is the tap for lag doff + j - kmap(q, e)  (MT<T>::toeplitz).
 
 // ---------------------------------------------------------------------------- forward
 template <typename T, int NK, int NW>
@@ -152,12 +297,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                                                        T *__restrict__ y, T *__restrict__ y2o,
                                                        T *__restrict__ bxo, Dims dm, MfmaPlan pl)
 {
-    typedef typename MT<T>::op_t op_t;
-    typedef Geo<NW> G;
-    constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW;
+    typedef MT<T> M;
+    typedef typename M::op_t op_t;
+    typedef typename M::hraw_t hraw_t;
+    typedef Geo<T, NW> G;
+    constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW, ES = M::ES;
     __shared__ __attribute__((aligned(16))) unsigned char u_rm[STEP * UROW];
     __shared__ __attribute__((aligned(16))) unsigned char y_st[STEP * YROW];
-    __shared__ uint16_t htab[NW][HTAB];
+    __shared__ hraw_t htab[NW][HTAB];
 
     int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
@@ -166,7 +313,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
     const int r = tid / G::LPR, a = tid % G::LPR;   // row layout: row r of the step, channels 8a..8a+7
-    const int j = l & 15, q = l >> 4;    // matrix layout
+    const int j = l & 15, q = l >> 4;               // matrix layout
     const int64_t d = dm.d, L = dm.L;
     const int64_t c0 = (int64_t)cb * CB;
     const int hl = dm.hl;
@@ -175,18 +322,18 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     {
         const int64_t cw = c0 + 16 * w;
         const int64_t grp = (cw < d) ? cw / dm.dg : 0;
-        const uint16_t *hg = (const uint16_t *)h + grp * hl;
+        const hraw_t *hg = (const hraw_t *)h + grp * hl;
         for (int i = l; i < HTAB; i += 64) {
             const int lag = i - HPAD;
-            htab[w][i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (uint16_t)0;
+            htab[w][i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
         }
     }
     __syncthreads();
     op_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
-        W0[i] = toeplitz_operand<T>(htab[w], 32 * i, j, q);
-        W1[i] = toeplitz_operand<T>(htab[w], 32 * i + 16, j, q);
+        W0[i] = M::toeplitz(htab[w], 32 * i, j, q);
+        W1[i] = M::toeplitz(htab[w], 32 * i + 16, j, q);
     }
 
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
@@ -195,30 +342,24 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 
     const bool cvalid = c0 + 8 * a < d;
     const int64_t col = b * L * d + c0 + 8 * a;            // element offset of this lane's columns
-    const int row_in_step = r;
 
     op_t A[NK];
 #pragma unroll
-    for (int i = 0; i < NK; ++i) {
-        uint4 z = make_uint4(0u, 0u, 0u, 0u);
-        __builtin_memcpy(&A[i], &z, 16);
-    }
+    for (int i = 0; i < NK; ++i) A[i] = M::zero_op();
 
-    unsigned char *u_wr = u_rm + row_in_step * UROW + 16 * a;
-    const unsigned char *u_rd = u_rm + (8 * q + (j >> 2)) * UROW + (16 * w + 4 * (j & 3)) * 2;
+    unsigned char *u_wr = u_rm + r * UROW + 8 * ES * a;
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
-    const unsigned char *y_rd = y_st + row_in_step * YROW + 32 * a;
+    const unsigned char *y_rd = y_st + r * YROW + 32 * a;
 
-    uint4 xr, Br, Cr;
-    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
-    auto fetch = [&](int64_t s, uint4 &xo, uint4 &Bo, uint4 &Co) {
-        const int64_t t = s * STEP + row_in_step;
-        xo = zero4; Bo = zero4; Co = zero4;
+    Row<T> xr, Br, Cr;
+    auto fetch = [&](int64_t s, Row<T> &xo, Row<T> &Bo, Row<T> &Co) {
+        const int64_t t = s * STEP + r;
+        xo = zero_row<T>(); Bo = zero_row<T>(); Co = zero_row<T>();
         if (cvalid && t < L) {
             const int64_t o = col + t * d;
-            xo = ldg16(x + o);
-            Bo = ldg16(B + o);
-            if (s >= s_lo) Co = ldg16(C + o);
+            xo = ldg_row(x + o);
+            Bo = ldg_row(B + o);
+            if (s >= s_lo) Co = ldg_row(C + o);
         }
     };
     fetch(s_first, xr, Br, Cr);
@@ -229,7 +370,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
                 const bool main_step = s >= s_lo;
-                uint4 xn = zero4, Bn = zero4, Cn = zero4;
+                Row<T> xn = zero_row<T>(), Bn = zero_row<T>(), Cn = zero_row<T>();
                 if (s + 1 < s_hi) fetch(s + 1, xn, Bn, Cn);
 
                 float xf[8], Bf[8], uf[8];
@@ -237,24 +378,19 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                 unpack8<T>(Br, Bf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
-                const uint4 up = pack8<T>(uf);
-                *(uint4 *)u_wr = up;
-                const int64_t t = s * STEP + row_in_step;
+                const Row<T> up = pack8<T>(uf);
+                lds_store_row<T>(u_wr, up);
+                const int64_t t = s * STEP + r;
                 const bool store_ok = main_step && cvalid && t < L;
-                if (bxo && store_ok) stg16(bxo + col + t * d, up);
+                if (bxo && store_ok) stg_row(bxo + col + t * d, up);
                 __syncthreads();
-                {
-                    const s16x4 lo = lds_read_tr(u_rd);
-                    const s16x4 hi = lds_read_tr(u_rd + 4 * UROW);
-                    short v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    __builtin_memcpy(&A[ph], v, 16);
-                }
+                A[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
                 if (main_step) {
                     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int i = 0; i < NK; ++i) {
-                        acc0 = MT<T>::mfma(A[(ph - i + NK) % NK], W0[i], acc0);
-                        acc1 = MT<T>::mfma(A[(ph - i + NK) % NK], W1[i], acc1);
+                        acc0 = M::mfma(A[(ph - i + NK) % NK], W0[i], acc0);
+                        acc1 = M::mfma(A[(ph - i + NK) % NK], W1[i], acc1);
                     }
                     *(f32x4 *)y_wr = acc0;
                     *(f32x4 *)(y_wr + 16 * YROW) = acc1;
@@ -268,8 +404,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                     unpack8<T>(Cr, Cf);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) yf[e] = Cf[e] * y2f[e];
-                    stg16(y + col + t * d, pack8<T>(yf));
-                    if (y2o) stg16(y2o + col + t * d, pack8<T>(y2f));
+                    stg_row(y + col + t * d, pack8<T>(yf));
+                    if (y2o) stg_row(y2o + col + t * d, pack8<T>(y2f));
                 }
                 xr = xn; Br = Bn; Cr = Cn;
                 ++s;
@@ -293,7 +429,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 // Filter gradient: dh[hl-1-lag] = sum g2[t,c] u[t-lag,c].  For the new u step the products
 // against the NK g2 steps in the ring are accumulated as ND = 2*NK-1 tiles
 //   P_delta[i][j] += sum_c G2[32*sigma + 16*delta + i, c] * U[32*sigma + j, c]
-// (a 16x16x32 MFMA contracts 16 channels x 2 row-halves), lag = 16*delta + i - j.  At the
+// (one 32-deep product contracts 16 channels x 2 row halves), lag = 16*delta + i - j.  At the
 // end the diagonals of the P tiles are summed in a fixed order into per-wave partials in
 // the workspace, and a second kernel adds the partials in a fixed order.
 template <typename T, int NK, int NW>
@@ -303,9 +439,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                                                        T *__restrict__ dB, T *__restrict__ dC,
                                                        float *__restrict__ ws, Dims dm, MfmaPlan pl)
 {
-    typedef typename MT<T>::op_t op_t;
-    typedef Geo<NW> G;
-    constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW;
+    typedef MT<T> M;
+    typedef typename M::op_t op_t;
+    typedef typename M::hraw_t hraw_t;
+    typedef Geo<T, NW> G;
+    constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW, ES = M::ES;
     constexpr int ND = 2 * NK - 1;
     constexpr int RING_ROWS = STEP * NK;
     constexpr int OFF_U = 0;                                // u of the current step, row-major
@@ -313,14 +451,15 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     constexpr int OFF_Y = OFF_G + RING_ROWS * UROW;         // y2 tile, fp32, row-major
     constexpr int OFF_D = OFF_Y + STEP * YROW;              // du tile, fp32, row-major
     constexpr int OFF_H = OFF_D + STEP * YROW;              // filter tables
-    constexpr int LDS_MAIN = OFF_H + NW * HTAB * 2;
+    constexpr int LDS_MAIN = OFF_H + NW * HTAB * (int)sizeof(hraw_t);
     constexpr int LDS_TAIL = NW * ND * 256 * 4;             // P tiles at the end
     constexpr int LDS_BYTES = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
     unsigned char *u_rm = smem + OFF_U, *g_rm = smem + OFF_G, *y_st = smem + OFF_Y, *d_st = smem + OFF_D;
-    uint16_t *htab = (uint16_t *)(smem + OFF_H);
+    hraw_t *htab = (hraw_t *)(smem + OFF_H);
 
-    int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int64_t wg_id = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    int64_t wg = wg_id;
     const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
     const int seg = (int)(wg % pl.nseg);
     const int64_t b = wg / pl.nseg;
@@ -335,18 +474,18 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
 
     {
         const int64_t grp = wave_valid ? (c0 + 16 * w) / dm.dg : 0;
-        const uint16_t *hg = (const uint16_t *)h + grp * hl;
+        const hraw_t *hg = (const hraw_t *)h + grp * hl;
         for (int i = l; i < HTAB; i += 64) {
             const int lag = i - HPAD;
-            htab[w * HTAB + i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (uint16_t)0;
+            htab[w * HTAB + i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
         }
     }
     __syncthreads();
     op_t W0[NK], W1[NK];
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
-        W0[i] = toeplitz_operand<T>(htab + w * HTAB, 32 * i, j, q);
-        W1[i] = toeplitz_operand<T>(htab + w * HTAB, 32 * i + 16, j, q);
+        W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
+        W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
     }
 
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
@@ -355,50 +494,42 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
 
     const bool cvalid = c0 + 8 * a < d;
     const int64_t col = b * L * d + c0 + 8 * a;
-    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
 
     op_t Au[NK], Ag[NK];      // Au[k]: u operand of a step; Ag[k]: time-reversed g2 operand of a step
-    uint4 dyq[NK];            // dy rows (row layout) waiting for their y2
+    Row<T> dyq[NK];           // dy rows (row layout) waiting for their y2
     f32x4 P[ND];
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
-        __builtin_memcpy(&Au[i], &zero4, 16);
-        __builtin_memcpy(&Ag[i], &zero4, 16);
-        dyq[i] = zero4;
+        Au[i] = M::zero_op();
+        Ag[i] = M::zero_op();
+        dyq[i] = zero_row<T>();
     }
 #pragma unroll
     for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // LDS addresses of this lane
-    unsigned char *u_wr = u_rm + r * UROW + 16 * a;
-    const int g_wr_off = r * UROW + 16 * a;                                   // + slot * STEP * UROW
-    const int tr_col = (16 * w + 4 * (j & 3)) * 2;
-    const unsigned char *u_tr = u_rm + (8 * q + (j >> 2)) * UROW + tr_col;
-    const int g_tr_off = (31 - 8 * q - (j >> 2)) * UROW + tr_col;             // reversed time order
-    const int nat_col = (16 * w + 8 * (q & 1)) * 2;                           // natural operand: 8 channels
-    const int nat_row = 16 * (q >> 1) + j;                                    // row half by lane quad
-    const unsigned char *u_nat = u_rm + nat_row * UROW + nat_col;
+    const int rm_off = r * UROW + 8 * ES * a;                                 // row layout, 8 channels
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
     unsigned char *d_wr = d_st + (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
     const unsigned char *d_rd = d_st + r * YROW + 32 * a;
 
-    auto fetch = [&](int64_t sg, uint4 &xo, uint4 &Bo, uint4 &dyo, uint4 &Co) {
-        xo = zero4; Bo = zero4; dyo = zero4; Co = zero4;
+    auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
+        xo = zero_row<T>(); Bo = zero_row<T>(); dyo = zero_row<T>(); Co = zero_row<T>();
         if (cvalid) {
             const int64_t t = sg * STEP + r;
             if (t >= 0 && t < L) {
-                xo = ldg16(x + col + t * d);
-                Bo = ldg16(B + col + t * d);
+                xo = ldg_row(x + col + t * d);
+                Bo = ldg_row(B + col + t * d);
             }
             const int64_t t2 = t + (NK - 1) * STEP;
             if (t2 >= 0 && t2 < L) {
-                dyo = ldg16(dy + col + t2 * d);
-                Co = ldg16(C + col + t2 * d);
+                dyo = ldg_row(dy + col + t2 * d);
+                Co = ldg_row(C + col + t2 * d);
             }
         }
     };
-    uint4 xr, Br, dyr, Cr;
+    Row<T> xr, Br, dyr, Cr;
     fetch(s_first, xr, Br, dyr, Cr);
 
     int64_t s = s_first;
@@ -408,7 +539,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
             if (s < s_hi) {
                 const bool main_step = s >= s_lo;
                 const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
-                uint4 xn = zero4, Bn = zero4, dyn = zero4, Cn = zero4;
+                Row<T> xn = zero_row<T>(), Bn = zero_row<T>(), dyn = zero_row<T>(), Cn = zero_row<T>();
                 if (s + 1 < s_hi) fetch(s + 1, xn, Bn, dyn, Cn);
 
                 float xf[8], Bf[8], tf[8], cf[8], pf[8];
@@ -416,54 +547,42 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                 unpack8<T>(Br, Bf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[e] = xf[e] * Bf[e];
-                *(uint4 *)u_wr = pack8<T>(pf);
+                lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
                 unpack8<T>(dyr, tf);
                 unpack8<T>(Cr, cf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[e] = tf[e] * cf[e];
-                *(uint4 *)(g_rm + slot_new * STEP * UROW + g_wr_off) = pack8<T>(pf);
+                unsigned char *g_slot = g_rm + slot_new * STEP * UROW;
+                lds_store_row<T>(g_slot + rm_off, pack8<T>(pf));
                 dyq[slot_new] = dyr;
                 __syncthreads();
-                {
-                    const s16x4 lo = lds_read_tr(u_tr);
-                    const s16x4 hi = lds_read_tr(u_tr + 4 * UROW);
-                    short v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    __builtin_memcpy(&Au[ph], v, 16);
-                    const unsigned char *gp = g_rm + slot_new * STEP * UROW + g_tr_off;
-                    const s16x4 glo = lds_read_tr(gp);
-                    const s16x4 ghi = lds_read_tr(gp - 4 * UROW);
-                    short gv[8] = {glo[0], glo[1], glo[2], glo[3], ghi[0], ghi[1], ghi[2], ghi[3]};
-                    __builtin_memcpy(&Ag[slot_new], gv, 16);
-                }
+                Au[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
+                Ag[slot_new] = M::load_operand(g_slot, UROW, w, j, q, true);
                 if (main_step) {
                     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
                     f32x4 dac0 = {0.f, 0.f, 0.f, 0.f}, dac1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int i = 0; i < NK; ++i) {
-                        acc0 = MT<T>::mfma(Au[(ph - i + NK) % NK], W0[i], acc0);
-                        acc1 = MT<T>::mfma(Au[(ph - i + NK) % NK], W1[i], acc1);
+                        acc0 = M::mfma(Au[(ph - i + NK) % NK], W0[i], acc0);
+                        acc1 = M::mfma(Au[(ph - i + NK) % NK], W1[i], acc1);
                         // g2 of step s+i sits in slot (ph+i) % NK
-                        dac0 = MT<T>::mfma(Ag[(ph + i) % NK], W1[i], dac0);   // output rows 0..15
-                        dac1 = MT<T>::mfma(Ag[(ph + i) % NK], W0[i], dac1);   // output rows 16..31
+                        dac0 = M::mfma(Ag[(ph + i) % NK], W1[i], dac0);   // output rows 0..15
+                        dac1 = M::mfma(Ag[(ph + i) % NK], W0[i], dac1);   // output rows 16..31
                     }
                     *(f32x4 *)y_wr = acc0;
                     *(f32x4 *)(y_wr + 16 * YROW) = acc1;
                     *(f32x4 *)d_wr = dac0;
                     *(f32x4 *)(d_wr + 16 * YROW) = dac1;
-                    // filter-gradient tiles: natural-layout operands, 8 channels of two row halves
-                    op_t un;
-                    {
-                        const uint4 t4 = *(const uint4 *)u_nat;
-                        __builtin_memcpy(&un, &t4, 16);
-                    }
+                    // filter-gradient tiles: natural-layout operands (rows j and 16+j of a 32-row window)
+                    const op_t un = M::load_natural(u_rm + j * UROW, u_rm + (16 + j) * UROW, w, q);
 #pragma unroll
                     for (int dl = 0; dl < ND; ++dl) {
-                        int row = STEP * ph + 16 * dl + nat_row;           // ring row of this lane's g2 row
-                        row = (row >= RING_ROWS) ? row - RING_ROWS : row;
-                        const uint4 t4 = *(const uint4 *)(g_rm + row * UROW + nat_col);
-                        op_t gn;
-                        __builtin_memcpy(&gn, &t4, 16);
-                        P[dl] = MT<T>::mfma(gn, un, P[dl]);
+                        int row0 = STEP * ph + 16 * dl + j;              // ring rows of the window's two halves
+                        int row1 = row0 + 16;
+                        row0 = (row0 >= RING_ROWS) ? row0 - RING_ROWS : row0;
+                        row1 = (row1 >= RING_ROWS) ? row1 - RING_ROWS : row1;
+                        const op_t gn = M::load_natural(g_rm + row0 * UROW, g_rm + row1 * UROW, w, q);
+                        P[dl] = M::mfma(gn, un, P[dl]);
                     }
                 }
                 __syncthreads();
@@ -478,7 +597,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         unpack8<T>(dyq[ph], dyf);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = dyf[e] * y2f[e];
-                        stg16(dC + o, pack8<T>(of));
+                        stg_row(dC + o, pack8<T>(of));
                     }
                     {
                         const f32x4 p0 = *(const f32x4 *)d_rd;
@@ -487,10 +606,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         float of[8];
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * Bf[e];
-                        stg16(dx + o, pack8<T>(of));
+                        stg_row(dx + o, pack8<T>(of));
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * xf[e];
-                        stg16(dB + o, pack8<T>(of));
+                        stg_row(dB + o, pack8<T>(of));
                     }
                 }
                 xr = xn; Br = Bn; dyr = dyn; Cr = Cn;
@@ -508,7 +627,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         for (int v = 0; v < 4; ++v) pt[dl * 256 + (4 * q + v) * 16 + j] = P[dl][v];
     __syncthreads();
     if (wave_valid) {
-        float *out = ws + ((size_t)xcd_contiguous_id(blockIdx.x, gridDim.x) * NW + w) * 128;
+        float *out = ws + ((size_t)wg_id * NW + w) * 128;
         for (int lag = l; lag < 128; lag += 64) {
             const int d0 = lag >> 4, rr = lag & 15;
             float sum = 0.f;
@@ -561,11 +680,13 @@ int env_int(const char *name, int dflt)
 
 // Waves per workgroup: wider workgroups read wider rows (16*NW channels, 32*NW bytes), which
 // the memory system rewards; narrow tensors fall back to what their width fills.
-int choose_nw(const Dims &dm)
+// fp32 doubles the register state per wave (operand tiles hold 8 floats), which caps the
+// forward at 8 waves and the backward at 4.
+int choose_nw(const Dims &dm, bool fp32)
 {
     static const int forced = env_int("GCG_MFMA_NW", 0);   // tuning override: 4, 8 or 16
-    if (forced == 4 || forced == 8 || forced == 16) return forced;
-    if (dm.d >= 256) return 16;
+    if (forced == 4 || forced == 8 || (forced == 16 && !fp32)) return forced;
+    if (dm.d >= 256 && !fp32) return 16;
     if (dm.d >= 128) return 8;
     return 4;
 }
@@ -600,7 +721,8 @@ template <typename T, int NK, int NW>
 int fwd_launch(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
                const Dims &dm, hipStream_t st)
 {
-    const MfmaPlan p = plan(dm, NW, 16, 16);   // ~124 registers: 4 waves per SIMD
+    // 16-bit: ~112 registers, 4 waves per SIMD; fp32: ~200 registers, 2 waves per SIMD
+    const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((mfma_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)x,
                        (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
@@ -611,11 +733,12 @@ template <typename T, int NK>
 int fwd_nk(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
            const Dims &dm, hipStream_t st)
 {
-    switch (choose_nw(dm)) {
-    case 16: return fwd_launch<T, NK, 16>(x, B, C, h, y, y2, bx, dm, st);
-    case 8:  return fwd_launch<T, NK, 8>(x, B, C, h, y, y2, bx, dm, st);
-    default: return fwd_launch<T, NK, 4>(x, B, C, h, y, y2, bx, dm, st);
+    const int nw = choose_nw(dm, sizeof(T) == 4);
+    if constexpr (sizeof(T) == 2) {
+        if (nw == 16) return fwd_launch<T, NK, 16>(x, B, C, h, y, y2, bx, dm, st);
     }
+    if (nw == 8) return fwd_launch<T, NK, 8>(x, B, C, h, y, y2, bx, dm, st);
+    return fwd_launch<T, NK, 4>(x, B, C, h, y, y2, bx, dm, st);
 }
 
 template <typename T>
@@ -635,7 +758,8 @@ int fwd_t(const void *x, const void *B, const void *C, const void *h, void *y, v
 
 bool mfma_supported(int dtype, const Dims &dm)
 {
-    return (dtype == GCG_BF16 || dtype == GCG_F16) && dm.hl <= 128 && dm.dg % 16 == 0;
+    (void)dtype;   // bf16, f16 and fp32 all have a matrix-core form
+    return dm.hl <= 128 && dm.dg % 16 == 0;
 }
 
 int mfma_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h, void *y,
@@ -643,6 +767,7 @@ int mfma_fwd_launch(int dtype, const void *x, const void *B, const void *C, cons
 {
     if (dtype == GCG_BF16) return fwd_t<bf16_t>(x, B, C, h, y, y2, bx, dm, st);
     if (dtype == GCG_F16) return fwd_t<f16_t>(x, B, C, h, y, y2, bx, dm, st);
+    if (dtype == GCG_F32) return fwd_t<float>(x, B, C, h, y, y2, bx, dm, st);
     return (int)hipErrorInvalidValue;
 }
 
@@ -652,20 +777,21 @@ namespace {
 
 // The backward holds about twice the forward's register state per wave, so it runs two
 // waves per SIMD and at most 8 waves (128 channels, 256-byte rows) per workgroup.
-int choose_nw_bwd(const Dims &dm)
+int choose_nw_bwd(const Dims &dm, bool fp32)
 {
     static const int forced = env_int("GCG_MFMA_BWD_NW", 0);   // tuning override: 4 or 8
-    if (forced == 4 || forced == 8) return forced;
-    return dm.d >= 128 ? 8 : 4;
+    if (forced == 4 || (forced == 8 && !fp32)) return forced;
+    return (dm.d >= 128 && !fp32) ? 8 : 4;
 }
 
-MfmaPlan plan_bwd(const Dims &dm) { return plan(dm, choose_nw_bwd(dm), 16, 8); }
+// 16-bit: two waves per SIMD (8 per CU); fp32: one (4 per CU)
+MfmaPlan plan_bwd(const Dims &dm, bool fp32) { return plan(dm, choose_nw_bwd(dm, fp32), 16, fp32 ? 4 : 8); }
 
 template <typename T, int NK, int NW>
 int bwd_launch(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
                void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    const MfmaPlan p = plan_bwd(dm);
+    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
@@ -682,7 +808,9 @@ template <typename T, int NK>
 int bwd_nk(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
            void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    if (choose_nw_bwd(dm) == 8) return bwd_launch<T, NK, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    if constexpr (sizeof(T) == 2) {
+        if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    }
     return bwd_launch<T, NK, 4>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
 }
 
@@ -701,9 +829,9 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
 
 } // namespace
 
-size_t mfma_bwd_workspace(const Dims &dm)
+size_t mfma_bwd_workspace(int dtype, const Dims &dm)
 {
-    const MfmaPlan p = plan_bwd(dm);
+    const MfmaPlan p = plan_bwd(dm, dtype == GCG_F32);
     return (size_t)p.nwg * p.nw * 128 * sizeof(float);
 }
 
@@ -712,6 +840,7 @@ int mfma_bwd_launch(int dtype, const void *dy, const void *x, const void *B, con
 {
     if (dtype == GCG_BF16) return bwd_t<bf16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     if (dtype == GCG_F16) return bwd_t<f16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    if (dtype == GCG_F32) return bwd_t<float>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     return (int)hipErrorInvalidValue;
 }
 

@@ -50,7 +50,6 @@ def test_argument_errors_need_no_device(gcg_lib):
     assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 7, 0, 9, None) == -1
     # forced family that cannot take the shape
     assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 200, 1, 3, None) == -2   # mfma, hl > 128
-    assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 128, 0, 3, None) == -2   # mfma, fp32
     assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 16, 9, 0, 2, None) == -2     # window, hl > 8
     assert gcg_lib.gcg_fwd(p, p, p, p, p, None, None, 1, 64, 2, 8, 64, 1, 3, None) == -2     # mfma, dg % 16
     # backward without workspace
@@ -66,7 +65,8 @@ def test_algo_selection(gcg_lib):
     assert _lib.select_algo(2, 8192, 256, 16, 128, bf, backward=True) == "mfma"
     assert _lib.select_algo(1, 32768, 512, 16, 7, bf) == "window"         # Hyena-SE
     assert _lib.select_algo(1, 2048, 16, 16, 7, f32) == "window"          # fp32 SE config
-    assert _lib.select_algo(2, 8192, 256, 16, 128, f32) == "direct"       # fp32 keeps full precision on the VALU
+    assert _lib.select_algo(2, 8192, 256, 16, 128, f32) == "mfma"         # fp32 MFMA keeps fp32 accuracy
+    assert _lib.select_algo(2, 8192, 256, 4, 128, f32) == "direct"        # narrow groups stay on the vector ALUs
     assert _lib.select_algo(1, 512, 4, 16, 300, bf) == "direct"           # filter longer than a chunk
     assert _lib.select_algo(1, 512, 64, 1, 64, bf) == "direct"            # one channel per filter
 

@@ -20,7 +20,7 @@ def algos_for(hl, dg, dtype):
     out = ["direct"]
     if hl <= 8 and dg % 4 == 0:
         out.append("window")
-    if hl <= 128 and dg % 16 == 0 and dtype != torch.float32:
+    if hl <= 128 and dg % 16 == 0:
         out.append("mfma")
     return out
 
