@@ -31,7 +31,7 @@ HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 
 # HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script scaled by a 256 MiB copy in the same run (profiles/mr_fwdbwd_7b_hbm_traffic.md).
+# this script scaled by a 256 MiB copy in the same run (the repository keeps the profiler summary).
 # Counters cannot be read from inside the process; configurations without a profile report null.
 MEASURED_TRAFFIC_BYTES = {
     ("mr_fwdbwd_7b", "gcg_bwd hl=128 mfma"): 935785 * 1024,

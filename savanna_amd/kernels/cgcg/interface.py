@@ -46,20 +46,11 @@ class TwoPassChunkedGateConvGate(torch.autograd.Function):
 
 
 def two_pass_chunked_gate_conv_gate(
-    x: torch.Tensor,
-    B: torch.Tensor,
-    C: torch.Tensor,
-    h: torch.Tensor,
-    bs: int,
-    seqlen: int,
-    g: int,
-    dg: int,
+    x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, h: torch.Tensor,
+    bs: int, seqlen: int, g: int, dg: int,
     schedule: str = "default",
-    fwd_autotune: bool = False,
-    bwd_autotune: bool = True,
-    fused_bwd: bool = True,
-    fwd_kernel_cfg: FwdKernelConfigRefactor = None,
-    bwd_kernel_cfg: BwdKernelConfigRefactor = None,
+    fwd_autotune: bool = False, bwd_autotune: bool = True, fused_bwd: bool = True,
+    fwd_kernel_cfg: FwdKernelConfigRefactor = None, bwd_kernel_cfg: BwdKernelConfigRefactor = None,
 ):
     """Gate -> causal FIR convolution -> gate, differentiable in x, B, C and h.
 

@@ -8,25 +8,13 @@ from .... import _lib
 
 
 def two_pass_fwd_grouped(
-    x: torch.Tensor,
-    B: torch.Tensor,
-    C: torch.Tensor,
-    h: torch.Tensor,
-    y: torch.Tensor = None,
-    return_bx: bool = True,
-    return_y2: bool = True,
-    verbose: bool = False,
-    schedule: str = "default",
-    autotune: bool = True,
-    CHUNK_SIZE: int = None,
-    BLOCK_D: int = None,
-    CHUNK_TILES_PER_PROGRAM: int = 1,
-    THREADBLOCK_SWIZZLE: str = "row",
-    num_warps: int = 4,
-    num_stages: int = 3,
-    num_ctas: int = 1,
-    maxnreg: int = None,
-    warmup: bool = False,
+    x: torch.Tensor, B: torch.Tensor, C: torch.Tensor, h: torch.Tensor,
+    y: torch.Tensor = None, return_bx: bool = True, return_y2: bool = True,
+    verbose: bool = False, schedule: str = "default", autotune: bool = True,
+    # Triton tiling arguments of the reference signature, accepted and ignored
+    CHUNK_SIZE: int = None, BLOCK_D: int = None, CHUNK_TILES_PER_PROGRAM: int = 1,
+    THREADBLOCK_SWIZZLE: str = "row", num_warps: int = 4, num_stages: int = 3, num_ctas: int = 1,
+    maxnreg: int = None, warmup: bool = False,
     algo="auto",
 ):
     """Gated causal convolution y = C * conv(B * x, h) on the GPU.

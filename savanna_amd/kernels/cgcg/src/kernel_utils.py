@@ -19,15 +19,15 @@ _SWIZZLES = ("row", "col")
 
 @dataclass
 class KernelConfig:
-    CHUNK_SIZE: int
-    BLOCK_D: int
-    THREADBLOCK_SWIZZLE: str
-    schedule: str = "default"
-    USE_TMA: bool = False
+    CHUNK_SIZE: int                       # Triton: time rows per program
+    BLOCK_D: int                          # Triton: channels per program
+    THREADBLOCK_SWIZZLE: str              # "row" or "col" program ordering
+    schedule: str = "default"             # "default" or "persistent"
+    USE_TMA: bool = False                 # Hopper tensor-memory-accelerator variants
     FLUSH_TMA: bool = False
-    NUM_PIPELINE_STAGES: int = 0
+    NUM_PIPELINE_STAGES: int = 0          # tl.range pipelining, 0 or 1
     CHUNK_TILES_PER_PROGRAM: int = 1
-    num_warps: int = 4
+    num_warps: int = 4                    # Triton launch knobs from here on
     num_stages: int = 3
     num_ctas: int = 1
     maxnreg: Optional[int] = None
@@ -58,14 +58,14 @@ class KernelConfig:
 class FwdKernelConfigRefactor(KernelConfig):
     name: str = "fwd"
     version: str = "refactor"
-    RETURN_BX: bool = True
-    RETURN_Y2: bool = True
+    RETURN_BX: bool = True                # the reference forward also returns B*x ...
+    RETURN_Y2: bool = True                # ... and the convolution before the post-gate
 
 
 @dataclass
 class BwdKernelConfigRefactor:
     name: str = "bwd-refactor"
-    pre_conv_BLOCK_X: int = 128
+    pre_conv_BLOCK_X: int = 128           # tiles of the reference's gate-and-transpose kernels
     pre_conv_BLOCK_Y: int = 128
     pre_conv_num_warps: int = 4
     post_conv_BLOCK_X: int = 128

@@ -66,7 +66,7 @@ WORKLOADS = {
     "mr_fwd_1m": Workload("mr_fwd_1m", 1, 1048576, 256, 16, (128,), torch.bfloat16, False,
                           "Hyena-MR forward, bf16, B=1 L=1048576 D=4096 G=256 hl=128"),
 }
-# order of BASELINE.json's `configs`
+# the order in which the benchmark reports them
 WORKLOAD_ORDER = ("se_fwd_fp32", "mr_fwd_7b", "mr_fwdbwd_7b", "se_mr_fwdbwd_40b", "mr_fwd_1m")
 
 
