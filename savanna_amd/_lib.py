@@ -94,13 +94,17 @@ def _require_gpu(t: torch.Tensor) -> None:
         )
 
 
-def fwd(x, B, C, h, return_bx=False, return_y2=False, algo=ALGO_AUTO):
-    """y (and optionally bx, y2) for contiguous (bs, L, g, dg) inputs and (g, 1, hl) filter."""
+def fwd(x, B, C, h, return_bx=False, return_y2=False, algo=ALGO_AUTO, out=None):
+    """y (and optionally bx, y2) for contiguous (bs, L, g, dg) inputs and (g, 1, hl) filter.
+    ``out``: optional pre-allocated contiguous tensor of x's shape, dtype and device for y."""
     lib = load()
     _require_gpu(x)
     bs, L, g, dg = x.shape
     hl = h.shape[-1]
-    y = torch.empty_like(x)
+    if out is not None:
+        if out.shape != x.shape or out.dtype != x.dtype or out.device != x.device or not out.is_contiguous():
+            raise ValueError("out must be a contiguous tensor with the shape, dtype and device of x")
+    y = out if out is not None else torch.empty_like(x)
     y2 = torch.empty_like(x) if return_y2 else None
     bx = torch.empty_like(x) if return_bx else None
     if x.numel() == 0:

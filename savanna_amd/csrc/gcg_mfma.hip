@@ -338,12 +338,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
-    const int64_t s_first = (s_lo - (NK - 1) > 0) ? s_lo - (NK - 1) : 0;
 
     const bool cvalid = c0 + 8 * a < d;
     const int64_t col = b * L * d + c0 + 8 * a;            // element offset of this lane's columns
 
-    op_t A[NK];
+    op_t A[NK];            // A[(ph - i + NK) % NK]: operand of step s-i while step s runs in phase ph
 #pragma unroll
     for (int i = 0; i < NK; ++i) A[i] = M::zero_op();
 
@@ -359,17 +358,46 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
             const int64_t o = col + t * d;
             xo = ldg_row(x + o);
             Bo = ldg_row(B + o);
-            if (s >= s_lo) Co = ldg_row(C + o);
+            Co = ldg_row(C + o);
         }
     };
-    fetch(s_first, xr, Br, Cr);
+    fetch(s_lo, xr, Br, Cr);
 
-    int64_t s = s_first;
+    // A segment that starts inside the sequence first rebuilds the operands of the NK-1 steps
+    // before it.  Their rows are requested together, so the replay costs one memory latency
+    // instead of NK-1; step s_lo-i lands in ring slot NK-i, where phase 0 expects it.
+    if constexpr (NK > 1) {
+        if (s_lo > 0) {
+            Row<T> wx[NK - 1], wB[NK - 1];
+#pragma unroll
+            for (int i = 1; i < NK; ++i) {
+                const int64_t t = (s_lo - i) * STEP + r;
+                wx[i - 1] = zero_row<T>(); wB[i - 1] = zero_row<T>();
+                if (cvalid && t >= 0) {
+                    wx[i - 1] = ldg_row(x + col + t * d);
+                    wB[i - 1] = ldg_row(B + col + t * d);
+                }
+            }
+#pragma unroll
+            for (int i = 1; i < NK; ++i) {
+                float xf[8], Bf[8], uf[8];
+                unpack8<T>(wx[i - 1], xf);
+                unpack8<T>(wB[i - 1], Bf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
+                lds_store_row<T>(u_wr, pack8<T>(uf));
+                __syncthreads();
+                A[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
+                __syncthreads();
+            }
+        }
+    }
+
+    int64_t s = s_lo;
     while (s < s_hi) {
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
-                const bool main_step = s >= s_lo;
                 Row<T> xn = zero_row<T>(), Bn = zero_row<T>(), Cn = zero_row<T>();
                 if (s + 1 < s_hi) fetch(s + 1, xn, Bn, Cn);
 
@@ -381,11 +409,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                 const Row<T> up = pack8<T>(uf);
                 lds_store_row<T>(u_wr, up);
                 const int64_t t = s * STEP + r;
-                const bool store_ok = main_step && cvalid && t < L;
+                const bool store_ok = cvalid && t < L;
                 if (bxo && store_ok) stg_row(bxo + col + t * d, up);
                 __syncthreads();
                 A[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
-                if (main_step) {
+                {
                     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int i = 0; i < NK; ++i) {
@@ -490,13 +518,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
 
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
-    const int64_t s_first = s_lo - (NK - 1);                // may be negative: those rows read as zero
 
     const bool cvalid = c0 + 8 * a < d;
     const int64_t col = b * L * d + c0 + 8 * a;
 
-    op_t Au[NK], Ag[NK];      // Au[k]: u operand of a step; Ag[k]: time-reversed g2 operand of a step
-    Row<T> dyq[NK];           // dy rows (row layout) waiting for their y2
+    // While step s runs in phase ph:  Au[(ph - i + NK) % NK] is the u operand of step s-i,
+    // Ag[(ph + i) % NK] the time-reversed g2 operand of step s+i, dyq[(ph + i) % NK] dy of step s+i.
+    op_t Au[NK], Ag[NK];
+    Row<T> dyq[NK];
     f32x4 P[ND];
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
@@ -514,6 +543,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
     const unsigned char *d_rd = d_st + r * YROW + 32 * a;
 
+    // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the sequence)
     auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
         xo = zero_row<T>(); Bo = zero_row<T>(); dyo = zero_row<T>(); Co = zero_row<T>();
         if (cvalid) {
@@ -530,14 +560,43 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         }
     };
     Row<T> xr, Br, dyr, Cr;
-    fetch(s_first, xr, Br, dyr, Cr);
+    fetch(s_lo, xr, Br, dyr, Cr);
 
-    int64_t s = s_first;
+    // Lead-in: u of the NK-1 steps before the segment and g2 of its first NK-1 steps, i.e. the
+    // rows iterations s_lo-NK+1 .. s_lo-1 would have brought.  They are requested together,
+    // so the lead-in costs one memory latency instead of NK-1.
+    if constexpr (NK > 1) {
+        Row<T> wx[NK - 1], wB[NK - 1], wdy[NK - 1], wC[NK - 1];
+#pragma unroll
+        for (int i = 1; i < NK; ++i) fetch(s_lo - i, wx[i - 1], wB[i - 1], wdy[i - 1], wC[i - 1]);
+#pragma unroll
+        for (int i = 1; i < NK; ++i) {
+            // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
+            float f0[8], f1[8], pf[8];
+            unpack8<T>(wx[i - 1], f0);
+            unpack8<T>(wB[i - 1], f1);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
+            lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
+            unpack8<T>(wdy[i - 1], f0);
+            unpack8<T>(wC[i - 1], f1);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
+            unsigned char *g_slot = g_rm + (NK - 1 - i) * STEP * UROW;
+            lds_store_row<T>(g_slot + rm_off, pack8<T>(pf));
+            dyq[NK - 1 - i] = wdy[i - 1];
+            __syncthreads();
+            Au[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
+            Ag[NK - 1 - i] = M::load_operand(g_slot, UROW, w, j, q, true);
+            __syncthreads();
+        }
+    }
+
+    int64_t s = s_lo;
     while (s < s_hi) {
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
-                const bool main_step = s >= s_lo;
                 const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
                 Row<T> xn = zero_row<T>(), Bn = zero_row<T>(), dyn = zero_row<T>(), Cn = zero_row<T>();
                 if (s + 1 < s_hi) fetch(s + 1, xn, Bn, dyn, Cn);
@@ -558,14 +617,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                 __syncthreads();
                 Au[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
                 Ag[slot_new] = M::load_operand(g_slot, UROW, w, j, q, true);
-                if (main_step) {
+                {
                     f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
                     f32x4 dac0 = {0.f, 0.f, 0.f, 0.f}, dac1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                     for (int i = 0; i < NK; ++i) {
                         acc0 = M::mfma(Au[(ph - i + NK) % NK], W0[i], acc0);
                         acc1 = M::mfma(Au[(ph - i + NK) % NK], W1[i], acc1);
-                        // g2 of step s+i sits in slot (ph+i) % NK
                         dac0 = M::mfma(Ag[(ph + i) % NK], W1[i], dac0);   // output rows 0..15
                         dac1 = M::mfma(Ag[(ph + i) % NK], W0[i], dac1);   // output rows 16..31
                     }
@@ -587,7 +645,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                 }
                 __syncthreads();
                 const int64_t t = s * STEP + r;
-                if (main_step && cvalid && t < L) {
+                if (cvalid && t < L) {
                     const int64_t o = col + t * d;
                     {
                         const f32x4 p0 = *(const f32x4 *)y_rd;

@@ -38,9 +38,9 @@ def two_pass_fwd_grouped(
         raise ValueError(f"schedule {schedule} not implemented")
     if warmup:
         raise NotImplementedError("ahead-of-time warmup is a Triton notion; the HIP library is prebuilt")
-    if y is not None:
-        raise NotImplementedError("pre-allocated output is not supported")
     if verbose:
         name = _lib.select_algo(bs, seqlen, g, dg, h.shape[-1], x.dtype) if algo in ("auto", 0) else algo
         print(f"gcg fwd: {bs=} {seqlen=} {g=} {dg=} hl={h.shape[-1]} dtype={x.dtype} kernel={name}")
-    return _lib.fwd(x, B, C, h, return_bx=return_bx, return_y2=return_y2, algo=algo)
+    if y is not None:
+        y = y.reshape(x.shape)      # the reference takes a (bs, L, d) or (bs, L, g, dg) buffer (fwd.py:155-156)
+    return _lib.fwd(x, B, C, h, return_bx=return_bx, return_y2=return_y2, algo=algo, out=y)

@@ -78,3 +78,17 @@ def test_operator_modules(gcg_lib, kind):
     op32 = hyena.HyenaSEOperator(g * dg, g, hyena_se_len=7, cfg=hyena.CgcgConfig(cgcg_dtype="float32")).to(DEV)
     z32 = op32(x1, x2, v)
     assert z32.dtype == torch.bfloat16
+
+
+def test_preallocated_output(gcg_lib):
+    from savanna_amd.kernels.cgcg.src.fwd import two_pass_fwd_grouped
+
+    bs, L, g, dg = 1, 128, 2, 16
+    x, B, C = (torch.randn(bs, L, g, dg, device=DEV) for _ in range(3))
+    h = torch.randn(g, 1, 7, device=DEV)
+    buf = torch.full((bs, L, g * dg), float("nan"), device=DEV)
+    bx, y2, y = two_pass_fwd_grouped(x, B, C, h, y=buf, autotune=False, CHUNK_SIZE=128, BLOCK_D=16)
+    assert y.data_ptr() == buf.data_ptr() and torch.isfinite(buf).all()
+    ref = oracle.gcg_fwd_oracle(x.cpu(), B.cpu(), C.cpu(), h.cpu(), return_intermediates=True)
+    for got, want, n in zip((bx, y2, y), ref, ("bx", "y2", "y")):
+        assert_close(got, want, 1e-5, n)
