@@ -318,24 +318,6 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     const int64_t c0 = (int64_t)cb * CB;
     const int hl = dm.hl;
 
-    // filter table of this wave's group: htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0
-    {
-        const int64_t cw = c0 + 16 * w;
-        const int64_t grp = (cw < d) ? cw / dm.dg : 0;
-        const hraw_t *hg = (const hraw_t *)h + grp * hl;
-        for (int i = l; i < HTAB; i += 64) {
-            const int lag = i - HPAD;
-            htab[w][i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
-        }
-    }
-    __syncthreads();
-    op_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
-#pragma unroll
-    for (int i = 0; i < NK; ++i) {
-        W0[i] = M::toeplitz(htab[w], 32 * i, j, q);
-        W1[i] = M::toeplitz(htab[w], 32 * i + 16, j, q);
-    }
-
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
 
@@ -366,9 +348,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     // A segment that starts inside the sequence first rebuilds the operands of the NK-1 steps
     // before it.  Their rows are requested together, so the replay costs one memory latency
     // instead of NK-1; step s_lo-i lands in ring slot NK-i, where phase 0 expects it.
+    constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
+    Row<T> wx[NLEAD], wB[NLEAD];
     if constexpr (NK > 1) {
         if (s_lo > 0) {
-            Row<T> wx[NK - 1], wB[NK - 1];
 #pragma unroll
             for (int i = 1; i < NK; ++i) {
                 const int64_t t = (s_lo - i) * STEP + r;
@@ -378,6 +361,30 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                     wB[i - 1] = ldg_row(B + col + t * d);
                 }
             }
+        }
+    }
+
+    // While those rows are in flight: filter table of this wave's group,
+    // htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0, and the Toeplitz operand tiles.
+    {
+        const int64_t cw = c0 + 16 * w;
+        const int64_t grp = (cw < d) ? cw / dm.dg : 0;
+        const hraw_t *hg = (const hraw_t *)h + grp * hl;
+        for (int i = l; i < HTAB; i += 64) {
+            const int lag = i - HPAD;
+            htab[w][i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
+        }
+    }
+    __syncthreads();
+    op_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+        W0[i] = M::toeplitz(htab[w], 32 * i, j, q);
+        W1[i] = M::toeplitz(htab[w], 32 * i + 16, j, q);
+    }
+
+    if constexpr (NK > 1) {
+        if (s_lo > 0) {
 #pragma unroll
             for (int i = 1; i < NK; ++i) {
                 float xf[8], Bf[8], uf[8];
@@ -500,22 +507,6 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     const int hl = dm.hl;
     const bool wave_valid = c0 + 16 * w < d;
 
-    {
-        const int64_t grp = wave_valid ? (c0 + 16 * w) / dm.dg : 0;
-        const hraw_t *hg = (const hraw_t *)h + grp * hl;
-        for (int i = l; i < HTAB; i += 64) {
-            const int lag = i - HPAD;
-            htab[w * HTAB + i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
-        }
-    }
-    __syncthreads();
-    op_t W0[NK], W1[NK];
-#pragma unroll
-    for (int i = 0; i < NK; ++i) {
-        W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
-        W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
-    }
-
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
 
@@ -565,10 +556,31 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     // Lead-in: u of the NK-1 steps before the segment and g2 of its first NK-1 steps, i.e. the
     // rows iterations s_lo-NK+1 .. s_lo-1 would have brought.  They are requested together,
     // so the lead-in costs one memory latency instead of NK-1.
+    constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
+    Row<T> wx[NLEAD], wB[NLEAD], wdy[NLEAD], wC[NLEAD];
     if constexpr (NK > 1) {
-        Row<T> wx[NK - 1], wB[NK - 1], wdy[NK - 1], wC[NK - 1];
 #pragma unroll
         for (int i = 1; i < NK; ++i) fetch(s_lo - i, wx[i - 1], wB[i - 1], wdy[i - 1], wC[i - 1]);
+    }
+
+    // While those rows are in flight: the filter table of this wave's group and the Toeplitz tiles.
+    {
+        const int64_t grp = wave_valid ? (c0 + 16 * w) / dm.dg : 0;
+        const hraw_t *hg = (const hraw_t *)h + grp * hl;
+        for (int i = l; i < HTAB; i += 64) {
+            const int lag = i - HPAD;
+            htab[w * HTAB + i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
+        }
+    }
+    __syncthreads();
+    op_t W0[NK], W1[NK];
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+        W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
+        W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
+    }
+
+    if constexpr (NK > 1) {
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
             // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i

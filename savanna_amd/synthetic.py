@@ -65,6 +65,11 @@ WORKLOADS = {
                                  "Hyena-SE then Hyena-MR forward+backward, bf16, B=1 L=32768 D=8192 G=512"),
     "mr_fwd_1m": Workload("mr_fwd_1m", 1, 1048576, 256, 16, (128,), torch.bfloat16, False,
                           "Hyena-MR forward, bf16, B=1 L=1048576 D=4096 G=256 hl=128"),
+    # the shapes the reference's own benchmark scripts use (cgcg/tests/benchmark-7b.sh, benchmark-40b.sh)
+    "ref_bench_7b": Workload("ref_bench_7b", 8, 8192, 256, 16, (128,), torch.bfloat16, True,
+                             "Hyena-MR forward+backward, bf16, B=8 L=8192 D=4096 G=256 hl=128"),
+    "ref_bench_40b": Workload("ref_bench_40b", 2, 8192, 512, 16, (7,), torch.bfloat16, True,
+                              "Hyena-SE forward+backward, bf16, B=2 L=8192 D=8192 G=512 hl=7"),
 }
 # the order in which the benchmark reports them
 WORKLOAD_ORDER = ("se_fwd_fp32", "mr_fwd_7b", "mr_fwdbwd_7b", "se_mr_fwdbwd_40b", "mr_fwd_1m")
