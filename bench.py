@@ -81,7 +81,35 @@ class Op:
         return y
 
 
-def time_workload(wl, device, steps, warmup):
+def time_graph(ops, steps, warmup):
+    """One HIP graph holding a full rotation over the input sets, replayed; ms per step.
+    For launch-bound shapes this is how a caller would run the op."""
+    rounds = max(o.nsets for o in ops)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(rounds):
+            for op in ops:
+                op.run()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for _ in range(rounds):
+            for op in ops:
+                op.run()
+    replays = max(1, -(-steps // rounds))
+    for _ in range(max(1, warmup // rounds)):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(replays):
+        graph.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / (replays * rounds)
+
+
+def time_workload(wl, device, steps, warmup, graph=False):
     ops = [Op(wl, hl, device) for hl in wl.filters]
     dom = max(range(len(ops)), key=lambda i: ops[i].hl)     # dominant launch: longest filter
     for _ in range(warmup):
@@ -117,6 +145,11 @@ def time_workload(wl, device, steps, warmup):
         "kernel_hbm_frac": achieved / HBM_PEAK_GBS,
         "input_sets": [o.nsets for o in ops],
     }
+    if graph:
+        g_ms = time_graph(ops, steps, warmup)
+        res["graph_ms_per_step"] = g_ms
+        res["graph_tokens_per_s"] = wl.tokens / (g_ms * 1e-3)
+        res["graph_hbm_frac"] = wl.algorithmic_bytes() / (g_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
     del ops
     torch.cuda.empty_cache()
     return res
@@ -169,6 +202,8 @@ def main():
     ap.add_argument("--workload", default="mr_fwdbwd_7b", choices=list(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also time the other four configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--graph", action="store_true",
+                    help="also time the step replayed from a captured HIP graph (launch-bound shapes)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, so a counter profile of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -185,7 +220,7 @@ def main():
     _lib.load()
 
     wl = WORKLOADS[args.workload]
-    res = time_workload(wl, device, args.steps, args.warmup)
+    res = time_workload(wl, device, args.steps, args.warmup, graph=args.graph)
     line = {
         "metric": "Hyena-MR fwd+bwd tokens/s and HBM GB/s (% roofline) at 1 MI355X",
         "value": res["tokens_per_s"],
@@ -209,6 +244,8 @@ def main():
                      "kernel_ms": res["kernel_ms"], "algorithmic_bytes": res["kernel_bytes"],
                      "traffic": MEASURED_TRAFFIC_BYTES.get((wl.name, res["kernel"]))},
     }
+    if args.graph:
+        line["graph"] = {k: res[k] for k in ("graph_ms_per_step", "graph_tokens_per_s", "graph_hbm_frac")}
     if args.all:
         others = {}
         for name in WORKLOAD_ORDER:
@@ -216,7 +253,8 @@ def main():
                 continue
             w = WORKLOADS[name]
             k = args.steps if w.bs * w.L * w.d < (1 << 30) else max(3, args.steps // 10)
-            others[name] = time_workload(w, device, k, max(2, args.warmup // 2))
+            small = w.algorithmic_bytes() < (64 << 20)       # launch-bound: also report graph replay
+            others[name] = time_workload(w, device, k, max(2, args.warmup // 2), graph=small)
         line["all_configs"] = others
     if args.copy_calibration:
         src = torch.ones(256 << 20, dtype=torch.uint8, device=device)

@@ -81,7 +81,7 @@ template <typename T, int VV> __device__ __forceinline__ typename Vec<T, VV>::ra
     return r;
 }
 
-struct WinPlan { int v, nvec, nseg, ts, ncvb; int64_t nthreads, nwg; };
+struct WinPlan { int v, nvec, nseg, ts, ncvb, threads; int64_t nthreads, nwg; };
 
 
 // ---------------------------------------------------------------------------- forward
@@ -92,13 +92,13 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
                                                          T *__restrict__ bx, Dims dm, WinPlan pl)
 {
     typedef typename Vec<T, V>::raw raw_t;
-    // (batch, run, block of 256 channel vectors) come from the workgroup index, so row addresses
+    // (batch, run, block of channel vectors) come from the workgroup index, so row addresses
     // are wave-uniform and only the channel offset is per lane
     int64_t wg = blockIdx.x;
     const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
     const int seg = (int)(wg % pl.nseg);
     const int64_t b = wg / pl.nseg;
-    const int cv = cvb * 256 + (int)threadIdx.x;
+    const int cv = cvb * (int)blockDim.x + (int)threadIdx.x;
     if (cv >= pl.nvec) return;
     const int64_t gid = (b * pl.nseg + seg) * pl.nvec + cv;     // index of this lane's workspace slot
     (void)gid;
@@ -188,13 +188,13 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                                                          float *__restrict__ ws, Dims dm, WinPlan pl)
 {
     typedef typename Vec<T, V>::raw raw_t;
-    // (batch, run, block of 256 channel vectors) come from the workgroup index, so row addresses
+    // (batch, run, block of channel vectors) come from the workgroup index, so row addresses
     // are wave-uniform and only the channel offset is per lane
     int64_t wg = blockIdx.x;
     const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
     const int seg = (int)(wg % pl.nseg);
     const int64_t b = wg / pl.nseg;
-    const int cv = cvb * 256 + (int)threadIdx.x;
+    const int cv = cvb * (int)blockDim.x + (int)threadIdx.x;
     if (cv >= pl.nvec) return;
     const int64_t gid = (b * pl.nseg + seg) * pl.nvec + cv;     // index of this lane's workspace slot
     (void)gid;
@@ -350,10 +350,11 @@ WinPlan plan(const Dims &dm, int v)
     p.nvec = (int)(dm.d / v);
     p.ts = 128;
     // shorter runs when the problem is too small to fill the chip with 128-row runs
-    while (p.ts > 16 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 256 * 1024) p.ts >>= 1;
+    while (p.ts > 8 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 256 * 1024) p.ts >>= 1;
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);
     p.nthreads = dm.bs * p.nseg * p.nvec;       // workspace slots (one per lane with work)
-    p.ncvb = (p.nvec + 255) / 256;
+    p.threads = p.nvec >= 256 ? 256 : ((p.nvec + 63) / 64) * 64;   // narrow tensors: fewer idle lanes
+    p.ncvb = (p.nvec + p.threads - 1) / p.threads;
     p.nwg = dm.bs * p.nseg * p.ncvb;
     return p;
 }
@@ -367,7 +368,7 @@ int fwd_v(const void *x, const void *B, const void *C, const void *h, void *y, v
     const WinPlan p = plan(dm, V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((window_fwd_kernel<T, HL, V>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)x,
+    hipLaunchKernelGGL((window_fwd_kernel<T, HL, V>), dim3((unsigned)nwg), dim3(p.threads), 0, st, (const T *)x,
                        (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     return (int)hipGetLastError();
 }
@@ -379,7 +380,7 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
     const WinPlan p = plan(dm, BWD_V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V>), dim3((unsigned)nwg), dim3(256), 0, st, (const T *)dy,
+    hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V>), dim3((unsigned)nwg), dim3(p.threads), 0, st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
                        (float *)ws, dm, p);
     int e = (int)hipGetLastError();

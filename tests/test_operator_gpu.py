@@ -92,3 +92,65 @@ def test_preallocated_output(gcg_lib):
     ref = oracle.gcg_fwd_oracle(x.cpu(), B.cpu(), C.cpu(), h.cpu(), return_intermediates=True)
     for got, want, n in zip((bx, y2, y), ref, ("bx", "y2", "y")):
         assert_close(got, want, 1e-5, n)
+
+
+def test_runs_on_the_callers_stream(gcg_lib):
+    """Kernels are enqueued on torch's current stream, not on the null stream."""
+    from savanna_amd import _lib
+
+    bs, L, g, dg, hl = 2, 2048, 16, 16, 128
+    x, B, C, dy = (torch.randn(bs, L, g, dg, device=DEV, dtype=torch.bfloat16) for _ in range(4))
+    h = (torch.randn(g, 1, hl, device=DEV) / hl ** 0.5).to(torch.bfloat16)
+    _, _, y_ref = _lib.fwd(x, B, C, h)
+    grads_ref = _lib.bwd(dy, x, B, C, h)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        # work queued on the side stream first: the convolution must wait for it, which it only
+        # does when it is launched on the same stream
+        x2 = x.clone()
+        for _ in range(20):
+            x2 = x2 * 1.0
+        _, _, y = _lib.fwd(x2, B, C, h)
+        grads = _lib.bwd(dy, x2, B, C, h)
+    side.synchronize()
+    assert torch.equal(y, y_ref)
+    for a, b in zip(grads, grads_ref):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("hl,dtype", [(7, torch.float32), (128, torch.bfloat16)])
+def test_graph_capture_and_replay(gcg_lib, hl, dtype):
+    """The launch-bound small shapes are what a HIP graph is for: forward and backward are
+    captured once and replayed with new input contents; every replay must equal the eager result.
+    (The library itself allocates nothing and issues no memset; the tensors come from the
+    capture's private pool.)"""
+    from savanna_amd import _lib
+
+    bs, L, g, dg = 1, 2048, 16, 16
+    static = [torch.randn(bs, L, g, dg, device=DEV).to(dtype) for _ in range(4)]       # x, B, C, dy
+    h = (torch.randn(g, 1, hl, device=DEV) / hl ** 0.5).to(dtype)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):                      # warm-up on the capture stream
+        _lib.fwd(static[0], static[1], static[2], h)
+        _lib.bwd(static[3], static[0], static[1], static[2], h)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _, _, y_g = _lib.fwd(static[0], static[1], static[2], h)
+        grads_g = _lib.bwd(static[3], static[0], static[1], static[2], h)
+    for it in range(3):
+        fresh = [torch.randn(bs, L, g, dg, device=DEV).to(dtype) for _ in range(4)]
+        for dst, src in zip(static, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        _, _, y_e = _lib.fwd(fresh[0], fresh[1], fresh[2], h)       # eager work between replays
+        grads_e = _lib.bwd(fresh[3], fresh[0], fresh[1], fresh[2], h)
+        torch.cuda.synchronize()
+        assert torch.equal(y_g, y_e), f"replay {it}: y"
+        for a, b, n in zip(grads_g, grads_e, ("dx", "dB", "dC", "dh")):
+            assert torch.equal(a, b), f"replay {it}: {n}"
