@@ -121,3 +121,31 @@ def test_error_codes(gcg_lib):
     assert lib.gcg_bwd(dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(),
                        x.data_ptr(), x.data_ptr(), x.data_ptr(), h.data_ptr(), None, 0,
                        1, 64, 2, 16, 200, 1, 0, None) == -3
+
+
+@pytest.mark.parametrize("dtype,hl", [(torch.bfloat16, 128), (torch.float32, 7)])
+def test_misaligned_tensors_take_the_direct_kernels(gcg_lib, dtype, hl):
+    """The vector kernels need 16-byte aligned tensors; a view that starts one element into its
+    storage is re-routed to the element-wise direct kernels under automatic selection and is
+    refused when a vector family is forced."""
+    bs, L, g, dg = 1, 200, 2, 16
+    x, B, C, h, dy = inputs(bs, L, g, dg, hl, dtype, seed=7, dy_scale=0.1)
+    n = bs * L * g * dg
+
+    def shifted(t):
+        buf = torch.empty(n + 1, dtype=dtype, device=DEV)
+        v = buf[1:].view(bs, L, g, dg)
+        v.copy_(t)
+        assert v.data_ptr() % 16 != 0 and v.is_contiguous()
+        return v
+
+    xs, Bs, Cs, dys = shifted(x), shifted(B), shifted(C), shifted(dy)
+    hd = h.to(DEV)
+    _, _, y = _lib.fwd(xs, Bs, Cs, hd)
+    assert_close(y, oracle_fwd(x, B, C, h)[2], TOL[dtype], "y")
+    got = _lib.bwd(dys, xs, Bs, Cs, hd)
+    for o, r_, n_ in zip(got, oracle_bwd(dy, x, B, C, h), ("dx", "dB", "dC", "dh")):
+        assert_close(o, r_, TOL_DH[dtype] if n_ == "dh" else TOL[dtype], n_)
+    forced = "mfma" if hl > 8 else "window"
+    with pytest.raises(_lib.GcgError, match="not supported"):
+        _lib.fwd(xs, Bs, Cs, hd, algo=forced)
