@@ -9,6 +9,8 @@
 // channel vectors, so every row access of a wave is one contiguous segment.
 #include "gcg_common.h"
 
+#include <cstdlib>
+
 namespace gcg {
 namespace {
 
@@ -349,8 +351,11 @@ WinPlan plan(const Dims &dm, int v)
     p.v = v;
     p.nvec = (int)(dm.d / v);
     p.ts = 128;
-    // shorter runs when the problem is too small to fill the chip with 128-row runs
-    while (p.ts > 8 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 256 * 1024) p.ts >>= 1;
+    // 128-row runs measured best (64 and 256 are both ~10 % slower at the 7B and 40B shapes);
+    // shorter runs only when 128 would leave fewer than two workgroups per CU
+    while (p.ts > 8 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
+    static const char *env = getenv("GCG_WINDOW_ROWS");   // tuning override: rows per lane, a multiple of 8
+    if (env && atoi(env) >= 8 && atoi(env) % 8 == 0) p.ts = atoi(env);
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);
     p.nthreads = dm.bs * p.nseg * p.nvec;       // workspace slots (one per lane with work)
     p.threads = p.nvec >= 256 ? 256 : ((p.nvec + 63) / 64) * 64;   // narrow tensors: fewer idle lanes
