@@ -56,16 +56,42 @@ class Op:
             else:
                 t = make_inputs(wl.bs, wl.L, wl.g, wl.dg, hl, wl.dtype, seed=i, device=device,
                                 with_dy=wl.backward)
+            if wl.layout != "separate":
+                # kernel names: C = v, B = q, x = k
+                t["feat"] = torch.stack([t.pop("v"), t.pop("q"), t.pop("k")], dim=-1).contiguous()
             self.sets.append(t)
+        self.layout = wl.layout
         self.hl = hl
         self.backward = wl.backward
         self.i = 0
         n = wl.bs * wl.L * wl.d * wl.elem_bytes
         self.fwd_bytes, self.bwd_bytes = 4 * n, 7 * n
 
+    def run_features(self, t, ev):
+        """Workloads whose inputs are one interleaved features tensor.  The whole op is bracketed:
+        for "gathered" the gathers and the re-assembly of the feature gradient are part of it."""
+        feat, h = t["feat"], t["h"]
+        if ev is not None:
+            ev[0].record()
+        if self.layout == "interleaved":
+            y = _lib.fwd_interleaved(feat, h)
+            if self.backward:
+                _lib.bwd_interleaved(t["dy"], feat, h)
+        else:
+            C, B, x = (feat[..., i].contiguous() for i in range(3))     # cgcg/interface.py:51-54
+            _, _, y = _lib.fwd(x, B, C, h)
+            if self.backward:
+                dx, dB, dC, _ = _lib.bwd(t["dy"], x, B, C, h)
+                torch.stack([dC, dB, dx], dim=-1)                        # autograd of unbind (block.py:886-890)
+        if ev is not None:
+            ev[1].record()
+        return y
+
     def run(self, ev=None):
         t = self.sets[self.i % self.nsets]
         self.i += 1
+        if self.layout != "separate":
+            return self.run_features(t, ev)
         # kernel names: B = q, x = k, C = v
         if ev is not None and not self.backward:
             ev[0].record()
@@ -130,6 +156,9 @@ def time_workload(wl, device, steps, warmup, graph=False):
     kern_bytes = op.bwd_bytes if op.backward else op.fwd_bytes
     kern_name = ("gcg_bwd" if op.backward else "gcg_fwd") + f" hl={op.hl} " + _lib.select_algo(
         wl.bs, wl.L, wl.g, wl.dg, op.hl, wl.dtype, op.backward)
+    if wl.layout != "separate":      # the bracket holds the whole op, not one launch
+        kern_bytes = op.fwd_bytes + (op.bwd_bytes if op.backward else 0)
+        kern_name = f"whole op ({wl.layout}) hl={op.hl}"
     achieved = kern_bytes / (kern_ms * 1e-3) / 1e9
     res = {
         "workload": wl.name,

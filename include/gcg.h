@@ -113,6 +113,40 @@ GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C,
 GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
                     int32_t dtype, int32_t backward);
 
+/*
+ * Forward on interleaved operands.
+ * Replaces the three gathers `x.contiguous()`, `B.contiguous()`, `C.contiguous()` of
+ * TwoPassChunkedGateConvGate.forward (savanna/kernels/triton_src/cgcg/interface.py:51-54)
+ * followed by two_pass_fwd_grouped, for the case those three arguments are the unbound
+ * thirds of one projected-features tensor, as the interleaved split of
+ * ParallelSequenceMixer.forward produces them (savanna/model/block.py:886-890:
+ * `rearrange(features, "b l (g dg p) -> b l g p dg", p=3).unbind(dim=3)` gives x1, x2, v,
+ * which the operators pass on as C = x1, B = x2, x = v, hyena.py:517-531, :825-840).
+ *
+ *   feat   (bs, L, g, dg, 3) contiguous: feat[..., 0] = C, feat[..., 1] = B, feat[..., 2] = x
+ *   y      out, (bs, L, g, dg)
+ */
+GCG_API int gcg_fwd_interleaved(const void *feat, const void *h, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, int32_t algo, void *stream);
+
+/*
+ * Backward on interleaved operands: the counterpart of gcg_bwd for gcg_fwd_interleaved.
+ * Replaces two_pass_bwd_refactor (src/bwd.py:347-474) plus the scatter of dx, dB, dC into
+ * the gradient of the features tensor that autograd performs for the unbind / rearrange of
+ * block.py:886-890.
+ *
+ *   dy      (bs, L, g, dg)
+ *   dfeat   out, (bs, L, g, dg, 3): dfeat[..., 0] = dC, [..., 1] = dB, [..., 2] = dx
+ *   dh      out, (g, 1, hl), overwritten
+ *   workspace, workspace_bytes   as for gcg_bwd, sized by gcg_bwd_workspace_bytes
+ */
+GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
+            void *dfeat, void *dh,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, int32_t algo, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,6 +25,7 @@ _DTYPES = {torch.float32: GCG_F32, torch.bfloat16: GCG_BF16, torch.float16: GCG_
 EXPORTS = (
     "gcg_strerror", "gcg_last_hip_error", "gcg_version", "gcg_fwd",
     "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_select_algo",
+    "gcg_fwd_interleaved", "gcg_bwd_interleaved",
 )
 
 _lock = threading.Lock()
@@ -62,6 +63,10 @@ def load() -> ctypes.CDLL:
         lib.gcg_bwd.restype = ctypes.c_int
         lib.gcg_select_algo.argtypes = [i64, i64, i32, i32, i32, i32, i32]
         lib.gcg_select_algo.restype = ctypes.c_int
+        lib.gcg_fwd_interleaved.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_fwd_interleaved.restype = ctypes.c_int
+        lib.gcg_bwd_interleaved.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_bwd_interleaved.restype = ctypes.c_int
         _lib = lib
         return lib
 
@@ -145,6 +150,63 @@ def bwd(dy, x, B, C, h, algo=ALGO_AUTO):
         )
     check(rc, "gcg_bwd")
     return dx, dB, dC, dh
+
+
+def _check_feat(feat, h):
+    if feat.dim() != 5 or feat.shape[-1] != 3 or not feat.is_contiguous():
+        raise ValueError("feat must be a contiguous (bs, L, g, dg, 3) tensor")
+    if h.dim() != 3 or h.shape[0] != feat.shape[2] or h.shape[1] != 1 or not h.is_contiguous():
+        raise ValueError("h must be a contiguous (g, 1, hl) tensor")
+    if h.dtype != feat.dtype or h.device != feat.device:
+        raise ValueError("feat and h must share dtype and device")
+
+
+def fwd_interleaved(feat, h, algo=ALGO_AUTO, out=None):
+    """y (bs, L, g, dg) for feat (bs, L, g, dg, 3) with feat[..., 0] = C, [..., 1] = B, [..., 2] = x."""
+    lib = load()
+    _require_gpu(feat)
+    _check_feat(feat, h)
+    bs, L, g, dg, _ = feat.shape
+    hl = h.shape[-1]
+    if out is not None:
+        if (out.shape != feat.shape[:4] or out.dtype != feat.dtype or out.device != feat.device
+                or not out.is_contiguous()):
+            raise ValueError("out must be a contiguous (bs, L, g, dg) tensor with the dtype and device of feat")
+    y = out if out is not None else torch.empty(feat.shape[:4], dtype=feat.dtype, device=feat.device)
+    if y.numel() == 0:
+        return y
+    with torch.cuda.device(feat.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_fwd_interleaved(feat.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg, hl,
+                                     dtype_code(feat.dtype), algo_code(algo), st)
+    check(rc, "gcg_fwd_interleaved")
+    return y
+
+
+def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO):
+    """(dfeat, dh): dfeat has feat's layout, dfeat[..., 0] = dC, [..., 1] = dB, [..., 2] = dx."""
+    lib = load()
+    _require_gpu(feat)
+    _check_feat(feat, h)
+    bs, L, g, dg, _ = feat.shape
+    hl = h.shape[-1]
+    if dy.shape != feat.shape[:4] or dy.dtype != feat.dtype or not dy.is_contiguous():
+        raise ValueError("dy must be a contiguous (bs, L, g, dg) tensor of feat's dtype")
+    dfeat = torch.empty_like(feat)
+    dh = torch.empty_like(h)
+    if dy.numel() == 0:
+        return dfeat, dh.zero_()
+    code, a = dtype_code(feat.dtype), algo_code(algo)
+    nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, a)
+    if nbytes == 0:
+        raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")
+    with torch.cuda.device(feat.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=feat.device)
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_bwd_interleaved(dy.data_ptr(), feat.data_ptr(), h.data_ptr(), dfeat.data_ptr(), dh.data_ptr(),
+                                     ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, a, st)
+    check(rc, "gcg_bwd_interleaved")
+    return dfeat, dh
 
 
 def select_algo(bs, L, g, dg, hl, dtype: torch.dtype, backward=False) -> str:

@@ -31,7 +31,7 @@ int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t 
 {
     if (bs <= 0 || L <= 0 || g <= 0 || dg <= 0 || hl <= 0) return GCG_ERR_BAD_ARG;
     if (dtype != GCG_F32 && dtype != GCG_BF16 && dtype != GCG_F16) return GCG_ERR_BAD_ARG;
-    dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg;
+    dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg; dm->es = 1;
     return GCG_OK;
 }
 
@@ -68,6 +68,14 @@ int finish(int hip_rc)
     return GCG_ERR_LAUNCH;
 }
 
+size_t elem_bytes(int dtype) { return dtype == GCG_F32 ? 4 : 2; }
+
+// pointer `elems` elements of `dtype` past p
+template <typename P> P *at(P *p, size_t elems, int dtype)
+{
+    return (P *)((uintptr_t)p + elems * elem_bytes(dtype));
+}
+
 } // namespace
 
 extern "C" {
@@ -87,7 +95,7 @@ GCG_API const char *gcg_strerror(int code)
 
 GCG_API int gcg_last_hip_error(void) { return tls_hip_error; }
 
-GCG_API int gcg_version(void) { return 100; }
+GCG_API int gcg_version(void) { return 101; }
 
 GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t backward)
 {
@@ -151,6 +159,59 @@ GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C,
     rc = check_device();
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
+    switch (a) {
+    case GCG_ALGO_DIRECT:
+        return finish(gcg::direct_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    case GCG_ALGO_WINDOW:
+        return finish(gcg::window_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    case GCG_ALGO_MFMA:
+        return finish(gcg::mfma_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
+// ---- interleaved operands: one (bs, L, g, dg, 3) tensor instead of three (bs, L, g, dg) ones
+
+GCG_API int gcg_fwd_interleaved(const void *feat, const void *h, void *y, int64_t bs, int64_t L, int32_t g, int32_t dg,
+                                int32_t hl, int32_t dtype, int32_t algo, void *stream)
+{
+    if (!feat || !h || !y) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    dm.es = 3;
+    const int a = resolve_algo(algo, dtype, dm, false, all_aligned16({feat, y}));
+    if (a < 0) return a;
+    rc = check_device();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const void *C = feat, *B = at(feat, 1, dtype), *x = at(feat, 2, dtype);
+    switch (a) {
+    case GCG_ALGO_DIRECT: return finish(gcg::direct_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
+    case GCG_ALGO_WINDOW: return finish(gcg::window_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
+    case GCG_ALGO_MFMA:   return finish(gcg::mfma_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
+GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *workspace,
+                                size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                                int32_t dtype, int32_t algo, void *stream)
+{
+    if (!dy || !feat || !h || !dfeat || !dh) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    dm.es = 3;
+    const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, feat, dfeat}));
+    if (a < 0) return a;
+    const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    const void *C = feat, *B = at(feat, 1, dtype), *x = at(feat, 2, dtype);
+    void *dC = dfeat, *dB = at(dfeat, 1, dtype), *dx = at(dfeat, 2, dtype);
     switch (a) {
     case GCG_ALGO_DIRECT:
         return finish(gcg::direct_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));

@@ -75,6 +75,11 @@ struct Dims {
     int64_t bs, L;
     int32_t g, dg, hl;
     int64_t d; // g * dg
+    // Element stride of the x, B, C operands and of dx, dB, dC.  1: three separate contiguous
+    // tensors.  3: one interleaved tensor (bs, L, g, dg, 3) with [..., 0] = C, [..., 1] = B,
+    // [..., 2] = x; the launchers then receive C = base, B = base + 1, x = base + 2 elements
+    // (and dC, dB, dx likewise).  y, y2, bx and dy are always plain.
+    int32_t es;
 };
 
 constexpr int kWave = 64;

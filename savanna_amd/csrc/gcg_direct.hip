@@ -38,6 +38,7 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(const T *__restrict__ x
     const int64_t c0 = (int64_t)ct * CT, c = c0 + cl, d = dm.d, L = dm.L;
     const bool cvalid = c < d;
     const int hl = dm.hl;
+    const int64_t es = dm.es;   // element stride of x, B, C (3 when they are interleaved in one tensor)
     const int64_t t0 = tt * TT;
     const T *hg = h + (cvalid ? (c / dm.dg) : 0) * hl;
 
@@ -57,7 +58,7 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(const T *__restrict__ x
             float v = 0.f;
             if (time >= 0 && time < L && c0 + cc < d) {
                 const int64_t off = (b * L + time) * d + c0 + cc;
-                v = ld(B, off) * ld(x, off);
+                v = ld(B, off * es) * ld(x, off * es);
             }
             us[row][cc] = v;
         }
@@ -86,8 +87,8 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(const T *__restrict__ x
         if (t < L) {
             const int64_t o = (b * L + t) * d + c;
             if (y2) Elem<T>::store(y2 + o, acc[r]);
-            if (bx) Elem<T>::store(bx + o, ld(B, o) * ld(x, o));
-            Elem<T>::store(y + o, ld(C, o) * acc[r]);
+            if (bx) Elem<T>::store(bx + o, ld(B, o * es) * ld(x, o * es));
+            Elem<T>::store(y + o, ld(C, o * es) * acc[r]);
         }
     }
 }
@@ -124,6 +125,7 @@ __global__ __launch_bounds__(256) void direct_bwd_kernel(const T *__restrict__ d
     const int64_t c0 = (int64_t)ct * CT, c = c0 + cl, d = dm.d, L = dm.L;
     const bool cvalid = c < d;
     const int hl = dm.hl, dg = dm.dg;
+    const int64_t es = dm.es;   // element stride of x, B, C, dx, dB, dC
     const T *hg = h + (cvalid ? (c / dg) : 0) * hl;
     const int64_t g0 = c0 / dg;                                            // first group in this tile
     const int64_t clast = (c0 + CT < d ? c0 + CT : d) - 1;
@@ -157,14 +159,14 @@ __global__ __launch_bounds__(256) void direct_bwd_kernel(const T *__restrict__ d
                 float v = 0.f;
                 if (time >= 0 && time < L && cok) {
                     const int64_t off = (b * L + time) * d + c0 + cc;
-                    v = ld(B, off) * ld(x, off);
+                    v = ld(B, off * es) * ld(x, off * es);
                 }
                 us[row][cc] = v;
                 time = gbase + row;
                 v = 0.f;
                 if (time < L && cok) {
                     const int64_t off = (b * L + time) * d + c0 + cc;
-                    v = ld(dy, off) * ld(C, off);
+                    v = ld(dy, off) * ld(C, off * es);
                 }
                 gs[row][cc] = v;
             }
@@ -227,9 +229,9 @@ __global__ __launch_bounds__(256) void direct_bwd_kernel(const T *__restrict__ d
                 const int64_t t = t0 + r0 + r;
                 if (t < L) {
                     const int64_t o = (b * L + t) * d + c;
-                    Elem<T>::store(dC + o, ld(dy, o) * y2a[r]);
-                    Elem<T>::store(dx + o, dua[r] * ld(B, o));
-                    Elem<T>::store(dB + o, dua[r] * ld(x, o));
+                    Elem<T>::store(dC + o * es, ld(dy, o) * y2a[r]);
+                    Elem<T>::store(dx + o * es, dua[r] * ld(B, o * es));
+                    Elem<T>::store(dB + o * es, dua[r] * ld(x, o * es));
                 }
             }
         }

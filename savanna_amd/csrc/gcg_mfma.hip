@@ -232,6 +232,58 @@ template <typename T> __device__ __forceinline__ void lds_store_row(unsigned cha
     for (int i = 0; i < MT<T>::RW; ++i) *(uint4 *)(p + 16 * i) = r.w[i];
 }
 
+template <typename T> __device__ __forceinline__ Row<T> lds_load_row(const unsigned char *p)
+{
+    Row<T> r;
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) r.w[i] = *(const uint4 *)(p + 16 * i);
+    return r;
+}
+
+// Interleaved operands (element stride 3): a lane's 8 channels of one row are 24 consecutive
+// elements, (C, B, x) per channel, i.e. three row vectors.  split_rows / join_rows convert
+// between that order and per-tensor channel vectors; every index is a compile-time constant.
+template <typename T>
+__device__ __forceinline__ void split_rows(const Row<T> (&p)[3], float (&xf)[8], float (&Bf)[8], float (&Cf)[8])
+{
+    float f[3][8];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) unpack8<T>(p[i], f[i]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        Cf[e] = f[(3 * e) / 8][(3 * e) % 8];
+        Bf[e] = f[(3 * e + 1) / 8][(3 * e + 1) % 8];
+        xf[e] = f[(3 * e + 2) / 8][(3 * e + 2) % 8];
+    }
+}
+template <typename T>
+__device__ __forceinline__ void join_rows(const float (&xf)[8], const float (&Bf)[8], const float (&Cf)[8],
+                                          Row<T> (&p)[3])
+{
+    float f[3][8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        f[(3 * e) / 8][(3 * e) % 8] = Cf[e];
+        f[(3 * e + 1) / 8][(3 * e + 1) % 8] = Bf[e];
+        f[(3 * e + 2) / 8][(3 * e + 2) % 8] = xf[e];
+    }
+#pragma unroll
+    for (int i = 0; i < 3; ++i) p[i] = pack8<T>(f[i]);
+}
+// One input row of a lane as three row vectors: (x, B, C) of separate tensors, or the three
+// thirds of the interleaved row.
+template <typename T, bool PK>
+__device__ __forceinline__ void in_floats(const Row<T> (&p)[3], float (&xf)[8], float (&Bf)[8], float (&Cf)[8])
+{
+    if constexpr (PK) {
+        split_rows<T>(p, xf, Bf, Cf);
+    } else {
+        unpack8<T>(p[0], xf);
+        unpack8<T>(p[1], Bf);
+        unpack8<T>(p[2], Cf);
+    }
+}
+
 // Streaming accesses: every tensor element is touched once, so loads and stores carry the
 // nontemporal hint (GCG_MFMA_NT=0 at build time turns it off for comparison).
 #ifndef GCG_XCD_SWIZZLE
@@ -291,7 +343,8 @@ struct MfmaPlan { int ncb, nseg, steps_per_seg, nw; int64_t nsteps, nwg; };
 // tile origins: element e of lane (j, q) is the tap for lag doff + j - kmap(q, e)  (MT<T>::toeplitz).
 
 // ---------------------------------------------------------------------------- forward
-template <typename T, int NK, int NW>
+// PK: x, B, C are interleaved in one tensor that starts at C (element stride 3).
+template <typename T, int NK, int NW, bool PK>
 __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__ x, const T *__restrict__ B,
                                                        const T *__restrict__ C, const T *__restrict__ h,
                                                        T *__restrict__ y, T *__restrict__ y2o,
@@ -332,34 +385,37 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
 
-    Row<T> xr, Br, Cr;
-    auto fetch = [&](int64_t s, Row<T> &xo, Row<T> &Bo, Row<T> &Co) {
-        const int64_t t = s * STEP + r;
-        xo = zero_row<T>(); Bo = zero_row<T>(); Co = zero_row<T>();
-        if (cvalid && t < L) {
-            const int64_t o = col + t * d;
-            xo = ldg_row(x + o);
-            Bo = ldg_row(B + o);
-            Co = ldg_row(C + o);
+    // a lane's input row: x, B, C vectors, or the three thirds of the interleaved row
+    auto load_in = [&](int64_t t, Row<T> (&p)[3], bool with_c) {
+        if constexpr (PK) {
+            const T *src = C + 3 * (col + t * d);
+            p[0] = ldg_row(src); p[1] = ldg_row(src + 8); p[2] = ldg_row(src + 16);
+        } else {
+            p[0] = ldg_row(x + col + t * d);
+            p[1] = ldg_row(B + col + t * d);
+            p[2] = with_c ? ldg_row(C + col + t * d) : zero_row<T>();
         }
     };
-    fetch(s_lo, xr, Br, Cr);
+    Row<T> in[3];
+    auto fetch = [&](int64_t s, Row<T> (&p)[3]) {
+        const int64_t t = s * STEP + r;
+        p[0] = zero_row<T>(); p[1] = zero_row<T>(); p[2] = zero_row<T>();
+        if (cvalid && t < L) load_in(t, p, true);
+    };
+    fetch(s_lo, in);
 
     // A segment that starts inside the sequence first rebuilds the operands of the NK-1 steps
     // before it.  Their rows are requested together, so the replay costs one memory latency
     // instead of NK-1; step s_lo-i lands in ring slot NK-i, where phase 0 expects it.
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
-    Row<T> wx[NLEAD], wB[NLEAD];
+    Row<T> lead[NLEAD][3];
     if constexpr (NK > 1) {
         if (s_lo > 0) {
 #pragma unroll
             for (int i = 1; i < NK; ++i) {
                 const int64_t t = (s_lo - i) * STEP + r;
-                wx[i - 1] = zero_row<T>(); wB[i - 1] = zero_row<T>();
-                if (cvalid && t >= 0) {
-                    wx[i - 1] = ldg_row(x + col + t * d);
-                    wB[i - 1] = ldg_row(B + col + t * d);
-                }
+                lead[i - 1][0] = zero_row<T>(); lead[i - 1][1] = zero_row<T>(); lead[i - 1][2] = zero_row<T>();
+                if (cvalid && t >= 0) load_in(t, lead[i - 1], false);
             }
         }
     }
@@ -387,9 +443,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
         if (s_lo > 0) {
 #pragma unroll
             for (int i = 1; i < NK; ++i) {
-                float xf[8], Bf[8], uf[8];
-                unpack8<T>(wx[i - 1], xf);
-                unpack8<T>(wB[i - 1], Bf);
+                float xf[8], Bf[8], Cf[8], uf[8];
+                in_floats<T, PK>(lead[i - 1], xf, Bf, Cf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
                 lds_store_row<T>(u_wr, pack8<T>(uf));
@@ -405,12 +460,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
-                Row<T> xn = zero_row<T>(), Bn = zero_row<T>(), Cn = zero_row<T>();
-                if (s + 1 < s_hi) fetch(s + 1, xn, Bn, Cn);
+                Row<T> nx[3] = {zero_row<T>(), zero_row<T>(), zero_row<T>()};
+                if (s + 1 < s_hi) fetch(s + 1, nx);
 
-                float xf[8], Bf[8], uf[8];
-                unpack8<T>(xr, xf);
-                unpack8<T>(Br, Bf);
+                float xf[8], Bf[8], Cf[8], uf[8];
+                in_floats<T, PK>(in, xf, Bf, Cf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
                 const Row<T> up = pack8<T>(uf);
@@ -435,14 +489,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                     const f32x4 p0 = *(const f32x4 *)y_rd;
                     const f32x4 p1 = *(const f32x4 *)(y_rd + 16);
                     float y2f[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
-                    float Cf[8], yf[8];
-                    unpack8<T>(Cr, Cf);
+                    float yf[8];
 #pragma unroll
                     for (int e = 0; e < 8; ++e) yf[e] = Cf[e] * y2f[e];
                     stg_row(y + col + t * d, pack8<T>(yf));
                     if (y2o) stg_row(y2o + col + t * d, pack8<T>(y2f));
                 }
-                xr = xn; Br = Bn; Cr = Cn;
+                in[0] = nx[0]; in[1] = nx[1]; in[2] = nx[2];
                 ++s;
             }
         }
@@ -467,7 +520,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 // (one 32-deep product contracts 16 channels x 2 row halves), lag = 16*delta + i - j.  At the
 // end the diagonals of the P tiles are summed in a fixed order into per-wave partials in
 // the workspace, and a second kernel adds the partials in a fixed order.
-template <typename T, int NK, int NW>
+//
+// PK: x, B, C are interleaved in one tensor that starts at C, and dx, dB, dC in one that starts
+// at dC (element stride 3).  C of step sigma+NK-1 then arrives together with x, B of that step,
+// NK-1 iterations before they are used, and the outputs of a row leave as one interleaved row.
+// The early x, B rows wait in LDS: each lane parks its own two row vectors in a ring of NK-1
+// slots and reads them back itself, so the ring needs no barrier.
+template <typename T, int NK, int NW, bool PK>
 __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                        const T *__restrict__ B, const T *__restrict__ C,
                                                        const T *__restrict__ h, T *__restrict__ dx,
@@ -486,9 +545,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     constexpr int OFF_Y = OFF_G + RING_ROWS * UROW;         // y2 tile, fp32, row-major
     constexpr int OFF_D = OFF_Y + STEP * YROW;              // du tile, fp32, row-major
     constexpr int OFF_H = OFF_D + STEP * YROW;              // filter tables
-    constexpr int LDS_MAIN = OFF_H + NW * HTAB * (int)sizeof(hraw_t);
+    constexpr int OFF_XB = (OFF_H + NW * HTAB * (int)sizeof(hraw_t) + 15) & ~15;   // PK: waiting x, B rows
+    constexpr int XB_SLOTS = (PK && NK > 1) ? NK - 1 : 0;
+    constexpr int XB_VEC = G::NT * 16 * M::RW;              // one row vector of every lane
+    constexpr int LDS_MAIN = OFF_XB + XB_SLOTS * 2 * XB_VEC;
     constexpr int LDS_TAIL = NW * ND * 256 * 4;             // P tiles at the end
     constexpr int LDS_BYTES = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
+    static_assert(LDS_BYTES <= 160 * 1024, "workgroup exceeds the 160 KB of LDS");
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
     unsigned char *u_rm = smem + OFF_U, *g_rm = smem + OFF_G, *y_st = smem + OFF_Y, *d_st = smem + OFF_D;
     hraw_t *htab = (hraw_t *)(smem + OFF_H);
@@ -533,34 +596,57 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     unsigned char *d_wr = d_st + (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
     const unsigned char *d_rd = d_st + r * YROW + 32 * a;
+    unsigned char *xb_own = smem + OFF_XB + tid * 16 * M::RW;                 // PK: slot k at + k * 2 * XB_VEC
 
-    // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the sequence)
-    auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
-        xo = zero_row<T>(); Bo = zero_row<T>(); dyo = zero_row<T>(); Co = zero_row<T>();
+    // Rows of iteration sg.  Separate tensors: in[0], in[1] = x, B of step sg; in[2] = C and dyo = dy
+    // of step sg+NK-1.  PK: in[] = the interleaved row and dyo = dy of step sg+NK-1.  Zero outside
+    // the sequence.
+    auto fetch = [&](int64_t sg, Row<T> (&in)[3], Row<T> &dyo) {
+        in[0] = zero_row<T>(); in[1] = zero_row<T>(); in[2] = zero_row<T>(); dyo = zero_row<T>();
         if (cvalid) {
             const int64_t t = sg * STEP + r;
-            if (t >= 0 && t < L) {
-                xo = ldg_row(x + col + t * d);
-                Bo = ldg_row(B + col + t * d);
-            }
             const int64_t t2 = t + (NK - 1) * STEP;
-            if (t2 >= 0 && t2 < L) {
-                dyo = ldg_row(dy + col + t2 * d);
-                Co = ldg_row(C + col + t2 * d);
+            if constexpr (PK) {
+                if (t2 >= 0 && t2 < L) {
+                    const T *src = C + 3 * (col + t2 * d);
+                    in[0] = ldg_row(src); in[1] = ldg_row(src + 8); in[2] = ldg_row(src + 16);
+                    dyo = ldg_row(dy + col + t2 * d);
+                }
+            } else {
+                if (t >= 0 && t < L) {
+                    in[0] = ldg_row(x + col + t * d);
+                    in[1] = ldg_row(B + col + t * d);
+                }
+                if (t2 >= 0 && t2 < L) {
+                    dyo = ldg_row(dy + col + t2 * d);
+                    in[2] = ldg_row(C + col + t2 * d);
+                }
             }
         }
     };
-    Row<T> xr, Br, dyr, Cr;
-    fetch(s_lo, xr, Br, dyr, Cr);
+    Row<T> in[3], dyr;
+    fetch(s_lo, in, dyr);
 
     // Lead-in: u of the NK-1 steps before the segment and g2 of its first NK-1 steps, i.e. the
     // rows iterations s_lo-NK+1 .. s_lo-1 would have brought.  They are requested together,
     // so the lead-in costs one memory latency instead of NK-1.
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
-    Row<T> wx[NLEAD], wB[NLEAD], wdy[NLEAD], wC[NLEAD];
+    Row<T> lead[NLEAD][3], wdy[NLEAD];
+    Row<T> past[PK ? NLEAD : 1][3];            // PK: the interleaved rows of steps s_lo-1 .. s_lo-NK+1
     if constexpr (NK > 1) {
+        if constexpr (PK) {
 #pragma unroll
-        for (int i = 1; i < NK; ++i) fetch(s_lo - i, wx[i - 1], wB[i - 1], wdy[i - 1], wC[i - 1]);
+            for (int i = 1; i < NK; ++i) {
+                const int64_t t = (s_lo - i) * STEP + r;
+                past[i - 1][0] = zero_row<T>(); past[i - 1][1] = zero_row<T>(); past[i - 1][2] = zero_row<T>();
+                if (cvalid && t >= 0) {
+                    const T *src = C + 3 * (col + t * d);
+                    past[i - 1][0] = ldg_row(src); past[i - 1][1] = ldg_row(src + 8); past[i - 1][2] = ldg_row(src + 16);
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 1; i < NK; ++i) fetch(s_lo - i, lead[i - 1], wdy[i - 1]);
     }
 
     // While those rows are in flight: the filter table of this wave's group and the Toeplitz tiles.
@@ -584,16 +670,28 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
             // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
-            float f0[8], f1[8], pf[8];
-            unpack8<T>(wx[i - 1], f0);
-            unpack8<T>(wB[i - 1], f1);
+            float f0[8], f1[8], f2[8], tf[8], pf[8];
+            if constexpr (PK) {
+                in_floats<T, true>(past[i - 1], f0, f1, f2);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
-            lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
-            unpack8<T>(wdy[i - 1], f0);
-            unpack8<T>(wC[i - 1], f1);
+                for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
+                lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
+                // x, B of step s_lo+NK-1-i wait in ring slot (NK-1-i) % (NK-1) for iteration s_lo+NK-1-i
+                in_floats<T, true>(lead[i - 1], f0, f1, f2);
+                unsigned char *slot = xb_own + ((NK - 1 - i) % (NK - 1)) * 2 * XB_VEC;
+                lds_store_row<T>(slot, pack8<T>(f0));
+                lds_store_row<T>(slot + XB_VEC, pack8<T>(f1));
+            } else {
+                unpack8<T>(lead[i - 1][0], f0);
+                unpack8<T>(lead[i - 1][1], f1);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
+                for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
+                lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
+                unpack8<T>(lead[i - 1][2], f2);
+            }
+            unpack8<T>(wdy[i - 1], tf);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = tf[e] * f2[e];
             unsigned char *g_slot = g_rm + (NK - 1 - i) * STEP * UROW;
             lds_store_row<T>(g_slot + rm_off, pack8<T>(pf));
             dyq[NK - 1 - i] = wdy[i - 1];
@@ -604,23 +702,41 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         }
     }
 
+    int xb_slot = 0;      // PK: ring slot of step s (steps s_lo+k sit in slot k % (NK-1))
     int64_t s = s_lo;
     while (s < s_hi) {
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
                 const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
-                Row<T> xn = zero_row<T>(), Bn = zero_row<T>(), dyn = zero_row<T>(), Cn = zero_row<T>();
-                if (s + 1 < s_hi) fetch(s + 1, xn, Bn, dyn, Cn);
+                Row<T> nx[3] = {zero_row<T>(), zero_row<T>(), zero_row<T>()}, dyn = zero_row<T>();
+                if (s + 1 < s_hi) fetch(s + 1, nx, dyn);
 
                 float xf[8], Bf[8], tf[8], cf[8], pf[8];
-                unpack8<T>(xr, xf);
-                unpack8<T>(Br, Bf);
+                if constexpr (PK) {
+                    float xa[8], Ba[8];
+                    in_floats<T, true>(in, xa, Ba, cf);       // x, B, C of step s+NK-1
+                    if constexpr (NK > 1) {
+                        unsigned char *slot = xb_own + xb_slot * 2 * XB_VEC;
+                        const Row<T> xw = lds_load_row<T>(slot), Bw = lds_load_row<T>(slot + XB_VEC);
+                        lds_store_row<T>(slot, pack8<T>(xa));
+                        lds_store_row<T>(slot + XB_VEC, pack8<T>(Ba));
+                        xb_slot = (xb_slot + 1 == NK - 1) ? 0 : xb_slot + 1;
+                        unpack8<T>(xw, xf);
+                        unpack8<T>(Bw, Bf);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) { xf[e] = xa[e]; Bf[e] = Ba[e]; }
+                    }
+                } else {
+                    unpack8<T>(in[0], xf);
+                    unpack8<T>(in[1], Bf);
+                    unpack8<T>(in[2], cf);
+                }
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[e] = xf[e] * Bf[e];
                 lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
                 unpack8<T>(dyr, tf);
-                unpack8<T>(Cr, cf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[e] = tf[e] * cf[e];
                 unsigned char *g_slot = g_rm + slot_new * STEP * UROW;
@@ -659,30 +775,31 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                 const int64_t t = s * STEP + r;
                 if (cvalid && t < L) {
                     const int64_t o = col + t * d;
-                    {
-                        const f32x4 p0 = *(const f32x4 *)y_rd;
-                        const f32x4 p1 = *(const f32x4 *)(y_rd + 16);
-                        const float y2f[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
-                        float dyf[8], of[8];
-                        unpack8<T>(dyq[ph], dyf);
+                    const f32x4 p0 = *(const f32x4 *)y_rd;
+                    const f32x4 p1 = *(const f32x4 *)(y_rd + 16);
+                    const float y2f[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
+                    const f32x4 e0 = *(const f32x4 *)d_rd;
+                    const f32x4 e1 = *(const f32x4 *)(d_rd + 16);
+                    const float duf[8] = {e0[0], e0[1], e0[2], e0[3], e1[0], e1[1], e1[2], e1[3]};
+                    float dyf[8], oC[8], ox[8], oB[8];
+                    unpack8<T>(dyq[ph], dyf);
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) of[e] = dyf[e] * y2f[e];
-                        stg_row(dC + o, pack8<T>(of));
-                    }
-                    {
-                        const f32x4 p0 = *(const f32x4 *)d_rd;
-                        const f32x4 p1 = *(const f32x4 *)(d_rd + 16);
-                        const float duf[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
-                        float of[8];
+                    for (int e = 0; e < 8; ++e) oC[e] = dyf[e] * y2f[e];
+                    if constexpr (!PK) stg_row(dC + o, pack8<T>(oC));
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) of[e] = duf[e] * Bf[e];
-                        stg_row(dx + o, pack8<T>(of));
+                    for (int e = 0; e < 8; ++e) ox[e] = duf[e] * Bf[e];
+                    if constexpr (!PK) stg_row(dx + o, pack8<T>(ox));
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) of[e] = duf[e] * xf[e];
-                        stg_row(dB + o, pack8<T>(of));
+                    for (int e = 0; e < 8; ++e) oB[e] = duf[e] * xf[e];
+                    if constexpr (!PK) stg_row(dB + o, pack8<T>(oB));
+                    if constexpr (PK) {
+                        Row<T> po[3];
+                        join_rows<T>(ox, oB, oC, po);
+                        T *dst = dC + 3 * o;
+                        stg_row(dst, po[0]); stg_row(dst + 8, po[1]); stg_row(dst + 16, po[2]);
                     }
                 }
-                xr = xn; Br = Bn; dyr = dyn; Cr = Cn;
+                in[0] = nx[0]; in[1] = nx[1]; in[2] = nx[2]; dyr = dyn;
                 ++s;
             }
         }
@@ -794,8 +911,12 @@ int fwd_launch(const void *x, const void *B, const void *C, const void *h, void 
     // 16-bit: ~112 registers, 4 waves per SIMD; fp32: ~200 registers, 2 waves per SIMD
     const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((mfma_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)x,
-                       (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+    if (dm.es == 3)
+        hipLaunchKernelGGL((mfma_fwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+                           (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+    else
+        hipLaunchKernelGGL((mfma_fwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+                           (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     return (int)hipGetLastError();
 }
 
@@ -863,9 +984,14 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
 {
     const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)dy,
-                       (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
-                       (float *)ws, dm, p);
+    if (dm.es == 3)
+        hipLaunchKernelGGL((mfma_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+                           (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
+                           (T *)dC, (float *)ws, dm, p);
+    else
+        hipLaunchKernelGGL((mfma_bwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+                           (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
+                           (T *)dC, (float *)ws, dm, p);
     int e = (int)hipGetLastError();
     if (e) return e;
     const int64_t n = (int64_t)dm.g * dm.hl;

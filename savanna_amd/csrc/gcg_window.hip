@@ -83,11 +83,59 @@ template <typename T, int VV> __device__ __forceinline__ typename Vec<T, VV>::ra
     return r;
 }
 
+// Interleaved operands (element stride 3): a lane's V channels of one row are 3V consecutive
+// elements, (C, B, x) per channel, i.e. three raw vectors.  split3 / join3 convert between
+// that order and per-tensor channel vectors; every index is a compile-time constant.
+template <typename T, int V>
+__device__ __forceinline__ void split3(const typename Vec<T, V>::raw (&p)[3], float (&xf)[V], float (&Bf)[V],
+                                       float (&Cf)[V])
+{
+    float f[3][V];
+#pragma unroll
+    for (int i = 0; i < 3; ++i) unpackv<T, V>(p[i], f[i]);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        Cf[v] = f[(3 * v) / V][(3 * v) % V];
+        Bf[v] = f[(3 * v + 1) / V][(3 * v + 1) % V];
+        xf[v] = f[(3 * v + 2) / V][(3 * v + 2) % V];
+    }
+}
+template <typename T, int V>
+__device__ __forceinline__ void join3(const float (&xf)[V], const float (&Bf)[V], const float (&Cf)[V],
+                                      typename Vec<T, V>::raw (&p)[3])
+{
+    float f[3][V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+        f[(3 * v) / V][(3 * v) % V] = Cf[v];
+        f[(3 * v + 1) / V][(3 * v + 1) % V] = Bf[v];
+        f[(3 * v + 2) / V][(3 * v + 2) % V] = xf[v];
+    }
+#pragma unroll
+    for (int i = 0; i < 3; ++i) p[i] = packv<T, V>(f[i]);
+}
+
+// One input row of a lane: three raw vectors, (x, B, C) of separate tensors or the three
+// thirds of the interleaved row.
+template <typename T, int V, bool PK>
+__device__ __forceinline__ void row_floats(const typename Vec<T, V>::raw (&p)[3], float (&xf)[V], float (&Bf)[V],
+                                           float (&Cf)[V])
+{
+    if constexpr (PK) {
+        split3<T, V>(p, xf, Bf, Cf);
+    } else {
+        unpackv<T, V>(p[0], xf);
+        unpackv<T, V>(p[1], Bf);
+        unpackv<T, V>(p[2], Cf);
+    }
+}
+
 struct WinPlan { int v, nvec, nseg, ts, ncvb, threads; int64_t nthreads, nwg; };
 
 
 // ---------------------------------------------------------------------------- forward
-template <typename T, int HL, int V>
+// PK: x, B, C are interleaved in one tensor that starts at C (element stride 3).
+template <typename T, int HL, int V, bool PK>
 __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x, const T *__restrict__ B,
                                                          const T *__restrict__ C, const T *__restrict__ h,
                                                          T *__restrict__ y, T *__restrict__ y2,
@@ -117,6 +165,19 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
     const int64_t base = b * L * d + c;   // (b*L + t)*d is uniform, c per lane
 
+    // input rows: PK reads three consecutive vectors from the interleaved tensor
+    const int64_t ibase = PK ? 3 * base : base, irow = PK ? 3 * d : d;
+    auto load_in = [&](int64_t t, raw_t (&p)[3], bool with_c) {
+        if constexpr (PK) {
+            const T *q = C + ibase + t * irow;
+            p[0] = ldg<raw_t>(q); p[1] = ldg<raw_t>(q + V); p[2] = ldg<raw_t>(q + 2 * V);
+        } else {
+            p[0] = ldg<raw_t>(x + ibase + t * irow);
+            p[1] = ldg<raw_t>(B + ibase + t * irow);
+            p[2] = with_c ? ldg<raw_t>(C + ibase + t * irow) : zero_raw<T, V>();
+        }
+    };
+
     float ring[RING][V];
 #pragma unroll
     for (int s = 0; s < RING; ++s)
@@ -127,9 +188,10 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
     for (int i = 1; i < HL; ++i) {
         const int64_t t = t_start - i;
         if (t >= 0) {
-            float xf[V], Bf[V];
-            unpackv<T, V>(ldg<raw_t>(x + base + t * d), xf);
-            unpackv<T, V>(ldg<raw_t>(B + base + t * d), Bf);
+            raw_t p[3];
+            float xf[V], Bf[V], Cf[V];
+            load_in(t, p, false);
+            row_floats<T, V, PK>(p, xf, Bf, Cf);
 #pragma unroll
             for (int v = 0; v < V; ++v) ring[RING - i][v] = xf[v] * Bf[v];
         }
@@ -140,16 +202,14 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
         for (int half = 0; half < RING / BATCH; ++half) {
             // rows are fetched BATCH at a time: enough loads in flight per lane without
             // pushing the register count past four waves per SIMD
-            raw_t xr[BATCH], Br[BATCH], Cr[BATCH];
+            raw_t in[BATCH][3];
 #pragma unroll
             for (int kk = 0; kk < BATCH; ++kk) {
                 const int64_t t = tb + half * BATCH + kk;
                 if (t < t_end) {
-                    xr[kk] = ldg<raw_t>(x + base + t * d);
-                    Br[kk] = ldg<raw_t>(B + base + t * d);
-                    Cr[kk] = ldg<raw_t>(C + base + t * d);
+                    load_in(t, in[kk], true);
                 } else {
-                    xr[kk] = zero_raw<T, V>(); Br[kk] = zero_raw<T, V>(); Cr[kk] = zero_raw<T, V>();
+                    in[kk][0] = zero_raw<T, V>(); in[kk][1] = zero_raw<T, V>(); in[kk][2] = zero_raw<T, V>();
                 }
             }
 #pragma unroll
@@ -157,9 +217,7 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
                 const int k = half * BATCH + kk;
                 const int64_t t = tb + k;
                 float xf[V], Bf[V], Cf[V], acc[V], out[V];
-                unpackv<T, V>(xr[kk], xf);
-                unpackv<T, V>(Br[kk], Bf);
-                unpackv<T, V>(Cr[kk], Cf);
+                row_floats<T, V, PK>(in[kk], xf, Bf, Cf);
 #pragma unroll
                 for (int v = 0; v < V; ++v) { ring[k][v] = xf[v] * Bf[v]; acc[v] = 0.f; }
 #pragma unroll
@@ -182,7 +240,10 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
 // Per lane: rows [t_start, t_end).  Row r is loaded at step r; dC[r] and the dh terms
 // of row r are produced at once (they look back), du[r-(HL-1)] is produced at step r
 // (it looks forward), so the walk runs HL-1 rows past t_end reading only dy and C.
-template <typename T, int HL, int V>
+// PK: x, B, C are interleaved in one tensor that starts at C, and dx, dB, dC in one that starts
+// at dC.  A row of the output then holds dC (ready at step r) next to dx, dB (ready HL-1 steps
+// later), so dC waits in a register ring like the raw x and B rows do.
+template <typename T, int HL, int V, bool PK>
 __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                          const T *__restrict__ B, const T *__restrict__ C,
                                                          const T *__restrict__ h, T *__restrict__ dx,
@@ -213,11 +274,14 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
     const int64_t base = b * L * d + c;   // (b*L + t)*d is uniform, c per lane
 
+    const int64_t ibase = PK ? 3 * base : base, irow = PK ? 3 * d : d;
+
     float ur[RING][V], gr[RING][V], dha[HL];
-    raw_t xs[RING], Bs[RING];
+    raw_t xs[RING], Bs[RING], dCs[PK ? RING : 1];
 #pragma unroll
     for (int s = 0; s < RING; ++s) {
         xs[s] = zero_raw<T, V>(); Bs[s] = zero_raw<T, V>();
+        if constexpr (PK) dCs[s] = zero_raw<T, V>();
 #pragma unroll
         for (int v = 0; v < V; ++v) { ur[s][v] = 0.f; gr[s][v] = 0.f; }
     }
@@ -227,9 +291,17 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
     for (int i = 1; i < HL; ++i) {
         const int64_t t = t_start - i;
         if (t >= 0) {
-            float xf[V], Bf[V];
-            unpackv<T, V>(ldg<raw_t>(x + base + t * d), xf);
-            unpackv<T, V>(ldg<raw_t>(B + base + t * d), Bf);
+            raw_t p[3];
+            float xf[V], Bf[V], Cf[V];
+            if constexpr (PK) {
+                const T *q = C + ibase + t * irow;
+                p[0] = ldg<raw_t>(q); p[1] = ldg<raw_t>(q + V); p[2] = ldg<raw_t>(q + 2 * V);
+            } else {
+                p[0] = ldg<raw_t>(x + ibase + t * irow);
+                p[1] = ldg<raw_t>(B + ibase + t * irow);
+                p[2] = zero_raw<T, V>();
+            }
+            row_floats<T, V, PK>(p, xf, Bf, Cf);
 #pragma unroll
             for (int v = 0; v < V; ++v) ur[RING - i][v] = xf[v] * Bf[v];
         }
@@ -241,38 +313,58 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
         for (int half = 0; half < RING / BATCH; ++half) {
             // rows are fetched BATCH at a time into staging registers; the x / B rings are only
             // overwritten slot by slot below, after the delayed du row has read them
-            raw_t dyr[BATCH], Cr[BATCH], xr[BATCH], Br[BATCH];
+            raw_t dyr[BATCH], in[BATCH][3];
 #pragma unroll
             for (int kk = 0; kk < BATCH; ++kk) {
                 const int64_t t = tb + half * BATCH + kk;
-                if (t < t_end) {
-                    xr[kk] = ldg<raw_t>(x + base + t * d);
-                    Br[kk] = ldg<raw_t>(B + base + t * d);
+                const bool ahead = t < L && t < t_stop;      // dy and C are read HL-1 rows past the run
+                if constexpr (PK) {
+                    if (ahead) {
+                        const T *q = C + ibase + t * irow;
+                        in[kk][0] = ldg<raw_t>(q); in[kk][1] = ldg<raw_t>(q + V); in[kk][2] = ldg<raw_t>(q + 2 * V);
+                        dyr[kk] = ldg<raw_t>(dy + base + t * d);
+                    } else {
+                        in[kk][0] = zero_raw<T, V>(); in[kk][1] = zero_raw<T, V>(); in[kk][2] = zero_raw<T, V>();
+                        dyr[kk] = zero_raw<T, V>();
+                    }
                 } else {
-                    xr[kk] = zero_raw<T, V>(); Br[kk] = zero_raw<T, V>();
-                }
-                if (t < L && t < t_stop) {
-                    dyr[kk] = ldg<raw_t>(dy + base + t * d);
-                    Cr[kk] = ldg<raw_t>(C + base + t * d);
-                } else {
-                    dyr[kk] = zero_raw<T, V>(); Cr[kk] = zero_raw<T, V>();
+                    if (t < t_end) {
+                        in[kk][0] = ldg<raw_t>(x + base + t * d);
+                        in[kk][1] = ldg<raw_t>(B + base + t * d);
+                    } else {
+                        in[kk][0] = zero_raw<T, V>(); in[kk][1] = zero_raw<T, V>();
+                    }
+                    if (ahead) {
+                        dyr[kk] = ldg<raw_t>(dy + base + t * d);
+                        in[kk][2] = ldg<raw_t>(C + base + t * d);
+                    } else {
+                        dyr[kk] = zero_raw<T, V>(); in[kk][2] = zero_raw<T, V>();
+                    }
                 }
             }
 #pragma unroll
             for (int kk = 0; kk < BATCH; ++kk) {
                 const int k = half * BATCH + kk;
                 const int64_t t = tb + k;
-                float dyf[V], Cf[V];
+                float dyf[V], xf[V], Bf[V], Cf[V];
                 unpackv<T, V>(dyr[kk], dyf);
-                unpackv<T, V>(Cr[kk], Cf);
+                if constexpr (PK) {
+                    row_floats<T, V, true>(in[kk], xf, Bf, Cf);
+                    xs[k] = packv<T, V>(xf);
+                    Bs[k] = packv<T, V>(Bf);
+                } else {
+                    unpackv<T, V>(in[kk][2], Cf);
+                    xs[k] = in[kk][0];
+                    Bs[k] = in[kk][1];
+                }
 #pragma unroll
                 for (int v = 0; v < V; ++v) gr[k][v] = dyf[v] * Cf[v];
-                xs[k] = xr[kk];
-                Bs[k] = Br[kk];
                 if (t < t_end) {
-                    float xf[V], Bf[V], y2v[V], o[V];
-                    unpackv<T, V>(xs[k], xf);
-                    unpackv<T, V>(Bs[k], Bf);
+                    float y2v[V], o[V];
+                    if constexpr (!PK) {
+                        unpackv<T, V>(xs[k], xf);
+                        unpackv<T, V>(Bs[k], Bf);
+                    }
 #pragma unroll
                     for (int v = 0; v < V; ++v) { ur[k][v] = xf[v] * Bf[v]; y2v[v] = 0.f; }
 #pragma unroll
@@ -288,12 +380,13 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                     }
 #pragma unroll
                     for (int v = 0; v < V; ++v) o[v] = dyf[v] * y2v[v];
-                    stg<raw_t>(dC + base + t * d, packv<T, V>(o));
+                    if constexpr (PK) dCs[k] = packv<T, V>(o);
+                    else stg<raw_t>(dC + base + t * d, packv<T, V>(o));
                 }
                 // du for row t-(HL-1): sum_j hr[j] * g2[row + j]
                 const int64_t orow = t - (HL - 1);
                 if (orow >= t_start && orow < t_end) {
-                    float du[V], xf[V], Bf[V], o[V];
+                    float du[V], xo[V], Bo[V], o[V];
 #pragma unroll
                     for (int v = 0; v < V; ++v) du[v] = 0.f;
 #pragma unroll
@@ -301,14 +394,25 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 #pragma unroll
                         for (int v = 0; v < V; ++v)
                             du[v] = fmaf(hr[j], gr[(k - (HL - 1) + j) & (RING - 1)][v], du[v]);
-                    unpackv<T, V>(xs[(k - (HL - 1)) & (RING - 1)], xf);
-                    unpackv<T, V>(Bs[(k - (HL - 1)) & (RING - 1)], Bf);
+                    unpackv<T, V>(xs[(k - (HL - 1)) & (RING - 1)], xo);
+                    unpackv<T, V>(Bs[(k - (HL - 1)) & (RING - 1)], Bo);
+                    if constexpr (PK) {
+                        float oB[V], oC[V];
+                        raw_t p[3];
 #pragma unroll
-                    for (int v = 0; v < V; ++v) o[v] = du[v] * Bf[v];
-                    stg<raw_t>(dx + base + orow * d, packv<T, V>(o));
+                        for (int v = 0; v < V; ++v) { o[v] = du[v] * Bo[v]; oB[v] = du[v] * xo[v]; }
+                        unpackv<T, V>(dCs[(k - (HL - 1)) & (RING - 1)], oC);
+                        join3<T, V>(o, oB, oC, p);
+                        T *q = dC + ibase + orow * irow;
+                        stg<raw_t>(q, p[0]); stg<raw_t>(q + V, p[1]); stg<raw_t>(q + 2 * V, p[2]);
+                    } else {
 #pragma unroll
-                    for (int v = 0; v < V; ++v) o[v] = du[v] * xf[v];
-                    stg<raw_t>(dB + base + orow * d, packv<T, V>(o));
+                        for (int v = 0; v < V; ++v) o[v] = du[v] * Bo[v];
+                        stg<raw_t>(dx + base + orow * d, packv<T, V>(o));
+#pragma unroll
+                        for (int v = 0; v < V; ++v) o[v] = du[v] * xo[v];
+                        stg<raw_t>(dB + base + orow * d, packv<T, V>(o));
+                    }
                 }
             }
         }
@@ -373,8 +477,12 @@ int fwd_v(const void *x, const void *B, const void *C, const void *h, void *y, v
     const WinPlan p = plan(dm, V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((window_fwd_kernel<T, HL, V>), dim3((unsigned)nwg), dim3(p.threads), 0, st, (const T *)x,
-                       (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+    if (dm.es == 3)
+        hipLaunchKernelGGL((window_fwd_kernel<T, HL, V, true>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+                           (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+    else
+        hipLaunchKernelGGL((window_fwd_kernel<T, HL, V, false>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+                           (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     return (int)hipGetLastError();
 }
 
@@ -385,9 +493,14 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
     const WinPlan p = plan(dm, BWD_V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V>), dim3((unsigned)nwg), dim3(p.threads), 0, st, (const T *)dy,
-                       (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
-                       (float *)ws, dm, p);
+    if (dm.es == 3)
+        hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V, true>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+                           (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
+                           (T *)dC, (float *)ws, dm, p);
+    else
+        hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V, false>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+                           (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
+                           (T *)dC, (float *)ws, dm, p);
     int e = (int)hipGetLastError();
     if (e) return e;
     hipLaunchKernelGGL(window_dh_reduce_kernel<T>, dim3((unsigned)(dm.g * dm.hl)), dim3(256), 0, st,

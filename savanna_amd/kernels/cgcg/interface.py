@@ -10,6 +10,7 @@ import warnings
 
 import torch
 
+from ... import _lib
 from .src.bwd import two_pass_bwd_refactor
 from .src.fwd import two_pass_fwd_grouped
 from .src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor  # noqa: F401
@@ -17,6 +18,32 @@ from .src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor  
 
 def _contig(t: torch.Tensor) -> torch.Tensor:
     return t if t.is_contiguous() else t.contiguous()
+
+
+def interleaved_source(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor):
+    """The (bs, L, g, dg, 3) tensor whose thirds [..., 0], [..., 1], [..., 2] are C, B, x, or None.
+
+    The interleaved split of the projected features (savanna/model/block.py:886-890,
+    ``rearrange(features, "b l (g dg p) -> b l g p dg", p=3).unbind(dim=3)`` -> x1, x2, v, passed on
+    as C, B, x) hands the operator three views of one buffer with element stride 3.  The reference
+    gathers each into its own tensor (interface.py:51-54); the HIP kernels read the buffer as it is.
+    """
+    if not (x.shape == B.shape == C.shape and x.dim() == 4 and x.dtype == B.dtype == C.dtype):
+        return None
+    if not (x.device == B.device == C.device):
+        return None
+    bs, L, g, dg = x.shape
+    want = (L * g * dg * 3, g * dg * 3, dg * 3, 3)
+    for t in (x, B, C):
+        if any(n > 1 and st != w for n, st, w in zip(t.shape, t.stride(), want)):
+            return None
+    base = C.untyped_storage().data_ptr()
+    if x.untyped_storage().data_ptr() != base or B.untyped_storage().data_ptr() != base:
+        return None
+    o = C.storage_offset()
+    if B.storage_offset() != o + 1 or x.storage_offset() != o + 2:
+        return None
+    return torch.as_strided(C, (bs, L, g, dg, 3), want + (1,), o)
 
 
 class TwoPassChunkedGateConvGate(torch.autograd.Function):
@@ -29,15 +56,31 @@ class TwoPassChunkedGateConvGate(torch.autograd.Function):
         schedule = schedule if fwd_autotune else fwd_kernel_cfg.schedule
         assert x.shape == torch.Size([bs, seqlen, g, dg])
         assert x.shape == B.shape == C.shape
+        ctx.input_shape = (bs, seqlen, g, dg)
+        feat = interleaved_source(x, B, C) if x.numel() > 0 else None
+        ctx.interleaved = feat is not None
+        if feat is not None:
+            # three views of one interleaved buffer: no gathers, one fused read
+            assert h.dim() == 3 and h.shape[0] == g and h.shape[1] == 1, "h must be (g, 1, hl)"
+            if schedule != "default":
+                raise NotImplementedError("Skip persistent for now") if schedule == "persistent" else \
+                    ValueError(f"schedule {schedule} not implemented")
+            h = _contig(h)
+            y = _lib.fwd_interleaved(feat, h)
+            ctx.save_for_backward(feat, h)
+            return y
         x, B, C, h = _contig(x), _contig(B), _contig(C), _contig(h)
         _, _, y = two_pass_fwd_grouped(x, B, C, h, autotune=fwd_autotune, schedule=schedule,
                                        return_bx=False, return_y2=False)
         ctx.save_for_backward(x, B, C, h)
-        ctx.input_shape = (bs, seqlen, g, dg)
         return y
 
     @staticmethod
     def backward(ctx, dy):
+        if ctx.interleaved:
+            feat, h = ctx.saved_tensors
+            dfeat, dh = _lib.bwd_interleaved(_contig(dy), feat, h)
+            return (dfeat[..., 2], dfeat[..., 1], dfeat[..., 0], dh) + (None,) * 10
         x, B, C, h = ctx.saved_tensors
         bs, seqlen, g, dg = ctx.input_shape
         dx, dB, dC, dh = two_pass_bwd_refactor(dy=_contig(dy), x=x, B=B, C=C, h=h,
@@ -70,3 +113,34 @@ def two_pass_chunked_gate_conv_gate(
         x, B, C, h, bs, seqlen, g, dg, schedule, fwd_autotune, fwd_kernel_cfg,
         fused_bwd, bwd_autotune, bwd_kernel_cfg,
     )
+
+
+class InterleavedGateConvGate(torch.autograd.Function):
+    """The same operator on the interleaved features tensor itself, so that the gradient is
+    produced in the features' layout and autograd has nothing to re-assemble."""
+
+    @staticmethod
+    def forward(ctx, feat, h):
+        feat, h = _contig(feat), _contig(h)
+        y = _lib.fwd_interleaved(feat, h)
+        ctx.save_for_backward(feat, h)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        feat, h = ctx.saved_tensors
+        dfeat, dh = _lib.bwd_interleaved(_contig(dy), feat, h)
+        return dfeat, dh
+
+
+def two_pass_chunked_gate_conv_gate_interleaved(features: torch.Tensor, h: torch.Tensor,
+                                                bs: int, seqlen: int, g: int, dg: int) -> torch.Tensor:
+    """y = x1 * conv(x2 * v, h) for projected features laid out "(g dg p)" with p = (x1, x2, v)
+    fastest, i.e. the tensor savanna/model/block.py:886-890 splits before calling the mixer.
+
+    features: (bs, seqlen, 3*g*dg) or (bs, seqlen, g, dg, 3); h: (g, 1, hl).  Returns (bs, seqlen, g, dg).
+    Equivalent to ``two_pass_chunked_gate_conv_gate(x=v, B=x2, C=x1, h=h, ...)`` on the split views.
+    """
+    assert features.numel() == bs * seqlen * g * dg * 3, "features must hold 3*g*dg values per position"
+    assert h.dim() == 3 and h.shape[0] == g and h.shape[1] == 1, "h must be (g, 1, hl)"
+    return InterleavedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3), h)

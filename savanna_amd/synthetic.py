@@ -27,6 +27,11 @@ class Workload:
     dtype: torch.dtype
     backward: bool
     about: str
+    # "separate": q, k, v are three contiguous tensors.  "interleaved": they are the thirds of one
+    # (bs, L, g, dg, 3) projected-features tensor and the kernels read it as it is.  "gathered": same
+    # features tensor, handled the way the reference does (three strided gathers before the forward,
+    # re-assembly of the feature gradient after the backward) around the separate-tensor kernels.
+    layout: str = "separate"
 
     @property
     def d(self) -> int:
@@ -70,6 +75,19 @@ WORKLOADS = {
                              "Hyena-MR forward+backward, bf16, B=8 L=8192 D=4096 G=256 hl=128"),
     "ref_bench_40b": Workload("ref_bench_40b", 2, 8192, 512, 16, (7,), torch.bfloat16, True,
                               "Hyena-SE forward+backward, bf16, B=2 L=8192 D=8192 G=512 hl=7"),
+    # Hyena-MR at the 7B layer shape fed from the interleaved projected features (block.py:886-890)
+    "mr_fwdbwd_7b_interleaved": Workload("mr_fwdbwd_7b_interleaved", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
+                                         "Hyena-MR forward+backward on interleaved features, bf16, B=2 L=8192 D=4096 "
+                                         "G=256 hl=128", layout="interleaved"),
+    "mr_fwdbwd_7b_gathered": Workload("mr_fwdbwd_7b_gathered", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
+                                      "the same with the reference's data flow: three gathers, separate-tensor "
+                                      "kernels, feature gradient re-assembled", layout="gathered"),
+    "se_fwdbwd_40b_interleaved": Workload("se_fwdbwd_40b_interleaved", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
+                                          "Hyena-SE forward+backward on interleaved features, bf16, B=1 L=32768 "
+                                          "D=8192 G=512 hl=7", layout="interleaved"),
+    "se_fwdbwd_40b_gathered": Workload("se_fwdbwd_40b_gathered", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
+                                       "the same with three gathers, separate-tensor kernels and re-assembly",
+                                       layout="gathered"),
 }
 # the order in which the benchmark reports them
 WORKLOAD_ORDER = ("se_fwd_fp32", "mr_fwd_7b", "mr_fwdbwd_7b", "se_mr_fwdbwd_40b", "mr_fwd_1m")
