@@ -189,7 +189,7 @@ GCG_API int gcg_fwd_interleaved(const void *feat, const void *h, void *y, int64_
     switch (a) {
     case GCG_ALGO_DIRECT: return finish(gcg::direct_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
     case GCG_ALGO_WINDOW: return finish(gcg::window_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
-    case GCG_ALGO_MFMA:   return finish(gcg::mfma_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
+    case GCG_ALGO_MFMA:   return finish(gcg::mfma_il_fwd_launch(dtype, feat, h, y, dm, st));
     }
     return GCG_ERR_BAD_ARG;
 }
@@ -218,7 +218,7 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
     case GCG_ALGO_WINDOW:
         return finish(gcg::window_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
     case GCG_ALGO_MFMA:
-        return finish(gcg::mfma_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+        return finish(gcg::mfma_il_bwd_launch(dtype, dy, feat, h, dfeat, dh, workspace, dm, st));
     }
     return GCG_ERR_BAD_ARG;
 }

@@ -84,6 +84,12 @@ struct Dims {
 
 constexpr int kWave = 64;
 
+
+// interleaved operands: feat / dfeat are (bs, L, g, dg, 3) with [..., 0] = C, [..., 1] = B, [..., 2] = x
+int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st);
+int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
+                       void *ws, const Dims &dm, hipStream_t st);
+
 } // namespace gcg
 
 // Host-side launchers, one translation unit per kernel family.  Each returns a
@@ -113,5 +119,16 @@ size_t mfma_bwd_workspace(int dtype, const Dims &dm);
 int mfma_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C,
                     const void *h, void *dx, void *dB, void *dC, void *dh, void *ws,
                     const Dims &dm, hipStream_t st);
+
+
+// interleaved operands: feat / dfeat are (bs, L, g, dg, 3) with [..., 0] = C, [..., 1] = B, [..., 2] = x
+int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st);
+int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
+                       void *ws, const Dims &dm, hipStream_t st);
+
+// interleaved operands: feat / dfeat are (bs, L, g, dg, 3) with [..., 0] = C, [..., 1] = B, [..., 2] = x
+int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st);
+int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
+                       void *ws, const Dims &dm, hipStream_t st);
 
 } // namespace gcg

@@ -1,0 +1,617 @@
+// Matrix-core kernels on interleaved operands: x, B, C are the thirds of one (bs, L, g, dg, 3)
+// projected-features tensor, [..., 0] = C, [..., 1] = B, [..., 2] = x, and the backward writes
+// dC, dB, dx in the same interleaved layout.
+//
+// The product side is the one of gcg_mfma.hip (same operand tiles, same order of operations,
+// so results agree bit for bit with the separate-tensor kernels).  The memory side differs: a
+// row of the workgroup's 16*NW channels is 48*NW elements of (C, B, x) triples, and a lane
+// takes 12 bytes of it per row -- two channels at 16 bits, one at fp32 -- so that the 64 lanes
+// of a load or store cover one contiguous 768-byte run.  (Eight channels per lane, as in the
+// separate-tensor kernels, would put lanes 48 bytes apart and make every access touch three
+// times the cache lines it uses; measured at 0.72x the bandwidth.)  With 12 bytes per row a
+// lane owns NR = 4 (16-bit) or 8 (fp32) rows of a 32-row step, RP = 32/NR rows apart.
+#include "gcg_mfma_tile.h"
+
+namespace gcg {
+namespace {
+
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+
+template <typename T, int NW> struct GeoIL {
+    static constexpr int CH = 4 / MT<T>::ES;                    // channels per lane
+    static constexpr int LPR = 16 * NW / CH;                    // lanes per row
+    static constexpr int RP = 64 * NW / LPR;                    // rows covered by one pass of the workgroup
+    static constexpr int NR = STEP / RP;                        // rows per lane and step
+    static_assert(NR * CH == 8, "a lane holds eight elements per tensor and step");
+};
+
+// 12-byte pieces are only 4-byte aligned; global memory takes that
+__device__ __forceinline__ u32x3 ldg12(const void *p) { return __builtin_nontemporal_load((const u32x3 *)p); }
+__device__ __forceinline__ void stg12(void *p, const u32x3 &v) { __builtin_nontemporal_store(v, (u32x3 *)p); }
+__device__ __forceinline__ uint32_t ldg4(const void *p) { return __builtin_nontemporal_load((const uint32_t *)p); }
+__device__ __forceinline__ void stg4(void *p, uint32_t v) { __builtin_nontemporal_store(v, (uint32_t *)p); }
+
+// A lane's pieces of one step <-> per-tensor values; element e = k * CH + c is row k, channel c.
+// 16 bits: a piece holds [C0 B0 | x0 C1 | B1 x1]; fp32: [C | B | x].
+template <typename T, int NR>
+__device__ __forceinline__ void il_split(const u32x3 (&p)[NR], float (&xf)[8], float (&Bf)[8], float (&Cf)[8])
+{
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+        if constexpr (MT<T>::ES == 4) {
+            Cf[k] = __uint_as_float(p[k][0]);
+            Bf[k] = __uint_as_float(p[k][1]);
+            xf[k] = __uint_as_float(p[k][2]);
+        } else {
+            MT<T>::unpack2(p[k][0], Cf[2 * k], Bf[2 * k]);
+            MT<T>::unpack2(p[k][1], xf[2 * k], Cf[2 * k + 1]);
+            MT<T>::unpack2(p[k][2], Bf[2 * k + 1], xf[2 * k + 1]);
+        }
+    }
+}
+template <typename T, int NR>
+__device__ __forceinline__ void il_join(const float (&xf)[8], const float (&Bf)[8], const float (&Cf)[8],
+                                        u32x3 (&p)[NR])
+{
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+        if constexpr (MT<T>::ES == 4) {
+            p[k][0] = __float_as_uint(Cf[k]);
+            p[k][1] = __float_as_uint(Bf[k]);
+            p[k][2] = __float_as_uint(xf[k]);
+        } else {
+            p[k][0] = MT<T>::pack2(Cf[2 * k], Bf[2 * k]);
+            p[k][1] = MT<T>::pack2(xf[2 * k], Cf[2 * k + 1]);
+            p[k][2] = MT<T>::pack2(Bf[2 * k + 1], xf[2 * k + 1]);
+        }
+    }
+}
+// the 4-byte unit of a plain tensor: CH elements of one row
+template <typename T> __device__ __forceinline__ uint32_t pack_unit(const float *f)
+{
+    if constexpr (MT<T>::ES == 4) return __float_as_uint(f[0]);
+    else return MT<T>::pack2(f[0], f[1]);
+}
+// NR units in a row vector: unpack8 then yields them in element order e = k * CH + c
+template <typename T, int NR> __device__ __forceinline__ Row<T> units_row(const uint32_t (&u)[NR])
+{
+    Row<T> r;
+    r.w[0] = make_uint4(u[0], u[1], u[2], u[3]);
+    if constexpr (NR == 8) r.w[1] = make_uint4(u[4], u[5], u[6], u[7]);
+    return r;
+}
+
+// ---------------------------------------------------------------------------- forward
+template <typename T, int NK, int NW>
+__global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restrict__ feat, const T *__restrict__ h,
+                                                          T *__restrict__ y, Dims dm, MfmaPlan pl)
+{
+    typedef MT<T> M;
+    typedef typename M::op_t op_t;
+    typedef typename M::hraw_t hraw_t;
+    typedef Geo<T, NW> G;
+    typedef GeoIL<T, NW> I;
+    constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW;
+    constexpr int CH = I::CH, LPR = I::LPR, RP = I::RP, NR = I::NR;
+    __shared__ __attribute__((aligned(16))) unsigned char u_rm[STEP * UROW];
+    __shared__ __attribute__((aligned(16))) unsigned char y_st[STEP * YROW];
+    __shared__ hraw_t htab[NW][HTAB];
+
+    int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
+    const int seg = (int)(wg % pl.nseg);
+    const int64_t b = wg / pl.nseg;
+
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+    const int rr = tid / LPR, a = tid % LPR;        // memory layout: rows rr + RP*k, channels CH*a ..
+    const int j = l & 15, q = l >> 4;               // matrix layout
+    const int64_t d = dm.d, L = dm.L;
+    const int64_t c0 = (int64_t)cb * CB;
+    const int hl = dm.hl;
+
+    const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
+    const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
+
+    const bool cvalid = c0 + CH * a < d;
+    const int64_t col = b * L * d + c0 + CH * a;           // element offset of this lane's columns
+
+    op_t A[NK];            // A[(ph - i + NK) % NK]: operand of step s-i while step s runs in phase ph
+#pragma unroll
+    for (int i = 0; i < NK; ++i) A[i] = M::zero_op();
+
+    unsigned char *u_wr = u_rm + rr * UROW + 4 * a;
+    unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
+    const unsigned char *y_rd = y_st + rr * YROW + 4 * CH * a;
+
+    auto fetch = [&](int64_t s, u32x3 (&p)[NR]) {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            const int64_t t = s * STEP + rr + RP * k;
+            p[k] = u32x3{0u, 0u, 0u};
+            if (cvalid && t >= 0 && t < L) p[k] = ldg12(feat + 3 * (col + t * d));
+        }
+    };
+    auto store_u = [&](const float (&uf)[8]) {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) *(uint32_t *)(u_wr + RP * k * UROW) = pack_unit<T>(&uf[CH * k]);
+    };
+    u32x3 in[NR];
+    fetch(s_lo, in);
+
+    // A segment that starts inside the sequence first rebuilds the operands of the NK-1 steps
+    // before it; their rows are requested together (one memory latency instead of NK-1) and
+    // step s_lo-i lands in ring slot NK-i, where phase 0 expects it.
+    constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
+    u32x3 lead[NLEAD][NR];
+    if constexpr (NK > 1) {
+        if (s_lo > 0) {
+#pragma unroll
+            for (int i = 1; i < NK; ++i) fetch(s_lo - i, lead[i - 1]);
+        }
+    }
+
+    // filter table of this wave's group, htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0
+    {
+        const int64_t cw = c0 + 16 * w;
+        const int64_t grp = (cw < d) ? cw / dm.dg : 0;
+        const hraw_t *hg = (const hraw_t *)h + grp * hl;
+        for (int i = l; i < HTAB; i += 64) {
+            const int lag = i - HPAD;
+            htab[w][i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
+        }
+    }
+    __syncthreads();
+    op_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+        W0[i] = M::toeplitz(htab[w], 32 * i, j, q);
+        W1[i] = M::toeplitz(htab[w], 32 * i + 16, j, q);
+    }
+
+    if constexpr (NK > 1) {
+        if (s_lo > 0) {
+#pragma unroll
+            for (int i = 1; i < NK; ++i) {
+                float xf[8], Bf[8], Cf[8], uf[8];
+                il_split<T, NR>(lead[i - 1], xf, Bf, Cf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
+                store_u(uf);
+                __syncthreads();
+                A[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
+                __syncthreads();
+            }
+        }
+    }
+
+    int64_t s = s_lo;
+    while (s < s_hi) {
+#pragma unroll
+        for (int ph = 0; ph < NK; ++ph) {
+            if (s < s_hi) {
+                u32x3 nx[NR];
+#pragma unroll
+                for (int k = 0; k < NR; ++k) nx[k] = u32x3{0u, 0u, 0u};
+                if (s + 1 < s_hi) fetch(s + 1, nx);
+
+                float xf[8], Bf[8], Cf[8], uf[8];
+                il_split<T, NR>(in, xf, Bf, Cf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
+                store_u(uf);
+                __syncthreads();
+                A[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
+                {
+                    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int i = 0; i < NK; ++i) {
+                        acc0 = M::mfma(A[(ph - i + NK) % NK], W0[i], acc0);
+                        acc1 = M::mfma(A[(ph - i + NK) % NK], W1[i], acc1);
+                    }
+                    *(f32x4 *)y_wr = acc0;
+                    *(f32x4 *)(y_wr + 16 * YROW) = acc1;
+                }
+                __syncthreads();
+#pragma unroll
+                for (int k = 0; k < NR; ++k) {
+                    const int64_t t = s * STEP + rr + RP * k;
+                    if (cvalid && t < L) {
+                        float yf[CH];
+#pragma unroll
+                        for (int c = 0; c < CH; ++c)
+                            yf[c] = Cf[CH * k + c] * *(const float *)(y_rd + RP * k * YROW + 4 * c);
+                        stg4(y + col + t * d, pack_unit<T>(yf));
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < NR; ++k) in[k] = nx[k];
+                ++s;
+            }
+        }
+    }
+}
+
+// --------------------------------------------------------------------------- backward
+// Same schedule as the separate-tensor backward: iteration sigma produces the outputs of step
+// sigma from u of steps sigma-NK+1..sigma and g2 = dy*C of steps sigma..sigma+NK-1.  In the
+// interleaved tensor C of step sigma+NK-1 arrives together with x, B of that step, NK-1
+// iterations before those are used, and the outputs of a row leave as one interleaved row.
+// The early x, B values wait in LDS: each lane parks its own two row vectors in a ring of NK-1
+// slots and reads them back itself, so the ring needs no barrier.
+template <typename T, int NK, int NW>
+__global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ feat,
+                                                          const T *__restrict__ h, T *__restrict__ dfeat,
+                                                          float *__restrict__ ws, Dims dm, MfmaPlan pl)
+{
+    typedef MT<T> M;
+    typedef typename M::op_t op_t;
+    typedef typename M::hraw_t hraw_t;
+    typedef Geo<T, NW> G;
+    typedef GeoIL<T, NW> I;
+    constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW;
+    constexpr int CH = I::CH, LPR = I::LPR, RP = I::RP, NR = I::NR;
+    constexpr int ND = 2 * NK - 1;
+    constexpr int RING_ROWS = STEP * NK;
+    constexpr int OFF_U = 0;                                // u of the current step, row-major
+    constexpr int OFF_G = OFF_U + STEP * UROW;              // g2 ring, NK steps, row-major
+    constexpr int OFF_Y = OFF_G + RING_ROWS * UROW;         // y2 tile, fp32, row-major
+    constexpr int OFF_D = OFF_Y + STEP * YROW;              // du tile, fp32, row-major
+    constexpr int OFF_H = OFF_D + STEP * YROW;              // filter tables
+    constexpr int OFF_XB = (OFF_H + NW * HTAB * (int)sizeof(hraw_t) + 15) & ~15;   // waiting x, B values
+    constexpr int XB_SLOTS = NK > 1 ? NK - 1 : 0;
+    constexpr int XB_VEC = G::NT * 16 * M::RW;              // one row vector of every lane
+    constexpr int LDS_MAIN = OFF_XB + XB_SLOTS * 2 * XB_VEC;
+    constexpr int LDS_TAIL = NW * ND * 256 * 4;             // P tiles at the end
+    constexpr int LDS_BYTES = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
+    static_assert(LDS_BYTES <= 160 * 1024, "workgroup exceeds the 160 KB of LDS");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
+    unsigned char *u_rm = smem + OFF_U, *g_rm = smem + OFF_G, *y_st = smem + OFF_Y, *d_st = smem + OFF_D;
+    hraw_t *htab = (hraw_t *)(smem + OFF_H);
+
+    const int64_t wg_id = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    int64_t wg = wg_id;
+    const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
+    const int seg = (int)(wg % pl.nseg);
+    const int64_t b = wg / pl.nseg;
+
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+    const int rr = tid / LPR, a = tid % LPR;        // memory layout: rows rr + RP*k, channels CH*a ..
+    const int j = l & 15, q = l >> 4;               // matrix layout
+    const int64_t d = dm.d, L = dm.L;
+    const int64_t c0 = (int64_t)cb * CB;
+    const int hl = dm.hl;
+    const bool wave_valid = c0 + 16 * w < d;
+
+    const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
+    const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
+
+    const bool cvalid = c0 + CH * a < d;
+    const int64_t col = b * L * d + c0 + CH * a;
+
+    // While step s runs in phase ph:  Au[(ph - i + NK) % NK] is the u operand of step s-i,
+    // Ag[(ph + i) % NK] the time-reversed g2 operand of step s+i, dyq[(ph + i) % NK] dy of step s+i.
+    op_t Au[NK], Ag[NK];
+    Row<T> dyq[NK];
+    f32x4 P[ND];
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+        Au[i] = M::zero_op();
+        Ag[i] = M::zero_op();
+        dyq[i] = zero_row<T>();
+    }
+#pragma unroll
+    for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // LDS addresses of this lane
+    const int rm_off = rr * UROW + 4 * a;                                     // memory layout, row rr
+    unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
+    unsigned char *d_wr = d_st + (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
+    const unsigned char *y_rd = y_st + rr * YROW + 4 * CH * a;
+    const unsigned char *d_rd = d_st + rr * YROW + 4 * CH * a;
+    unsigned char *xb_own = smem + OFF_XB + tid * 16 * M::RW;                 // slot k at + k * 2 * XB_VEC
+
+    // interleaved rows and dy of one step (zero outside the sequence)
+    auto fetch_feat = [&](int64_t step, u32x3 (&p)[NR]) {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            const int64_t t = step * STEP + rr + RP * k;
+            p[k] = u32x3{0u, 0u, 0u};
+            if (cvalid && t >= 0 && t < L) p[k] = ldg12(feat + 3 * (col + t * d));
+        }
+    };
+    auto fetch_dy = [&](int64_t step, Row<T> &o) {
+        uint32_t u[NR];
+#pragma unroll
+        for (int k = 0; k < NR; ++k) {
+            const int64_t t = step * STEP + rr + RP * k;
+            u[k] = 0u;
+            if (cvalid && t >= 0 && t < L) u[k] = ldg4(dy + col + t * d);
+        }
+        o = units_row<T, NR>(u);
+    };
+    auto store_rows = [&](unsigned char *tile, const float (&f)[8]) {
+#pragma unroll
+        for (int k = 0; k < NR; ++k) *(uint32_t *)(tile + rm_off + RP * k * UROW) = pack_unit<T>(&f[CH * k]);
+    };
+
+    // iteration sigma brings the interleaved rows and dy of step sigma+NK-1
+    u32x3 in[NR];
+    Row<T> dyr;
+    fetch_feat(s_lo + NK - 1, in);
+    fetch_dy(s_lo + NK - 1, dyr);
+
+    // Lead-in: the rows of the NK-1 steps before the segment (for u) and of its first NK-1 steps
+    // (for g2, and x, B to wait in the ring), i.e. what iterations s_lo-NK+1 .. s_lo-1 would have
+    // brought.  Requested together, so the lead-in costs one memory latency instead of NK-1.
+    constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
+    u32x3 past[NLEAD][NR], lead[NLEAD][NR];
+    Row<T> wdy[NLEAD];
+    if constexpr (NK > 1) {
+#pragma unroll
+        for (int i = 1; i < NK; ++i) {
+            fetch_feat(s_lo - i, past[i - 1]);
+            fetch_feat(s_lo + NK - 1 - i, lead[i - 1]);
+            fetch_dy(s_lo + NK - 1 - i, wdy[i - 1]);
+        }
+    }
+
+    // While those rows are in flight: the filter table of this wave's group and the Toeplitz tiles.
+    {
+        const int64_t grp = wave_valid ? (c0 + 16 * w) / dm.dg : 0;
+        const hraw_t *hg = (const hraw_t *)h + grp * hl;
+        for (int i = l; i < HTAB; i += 64) {
+            const int lag = i - HPAD;
+            htab[w * HTAB + i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
+        }
+    }
+    __syncthreads();
+    op_t W0[NK], W1[NK];
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+        W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
+        W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
+    }
+
+    if constexpr (NK > 1) {
+#pragma unroll
+        for (int i = 1; i < NK; ++i) {
+            // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
+            float f0[8], f1[8], f2[8], tf[8], pf[8];
+            il_split<T, NR>(past[i - 1], f0, f1, f2);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
+            store_rows(u_rm, pf);
+            // x, B of step s_lo+NK-1-i wait in ring slot (NK-1-i) % (NK-1) for iteration s_lo+NK-1-i
+            il_split<T, NR>(lead[i - 1], f0, f1, f2);
+            unsigned char *slot = xb_own + ((NK - 1 - i) % (NK - 1)) * 2 * XB_VEC;
+            lds_store_row<T>(slot, pack8<T>(f0));
+            lds_store_row<T>(slot + XB_VEC, pack8<T>(f1));
+            unpack8<T>(wdy[i - 1], tf);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = tf[e] * f2[e];
+            unsigned char *g_slot = g_rm + (NK - 1 - i) * STEP * UROW;
+            store_rows(g_slot, pf);
+            dyq[NK - 1 - i] = wdy[i - 1];
+            __syncthreads();
+            Au[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
+            Ag[NK - 1 - i] = M::load_operand(g_slot, UROW, w, j, q, true);
+            __syncthreads();
+        }
+    }
+
+    int xb_slot = 0;      // ring slot of step s (step s_lo+k sits in slot k % (NK-1))
+    int64_t s = s_lo;
+    while (s < s_hi) {
+#pragma unroll
+        for (int ph = 0; ph < NK; ++ph) {
+            if (s < s_hi) {
+                const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
+                u32x3 nx[NR];
+                Row<T> dyn = zero_row<T>();
+#pragma unroll
+                for (int k = 0; k < NR; ++k) nx[k] = u32x3{0u, 0u, 0u};
+                if (s + 1 < s_hi) {
+                    fetch_feat(s + NK, nx);
+                    fetch_dy(s + NK, dyn);
+                }
+
+                float xf[8], Bf[8], tf[8], cf[8], pf[8];
+                {
+                    float xa[8], Ba[8];
+                    il_split<T, NR>(in, xa, Ba, cf);          // x, B, C of step s+NK-1
+                    if constexpr (NK > 1) {
+                        unsigned char *slot = xb_own + xb_slot * 2 * XB_VEC;
+                        const Row<T> xw = lds_load_row<T>(slot), Bw = lds_load_row<T>(slot + XB_VEC);
+                        lds_store_row<T>(slot, pack8<T>(xa));
+                        lds_store_row<T>(slot + XB_VEC, pack8<T>(Ba));
+                        xb_slot = (xb_slot + 1 == NK - 1) ? 0 : xb_slot + 1;
+                        unpack8<T>(xw, xf);
+                        unpack8<T>(Bw, Bf);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) { xf[e] = xa[e]; Bf[e] = Ba[e]; }
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pf[e] = xf[e] * Bf[e];
+                store_rows(u_rm, pf);
+                unpack8<T>(dyr, tf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pf[e] = tf[e] * cf[e];
+                unsigned char *g_slot = g_rm + slot_new * STEP * UROW;
+                store_rows(g_slot, pf);
+                dyq[slot_new] = dyr;
+                __syncthreads();
+                Au[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
+                Ag[slot_new] = M::load_operand(g_slot, UROW, w, j, q, true);
+                {
+                    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+                    f32x4 dac0 = {0.f, 0.f, 0.f, 0.f}, dac1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int i = 0; i < NK; ++i) {
+                        acc0 = M::mfma(Au[(ph - i + NK) % NK], W0[i], acc0);
+                        acc1 = M::mfma(Au[(ph - i + NK) % NK], W1[i], acc1);
+                        dac0 = M::mfma(Ag[(ph + i) % NK], W1[i], dac0);   // output rows 0..15
+                        dac1 = M::mfma(Ag[(ph + i) % NK], W0[i], dac1);   // output rows 16..31
+                    }
+                    *(f32x4 *)y_wr = acc0;
+                    *(f32x4 *)(y_wr + 16 * YROW) = acc1;
+                    *(f32x4 *)d_wr = dac0;
+                    *(f32x4 *)(d_wr + 16 * YROW) = dac1;
+                    // filter-gradient tiles: natural-layout operands (rows j and 16+j of a 32-row window)
+                    const op_t un = M::load_natural(u_rm + j * UROW, u_rm + (16 + j) * UROW, w, q);
+#pragma unroll
+                    for (int dl = 0; dl < ND; ++dl) {
+                        int row0 = STEP * ph + 16 * dl + j;              // ring rows of the window's two halves
+                        int row1 = row0 + 16;
+                        row0 = (row0 >= RING_ROWS) ? row0 - RING_ROWS : row0;
+                        row1 = (row1 >= RING_ROWS) ? row1 - RING_ROWS : row1;
+                        const op_t gn = M::load_natural(g_rm + row0 * UROW, g_rm + row1 * UROW, w, q);
+                        P[dl] = M::mfma(gn, un, P[dl]);
+                    }
+                }
+                __syncthreads();
+                {
+                    float dyf[8], oC[8], ox[8], oB[8];
+                    unpack8<T>(dyq[ph], dyf);
+#pragma unroll
+                    for (int k = 0; k < NR; ++k)
+#pragma unroll
+                        for (int c = 0; c < CH; ++c) {
+                            const int e = CH * k + c;
+                            const float y2v = *(const float *)(y_rd + RP * k * YROW + 4 * c);
+                            const float duv = *(const float *)(d_rd + RP * k * YROW + 4 * c);
+                            oC[e] = dyf[e] * y2v;
+                            ox[e] = duv * Bf[e];
+                            oB[e] = duv * xf[e];
+                        }
+                    u32x3 po[NR];
+                    il_join<T, NR>(ox, oB, oC, po);
+#pragma unroll
+                    for (int k = 0; k < NR; ++k) {
+                        const int64_t t = s * STEP + rr + RP * k;
+                        if (cvalid && t < L) stg12(dfeat + 3 * (col + t * d), po[k]);
+                    }
+                }
+#pragma unroll
+                for (int k = 0; k < NR; ++k) in[k] = nx[k];
+                dyr = dyn;
+                ++s;
+            }
+        }
+    }
+
+    // diagonal sums of the P tiles -> per-wave filter-gradient partials
+    __syncthreads();
+    float *pt = (float *)smem + w * ND * 256;
+#pragma unroll
+    for (int dl = 0; dl < ND; ++dl)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) pt[dl * 256 + (4 * q + v) * 16 + j] = P[dl][v];
+    __syncthreads();
+    if (wave_valid) {
+        float *out = ws + ((size_t)wg_id * NW + w) * 128;
+        for (int lag = l; lag < 128; lag += 64) {
+            const int d0 = lag >> 4, r16 = lag & 15;
+            float sum = 0.f;
+            if (d0 < ND)
+                for (int jj = 0; jj + r16 < 16; ++jj) sum += pt[d0 * 256 + (jj + r16) * 16 + jj];
+            if (d0 + 1 < ND)
+                for (int ii = 0; ii < r16; ++ii) sum += pt[(d0 + 1) * 256 + ii * 16 + ii + 16 - r16];
+            out[lag] = sum;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------- launch
+template <typename T, int NK, int NW>
+int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
+{
+    const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16);
+    if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((mfma_il_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)feat,
+                       (const T *)h, (T *)y, dm, p);
+    return (int)hipGetLastError();
+}
+
+template <typename T, int NK> int fwd_nk(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
+{
+    const int nw = choose_nw(dm, sizeof(T) == 4);
+    if constexpr (sizeof(T) == 2) {
+        if (nw == 16) return fwd_launch<T, NK, 16>(feat, h, y, dm, st);
+    }
+    if (nw == 8) return fwd_launch<T, NK, 8>(feat, h, y, dm, st);
+    return fwd_launch<T, NK, 4>(feat, h, y, dm, st);
+}
+
+template <typename T> int fwd_t(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
+{
+    switch (nk_for(dm.hl)) {
+    case 1: return fwd_nk<T, 1>(feat, h, y, dm, st);
+    case 2: return fwd_nk<T, 2>(feat, h, y, dm, st);
+    case 3: return fwd_nk<T, 3>(feat, h, y, dm, st);
+    case 4: return fwd_nk<T, 4>(feat, h, y, dm, st);
+    default: return fwd_nk<T, 5>(feat, h, y, dm, st);
+    }
+}
+
+// same plan as the separate-tensor backward, so gcg_bwd_workspace_bytes covers both
+template <typename T, int NK, int NW>
+int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *ws, const Dims &dm,
+               hipStream_t st)
+{
+    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
+    if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL((mfma_il_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)dy,
+                       (const T *)feat, (const T *)h, (T *)dfeat, (float *)ws, dm, p);
+    int e = (int)hipGetLastError();
+    if (e) return e;
+    const int64_t n = (int64_t)dm.g * dm.hl;
+    hipLaunchKernelGGL(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       (const float *)ws, (T *)dh, dm, p);
+    return (int)hipGetLastError();
+}
+
+template <typename T, int NK>
+int bwd_nk(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *ws, const Dims &dm,
+           hipStream_t st)
+{
+    if constexpr (sizeof(T) == 2) {
+        if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, feat, h, dfeat, dh, ws, dm, st);
+    }
+    return bwd_launch<T, NK, 4>(dy, feat, h, dfeat, dh, ws, dm, st);
+}
+
+template <typename T>
+int bwd_t(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *ws, const Dims &dm,
+          hipStream_t st)
+{
+    switch (nk_for(dm.hl)) {
+    case 1: return bwd_nk<T, 1>(dy, feat, h, dfeat, dh, ws, dm, st);
+    case 2: return bwd_nk<T, 2>(dy, feat, h, dfeat, dh, ws, dm, st);
+    case 3: return bwd_nk<T, 3>(dy, feat, h, dfeat, dh, ws, dm, st);
+    case 4: return bwd_nk<T, 4>(dy, feat, h, dfeat, dh, ws, dm, st);
+    default: return bwd_nk<T, 5>(dy, feat, h, dfeat, dh, ws, dm, st);
+    }
+}
+
+} // namespace
+
+int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
+{
+    if (dtype == GCG_BF16) return fwd_t<bf16_t>(feat, h, y, dm, st);
+    if (dtype == GCG_F16) return fwd_t<f16_t>(feat, h, y, dm, st);
+    if (dtype == GCG_F32) return fwd_t<float>(feat, h, y, dm, st);
+    return (int)hipErrorInvalidValue;
+}
+
+int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
+                       void *ws, const Dims &dm, hipStream_t st)
+{
+    if (dtype == GCG_BF16) return bwd_t<bf16_t>(dy, feat, h, dfeat, dh, ws, dm, st);
+    if (dtype == GCG_F16) return bwd_t<f16_t>(dy, feat, h, dfeat, dh, ws, dm, st);
+    if (dtype == GCG_F32) return bwd_t<float>(dy, feat, h, dfeat, dh, ws, dm, st);
+    return (int)hipErrorInvalidValue;
+}
+
+} // namespace gcg

@@ -1,0 +1,375 @@
+// Shared pieces of the matrix-core kernels: element-type traits of the 32-deep banded-Toeplitz
+// product, the row-vector helpers, streaming loads and stores, the filter-gradient reduction
+// and the host-side launch plan.  Included by the separate-tensor kernels (gcg_mfma.hip) and
+// the interleaved-features kernels (gcg_mfma_il.hip).
+#pragma once
+#include "gcg_common.h"
+
+#include <cstdlib>
+
+namespace gcg {
+namespace {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int STEP = 32;          // time rows per step (contraction depth of one product)
+constexpr int HPAD = 32;          // filter table holds lags [-32, 160)
+constexpr int HTAB = 192;
+
+// Transposing LDS read: within each block of 16 lanes, lane i receives element (i % 4) of
+// the 8-byte rows addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4 of that block.
+__device__ __forceinline__ s16x4 lds_read_tr(const unsigned char *p)
+{
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3))) *)p);
+}
+
+// Per element type: the matrix operand, how it is fetched from a row-major LDS tile of
+// `urow` bytes per time row, and the 32-deep product.  Operand element e of the lane in
+// quad q stands for contraction index kmap(q, e); both factors of a product use the same map.
+template <typename T> struct MT;
+
+template <typename OP> struct MT16 {
+    static constexpr int ES = 2;                 // bytes per element
+    static constexpr int RW = 1;                 // 16-byte words per 8-channel row vector
+    static constexpr int UPAD = 32;              // row padding: consecutive rows start 8 banks apart
+    typedef OP op_t;
+    typedef uint16_t hraw_t;
+    static __device__ __forceinline__ int kmap(int q, int e) { return 8 * q + e; }
+    static __device__ __forceinline__ op_t zero_op()
+    {
+        op_t r;
+        const uint4 z = make_uint4(0u, 0u, 0u, 0u);
+        __builtin_memcpy(&r, &z, 16);
+        return r;
+    }
+    // time samples kmap(q, .) of channel 16w+j from rows row0 .. row0+31 (reversed: 31-k)
+    static __device__ __forceinline__ op_t load_operand(const unsigned char *tile, int urow, int w, int j, int q,
+                                                        bool reversed)
+    {
+        const int col = (16 * w + 4 * (j & 3)) * 2;
+        const int r0 = reversed ? 31 - 8 * q - (j >> 2) : 8 * q + (j >> 2);
+        const int r1 = reversed ? r0 - 4 : r0 + 4;
+        const s16x4 lo = lds_read_tr(tile + r0 * urow + col);
+        const s16x4 hi = lds_read_tr(tile + r1 * urow + col);
+        const short v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        op_t r;
+        __builtin_memcpy(&r, v, 16);
+        return r;
+    }
+    // natural-layout operand of the filter-gradient product: 8 channels of one of two rows;
+    // lane quad q takes row half q>>1 and channels 8*(q&1)..+7 of the wave's 16
+    static __device__ __forceinline__ op_t load_natural(const unsigned char *row_half0,
+                                                        const unsigned char *row_half1, int w, int q)
+    {
+        const unsigned char *p = ((q >> 1) ? row_half1 : row_half0) + (16 * w + 8 * (q & 1)) * 2;
+        const uint4 t4 = *(const uint4 *)p;
+        op_t r;
+        __builtin_memcpy(&r, &t4, 16);
+        return r;
+    }
+    static __device__ __forceinline__ op_t toeplitz(const hraw_t *htab, int doff, int j, int q)
+    {
+        uint16_t v[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = htab[doff + j - kmap(q, e) + HPAD];
+        op_t r;
+        __builtin_memcpy(&r, v, 16);
+        return r;
+    }
+};
+
+template <> struct MT<bf16_t> : MT16<bf16x8> {
+    static __device__ __forceinline__ f32x4 mfma(op_t a, op_t b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void unpack2(uint32_t p, float &lo, float &hi)
+    {
+        lo = __uint_as_float(p << 16);
+        hi = __uint_as_float(p & 0xffff0000u);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+};
+template <> struct MT<f16_t> : MT16<f16x8> {
+    static __device__ __forceinline__ f32x4 mfma(op_t a, op_t b, f32x4 c)
+    {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void unpack2(uint32_t p, float &lo, float &hi)
+    {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        h2 v;
+        __builtin_memcpy(&v, &p, 4);
+        lo = (float)v[0];
+        hi = (float)v[1];
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
+};
+
+struct F32x8 { float v[8]; };
+template <> struct MT<float> {
+    static constexpr int ES = 4;
+    static constexpr int RW = 2;
+    static constexpr int UPAD = 64;              // consecutive rows start 16 banks apart
+    typedef F32x8 op_t;
+    typedef float hraw_t;
+    // instruction e of the eight contracts time samples 4e .. 4e+3, one per lane quad
+    static __device__ __forceinline__ int kmap(int q, int e) { return 4 * e + q; }
+    static __device__ __forceinline__ op_t zero_op()
+    {
+        op_t r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r.v[e] = 0.f;
+        return r;
+    }
+    static __device__ __forceinline__ op_t load_operand(const unsigned char *tile, int urow, int w, int j, int q,
+                                                        bool reversed)
+    {
+        op_t r;
+        const int col = (16 * w + j) * 4;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const int k = kmap(q, e);
+            r.v[e] = *(const float *)(tile + (reversed ? 31 - k : k) * urow + col);
+        }
+        return r;
+    }
+    // element e: row half e>>2, channel 4q + (e&3) of the wave's 16
+    static __device__ __forceinline__ op_t load_natural(const unsigned char *row_half0,
+                                                        const unsigned char *row_half1, int w, int q)
+    {
+        const int col = (16 * w + 4 * q) * 4;
+        const f32x4 a = *(const f32x4 *)(row_half0 + col), b = *(const f32x4 *)(row_half1 + col);
+        op_t r;
+        r.v[0] = a[0]; r.v[1] = a[1]; r.v[2] = a[2]; r.v[3] = a[3];
+        r.v[4] = b[0]; r.v[5] = b[1]; r.v[6] = b[2]; r.v[7] = b[3];
+        return r;
+    }
+    static __device__ __forceinline__ op_t toeplitz(const hraw_t *htab, int doff, int j, int q)
+    {
+        op_t r;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) r.v[e] = htab[doff + j - kmap(q, e) + HPAD];
+        return r;
+    }
+    static __device__ __forceinline__ f32x4 mfma(const op_t &a, const op_t &b, f32x4 c)
+    {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[e], b.v[e], c, 0, 0, 0);
+        return c;
+    }
+};
+
+// A workgroup of NW waves owns CB = 16*NW adjacent channels; LDS rows are padded (see UPAD;
+// the fp32 result tile: consecutive rows start 4 banks apart).
+template <typename T, int NW> struct Geo {
+    static constexpr int CB = 16 * NW;                          // channels per workgroup
+    static constexpr int LPR = CB / 8;                          // lanes per row in the row layout (8 channels each)
+    static constexpr int UROW = CB * MT<T>::ES + MT<T>::UPAD;   // bytes per LDS row of u / g2
+    static constexpr int YROW = CB * 4 + 16;                    // bytes per LDS row of y2 / du
+    static constexpr int NT = 64 * NW;                          // threads
+};
+
+// A lane's 8 channels of one row: RW 16-byte words.
+template <typename T> struct Row { uint4 w[MT<T>::RW]; };
+
+template <typename T> __device__ __forceinline__ void unpack8(const Row<T> &r, float (&f)[8])
+{
+    if constexpr (MT<T>::ES == 4) {
+        f[0] = __uint_as_float(r.w[0].x); f[1] = __uint_as_float(r.w[0].y);
+        f[2] = __uint_as_float(r.w[0].z); f[3] = __uint_as_float(r.w[0].w);
+        f[4] = __uint_as_float(r.w[1].x); f[5] = __uint_as_float(r.w[1].y);
+        f[6] = __uint_as_float(r.w[1].z); f[7] = __uint_as_float(r.w[1].w);
+    } else {
+        MT<T>::unpack2(r.w[0].x, f[0], f[1]);
+        MT<T>::unpack2(r.w[0].y, f[2], f[3]);
+        MT<T>::unpack2(r.w[0].z, f[4], f[5]);
+        MT<T>::unpack2(r.w[0].w, f[6], f[7]);
+    }
+}
+template <typename T> __device__ __forceinline__ Row<T> pack8(const float (&f)[8])
+{
+    Row<T> r;
+    if constexpr (MT<T>::ES == 4) {
+        r.w[0] = make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]), __float_as_uint(f[2]), __float_as_uint(f[3]));
+        r.w[1] = make_uint4(__float_as_uint(f[4]), __float_as_uint(f[5]), __float_as_uint(f[6]), __float_as_uint(f[7]));
+    } else {
+        r.w[0] = make_uint4(MT<T>::pack2(f[0], f[1]), MT<T>::pack2(f[2], f[3]), MT<T>::pack2(f[4], f[5]),
+                            MT<T>::pack2(f[6], f[7]));
+    }
+    return r;
+}
+template <typename T> __device__ __forceinline__ Row<T> zero_row()
+{
+    Row<T> r;
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) r.w[i] = make_uint4(0u, 0u, 0u, 0u);
+    return r;
+}
+template <typename T> __device__ __forceinline__ void lds_store_row(unsigned char *p, const Row<T> &r)
+{
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) *(uint4 *)(p + 16 * i) = r.w[i];
+}
+
+template <typename T> __device__ __forceinline__ Row<T> lds_load_row(const unsigned char *p)
+{
+    Row<T> r;
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) r.w[i] = *(const uint4 *)(p + 16 * i);
+    return r;
+}
+
+// Streaming accesses: every tensor element is touched once, so loads and stores carry the
+// nontemporal hint (GCG_MFMA_NT=0 at build time turns it off for comparison).
+#ifndef GCG_XCD_SWIZZLE
+#define GCG_XCD_SWIZZLE 1
+#endif
+#ifndef GCG_MFMA_NT
+#define GCG_MFMA_NT 3
+#endif
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+template <typename T> __device__ __forceinline__ uint4 ldg16(const T *p);
+template <typename T> __device__ __forceinline__ void stg16(T *p, const uint4 &v);
+template <typename T> __device__ __forceinline__ Row<T> ldg_row(const T *p)
+{
+    Row<T> r;
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) r.w[i] = ldg16((const unsigned char *)p + 16 * i);
+    return r;
+}
+template <typename T> __device__ __forceinline__ void stg_row(T *p, const Row<T> &r)
+{
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) stg16((unsigned char *)p + 16 * i, r.w[i]);
+}
+template <typename T> __device__ __forceinline__ uint4 ldg16(const T *p)
+{
+#if GCG_MFMA_NT & 1
+    const u32x4 v = __builtin_nontemporal_load((const u32x4 *)p);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+#else
+    return *(const uint4 *)p;
+#endif
+}
+template <typename T> __device__ __forceinline__ void stg16(T *p, const uint4 &v)
+{
+#if GCG_MFMA_NT & 2
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, (u32x4 *)p);
+#else
+    *(uint4 *)p = v;
+#endif
+}
+
+// Workgroups are dealt to the 8 XCDs round-robin by index.  Re-labelling them so that each XCD
+// receives a contiguous run of (batch, segment, channel-block) triples makes the workgroups of
+// one XCD cover whole tensor rows between them, which its L2 and the memory channels prefer.
+__device__ __forceinline__ int64_t xcd_contiguous_id(int64_t id, int64_t n)
+{
+#if GCG_XCD_SWIZZLE
+    if ((n & 7) == 0) return (id & 7) * (n >> 3) + (id >> 3);
+#endif
+    return id;
+}
+
+struct MfmaPlan { int ncb, nseg, steps_per_seg, nw; int64_t nsteps, nwg; };
+
+// Operand tile of the banded Toeplitz matrix at row offset doff = (out time) - (in time) of the
+// tile origins: element e of lane (j, q) is the tap for lag doff + j - kmap(q, e)  (MT<T>::toeplitz).
+
+
+// dh[grp][k] = sum of the per-wave partials of the 16-channel blocks of the group
+template <typename T>
+__global__ __launch_bounds__(256) void mfma_dh_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dh,
+                                                             Dims dm, MfmaPlan pl)
+{
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (int64_t)dm.g * dm.hl) return;
+    const int64_t grp = i / dm.hl;
+    const int lag = dm.hl - 1 - (int)(i % dm.hl);
+    const int bpg = dm.dg / 16;                          // 16-channel blocks per group
+    const int64_t slots = (int64_t)pl.ncb * pl.nw;       // block slots per (batch, segment)
+    float sum = 0.f;
+    for (int64_t p = 0; p < dm.bs * pl.nseg; ++p)
+        for (int k = 0; k < bpg; ++k)
+            sum += ws[(p * slots + grp * bpg + k) * 128 + lag];
+    Elem<T>::store(dh + i, sum);
+}
+
+int cu_count()
+{
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            n = v;
+        else
+            n = 256;
+    }
+    return n;
+}
+
+int env_int(const char *name, int dflt)
+{
+    const char *v = getenv(name);
+    return (v && atoi(v) > 0) ? atoi(v) : dflt;
+}
+
+// Waves per workgroup: wider workgroups read wider rows (16*NW channels, 32*NW bytes), which
+// the memory system rewards; narrow tensors fall back to what their width fills.
+// fp32 doubles the register state per wave (operand tiles hold 8 floats), which caps the
+// forward at 8 waves and the backward at 4.
+int choose_nw(const Dims &dm, bool fp32)
+{
+    static const int forced = env_int("GCG_MFMA_NW", 0);   // tuning override: 4, 8 or 16
+    if (forced == 4 || forced == 8 || (forced == 16 && !fp32)) return forced;
+    if (dm.d >= 256 && !fp32) return 16;
+    if (dm.d >= 128) return 8;
+    return 4;
+}
+
+MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu)
+{
+    MfmaPlan p;
+    const int cb = 16 * nw;
+    p.nw = nw;
+    p.ncb = (int)((dm.d + cb - 1) / cb);
+    p.nsteps = (dm.L + STEP - 1) / STEP;
+    const int wg_per_cu = waves_per_cu / nw > 0 ? waves_per_cu / nw : 1;
+    int64_t cols = dm.bs * p.ncb;
+    int64_t want = ((int64_t)cu_count() * wg_per_cu + cols - 1) / cols;   // segments to fill the chip
+    int64_t max_seg = p.nsteps / min_steps;
+    if (max_seg < 1) max_seg = 1;
+    if (want > max_seg) want = max_seg;
+    if (want < 1) want = 1;
+    static const int forced = env_int("GCG_MFMA_STEPS_PER_SEG", 0);        // tuning override
+    int64_t sps = (p.nsteps + want - 1) / want;
+    if (forced > 0) sps = forced;
+    p.steps_per_seg = (int)sps;
+    p.nseg = (int)((p.nsteps + sps - 1) / sps);
+    p.nwg = dm.bs * p.nseg * p.ncb;
+    return p;
+}
+
+// input steps an output step reaches back over: lags up to hl-1 from rows 0..31 of the step
+int nk_for(int hl) { const int n = (hl + 30) / 32 + 1; return n > 5 ? 5 : n; }
+
+// The backward holds about twice the forward's register state per wave, so it runs two
+// waves per SIMD and at most 8 waves (128 channels, 256-byte rows) per workgroup.
+int choose_nw_bwd(const Dims &dm, bool fp32)
+{
+    static const int forced = env_int("GCG_MFMA_BWD_NW", 0);   // tuning override: 4 or 8
+    if (forced == 4 || (forced == 8 && !fp32)) return forced;
+    return (dm.d >= 128 && !fp32) ? 8 : 4;
+}
+
+// 16-bit: two waves per SIMD (8 per CU); fp32: one (4 per CU)
+MfmaPlan plan_bwd(const Dims &dm, bool fp32) { return plan(dm, choose_nw_bwd(dm, fp32), 16, fp32 ? 4 : 8); }
+
+} // namespace
+} // namespace gcg
