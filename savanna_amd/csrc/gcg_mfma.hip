@@ -26,7 +26,8 @@ namespace gcg {
 namespace {
 
 // ---------------------------------------------------------------------------- forward
-template <typename T, int NK, int NW>
+// EXTRA: also write the convolution before the post-gate (y2o) and the pre-gate product (bxo).
+template <typename T, int NK, int NW, bool EXTRA>
 __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__ x, const T *__restrict__ B,
                                                        const T *__restrict__ C, const T *__restrict__ h,
                                                        T *__restrict__ y, T *__restrict__ y2o,
@@ -56,8 +57,17 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
 
-    const bool cvalid = c0 + 8 * a < d;
-    const int64_t col = b * L * d + c0 + 8 * a;            // element offset of this lane's columns
+    // Windows over rows [t0, t1) of this batch row; a lane's offset is lane_off + step_off(s).
+    const int64_t t0 = (s_lo - (NK - 1)) * STEP > 0 ? (s_lo - (NK - 1)) * STEP : 0;
+    const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
+    const int64_t row_bytes = d * ES, win_bytes = (t1 - t0) * row_bytes;
+    const int64_t origin = (b * L + t0) * d;
+    const win_t wx = make_window(x + origin, win_bytes), wB = make_window(B + origin, win_bytes);
+    const win_t wC = make_window(C + origin, win_bytes), wy = make_window(y + origin, win_bytes);
+    const win_t wy2 = make_window(EXTRA && y2o ? y2o + origin : y + origin, EXTRA && y2o ? win_bytes : 0);
+    const win_t wbx = make_window(EXTRA && bxo ? bxo + origin : y + origin, EXTRA && bxo ? win_bytes : 0);
+    const uint32_t lane_off = (uint32_t)(r * row_bytes + (c0 + 8 * a) * ES) + (c0 + 8 * a < d ? 0u : WIN_OFF);
+    auto step_off = [&](int64_t s) { return (uint32_t)((s * STEP - t0) * row_bytes); };
 
     op_t A[NK];            // A[(ph - i + NK) % NK]: operand of step s-i while step s runs in phase ph
 #pragma unroll
@@ -69,33 +79,25 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 
     Row<T> xr, Br, Cr;
     auto fetch = [&](int64_t s, Row<T> &xo, Row<T> &Bo, Row<T> &Co) {
-        const int64_t t = s * STEP + r;
-        xo = zero_row<T>(); Bo = zero_row<T>(); Co = zero_row<T>();
-        if (cvalid && t < L) {
-            const int64_t o = col + t * d;
-            xo = ldg_row(x + o);
-            Bo = ldg_row(B + o);
-            Co = ldg_row(C + o);
-        }
+        const uint32_t o = lane_off + step_off(s);
+        xo = ldw_row<T>(wx, o);
+        Bo = ldw_row<T>(wB, o);
+        Co = ldw_row<T>(wC, o);
     };
     fetch(s_lo, xr, Br, Cr);
 
-    // A segment that starts inside the sequence first rebuilds the operands of the NK-1 steps
-    // before it.  Their rows are requested together, so the replay costs one memory latency
-    // instead of NK-1; step s_lo-i lands in ring slot NK-i, where phase 0 expects it.
+    // The operands of the NK-1 steps before the segment are rebuilt first (zero before the
+    // start of the sequence).  Their rows are requested together, so the replay costs one
+    // memory latency instead of NK-1; step s_lo-i lands in ring slot NK-i, where phase 0
+    // expects it.
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
-    Row<T> wx[NLEAD], wB[NLEAD];
+    Row<T> lx[NLEAD], lB[NLEAD];
     if constexpr (NK > 1) {
-        if (s_lo > 0) {
 #pragma unroll
-            for (int i = 1; i < NK; ++i) {
-                const int64_t t = (s_lo - i) * STEP + r;
-                wx[i - 1] = zero_row<T>(); wB[i - 1] = zero_row<T>();
-                if (cvalid && t >= 0) {
-                    wx[i - 1] = ldg_row(x + col + t * d);
-                    wB[i - 1] = ldg_row(B + col + t * d);
-                }
-            }
+        for (int i = 1; i < NK; ++i) {
+            const uint32_t o = lane_off + step_off(s_lo - i);
+            lx[i - 1] = ldw_row<T>(wx, o);
+            lB[i - 1] = ldw_row<T>(wB, o);
         }
     }
 
@@ -119,19 +121,17 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     }
 
     if constexpr (NK > 1) {
-        if (s_lo > 0) {
 #pragma unroll
-            for (int i = 1; i < NK; ++i) {
-                float xf[8], Bf[8], uf[8];
-                unpack8<T>(wx[i - 1], xf);
-                unpack8<T>(wB[i - 1], Bf);
+        for (int i = 1; i < NK; ++i) {
+            float xf[8], Bf[8], uf[8];
+            unpack8<T>(lx[i - 1], xf);
+            unpack8<T>(lB[i - 1], Bf);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
-                lds_store_row<T>(u_wr, pack8<T>(uf));
-                __syncthreads();
-                A[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
-                __syncthreads();
-            }
+            for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
+            lds_store_row<T>(u_wr, pack8<T>(uf));
+            __syncthreads();
+            A[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
+            __syncthreads();
         }
     }
 
@@ -140,8 +140,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
-                Row<T> xn = zero_row<T>(), Bn = zero_row<T>(), Cn = zero_row<T>();
-                if (s + 1 < s_hi) fetch(s + 1, xn, Bn, Cn);
+                // rows of the next step; past the segment they fall outside the window
+                Row<T> xn, Bn, Cn;
+                fetch(s + 1, xn, Bn, Cn);
 
                 float xf[8], Bf[8], uf[8];
                 unpack8<T>(xr, xf);
@@ -150,9 +151,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                 for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
                 const Row<T> up = pack8<T>(uf);
                 lds_store_row<T>(u_wr, up);
-                const int64_t t = s * STEP + r;
-                const bool store_ok = cvalid && t < L;
-                if (bxo && store_ok) stg_row(bxo + col + t * d, up);
+                const uint32_t o = lane_off + step_off(s);
+                if constexpr (EXTRA) stw_row<T>(wbx, o, up);
                 __syncthreads();
                 A[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
                 {
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                     *(f32x4 *)(y_wr + 16 * YROW) = acc1;
                 }
                 __syncthreads();
-                if (store_ok) {
+                {
                     const f32x4 p0 = *(const f32x4 *)y_rd;
                     const f32x4 p1 = *(const f32x4 *)(y_rd + 16);
                     float y2f[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
@@ -174,8 +174,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                     unpack8<T>(Cr, Cf);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) yf[e] = Cf[e] * y2f[e];
-                    stg_row(y + col + t * d, pack8<T>(yf));
-                    if (y2o) stg_row(y2o + col + t * d, pack8<T>(y2f));
+                    stw_row<T>(wy, o, pack8<T>(yf));
+                    if constexpr (EXTRA) stw_row<T>(wy2, o, pack8<T>(y2f));
                 }
                 xr = xn; Br = Bn; Cr = Cn;
                 ++s;
@@ -245,8 +245,19 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
 
-    const bool cvalid = c0 + 8 * a < d;
-    const int64_t col = b * L * d + c0 + 8 * a;
+    // Windows of this batch row: x, B and the outputs over rows [t0, t1), dy and C over [t0, t2)
+    // (the backward looks NK-1 steps ahead for g2).  A lane's offset is lane_off + step_off(s).
+    const int64_t t0 = (s_lo - (NK - 1)) * STEP > 0 ? (s_lo - (NK - 1)) * STEP : 0;
+    const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
+    const int64_t t2 = (s_hi + NK - 1) * STEP < L ? (s_hi + NK - 1) * STEP : L;
+    const int64_t row_bytes = d * ES, origin = (b * L + t0) * d;
+    const int64_t near_bytes = (t1 - t0) * row_bytes, far_bytes = (t2 - t0) * row_bytes;
+    const win_t wx = make_window(x + origin, near_bytes), wB = make_window(B + origin, near_bytes);
+    const win_t wdy = make_window(dy + origin, far_bytes), wC = make_window(C + origin, far_bytes);
+    const win_t wdx = make_window(dx + origin, near_bytes), wdB = make_window(dB + origin, near_bytes);
+    const win_t wdC = make_window(dC + origin, near_bytes);
+    const uint32_t lane_off = (uint32_t)(r * row_bytes + (c0 + 8 * a) * ES) + (c0 + 8 * a < d ? 0u : WIN_OFF);
+    auto step_off = [&](int64_t sg) { return (uint32_t)((sg * STEP - t0) * row_bytes); };
 
     // While step s runs in phase ph:  Au[(ph - i + NK) % NK] is the u operand of step s-i,
     // Ag[(ph + i) % NK] the time-reversed g2 operand of step s+i, dyq[(ph + i) % NK] dy of step s+i.
@@ -269,21 +280,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
     const unsigned char *d_rd = d_st + r * YROW + 32 * a;
 
-    // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the sequence)
+    // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the windows)
     auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
-        xo = zero_row<T>(); Bo = zero_row<T>(); dyo = zero_row<T>(); Co = zero_row<T>();
-        if (cvalid) {
-            const int64_t t = sg * STEP + r;
-            if (t >= 0 && t < L) {
-                xo = ldg_row(x + col + t * d);
-                Bo = ldg_row(B + col + t * d);
-            }
-            const int64_t t2 = t + (NK - 1) * STEP;
-            if (t2 >= 0 && t2 < L) {
-                dyo = ldg_row(dy + col + t2 * d);
-                Co = ldg_row(C + col + t2 * d);
-            }
-        }
+        const uint32_t o = lane_off + step_off(sg), o2 = lane_off + step_off(sg + NK - 1);
+        xo = ldw_row<T>(wx, o);
+        Bo = ldw_row<T>(wB, o);
+        dyo = ldw_row<T>(wdy, o2);
+        Co = ldw_row<T>(wC, o2);
     };
     Row<T> xr, Br, dyr, Cr;
     fetch(s_lo, xr, Br, dyr, Cr);
@@ -292,10 +295,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     // rows iterations s_lo-NK+1 .. s_lo-1 would have brought.  They are requested together,
     // so the lead-in costs one memory latency instead of NK-1.
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
-    Row<T> wx[NLEAD], wB[NLEAD], wdy[NLEAD], wC[NLEAD];
+    Row<T> wx_[NLEAD], wB_[NLEAD], wdy_[NLEAD], wC_[NLEAD];
     if constexpr (NK > 1) {
 #pragma unroll
-        for (int i = 1; i < NK; ++i) fetch(s_lo - i, wx[i - 1], wB[i - 1], wdy[i - 1], wC[i - 1]);
+        for (int i = 1; i < NK; ++i) fetch(s_lo - i, wx_[i - 1], wB_[i - 1], wdy_[i - 1], wC_[i - 1]);
     }
 
     // While those rows are in flight: the filter table of this wave's group and the Toeplitz tiles.
@@ -320,18 +323,18 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         for (int i = 1; i < NK; ++i) {
             // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
             float f0[8], f1[8], pf[8];
-            unpack8<T>(wx[i - 1], f0);
-            unpack8<T>(wB[i - 1], f1);
+            unpack8<T>(wx_[i - 1], f0);
+            unpack8<T>(wB_[i - 1], f1);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
             lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
-            unpack8<T>(wdy[i - 1], f0);
-            unpack8<T>(wC[i - 1], f1);
+            unpack8<T>(wdy_[i - 1], f0);
+            unpack8<T>(wC_[i - 1], f1);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
             unsigned char *g_slot = g_rm + (NK - 1 - i) * STEP * UROW;
             lds_store_row<T>(g_slot + rm_off, pack8<T>(pf));
-            dyq[NK - 1 - i] = wdy[i - 1];
+            dyq[NK - 1 - i] = wdy_[i - 1];
             __syncthreads();
             Au[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
             Ag[NK - 1 - i] = M::load_operand(g_slot, UROW, w, j, q, true);
@@ -345,8 +348,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
                 const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
-                Row<T> xn = zero_row<T>(), Bn = zero_row<T>(), dyn = zero_row<T>(), Cn = zero_row<T>();
-                if (s + 1 < s_hi) fetch(s + 1, xn, Bn, dyn, Cn);
+                // rows of the next iteration; past the segment they fall outside the windows
+                Row<T> xn, Bn, dyn, Cn;
+                fetch(s + 1, xn, Bn, dyn, Cn);
 
                 float xf[8], Bf[8], tf[8], cf[8], pf[8];
                 unpack8<T>(xr, xf);
@@ -391,9 +395,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                     }
                 }
                 __syncthreads();
-                const int64_t t = s * STEP + r;
-                if (cvalid && t < L) {
-                    const int64_t o = col + t * d;
+                {
+                    const uint32_t o = lane_off + step_off(s);
                     {
                         const f32x4 p0 = *(const f32x4 *)y_rd;
                         const f32x4 p1 = *(const f32x4 *)(y_rd + 16);
@@ -402,7 +405,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         unpack8<T>(dyq[ph], dyf);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = dyf[e] * y2f[e];
-                        stg_row(dC + o, pack8<T>(of));
+                        stw_row<T>(wdC, o, pack8<T>(of));
                     }
                     {
                         const f32x4 p0 = *(const f32x4 *)d_rd;
@@ -411,10 +414,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         float of[8];
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * Bf[e];
-                        stg_row(dx + o, pack8<T>(of));
+                        stw_row<T>(wdx, o, pack8<T>(of));
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * xf[e];
-                        stg_row(dB + o, pack8<T>(of));
+                        stw_row<T>(wdB, o, pack8<T>(of));
                     }
                 }
                 xr = xn; Br = Bn; dyr = dyn; Cr = Cn;
@@ -450,10 +453,14 @@ int fwd_launch(const void *x, const void *B, const void *C, const void *h, void 
                const Dims &dm, hipStream_t st)
 {
     // 16-bit: ~112 registers, 4 waves per SIMD; fp32: ~200 registers, 2 waves per SIMD
-    const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16);
+    const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((mfma_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)x,
-                       (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+    if (y2 || bx)
+        hipLaunchKernelGGL((mfma_fwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+                           (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+    else
+        hipLaunchKernelGGL((mfma_fwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+                           (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     return (int)hipGetLastError();
 }
 

@@ -15,8 +15,6 @@
 namespace gcg {
 namespace {
 
-typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
-
 template <typename T, int NW> struct GeoIL {
     static constexpr int CH = 4 / MT<T>::ES;                    // channels per lane
     static constexpr int LPR = 16 * NW / CH;                    // lanes per row
@@ -24,12 +22,6 @@ template <typename T, int NW> struct GeoIL {
     static constexpr int NR = STEP / RP;                        // rows per lane and step
     static_assert(NR * CH == 8, "a lane holds eight elements per tensor and step");
 };
-
-// 12-byte pieces are only 4-byte aligned; global memory takes that
-__device__ __forceinline__ u32x3 ldg12(const void *p) { return __builtin_nontemporal_load((const u32x3 *)p); }
-__device__ __forceinline__ void stg12(void *p, const u32x3 &v) { __builtin_nontemporal_store(v, (u32x3 *)p); }
-__device__ __forceinline__ uint32_t ldg4(const void *p) { return __builtin_nontemporal_load((const uint32_t *)p); }
-__device__ __forceinline__ void stg4(void *p, uint32_t v) { __builtin_nontemporal_store(v, (uint32_t *)p); }
 
 // A lane's pieces of one step <-> per-tensor values; element e = k * CH + c is row k, channel c.
 // 16 bits: a piece holds [C0 B0 | x0 C1 | B1 x1]; fp32: [C | B | x].
@@ -112,8 +104,18 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
 
+    // Windows over rows [t0, t1) of this batch row (12-byte pieces are only 4-byte aligned, which
+    // buffer accesses take).  A lane's offset into y is lane_off + k * pass_off + step_off(s); into
+    // the features three times that.
+    const int64_t t0 = (s_lo - (NK - 1)) * STEP > 0 ? (s_lo - (NK - 1)) * STEP : 0;
+    const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
+    const int64_t row_bytes = d * M::ES, win_bytes = (t1 - t0) * row_bytes;
+    const int64_t origin = (b * L + t0) * d;
+    const win_t wf = make_window(feat + 3 * origin, 3 * win_bytes), wy = make_window(y + origin, win_bytes);
     const bool cvalid = c0 + CH * a < d;
-    const int64_t col = b * L * d + c0 + CH * a;           // element offset of this lane's columns
+    const uint32_t lane_off = (uint32_t)(rr * row_bytes + (c0 + CH * a) * M::ES);
+    const uint32_t pass_off = (uint32_t)(RP * row_bytes), bad = cvalid ? 0u : WIN_OFF;
+    auto step_off = [&](int64_t s) { return (uint32_t)((s * STEP - t0) * row_bytes); };
 
     op_t A[NK];            // A[(ph - i + NK) % NK]: operand of step s-i while step s runs in phase ph
 #pragma unroll
@@ -124,12 +126,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     const unsigned char *y_rd = y_st + rr * YROW + 4 * CH * a;
 
     auto fetch = [&](int64_t s, u32x3 (&p)[NR]) {
+        const uint32_t o = lane_off + step_off(s);
 #pragma unroll
-        for (int k = 0; k < NR; ++k) {
-            const int64_t t = s * STEP + rr + RP * k;
-            p[k] = u32x3{0u, 0u, 0u};
-            if (cvalid && t >= 0 && t < L) p[k] = ldg12(feat + 3 * (col + t * d));
-        }
+        for (int k = 0; k < NR; ++k) p[k] = ldw12(wf, 3 * (o + k * pass_off) + bad);
     };
     auto store_u = [&](const float (&uf)[8]) {
 #pragma unroll
@@ -144,10 +143,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
     u32x3 lead[NLEAD][NR];
     if constexpr (NK > 1) {
-        if (s_lo > 0) {
 #pragma unroll
-            for (int i = 1; i < NK; ++i) fetch(s_lo - i, lead[i - 1]);
-        }
+        for (int i = 1; i < NK; ++i) fetch(s_lo - i, lead[i - 1]);
     }
 
     // filter table of this wave's group, htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0
@@ -169,18 +166,16 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     }
 
     if constexpr (NK > 1) {
-        if (s_lo > 0) {
 #pragma unroll
-            for (int i = 1; i < NK; ++i) {
-                float xf[8], Bf[8], Cf[8], uf[8];
-                il_split<T, NR>(lead[i - 1], xf, Bf, Cf);
+        for (int i = 1; i < NK; ++i) {
+            float xf[8], Bf[8], Cf[8], uf[8];
+            il_split<T, NR>(lead[i - 1], xf, Bf, Cf);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
-                store_u(uf);
-                __syncthreads();
-                A[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
-                __syncthreads();
-            }
+            for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
+            store_u(uf);
+            __syncthreads();
+            A[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
+            __syncthreads();
         }
     }
 
@@ -189,10 +184,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
-                u32x3 nx[NR];
-#pragma unroll
-                for (int k = 0; k < NR; ++k) nx[k] = u32x3{0u, 0u, 0u};
-                if (s + 1 < s_hi) fetch(s + 1, nx);
+                u32x3 nx[NR];        // rows of the next step; past the segment they fall outside the window
+                fetch(s + 1, nx);
 
                 float xf[8], Bf[8], Cf[8], uf[8];
                 il_split<T, NR>(in, xf, Bf, Cf);
@@ -212,16 +205,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
                     *(f32x4 *)(y_wr + 16 * YROW) = acc1;
                 }
                 __syncthreads();
+                const uint32_t o = lane_off + step_off(s) + bad;
 #pragma unroll
                 for (int k = 0; k < NR; ++k) {
-                    const int64_t t = s * STEP + rr + RP * k;
-                    if (cvalid && t < L) {
-                        float yf[CH];
+                    float yf[CH];
 #pragma unroll
-                        for (int c = 0; c < CH; ++c)
-                            yf[c] = Cf[CH * k + c] * *(const float *)(y_rd + RP * k * YROW + 4 * c);
-                        stg4(y + col + t * d, pack_unit<T>(yf));
-                    }
+                    for (int c = 0; c < CH; ++c)
+                        yf[c] = Cf[CH * k + c] * *(const float *)(y_rd + RP * k * YROW + 4 * c);
+                    stw4(wy, o + k * pass_off, pack_unit<T>(yf));
                 }
 #pragma unroll
                 for (int k = 0; k < NR; ++k) in[k] = nx[k];
@@ -285,8 +276,19 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
 
+    // Windows of this batch row: the outputs over rows [t0, t1), the features and dy over
+    // [t0, t2) (the backward looks NK-1 steps ahead for g2).
+    const int64_t t0 = (s_lo - (NK - 1)) * STEP > 0 ? (s_lo - (NK - 1)) * STEP : 0;
+    const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
+    const int64_t t2 = (s_hi + NK - 1) * STEP < L ? (s_hi + NK - 1) * STEP : L;
+    const int64_t row_bytes = d * M::ES, origin = (b * L + t0) * d;
+    const win_t wf = make_window(feat + 3 * origin, 3 * (t2 - t0) * row_bytes);
+    const win_t wdyw = make_window(dy + origin, (t2 - t0) * row_bytes);
+    const win_t wdf = make_window(dfeat + 3 * origin, 3 * (t1 - t0) * row_bytes);
     const bool cvalid = c0 + CH * a < d;
-    const int64_t col = b * L * d + c0 + CH * a;
+    const uint32_t lane_off = (uint32_t)(rr * row_bytes + (c0 + CH * a) * M::ES);
+    const uint32_t pass_off = (uint32_t)(RP * row_bytes), bad = cvalid ? 0u : WIN_OFF;
+    auto step_off = [&](int64_t sg) { return (uint32_t)((sg * STEP - t0) * row_bytes); };
 
     // While step s runs in phase ph:  Au[(ph - i + NK) % NK] is the u operand of step s-i,
     // Ag[(ph + i) % NK] the time-reversed g2 operand of step s+i, dyq[(ph + i) % NK] dy of step s+i.
@@ -312,22 +314,16 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
 
     // interleaved rows and dy of one step (zero outside the sequence)
     auto fetch_feat = [&](int64_t step, u32x3 (&p)[NR]) {
+        const uint32_t o = lane_off + step_off(step);
 #pragma unroll
-        for (int k = 0; k < NR; ++k) {
-            const int64_t t = step * STEP + rr + RP * k;
-            p[k] = u32x3{0u, 0u, 0u};
-            if (cvalid && t >= 0 && t < L) p[k] = ldg12(feat + 3 * (col + t * d));
-        }
+        for (int k = 0; k < NR; ++k) p[k] = ldw12(wf, 3 * (o + k * pass_off) + bad);
     };
-    auto fetch_dy = [&](int64_t step, Row<T> &o) {
+    auto fetch_dy = [&](int64_t step, Row<T> &out) {
+        const uint32_t o = lane_off + step_off(step) + bad;
         uint32_t u[NR];
 #pragma unroll
-        for (int k = 0; k < NR; ++k) {
-            const int64_t t = step * STEP + rr + RP * k;
-            u[k] = 0u;
-            if (cvalid && t >= 0 && t < L) u[k] = ldg4(dy + col + t * d);
-        }
-        o = units_row<T, NR>(u);
+        for (int k = 0; k < NR; ++k) u[k] = ldw4(wdyw, o + k * pass_off);
+        out = units_row<T, NR>(u);
     };
     auto store_rows = [&](unsigned char *tile, const float (&f)[8]) {
 #pragma unroll
@@ -406,14 +402,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
                 const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
-                u32x3 nx[NR];
-                Row<T> dyn = zero_row<T>();
-#pragma unroll
-                for (int k = 0; k < NR; ++k) nx[k] = u32x3{0u, 0u, 0u};
-                if (s + 1 < s_hi) {
-                    fetch_feat(s + NK, nx);
-                    fetch_dy(s + NK, dyn);
-                }
+                u32x3 nx[NR];        // rows of the next iteration; past the segment's reach they are
+                Row<T> dyn;          // outside the windows
+                fetch_feat(s + NK, nx);
+                fetch_dy(s + NK, dyn);
 
                 float xf[8], Bf[8], tf[8], cf[8], pf[8];
                 {
@@ -487,11 +479,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
                         }
                     u32x3 po[NR];
                     il_join<T, NR>(ox, oB, oC, po);
+                    const uint32_t o = lane_off + step_off(s);
 #pragma unroll
-                    for (int k = 0; k < NR; ++k) {
-                        const int64_t t = s * STEP + rr + RP * k;
-                        if (cvalid && t < L) stg12(dfeat + 3 * (col + t * d), po[k]);
-                    }
+                    for (int k = 0; k < NR; ++k) stw12(wdf, 3 * (o + k * pass_off) + bad, po[k]);
                 }
 #pragma unroll
                 for (int k = 0; k < NR; ++k) in[k] = nx[k];
@@ -527,7 +517,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
 template <typename T, int NK, int NW>
 int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
 {
-    const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16);
+    const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((mfma_il_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)feat,
                        (const T *)h, (T *)y, dm, p);

@@ -265,6 +265,63 @@ template <typename T> __device__ __forceinline__ void stg16(T *p, const uint4 &v
 #endif
 }
 
+// Tensor windows.  A workgroup addresses each tensor through a buffer descriptor that covers
+// the rows it touches: byte offsets are 32-bit, a load outside the window returns zero and a
+// store outside it is dropped.  Rows before the sequence start (negative offsets, which wrap
+// past the window) and after its end thus need no test, and a lane whose channels lie beyond
+// the tensor adds WIN_OFF to its offsets.  With no branch around any load or store the
+// instruction stream of a step is straight-line, and the compiler's wait-count insertion can
+// tell exactly how many accesses are in flight; across a divergent branch it cannot, and it
+// then waits for every outstanding load -- the prefetch of the next step included.
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+typedef __amdgpu_buffer_rsrc_t win_t;
+constexpr uint32_t WIN_OFF = 0x80000000u;           // offsets at or above this are outside every window
+constexpr int64_t WIN_MAX_BYTES = (1ll << 31) - (1ll << 27);
+constexpr int WIN_NT = (GCG_MFMA_NT & 1) ? 2 : 0, WIN_NT_ST = (GCG_MFMA_NT & 2) ? 2 : 0;   // cache policy: nt
+
+__device__ __forceinline__ win_t make_window(const void *base, int64_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 ldw16(win_t w, uint32_t off)
+{
+    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(w, (int)off, 0, WIN_NT);
+    return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void stw16(win_t w, uint32_t off, const uint4 &v)
+{
+    const u32x4 t = {v.x, v.y, v.z, v.w};
+    __builtin_amdgcn_raw_buffer_store_b128(t, w, (int)off, 0, WIN_NT_ST);
+}
+__device__ __forceinline__ u32x3 ldw12(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b96(w, (int)off, 0, WIN_NT);
+}
+__device__ __forceinline__ void stw12(win_t w, uint32_t off, const u32x3 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b96(v, w, (int)off, 0, WIN_NT_ST);
+}
+__device__ __forceinline__ uint32_t ldw4(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b32(w, (int)off, 0, WIN_NT);
+}
+__device__ __forceinline__ void stw4(win_t w, uint32_t off, uint32_t v)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(v, w, (int)off, 0, WIN_NT_ST);
+}
+template <typename T> __device__ __forceinline__ Row<T> ldw_row(win_t w, uint32_t off)
+{
+    Row<T> r;
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) r.w[i] = ldw16(w, off + 16 * i);
+    return r;
+}
+template <typename T> __device__ __forceinline__ void stw_row(win_t w, uint32_t off, const Row<T> &r)
+{
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) stw16(w, off + 16 * i, r.w[i]);
+}
+
 // Workgroups are dealt to the 8 XCDs round-robin by index.  Re-labelling them so that each XCD
 // receives a contiguous run of (batch, segment, channel-block) triples makes the workgroups of
 // one XCD cover whole tensor rows between them, which its L2 and the memory channels prefer.
@@ -333,7 +390,9 @@ int choose_nw(const Dims &dm, bool fp32)
     return 4;
 }
 
-MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu)
+// elem_bytes: size of one element; segments are kept short enough for the widest window (an
+// interleaved tensor, 3 * d elements per row) to stay below WIN_MAX_BYTES.
+MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu, int elem_bytes)
 {
     MfmaPlan p;
     const int cb = 16 * nw;
@@ -350,6 +409,8 @@ MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu)
     static const int forced = env_int("GCG_MFMA_STEPS_PER_SEG", 0);        // tuning override
     int64_t sps = (p.nsteps + want - 1) / want;
     if (forced > 0) sps = forced;
+    const int64_t cap = WIN_MAX_BYTES / (STEP * 3 * dm.d * elem_bytes) - 2 * 5;   // rows of NK-1 steps either side
+    if (sps > cap) sps = cap > 1 ? cap : 1;
     p.steps_per_seg = (int)sps;
     p.nseg = (int)((p.nsteps + sps - 1) / sps);
     p.nwg = dm.bs * p.nseg * p.ncb;
@@ -369,7 +430,10 @@ int choose_nw_bwd(const Dims &dm, bool fp32)
 }
 
 // 16-bit: two waves per SIMD (8 per CU); fp32: one (4 per CU)
-MfmaPlan plan_bwd(const Dims &dm, bool fp32) { return plan(dm, choose_nw_bwd(dm, fp32), 16, fp32 ? 4 : 8); }
+MfmaPlan plan_bwd(const Dims &dm, bool fp32)
+{
+    return plan(dm, choose_nw_bwd(dm, fp32), 16, fp32 ? 4 : 8, fp32 ? 4 : 2);
+}
 
 } // namespace
 } // namespace gcg
