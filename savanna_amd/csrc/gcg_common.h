@@ -70,6 +70,75 @@ template <> struct Elem<f16_t> {
     }
 };
 
+// ---- tensor windows --------------------------------------------------------------------
+// A kernel addresses each tensor through a buffer descriptor that covers the rows it touches:
+// byte offsets are 32-bit, a load outside the window returns zero and a store outside it is
+// dropped.  Rows before the sequence start (negative offsets, which wrap past the window) and
+// after its end thus need no test, and a lane whose channels lie beyond the tensor adds WIN_OFF
+// to its offsets.  With no branch around any load or store the instruction stream is
+// straight-line, and the compiler's wait-count insertion can tell exactly how many accesses are
+// in flight; across a branch it cannot, and it then waits for every outstanding access.
+// Every element is touched once, so accesses carry the nontemporal hint.
+typedef uint32_t u32x1 __attribute__((ext_vector_type(1)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t win_t;
+constexpr uint32_t WIN_OFF = 0x80000000u;           // offsets at or above this are outside every window
+constexpr int64_t WIN_MAX_BYTES = (1ll << 31) - (1ll << 27);
+#ifndef GCG_NT
+#define GCG_NT 3                                    // bit 0: loads, bit 1: stores
+#endif
+constexpr int WIN_NT = (GCG_NT & 1) ? 2 : 0, WIN_NT_ST = (GCG_NT & 2) ? 2 : 0;   // cache policy "nt"
+
+__device__ __forceinline__ win_t make_window(const void *base, int64_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)(bytes > 0 ? bytes : 0), 0x00020000);
+}
+template <typename R> __device__ __forceinline__ R win_load(win_t w, uint32_t off);
+template <> __device__ __forceinline__ uint32_t win_load<uint32_t>(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b32(w, (int)off, 0, WIN_NT);
+}
+template <> __device__ __forceinline__ u32x1 win_load<u32x1>(win_t w, uint32_t off)
+{
+    u32x1 r;
+    r[0] = __builtin_amdgcn_raw_buffer_load_b32(w, (int)off, 0, WIN_NT);
+    return r;
+}
+template <> __device__ __forceinline__ u32x2 win_load<u32x2>(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b64(w, (int)off, 0, WIN_NT);
+}
+template <> __device__ __forceinline__ u32x3 win_load<u32x3>(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b96(w, (int)off, 0, WIN_NT);
+}
+template <> __device__ __forceinline__ u32x4 win_load<u32x4>(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b128(w, (int)off, 0, WIN_NT);
+}
+__device__ __forceinline__ void win_store(win_t w, uint32_t off, uint32_t v)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(v, w, (int)off, 0, WIN_NT_ST);
+}
+__device__ __forceinline__ void win_store(win_t w, uint32_t off, const u32x1 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(v[0], w, (int)off, 0, WIN_NT_ST);
+}
+__device__ __forceinline__ void win_store(win_t w, uint32_t off, const u32x2 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b64(v, w, (int)off, 0, WIN_NT_ST);
+}
+__device__ __forceinline__ void win_store(win_t w, uint32_t off, const u32x3 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b96(v, w, (int)off, 0, WIN_NT_ST);
+}
+__device__ __forceinline__ void win_store(win_t w, uint32_t off, const u32x4 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(v, w, (int)off, 0, WIN_NT_ST);
+}
+
 // ---- launch descriptors shared by host dispatch and kernels --------------------------
 struct Dims {
     int64_t bs, L;

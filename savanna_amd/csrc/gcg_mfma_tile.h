@@ -223,92 +223,24 @@ template <typename T> __device__ __forceinline__ Row<T> lds_load_row(const unsig
     return r;
 }
 
-// Streaming accesses: every tensor element is touched once, so loads and stores carry the
-// nontemporal hint (GCG_MFMA_NT=0 at build time turns it off for comparison).
 #ifndef GCG_XCD_SWIZZLE
 #define GCG_XCD_SWIZZLE 1
 #endif
-#ifndef GCG_MFMA_NT
-#define GCG_MFMA_NT 3
-#endif
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-template <typename T> __device__ __forceinline__ uint4 ldg16(const T *p);
-template <typename T> __device__ __forceinline__ void stg16(T *p, const uint4 &v);
-template <typename T> __device__ __forceinline__ Row<T> ldg_row(const T *p)
-{
-    Row<T> r;
-#pragma unroll
-    for (int i = 0; i < MT<T>::RW; ++i) r.w[i] = ldg16((const unsigned char *)p + 16 * i);
-    return r;
-}
-template <typename T> __device__ __forceinline__ void stg_row(T *p, const Row<T> &r)
-{
-#pragma unroll
-    for (int i = 0; i < MT<T>::RW; ++i) stg16((unsigned char *)p + 16 * i, r.w[i]);
-}
-template <typename T> __device__ __forceinline__ uint4 ldg16(const T *p)
-{
-#if GCG_MFMA_NT & 1
-    const u32x4 v = __builtin_nontemporal_load((const u32x4 *)p);
-    return make_uint4(v[0], v[1], v[2], v[3]);
-#else
-    return *(const uint4 *)p;
-#endif
-}
-template <typename T> __device__ __forceinline__ void stg16(T *p, const uint4 &v)
-{
-#if GCG_MFMA_NT & 2
-    const u32x4 t = {v.x, v.y, v.z, v.w};
-    __builtin_nontemporal_store(t, (u32x4 *)p);
-#else
-    *(uint4 *)p = v;
-#endif
-}
 
-// Tensor windows.  A workgroup addresses each tensor through a buffer descriptor that covers
-// the rows it touches: byte offsets are 32-bit, a load outside the window returns zero and a
-// store outside it is dropped.  Rows before the sequence start (negative offsets, which wrap
-// past the window) and after its end thus need no test, and a lane whose channels lie beyond
-// the tensor adds WIN_OFF to its offsets.  With no branch around any load or store the
-// instruction stream of a step is straight-line, and the compiler's wait-count insertion can
-// tell exactly how many accesses are in flight; across a divergent branch it cannot, and it
-// then waits for every outstanding load -- the prefetch of the next step included.
-typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
-typedef __amdgpu_buffer_rsrc_t win_t;
-constexpr uint32_t WIN_OFF = 0x80000000u;           // offsets at or above this are outside every window
-constexpr int64_t WIN_MAX_BYTES = (1ll << 31) - (1ll << 27);
-constexpr int WIN_NT = (GCG_MFMA_NT & 1) ? 2 : 0, WIN_NT_ST = (GCG_MFMA_NT & 2) ? 2 : 0;   // cache policy: nt
-
-__device__ __forceinline__ win_t make_window(const void *base, int64_t bytes)
-{
-    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)bytes, 0x00020000);
-}
+// 16-, 12- and 4-byte accesses of a tensor window (gcg_common.h)
 __device__ __forceinline__ uint4 ldw16(win_t w, uint32_t off)
 {
-    const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(w, (int)off, 0, WIN_NT);
+    const u32x4 v = win_load<u32x4>(w, off);
     return make_uint4(v[0], v[1], v[2], v[3]);
 }
 __device__ __forceinline__ void stw16(win_t w, uint32_t off, const uint4 &v)
 {
-    const u32x4 t = {v.x, v.y, v.z, v.w};
-    __builtin_amdgcn_raw_buffer_store_b128(t, w, (int)off, 0, WIN_NT_ST);
+    win_store(w, off, u32x4{v.x, v.y, v.z, v.w});
 }
-__device__ __forceinline__ u32x3 ldw12(win_t w, uint32_t off)
-{
-    return __builtin_amdgcn_raw_buffer_load_b96(w, (int)off, 0, WIN_NT);
-}
-__device__ __forceinline__ void stw12(win_t w, uint32_t off, const u32x3 &v)
-{
-    __builtin_amdgcn_raw_buffer_store_b96(v, w, (int)off, 0, WIN_NT_ST);
-}
-__device__ __forceinline__ uint32_t ldw4(win_t w, uint32_t off)
-{
-    return __builtin_amdgcn_raw_buffer_load_b32(w, (int)off, 0, WIN_NT);
-}
-__device__ __forceinline__ void stw4(win_t w, uint32_t off, uint32_t v)
-{
-    __builtin_amdgcn_raw_buffer_store_b32(v, w, (int)off, 0, WIN_NT_ST);
-}
+__device__ __forceinline__ u32x3 ldw12(win_t w, uint32_t off) { return win_load<u32x3>(w, off); }
+__device__ __forceinline__ void stw12(win_t w, uint32_t off, const u32x3 &v) { win_store(w, off, v); }
+__device__ __forceinline__ uint32_t ldw4(win_t w, uint32_t off) { return win_load<uint32_t>(w, off); }
+__device__ __forceinline__ void stw4(win_t w, uint32_t off, uint32_t v) { win_store(w, off, v); }
 template <typename T> __device__ __forceinline__ Row<T> ldw_row(win_t w, uint32_t off)
 {
     Row<T> r;

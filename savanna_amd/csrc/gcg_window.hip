@@ -16,22 +16,42 @@ namespace {
 
 constexpr int RING = 8;
 constexpr int BATCH = 4;   // rows fetched together
+constexpr int HALO_BURST = 4;   // halo rows fetched together
 
-typedef uint32_t u32v2 __attribute__((ext_vector_type(2)));
-typedef uint32_t u32v4 __attribute__((ext_vector_type(4)));
 
 // A lane's row vector: VV channels as raw 32-bit words (fp32: one channel per word;
 // bf16 / f16: two).  VV = 4 everywhere, or 8 for the 16-bit types (16-byte accesses).
 template <typename T, int VV> struct Vec;
-template <> struct Vec<float, 4> { typedef u32v4 raw; static constexpr int W = 4; };
-template <> struct Vec<bf16_t, 4> { typedef u32v2 raw; static constexpr int W = 2; };
-template <> struct Vec<f16_t, 4> { typedef u32v2 raw; static constexpr int W = 2; };
-template <> struct Vec<bf16_t, 8> { typedef u32v4 raw; static constexpr int W = 4; };
-template <> struct Vec<f16_t, 8> { typedef u32v4 raw; static constexpr int W = 4; };
-
-// every row is read once and written once: stream past the caches
-template <typename R> __device__ __forceinline__ R ldg(const void *p) { return __builtin_nontemporal_load((const R *)p); }
-template <typename R> __device__ __forceinline__ void stg(void *p, const R &v) { __builtin_nontemporal_store(v, (R *)p); }
+template <> struct Vec<float, 4> { typedef u32x4 raw; static constexpr int W = 4; };
+template <> struct Vec<bf16_t, 4> { typedef u32x2 raw; static constexpr int W = 2; };
+template <> struct Vec<f16_t, 4> { typedef u32x2 raw; static constexpr int W = 2; };
+template <> struct Vec<bf16_t, 8> { typedef u32x4 raw; static constexpr int W = 4; };
+// one 32-bit word per row: the lane width of the interleaved kernels, whose row piece
+// (C, B, x per channel) is then 12 contiguous bytes
+template <> struct Vec<float, 1> { typedef u32x1 raw; static constexpr int W = 1; };
+template <> struct Vec<bf16_t, 2> { typedef u32x1 raw; static constexpr int W = 1; };
+template <> struct Vec<f16_t, 2> { typedef u32x1 raw; static constexpr int W = 1; };
+// the three words of an interleaved row piece in one 12-byte access
+__device__ __forceinline__ void load_piece(win_t w, uint32_t off, u32x1 (&p)[3])
+{
+    const u32x3 v = win_load<u32x3>(w, off);
+    p[0][0] = v[0]; p[1][0] = v[1]; p[2][0] = v[2];
+}
+__device__ __forceinline__ void store_piece(win_t w, uint32_t off, const u32x1 (&p)[3])
+{
+    win_store(w, off, u32x3{p[0][0], p[1][0], p[2][0]});
+}
+template <typename R> __device__ __forceinline__ void load_piece(win_t w, uint32_t off, R (&p)[3])
+{
+    constexpr int NB = sizeof(R);
+    p[0] = win_load<R>(w, off); p[1] = win_load<R>(w, off + NB); p[2] = win_load<R>(w, off + 2 * NB);
+}
+template <typename R> __device__ __forceinline__ void store_piece(win_t w, uint32_t off, const R (&p)[3])
+{
+    constexpr int NB = sizeof(R);
+    win_store(w, off, p[0]); win_store(w, off + NB, p[1]); win_store(w, off + 2 * NB, p[2]);
+}
+template <> struct Vec<f16_t, 8> { typedef u32x4 raw; static constexpr int W = 4; };
 
 template <typename T> struct Word;   // conversions of one 32-bit word
 template <> struct Word<float> {
@@ -135,14 +155,18 @@ struct WinPlan { int v, nvec, nseg, ts, ncvb, threads; int64_t nthreads, nwg; };
 
 // ---------------------------------------------------------------------------- forward
 // PK: x, B, C are interleaved in one tensor that starts at C (element stride 3).
-template <typename T, int HL, int V, bool PK>
+// EXTRA: also write the convolution before the post-gate (y2) and the pre-gate product (bx).
+// Tensors are addressed through windows over the rows of this run, so no load or store sits
+// behind a branch: rows before the sequence start read as zero, rows past the run are dropped.
+template <typename T, int HL, int V, bool PK, bool EXTRA>
 __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x, const T *__restrict__ B,
                                                          const T *__restrict__ C, const T *__restrict__ h,
                                                          T *__restrict__ y, T *__restrict__ y2,
                                                          T *__restrict__ bx, Dims dm, WinPlan pl)
 {
     typedef typename Vec<T, V>::raw raw_t;
-    // (batch, run, block of channel vectors) come from the workgroup index, so row addresses
+    constexpr int ES = sizeof(T), IS = PK ? 3 : 1;     // element bytes, element stride of the inputs
+    // (batch, run, block of channel vectors) come from the workgroup index, so row offsets
     // are wave-uniform and only the channel offset is per lane
     int64_t wg = blockIdx.x;
     const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
@@ -150,8 +174,6 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
     const int64_t b = wg / pl.nseg;
     const int cv = cvb * (int)blockDim.x + (int)threadIdx.x;
     if (cv >= pl.nvec) return;
-    const int64_t gid = (b * pl.nseg + seg) * pl.nvec + cv;     // index of this lane's workspace slot
-    (void)gid;
     const int64_t L = dm.L, d = dm.d;
     const int64_t c = (int64_t)cv * V;
     const int hl = dm.hl;
@@ -163,18 +185,23 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
-    const int64_t base = b * L * d + c;   // (b*L + t)*d is uniform, c per lane
-
-    // input rows: PK reads three consecutive vectors from the interleaved tensor
-    const int64_t ibase = PK ? 3 * base : base, irow = PK ? 3 * d : d;
+    const int64_t t0 = t_start - (HL - 1) > 0 ? t_start - (HL - 1) : 0;       // first row of the windows
+    const int64_t origin = (b * L + t0) * d, rows = t_end - t0;
+    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow;               // bytes per row: outputs, inputs
+    const win_t wx = make_window((PK ? C : x) + IS * origin, rows * irow);
+    const win_t wB = make_window(B + origin, PK ? 0 : rows * irow), wC = make_window(C + origin, PK ? 0 : rows * irow);
+    const win_t wy = make_window(y + origin, rows * orow);
+    const win_t wy2 = make_window(EXTRA && y2 ? y2 + origin : y + origin, EXTRA && y2 ? rows * orow : 0);
+    const win_t wbx = make_window(EXTRA && bx ? bx + origin : y + origin, EXTRA && bx ? rows * orow : 0);
+    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = IS * lane_o;
     auto load_in = [&](int64_t t, raw_t (&p)[3], bool with_c) {
+        const uint32_t o = lane_i + (uint32_t)(t - t0) * irow;
         if constexpr (PK) {
-            const T *q = C + ibase + t * irow;
-            p[0] = ldg<raw_t>(q); p[1] = ldg<raw_t>(q + V); p[2] = ldg<raw_t>(q + 2 * V);
+            load_piece(wx, o, p);
         } else {
-            p[0] = ldg<raw_t>(x + ibase + t * irow);
-            p[1] = ldg<raw_t>(B + ibase + t * irow);
-            p[2] = with_c ? ldg<raw_t>(C + ibase + t * irow) : zero_raw<T, V>();
+            p[0] = win_load<raw_t>(wx, o);
+            p[1] = win_load<raw_t>(wB, o);
+            p[2] = with_c ? win_load<raw_t>(wC, o) : zero_raw<T, V>();
         }
     };
 
@@ -184,53 +211,59 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
 #pragma unroll
         for (int v = 0; v < V; ++v) ring[s][v] = 0.f;
     // halo: rows t_start-(HL-1) .. t_start-1 go to slots (t & 7); t_start is a multiple of 8
+    // (fetched HALO_BURST rows at a time, so the staging registers stay below the main loop's)
 #pragma unroll
-    for (int i = 1; i < HL; ++i) {
-        const int64_t t = t_start - i;
-        if (t >= 0) {
-            raw_t p[3];
+    for (int i0 = 1; i0 < HL; i0 += HALO_BURST) {
+        raw_t halo[HALO_BURST][3];
+#pragma unroll
+        for (int i = i0; i < i0 + HALO_BURST && i < HL; ++i) load_in(t_start - i, halo[i - i0], false);
+#pragma unroll
+        for (int i = i0; i < i0 + HALO_BURST && i < HL; ++i) {
             float xf[V], Bf[V], Cf[V];
-            load_in(t, p, false);
-            row_floats<T, V, PK>(p, xf, Bf, Cf);
+            row_floats<T, V, PK>(halo[i - i0], xf, Bf, Cf);
 #pragma unroll
             for (int v = 0; v < V; ++v) ring[RING - i][v] = xf[v] * Bf[v];
         }
     }
 
+    // Rows are fetched BATCH at a time.  At 16 bits one batch ahead: while a batch is worked on,
+    // the loads of the next are in flight (past the run they fall outside the windows and cost
+    // nothing).  At fp32 the second staging buffer would cost a wave per SIMD; measured slower.
+    constexpr bool AHEAD = sizeof(T) == 2;
+    raw_t in[AHEAD ? 2 : 1][BATCH][3];
+    if constexpr (AHEAD) {
+#pragma unroll
+        for (int kk = 0; kk < BATCH; ++kk) load_in(t_start + kk, in[0][kk], true);
+    }
     for (int64_t tb = t_start; tb < t_end; tb += RING) {
 #pragma unroll
         for (int half = 0; half < RING / BATCH; ++half) {
-            // rows are fetched BATCH at a time: enough loads in flight per lane without
-            // pushing the register count past four waves per SIMD
-            raw_t in[BATCH][3];
+            constexpr int NB = RING / BATCH;
+            const int cur = AHEAD ? half % 2 : 0, nxt = AHEAD ? (half + 1) % 2 : 0;
+            static_assert(NB % 2 == 0, "the staging buffers alternate with the batches of a ring turn");
 #pragma unroll
-            for (int kk = 0; kk < BATCH; ++kk) {
-                const int64_t t = tb + half * BATCH + kk;
-                if (t < t_end) {
-                    load_in(t, in[kk], true);
-                } else {
-                    in[kk][0] = zero_raw<T, V>(); in[kk][1] = zero_raw<T, V>(); in[kk][2] = zero_raw<T, V>();
-                }
-            }
+            for (int kk = 0; kk < BATCH; ++kk)
+                load_in(tb + (half + (AHEAD ? 1 : 0)) * BATCH + kk, in[nxt][kk], true);
 #pragma unroll
             for (int kk = 0; kk < BATCH; ++kk) {
                 const int k = half * BATCH + kk;
                 const int64_t t = tb + k;
                 float xf[V], Bf[V], Cf[V], acc[V], out[V];
-                row_floats<T, V, PK>(in[kk], xf, Bf, Cf);
+                row_floats<T, V, PK>(in[cur][kk], xf, Bf, Cf);
 #pragma unroll
                 for (int v = 0; v < V; ++v) { ring[k][v] = xf[v] * Bf[v]; acc[v] = 0.f; }
 #pragma unroll
                 for (int j = HL - 1; j >= 0; --j)
 #pragma unroll
                     for (int v = 0; v < V; ++v) acc[v] = fmaf(hr[j], ring[(k - j) & (RING - 1)][v], acc[v]);
-                if (t < t_end) {
-                    if (y2) stg<raw_t>(y2 + base + t * d, packv<T, V>(acc));
-                    if (bx) stg<raw_t>(bx + base + t * d, packv<T, V>(ring[k]));
-#pragma unroll
-                    for (int v = 0; v < V; ++v) out[v] = Cf[v] * acc[v];
-                    stg<raw_t>(y + base + t * d, packv<T, V>(out));
+                const uint32_t o = lane_o + (uint32_t)(t - t0) * orow;
+                if constexpr (EXTRA) {
+                    win_store(wy2, o, packv<T, V>(acc));
+                    win_store(wbx, o, packv<T, V>(ring[k]));
                 }
+#pragma unroll
+                for (int v = 0; v < V; ++v) out[v] = Cf[v] * acc[v];
+                win_store(wy, o, packv<T, V>(out));
             }
         }
     }
@@ -243,6 +276,10 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
 // PK: x, B, C are interleaved in one tensor that starts at C, and dx, dB, dC in one that starts
 // at dC.  A row of the output then holds dC (ready at step r) next to dx, dB (ready HL-1 steps
 // later), so dC waits in a register ring like the raw x and B rows do.
+// Windows: x and B end with the run, dy and C HL-1 rows later, the outputs start with the run;
+// every row outside reads as zero or is dropped, so the walk has no branch around an access.
+// (occupancy floor: three workgroups per CU at 16 bits, two at fp32, so that the scheduler
+// does not trade waves for longer load batches)
 template <typename T, int HL, int V, bool PK>
 __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                          const T *__restrict__ B, const T *__restrict__ C,
@@ -251,8 +288,7 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                                                          float *__restrict__ ws, Dims dm, WinPlan pl)
 {
     typedef typename Vec<T, V>::raw raw_t;
-    // (batch, run, block of channel vectors) come from the workgroup index, so row addresses
-    // are wave-uniform and only the channel offset is per lane
+    constexpr int ES = sizeof(T), IS = PK ? 3 : 1;
     int64_t wg = blockIdx.x;
     const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
     const int seg = (int)(wg % pl.nseg);
@@ -260,7 +296,6 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
     const int cv = cvb * (int)blockDim.x + (int)threadIdx.x;
     if (cv >= pl.nvec) return;
     const int64_t gid = (b * pl.nseg + seg) * pl.nvec + cv;     // index of this lane's workspace slot
-    (void)gid;
     const int64_t L = dm.L, d = dm.d;
     const int64_t c = (int64_t)cv * V;
     const int hl = dm.hl;
@@ -272,9 +307,20 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
-    const int64_t base = b * L * d + c;   // (b*L + t)*d is uniform, c per lane
-
-    const int64_t ibase = PK ? 3 * base : base, irow = PK ? 3 * d : d;
+    const int64_t t_stop = t_end + (HL - 1);                     // exclusive bound of the walk
+    const int64_t t0 = t_start - (HL - 1) > 0 ? t_start - (HL - 1) : 0;
+    const int64_t t_far = t_stop < L ? t_stop : L;
+    const int64_t origin = (b * L + t0) * d, out_origin = (b * L + t_start) * d;
+    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow;
+    // PK: wx is the interleaved tensor and reaches as far as dy (C is part of it)
+    const win_t wx = make_window((PK ? C : x) + IS * origin, ((PK ? t_far : t_end) - t0) * irow);
+    const win_t wB = make_window(B + origin, PK ? 0 : (t_end - t0) * irow);
+    const win_t wC = make_window(C + origin, PK ? 0 : (t_far - t0) * irow);
+    const win_t wdy = make_window(dy + origin, (t_far - t0) * orow);
+    const win_t wdC = make_window(dC + IS * out_origin, (t_end - t_start) * irow);
+    const win_t wdx = make_window(dx + out_origin, PK ? 0 : (t_end - t_start) * irow);
+    const win_t wdB = make_window(dB + out_origin, PK ? 0 : (t_end - t_start) * irow);
+    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = IS * lane_o;
 
     float ur[RING][V], gr[RING][V], dha[HL];
     raw_t xs[RING], Bs[RING], dCs[PK ? RING : 1];
@@ -288,26 +334,28 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 #pragma unroll
     for (int j = 0; j < HL; ++j) dha[j] = 0.f;
 #pragma unroll
-    for (int i = 1; i < HL; ++i) {
-        const int64_t t = t_start - i;
-        if (t >= 0) {
-            raw_t p[3];
-            float xf[V], Bf[V], Cf[V];
+    for (int i0 = 1; i0 < HL; i0 += HALO_BURST) {
+        raw_t halo[HALO_BURST][3];
+#pragma unroll
+        for (int i = i0; i < i0 + HALO_BURST && i < HL; ++i) {
+            const uint32_t o = lane_i + (uint32_t)(t_start - i - t0) * irow;
             if constexpr (PK) {
-                const T *q = C + ibase + t * irow;
-                p[0] = ldg<raw_t>(q); p[1] = ldg<raw_t>(q + V); p[2] = ldg<raw_t>(q + 2 * V);
+                load_piece(wx, o, halo[i - i0]);
             } else {
-                p[0] = ldg<raw_t>(x + ibase + t * irow);
-                p[1] = ldg<raw_t>(B + ibase + t * irow);
-                p[2] = zero_raw<T, V>();
+                halo[i - i0][0] = win_load<raw_t>(wx, o);
+                halo[i - i0][1] = win_load<raw_t>(wB, o);
+                halo[i - i0][2] = zero_raw<T, V>();
             }
-            row_floats<T, V, PK>(p, xf, Bf, Cf);
+        }
+#pragma unroll
+        for (int i = i0; i < i0 + HALO_BURST && i < HL; ++i) {
+            float xf[V], Bf[V], Cf[V];
+            row_floats<T, V, PK>(halo[i - i0], xf, Bf, Cf);
 #pragma unroll
             for (int v = 0; v < V; ++v) ur[RING - i][v] = xf[v] * Bf[v];
         }
     }
 
-    const int64_t t_stop = t_end + (HL - 1);  // exclusive bound of the walk
     for (int64_t tb = t_start; tb < t_stop; tb += RING) {
 #pragma unroll
         for (int half = 0; half < RING / BATCH; ++half) {
@@ -317,56 +365,41 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 #pragma unroll
             for (int kk = 0; kk < BATCH; ++kk) {
                 const int64_t t = tb + half * BATCH + kk;
-                const bool ahead = t < L && t < t_stop;      // dy and C are read HL-1 rows past the run
+                const uint32_t o = lane_i + (uint32_t)(t - t0) * irow;
                 if constexpr (PK) {
-                    if (ahead) {
-                        const T *q = C + ibase + t * irow;
-                        in[kk][0] = ldg<raw_t>(q); in[kk][1] = ldg<raw_t>(q + V); in[kk][2] = ldg<raw_t>(q + 2 * V);
-                        dyr[kk] = ldg<raw_t>(dy + base + t * d);
-                    } else {
-                        in[kk][0] = zero_raw<T, V>(); in[kk][1] = zero_raw<T, V>(); in[kk][2] = zero_raw<T, V>();
-                        dyr[kk] = zero_raw<T, V>();
-                    }
+                    load_piece(wx, o, in[kk]);
                 } else {
-                    if (t < t_end) {
-                        in[kk][0] = ldg<raw_t>(x + base + t * d);
-                        in[kk][1] = ldg<raw_t>(B + base + t * d);
-                    } else {
-                        in[kk][0] = zero_raw<T, V>(); in[kk][1] = zero_raw<T, V>();
-                    }
-                    if (ahead) {
-                        dyr[kk] = ldg<raw_t>(dy + base + t * d);
-                        in[kk][2] = ldg<raw_t>(C + base + t * d);
-                    } else {
-                        dyr[kk] = zero_raw<T, V>(); in[kk][2] = zero_raw<T, V>();
-                    }
+                    in[kk][0] = win_load<raw_t>(wx, o);
+                    in[kk][1] = win_load<raw_t>(wB, o);
+                    in[kk][2] = win_load<raw_t>(wC, o);
                 }
+                dyr[kk] = win_load<raw_t>(wdy, lane_o + (uint32_t)(t - t0) * orow);
             }
 #pragma unroll
             for (int kk = 0; kk < BATCH; ++kk) {
                 const int k = half * BATCH + kk;
                 const int64_t t = tb + k;
+                const bool in_run = t < t_end;          // uniform; past the run only g2 is wanted
                 float dyf[V], xf[V], Bf[V], Cf[V];
                 unpackv<T, V>(dyr[kk], dyf);
+                row_floats<T, V, PK>(in[kk], xf, Bf, Cf);
                 if constexpr (PK) {
-                    row_floats<T, V, true>(in[kk], xf, Bf, Cf);
                     xs[k] = packv<T, V>(xf);
                     Bs[k] = packv<T, V>(Bf);
                 } else {
-                    unpackv<T, V>(in[kk][2], Cf);
                     xs[k] = in[kk][0];
                     Bs[k] = in[kk][1];
                 }
 #pragma unroll
                 for (int v = 0; v < V; ++v) gr[k][v] = dyf[v] * Cf[v];
-                if (t < t_end) {
-                    float y2v[V], o[V];
-                    if constexpr (!PK) {
-                        unpackv<T, V>(xs[k], xf);
-                        unpackv<T, V>(Bs[k], Bf);
-                    }
+                {
+                    float y2v[V], o[V], gd[V];
 #pragma unroll
-                    for (int v = 0; v < V; ++v) { ur[k][v] = xf[v] * Bf[v]; y2v[v] = 0.f; }
+                    for (int v = 0; v < V; ++v) {
+                        ur[k][v] = in_run ? xf[v] * Bf[v] : 0.f;
+                        gd[v] = in_run ? gr[k][v] : 0.f;     // rows past the run belong to the next run's dh
+                        y2v[v] = 0.f;
+                    }
 #pragma unroll
                     for (int j = HL - 1; j >= 0; --j) {
                         float sacc = 0.f;
@@ -374,18 +407,19 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                         for (int v = 0; v < V; ++v) {
                             const float u = ur[(k - j) & (RING - 1)][v];
                             y2v[v] = fmaf(hr[j], u, y2v[v]);
-                            sacc = fmaf(gr[k][v], u, sacc);
+                            sacc = fmaf(gd[v], u, sacc);
                         }
                         dha[j] += sacc;
                     }
 #pragma unroll
                     for (int v = 0; v < V; ++v) o[v] = dyf[v] * y2v[v];
                     if constexpr (PK) dCs[k] = packv<T, V>(o);
-                    else stg<raw_t>(dC + base + t * d, packv<T, V>(o));
+                    else win_store(wdC, lane_o + (uint32_t)(t - t_start) * orow, packv<T, V>(o));
                 }
-                // du for row t-(HL-1): sum_j hr[j] * g2[row + j]
-                const int64_t orow = t - (HL - 1);
-                if (orow >= t_start && orow < t_end) {
+                // du for row t-(HL-1): sum_j hr[j] * g2[row + j]; rows before the run fall outside
+                // the output windows
+                {
+                    const int64_t out_t = t - (HL - 1);
                     float du[V], xo[V], Bo[V], o[V];
 #pragma unroll
                     for (int v = 0; v < V; ++v) du[v] = 0.f;
@@ -403,15 +437,16 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                         for (int v = 0; v < V; ++v) { o[v] = du[v] * Bo[v]; oB[v] = du[v] * xo[v]; }
                         unpackv<T, V>(dCs[(k - (HL - 1)) & (RING - 1)], oC);
                         join3<T, V>(o, oB, oC, p);
-                        T *q = dC + ibase + orow * irow;
-                        stg<raw_t>(q, p[0]); stg<raw_t>(q + V, p[1]); stg<raw_t>(q + 2 * V, p[2]);
+                        const uint32_t q = lane_i + (uint32_t)(out_t - t_start) * irow;
+                        store_piece(wdC, q, p);
                     } else {
+                        const uint32_t q = lane_o + (uint32_t)(out_t - t_start) * orow;
 #pragma unroll
                         for (int v = 0; v < V; ++v) o[v] = du[v] * Bo[v];
-                        stg<raw_t>(dx + base + orow * d, packv<T, V>(o));
+                        win_store(wdx, q, packv<T, V>(o));
 #pragma unroll
                         for (int v = 0; v < V; ++v) o[v] = du[v] * xo[v];
-                        stg<raw_t>(dB + base + orow * d, packv<T, V>(o));
+                        win_store(wdB, q, packv<T, V>(o));
                     }
                 }
             }
@@ -460,6 +495,8 @@ WinPlan plan(const Dims &dm, int v)
     while (p.ts > 8 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
     static const char *env = getenv("GCG_WINDOW_ROWS");   // tuning override: rows per lane, a multiple of 8
     if (env && atoi(env) >= 8 && atoi(env) % 8 == 0) p.ts = atoi(env);
+    // the rows of a run, its halo and an interleaved fp32 row width must fit one tensor window
+    while (p.ts > 8 && (int64_t)(p.ts + 2 * RING) * 3 * dm.d * 4 > WIN_MAX_BYTES) p.ts >>= 1;
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);
     p.nthreads = dm.bs * p.nseg * p.nvec;       // workspace slots (one per lane with work)
     p.threads = p.nvec >= 256 ? 256 : ((p.nvec + 63) / 64) * 64;   // narrow tensors: fewer idle lanes
@@ -469,19 +506,29 @@ WinPlan plan(const Dims &dm, int v)
 }
 
 constexpr int BWD_V = 4;   // the backward keeps four rings per lane: 4 channels is what fits
+// interleaved operands: the lane width that makes a row piece 12 contiguous bytes
+template <typename T> constexpr int il_v() { return 4 / (int)sizeof(T); }
 
 template <typename T, int HL, int V>
 int fwd_v(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
           const Dims &dm, hipStream_t st)
 {
+    if (dm.es == 3) {
+        constexpr int VI = il_v<T>();
+        const WinPlan p = plan(dm, VI);
+        if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+        hipLaunchKernelGGL((window_fwd_kernel<T, HL, VI, true, false>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+                           (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+        return (int)hipGetLastError();
+    }
     const WinPlan p = plan(dm, V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    if (dm.es == 3)
-        hipLaunchKernelGGL((window_fwd_kernel<T, HL, V, true>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+    if (y2 || bx)
+        hipLaunchKernelGGL((window_fwd_kernel<T, HL, V, false, true>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     else
-        hipLaunchKernelGGL((window_fwd_kernel<T, HL, V, false>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+        hipLaunchKernelGGL((window_fwd_kernel<T, HL, V, false, false>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     return (int)hipGetLastError();
 }
@@ -490,11 +537,11 @@ template <typename T, int HL>
 int bwd_t(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
           void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    const WinPlan p = plan(dm, BWD_V);
+    const WinPlan p = plan(dm, dm.es == 3 ? il_v<T>() : BWD_V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (dm.es == 3)
-        hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V, true>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+        hipLaunchKernelGGL((window_bwd_kernel<T, HL, il_v<T>(), true>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
                            (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
     else
@@ -539,7 +586,8 @@ int bwd_hl(const void *dy, const void *x, const void *B, const void *C, const vo
 
 bool window_supported(const Dims &dm)
 {
-    return dm.hl <= RING && dm.dg % 4 == 0 && (int64_t)dm.g * dm.hl <= 0x7fffffffLL;
+    return dm.hl <= RING && dm.dg % 4 == 0 && (int64_t)dm.g * dm.hl <= 0x7fffffffLL &&
+           (int64_t)(3 * RING) * 3 * dm.d * 4 <= WIN_MAX_BYTES;
 }
 
 int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h, void *y,
@@ -553,10 +601,16 @@ int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, co
     return (int)hipErrorInvalidValue;
 }
 
+// one figure for the separate-tensor backward (4 channels per lane) and the interleaved one
+// (2 or 1) of every element type: the largest of the three plans
 size_t window_bwd_workspace(const Dims &dm)
 {
-    const WinPlan p = plan(dm, BWD_V);
-    return (size_t)p.nthreads * dm.hl * sizeof(float);
+    int64_t n = 0;
+    for (int v : {1, 2, BWD_V}) {
+        const WinPlan p = plan(dm, v);
+        if (p.nthreads > n) n = p.nthreads;
+    }
+    return (size_t)n * dm.hl * sizeof(float);
 }
 
 int window_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C, const void *h,

@@ -70,7 +70,12 @@ def test_bwd_interleaved_small(gcg_lib, bs, L, g, dg, hl, dtype, algo):
     got = (dfeat[..., 2], dfeat[..., 1], dfeat[..., 0], dh)
     few_terms = algo == "mfma" and bs * L * dg < 256     # see test_parity_gpu.test_bwd_small
     for o, p, r, n in zip(got, plain, ref, ("dx", "dB", "dC", "dh")):
-        assert_same(o, p, dtype, n)
+        if n == "dh" and algo == "window":
+            # the interleaved register-window kernel gives a lane 2 (or 1) channels instead of 4, so
+            # the per-lane partial sums of dh group differently: same terms, another summation order
+            assert_close(o, p, TOL_DH[dtype], "dh (interleaved vs separate tensors)")
+        else:
+            assert_same(o, p, dtype, n)
         if not (n == "dh" and few_terms):
             assert_close(o, r, TOL_DH[dtype] if n == "dh" else TOL[dtype], n)
 
@@ -171,7 +176,10 @@ def test_benchmark_shapes_match_separate_tensors(gcg_lib, bs, L, g, dg, hl, dtyp
     torch.cuda.synchronize()
     assert torch.equal(y, y_p)
     assert torch.equal(dfeat[..., 0], dC) and torch.equal(dfeat[..., 1], dB) and torch.equal(dfeat[..., 2], dx)
-    assert torch.equal(dh, dh_p)
+    if hl > 8:
+        assert torch.equal(dh, dh_p)
+    else:       # register-window kernels: lanes of another width sum dh in another order
+        assert_close(dh, dh_p, TOL_DH[dtype], "dh")
 
 
 def test_interleaved_64bit_offsets(gcg_lib):
