@@ -164,3 +164,32 @@ def test_explicit_filter_recipe():
     assert f(64).shape == (8, 64)
     assert hyena.get_groups_and_group_sizes(4096, 256) == (4096, 256, 16)
     assert hyena.get_groups_and_group_sizes(8192, 512, world_size=8) == (1024, 64, 16)
+
+
+def test_interleaved_views_are_recognised_on_the_host():
+    """The split of block.py:886-888 gives three stride-3 views of one buffer; the autograd boundary
+    must find that buffer (and only then) so that it can skip the gathers."""
+    import torch
+    from einops import rearrange
+
+    from savanna_amd.kernels.cgcg.interface import interleaved_source
+
+    g, dg = 4, 16
+    feats = torch.randn(2, 5, 3 * g * dg)
+    x1, x2, v = rearrange(feats, "b l (g dg p) -> b l g p dg", p=3, g=g).unbind(dim=3)
+    src = interleaved_source(x=v, B=x2, C=x1)
+    assert src is not None and src.shape == (2, 5, g, dg, 3) and src.data_ptr() == feats.data_ptr()
+    assert torch.equal(src[..., 0], x1) and torch.equal(src[..., 1], x2) and torch.equal(src[..., 2], v)
+    # wrong order, gathered copies, a padded row stride, the non-interleaved split: not recognised
+    assert interleaved_source(x=x1, B=x2, C=v) is None
+    assert interleaved_source(x=v.contiguous(), B=x2, C=x1) is None
+    padded = torch.randn(2, 5, 3 * g * dg + 3)[:, :, 3:]
+    p1, p2, pv = rearrange(padded, "b l (g dg p) -> b l g p dg", p=3, g=g).unbind(dim=3)
+    assert interleaved_source(x=pv, B=p2, C=p1) is None
+    q1, q2, qv = rearrange(feats, "b l (p g dg) -> b l p g dg", p=3, g=g).unbind(dim=2)
+    assert interleaved_source(x=qv, B=q2, C=q1) is None
+    # an offset into a larger buffer is fine
+    big = torch.randn(3, 5, 3 * g * dg)
+    b1, b2, bv = rearrange(big[1:], "b l (g dg p) -> b l g p dg", p=3, g=g).unbind(dim=3)
+    src = interleaved_source(x=bv, B=b2, C=b1)
+    assert src is not None and src.data_ptr() == big[1:].data_ptr()
