@@ -56,7 +56,9 @@ class Op:
             else:
                 t = make_inputs(wl.bs, wl.L, wl.g, wl.dg, hl, wl.dtype, seed=i, device=device,
                                 with_dy=wl.backward)
-            if wl.layout != "separate":
+            if wl.layout == "dwconv":
+                t = {"x": t["k"], "h": t["h"], "dy": t.get("dy")}
+            elif wl.layout != "separate":
                 # kernel names: C = v, B = q, x = k
                 t["feat"] = torch.stack([t.pop("v"), t.pop("q"), t.pop("k")], dim=-1).contiguous()
             self.sets.append(t)
@@ -65,11 +67,20 @@ class Op:
         self.backward = wl.backward
         self.i = 0
         n = wl.bs * wl.L * wl.d * wl.elem_bytes
-        self.fwd_bytes, self.bwd_bytes = 4 * n, 7 * n
+        self.fwd_bytes, self.bwd_bytes = (2 * n, 3 * n) if wl.layout == "dwconv" else (4 * n, 7 * n)
 
     def run_features(self, t, ev):
         """Workloads whose inputs are one interleaved features tensor.  The whole op is bracketed:
         for "gathered" the gathers and the re-assembly of the feature gradient are part of it."""
+        if self.layout == "dwconv":
+            if ev is not None:
+                ev[0].record()
+            y = _lib.dwconv_fwd(t["x"], t["h"])
+            if self.backward:
+                _lib.dwconv_bwd(t["dy"], t["x"], t["h"])
+            if ev is not None:
+                ev[1].record()
+            return y
         feat, h = t["feat"], t["h"]
         if ev is not None:
             ev[0].record()

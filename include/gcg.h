@@ -147,6 +147,40 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
             int32_t dtype, int32_t algo, void *stream);
 
+/*
+ * Short causal depthwise convolution without gates: the featurizer that the hyena blocks apply to
+ * the projected features before splitting them.
+ * Replaces ParallelCausalDepthwiseConv1d.forward (savanna/model/operators/hyena/hyena.py:136-181,
+ * the F.conv1d path :159-176; called at savanna/model/block.py:873) together with the permutes
+ * to and from its (B, D, L) layout (block.py:867, :875): here the tensors stay (bs, L, g, dg) with
+ * the channel fastest, the layout of the dense projection before it and of gcg_fwd_interleaved
+ * after it.
+ *
+ *   y[b, t, c] = sum_k w[c / dg, 0, k] * x[b, t - (hl-1) + k, c]      (zero before the sequence)
+ *
+ *   x, y   (bs, L, g, dg);  w  (g, 1, hl), hl <= 8.  The reference's filters are one per
+ *          channel (weight (D, 1, K), hyena.py:108-110): g = D, dg = 1.  Supported: dg == 1 or
+ *          dg % 4 == 0, g * dg % 4 == 0, 16-byte aligned tensors; otherwise GCG_ERR_UNSUPPORTED.
+ */
+GCG_API int gcg_dwconv_fwd(const void *x, const void *w, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, void *stream);
+
+/* Workspace of gcg_dwconv_bwd (per-run partial sums of dw); 0 on invalid or unsupported arguments. */
+GCG_API size_t gcg_dwconv_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype);
+
+/*
+ * Backward of gcg_dwconv_fwd: what autograd derives for the F.conv1d of hyena.py:168-175
+ * (conv1d_input / conv1d_weight).
+ *   dx  out, (bs, L, g, dg);  dw  out, (g, 1, hl), overwritten, bit-reproducible
+ *   workspace  at least gcg_dwconv_bwd_workspace_bytes(...) bytes, 256-byte aligned
+ */
+GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *dx, void *dw,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,6 +26,7 @@ EXPORTS = (
     "gcg_strerror", "gcg_last_hip_error", "gcg_version", "gcg_fwd",
     "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_select_algo",
     "gcg_fwd_interleaved", "gcg_bwd_interleaved",
+    "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
 )
 
 _lock = threading.Lock()
@@ -67,6 +68,12 @@ def load() -> ctypes.CDLL:
         lib.gcg_fwd_interleaved.restype = ctypes.c_int
         lib.gcg_bwd_interleaved.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_bwd_interleaved.restype = ctypes.c_int
+        lib.gcg_dwconv_fwd.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, vp]
+        lib.gcg_dwconv_fwd.restype = ctypes.c_int
+        lib.gcg_dwconv_bwd_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32]
+        lib.gcg_dwconv_bwd_workspace_bytes.restype = sz
+        lib.gcg_dwconv_bwd.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, vp]
+        lib.gcg_dwconv_bwd.restype = ctypes.c_int
         _lib = lib
         return lib
 
@@ -207,6 +214,57 @@ def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO):
                                      ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, a, st)
     check(rc, "gcg_bwd_interleaved")
     return dfeat, dh
+
+
+def _check_dwconv(x, w):
+    if x.dim() != 4 or not x.is_contiguous():
+        raise ValueError("x must be a contiguous (bs, L, g, dg) tensor")
+    if w.dim() != 3 or w.shape[0] != x.shape[2] or w.shape[1] != 1 or not w.is_contiguous():
+        raise ValueError("w must be a contiguous (g, 1, hl) tensor")
+    if w.dtype != x.dtype or w.device != x.device:
+        raise ValueError("x and w must share dtype and device")
+
+
+def dwconv_fwd(x, w):
+    """y = causal depthwise convolution of x (bs, L, g, dg) with w (g, 1, hl), no gates."""
+    lib = load()
+    _require_gpu(x)
+    _check_dwconv(x, w)
+    bs, L, g, dg = x.shape
+    y = torch.empty_like(x)
+    if x.numel() == 0:
+        return y
+    with torch.cuda.device(x.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_dwconv_fwd(x.data_ptr(), w.data_ptr(), y.data_ptr(), bs, L, g, dg, w.shape[-1],
+                                dtype_code(x.dtype), st)
+    check(rc, "gcg_dwconv_fwd")
+    return y
+
+
+def dwconv_bwd(dy, x, w):
+    """(dx, dw) of dwconv_fwd."""
+    lib = load()
+    _require_gpu(x)
+    _check_dwconv(x, w)
+    if dy.shape != x.shape or dy.dtype != x.dtype or not dy.is_contiguous():
+        raise ValueError("dy must be a contiguous tensor of x's shape and dtype")
+    bs, L, g, dg = x.shape
+    hl = w.shape[-1]
+    dx, dw = torch.empty_like(x), torch.empty_like(w)
+    if x.numel() == 0:
+        return dx, dw.zero_()
+    code = dtype_code(x.dtype)
+    nbytes = lib.gcg_dwconv_bwd_workspace_bytes(bs, L, g, dg, hl, code)
+    if nbytes == 0:
+        check(-2, "gcg_dwconv_bwd_workspace_bytes")     # GCG_ERR_UNSUPPORTED
+    with torch.cuda.device(x.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_dwconv_bwd(dy.data_ptr(), x.data_ptr(), w.data_ptr(), dx.data_ptr(), dw.data_ptr(),
+                                ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, st)
+    check(rc, "gcg_dwconv_bwd")
+    return dx, dw
 
 
 def select_algo(bs, L, g, dg, hl, dtype: torch.dtype, backward=False) -> str:

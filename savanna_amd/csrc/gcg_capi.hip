@@ -95,7 +95,7 @@ GCG_API const char *gcg_strerror(int code)
 
 GCG_API int gcg_last_hip_error(void) { return tls_hip_error; }
 
-GCG_API int gcg_version(void) { return 101; }
+GCG_API int gcg_version(void) { return 102; }
 
 GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t backward)
 {
@@ -221,6 +221,44 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
         return finish(gcg::mfma_il_bwd_launch(dtype, dy, feat, h, dfeat, dh, workspace, dm, st));
     }
     return GCG_ERR_BAD_ARG;
+}
+
+// ---- ungated short causal depthwise convolution (featurizer)
+
+GCG_API int gcg_dwconv_fwd(const void *x, const void *w, void *y, int64_t bs, int64_t L, int32_t g, int32_t dg,
+                           int32_t hl, int32_t dtype, void *stream)
+{
+    if (!x || !w || !y) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    if (!gcg::dwconv_supported(dm) || !all_aligned16({x, y})) return GCG_ERR_UNSUPPORTED;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::dwconv_fwd_launch(dtype, x, w, y, dm, (hipStream_t)stream));
+}
+
+GCG_API size_t gcg_dwconv_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype)
+{
+    gcg::Dims dm;
+    if (make_dims(bs, L, g, dg, hl, dtype, &dm) || !gcg::dwconv_supported(dm)) return 0;
+    return (gcg::dwconv_bwd_workspace(dm) + 255) & ~(size_t)255;
+}
+
+GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *dx, void *dw, void *workspace,
+                           size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                           int32_t dtype, void *stream)
+{
+    if (!dy || !x || !w || !dx || !dw) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    if (!gcg::dwconv_supported(dm) || !all_aligned16({dy, x, dx})) return GCG_ERR_UNSUPPORTED;
+    const size_t need = gcg_dwconv_bwd_workspace_bytes(bs, L, g, dg, hl, dtype);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::dwconv_bwd_launch(dtype, dy, x, w, dx, dw, workspace, dm, (hipStream_t)stream));
 }
 
 } // extern "C"

@@ -200,4 +200,11 @@ int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, cons
 int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
                        void *ws, const Dims &dm, hipStream_t st);
 
+// ungated short causal depthwise convolution (the featurizer), (bs, L, g, dg) channel-fastest
+bool dwconv_supported(const Dims &dm);
+int dwconv_fwd_launch(int dtype, const void *x, const void *w, void *y, const Dims &dm, hipStream_t st);
+size_t dwconv_bwd_workspace(const Dims &dm);
+int dwconv_bwd_launch(int dtype, const void *dy, const void *x, const void *w, void *dx, void *dw, void *ws,
+                      const Dims &dm, hipStream_t st);
+
 } // namespace gcg

@@ -25,6 +25,7 @@ from typing import Optional
 import torch
 import torch.nn as nn
 
+from .. import _lib
 from ..kernels.cgcg.interface import two_pass_chunked_gate_conv_gate
 from ..kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
 
@@ -171,3 +172,52 @@ class HyenaSEOperator(_CgcgOperatorBase):
 
     def _filter(self, L: int) -> torch.Tensor:
         return self.short_conv_weight
+
+
+class _CausalDepthwiseConv(torch.autograd.Function):
+    """y[b, t, c] = sum_k w[c / dg, 0, k] x[b, t - (K-1) + k, c] on (b, l, g, dg) tensors."""
+
+    @staticmethod
+    def forward(ctx, x, w):
+        x = x if x.is_contiguous() else x.contiguous()
+        w = w if w.is_contiguous() else w.contiguous()
+        ctx.save_for_backward(x, w)
+        return _lib.dwconv_fwd(x, w)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        return _lib.dwconv_bwd(dy if dy.is_contiguous() else dy.contiguous(), x, w)
+
+
+class CausalDepthwiseConv1d(nn.Module):
+    """The featurizer conv of the hyena blocks: counterpart of ParallelCausalDepthwiseConv1d
+    (savanna/model/operators/hyena/hyena.py:76-181) on its torch path (:159-176), i.e. left
+    zero padding of K-1 and a cross-correlation, one filter per channel unless ``num_groups``
+    shares them ((num_groups, 1, K) weight, hyena.py:99-110, uniform(+-sqrt(1/K)) init, :128-130).
+
+    The reference module works on (B, D, L) and the block permutes around it (block.py:867-876);
+    ``forward_bld`` takes and returns (B, L, D) -- the layout of the projection before it and of
+    the interleaved operator after it -- and ``forward`` keeps the reference's (B, D, L) contract.
+    """
+
+    def __init__(self, d_model: int, kernel_size: int = 3, num_groups: Optional[int] = None,
+                 dtype=torch.float32, device=None):
+        super().__init__()
+        self.d_model, self.kernel_size = d_model, kernel_size
+        self.num_groups = d_model if num_groups is None else num_groups
+        assert d_model % self.num_groups == 0
+        self.group_dim = d_model // self.num_groups
+        bound = math.sqrt(1.0 / kernel_size)
+        w = torch.empty(self.num_groups, 1, kernel_size, dtype=dtype, device=device).uniform_(-bound, bound)
+        self.short_conv_weight = nn.Parameter(w)
+
+    def forward_bld(self, x: torch.Tensor) -> torch.Tensor:
+        b, l, d = x.shape
+        assert d == self.d_model
+        y = _CausalDepthwiseConv.apply(x.reshape(b, l, self.num_groups, self.group_dim),
+                                       self.short_conv_weight.to(x.dtype))
+        return y.reshape(b, l, d)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.forward_bld(x.permute(0, 2, 1)).permute(0, 2, 1)

@@ -31,6 +31,7 @@ class Workload:
     # (bs, L, g, dg, 3) projected-features tensor and the kernels read it as it is.  "gathered": same
     # features tensor, handled the way the reference does (three strided gathers before the forward,
     # re-assembly of the feature gradient after the backward) around the separate-tensor kernels.
+    # "dwconv": the ungated featurizer conv on one (bs, L, g, dg) tensor.
     layout: str = "separate"
 
     @property
@@ -46,6 +47,11 @@ class Workload:
         return torch.empty((), dtype=self.dtype).element_size()
 
     def algorithmic_bytes(self) -> int:
+        if self.layout == "dwconv":      # ungated: forward reads x, writes y; backward reads dy, x, writes dx
+            return (5 if self.backward else 2) * self.bs * self.L * self.d * self.elem_bytes * len(self.filters)
+        return self._gated_bytes()
+
+    def _gated_bytes(self) -> int:
         """Compulsory HBM traffic of one pass: forward reads q, k, v and writes y (4
         tensors); forward+backward adds reads of dy, q, k, v and writes of dq, dk, dv
         (11 tensors).  Filter and filter-gradient traffic (<= 256 KB) is not counted."""
@@ -88,6 +94,10 @@ WORKLOADS = {
     "se_fwdbwd_40b_gathered": Workload("se_fwdbwd_40b_gathered", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
                                        "the same with three gathers, separate-tensor kernels and re-assembly",
                                        layout="gathered"),
+    # the featurizer conv of a 7B layer: 3 * 4096 channels, one 3-tap filter per channel (block.py:873)
+    "featurizer_fwdbwd_7b": Workload("featurizer_fwdbwd_7b", 2, 8192, 12288, 1, (3,), torch.bfloat16, True,
+                                     "featurizer conv forward+backward, bf16, B=2 L=8192 channels=12288, one 3-tap "
+                                     "filter per channel", layout="dwconv"),
 }
 # the order in which the benchmark reports them
 WORKLOAD_ORDER = ("se_fwd_fp32", "mr_fwd_7b", "mr_fwdbwd_7b", "se_mr_fwdbwd_40b", "mr_fwd_1m")
