@@ -202,24 +202,6 @@ __global__ __launch_bounds__(256) void dwconv_bwd_kernel(const T *__restrict__ d
         }
 }
 
-// dw[grp][k]: sum over (batch, run) rows and, without per-channel filters, over the lanes of the group
-template <typename T, bool PCF>
-__global__ __launch_bounds__(256) void dwconv_dw_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dw,
-                                                               Dims dm, DwPlan pl)
-{
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= (int64_t)dm.g * dm.hl) return;
-    const int k = (int)(i / dm.g);                    // consecutive threads take consecutive filters
-    const int64_t grp = i % dm.g;
-    const int64_t nslot = PCF ? dm.d : pl.nvec;
-    const int lpg = PCF ? dm.dg : dm.dg / pl.v;       // slots per filter
-    const float *src = ws + (size_t)k * pl.nrows * nslot + grp * lpg;
-    float s = 0.f;
-    for (int64_t r = 0; r < pl.nrows; ++r)
-        for (int q = 0; q < lpg; ++q) s += src[r * nslot + q];
-    Elem<T>::store(dw + grp * dm.hl + k, s);
-}
-
 // Channels per lane: 4.  Eight (16-byte vectors at 16 bits) measured the same within noise at the
 // 7B featurizer shape (forward 160 vs 153 us, backward 265 vs 269 us) and stays a tuning override.
 int lane_width(int dtype, const Dims &dm)
@@ -266,10 +248,9 @@ int bwd_launch(const void *dy, const void *x, const void *w, void *dx, void *dw,
                        (const T *)dy, (const T *)x, (const T *)w, (T *)dx, (float *)ws, dm, p);
     int e = (int)hipGetLastError();
     if (e) return e;
-    const int64_t n = (int64_t)dm.g * dm.hl;
-    hipLaunchKernelGGL((dwconv_dw_reduce_kernel<T, PCF>), dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
-                       (const float *)ws, (T *)dw, dm, p);
-    return (int)hipGetLastError();
+    // partials are ws[tap][(batch, run)][slot], slot = channel (per-channel filters) or lane
+    return launch_colsum_reduce<T>((const float *)ws, (T *)dw, p.nrows, PCF ? dm.d : p.nvec, PCF ? dm.dg : dm.dg / V,
+                                   dm.g, dm.hl, st);
 }
 
 template <typename T, int V, bool PCF> int fwd_hl(const void *x, const void *w, void *y, const Dims &dm, hipStream_t st)

@@ -89,5 +89,50 @@ template <typename T, int VV> __device__ __forceinline__ typename Vec<T, VV>::ra
     return r;
 }
 
+
+// Filter-gradient reduction shared by the register-window kernels.  The walk kernels leave
+// partials ws[tap][row][col]: one row per (batch, run), one column per lane (or per channel);
+// filter f owns the lpg adjacent columns [f * lpg, (f+1) * lpg).  out[f * ntap + tap] is their
+// sum over all rows.  A workgroup takes a tile of whole filters at most 64 columns wide (one
+// filter if it is wider) and 4 row slices: its 64-lane rows read contiguous runs of a partial
+// row, every thread adds its terms in a fixed order, and the slices and columns of a filter are
+// then combined in a fixed order -- the result is bit-reproducible.
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_reduce_kernel(const float *__restrict__ ws, T *__restrict__ out,
+                                                            int64_t nrow, int64_t ncol, int lpg, int nfilt, int ntap)
+{
+    __shared__ float red[4][64];
+    const int fpb = lpg >= 64 ? 1 : 64 / lpg;                 // filters per workgroup
+    const int tap = blockIdx.y;
+    const int64_t f0 = (int64_t)blockIdx.x * fpb;
+    const int nf = (int)((f0 + fpb <= nfilt) ? fpb : nfilt - f0);
+    const int width = nf * lpg;                                // columns of the tile
+    const int c = threadIdx.x & 63, slice = threadIdx.x >> 6;
+    const float *src = ws + (size_t)tap * nrow * ncol + f0 * lpg;
+    float s = 0.f;
+    for (int cc = c; cc < width; cc += 64)                     // more than one column only for one wide filter
+        for (int64_t r = slice; r < nrow; r += 4) s += src[r * ncol + cc];
+    red[slice][c] = s;
+    __syncthreads();
+    if ((int)threadIdx.x < nf) {
+        const int lo = lpg >= 64 ? 0 : (int)threadIdx.x * lpg, n = lpg >= 64 ? 64 : lpg;
+        float t = 0.f;
+        for (int q = 0; q < n; ++q)
+            for (int sl = 0; sl < 4; ++sl) t += red[sl][lo + q];
+        Elem<T>::store(out + (f0 + threadIdx.x) * ntap + tap, t);
+    }
+}
+
+template <typename T>
+inline int launch_colsum_reduce(const float *ws, T *out, int64_t nrow, int64_t ncol, int lpg, int nfilt, int ntap,
+                                hipStream_t st)
+{
+    const int fpb = lpg >= 64 ? 1 : 64 / lpg;
+    const unsigned nbx = (unsigned)((nfilt + fpb - 1) / fpb);
+    hipLaunchKernelGGL(colsum_reduce_kernel<T>, dim3(nbx, (unsigned)ntap), dim3(256), 0, st, ws, out, nrow, ncol, lpg,
+                       nfilt, ntap);
+    return (int)hipGetLastError();
+}
+
 } // namespace
 } // namespace gcg

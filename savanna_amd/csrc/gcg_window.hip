@@ -375,31 +375,6 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
         if (j < hl) slot[(size_t)(hl - 1 - j) * pl.nthreads] = dha[j];
 }
 
-// One workgroup per (group, tap): fixed-order strided sums, then a fixed LDS tree.
-template <typename T>
-__global__ __launch_bounds__(256) void window_dh_reduce_kernel(const float *__restrict__ ws, T *__restrict__ dh,
-                                                               Dims dm, WinPlan pl)
-{
-    __shared__ float red[256];
-    const int grp = blockIdx.x / dm.hl, k = blockIdx.x % dm.hl;
-    const int lpg = dm.dg / pl.v;                    // lanes (channel vectors) per group
-    const int64_t nrow = dm.bs * pl.nseg;            // (batch, segment) pairs
-    const int64_t nterm = nrow * lpg;
-    const float *src = ws + (size_t)k * pl.nthreads;
-    float s = 0.f;
-    for (int64_t i = threadIdx.x; i < nterm; i += 256) {
-        const int64_t row = i / lpg, l = i % lpg;
-        s += src[row * pl.nvec + (int64_t)grp * lpg + l];
-    }
-    red[threadIdx.x] = s;
-    __syncthreads();
-    for (int w = 128; w > 0; w >>= 1) {
-        if ((int)threadIdx.x < w) red[threadIdx.x] += red[threadIdx.x + w];
-        __syncthreads();
-    }
-    if (threadIdx.x == 0) Elem<T>::store(dh + (size_t)grp * dm.hl + k, red[0]);
-}
-
 WinPlan plan(const Dims &dm, int v)
 {
     WinPlan p;
@@ -466,9 +441,8 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
                            (T *)dC, (float *)ws, dm, p);
     int e = (int)hipGetLastError();
     if (e) return e;
-    hipLaunchKernelGGL(window_dh_reduce_kernel<T>, dim3((unsigned)(dm.g * dm.hl)), dim3(256), 0, st,
-                       (const float *)ws, (T *)dh, dm, p);
-    return (int)hipGetLastError();
+    // partials are ws[tap][(batch, run)][lane]; a filter owns dg / v adjacent lanes
+    return launch_colsum_reduce<T>((const float *)ws, (T *)dh, dm.bs * p.nseg, p.nvec, dm.dg / p.v, dm.g, dm.hl, st);
 }
 
 // Four channels per lane in both directions.  Eight (16-byte vectors for the 16-bit types) was
