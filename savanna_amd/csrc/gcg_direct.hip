@@ -4,8 +4,8 @@
 // halo is staged once in LDS as fp32; each lane then owns one channel and 16
 // consecutive time rows and walks the taps in blocks of 16, holding 16 taps and a
 // 31-sample window in registers so that a block costs 47 LDS reads for 256 FMAs.
-// This is the fp32 path (matrix cores would round the operands) and the fallback
-// for shapes the MFMA and register-window kernels do not take.
+// This is the fallback for shapes the MFMA and register-window kernels do not take (filters
+// longer than 128 taps, narrow or odd group widths, misaligned tensors).
 #include "gcg_common.h"
 
 namespace gcg {

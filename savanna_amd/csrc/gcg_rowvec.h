@@ -110,8 +110,17 @@ __global__ __launch_bounds__(256) void colsum_reduce_kernel(const float *__restr
     const int c = threadIdx.x & 63, slice = threadIdx.x >> 6;
     const float *src = ws + (size_t)tap * nrow * ncol + f0 * lpg;
     float s = 0.f;
-    for (int cc = c; cc < width; cc += 64)                     // more than one column only for one wide filter
-        for (int64_t r = slice; r < nrow; r += 4) s += src[r * ncol + cc];
+    for (int cc = c; cc < width; cc += 64) {                   // more than one column only for one wide filter
+        int64_t r = slice;
+        for (; r + 28 < nrow; r += 32) {                       // eight loads in flight, added in row order
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) v[i] = src[(r + 4 * i) * ncol + cc];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s += v[i];
+        }
+        for (; r < nrow; r += 4) s += src[r * ncol + cc];
+    }
     red[slice][c] = s;
     __syncthreads();
     if ((int)threadIdx.x < nf) {
