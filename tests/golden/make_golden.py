@@ -29,7 +29,30 @@ CASES = {
 }
 
 
+def featurizer_case():
+    """The featurizer conv as ParallelCausalDepthwiseConv1d.forward computes it on (B, D, L)
+    (savanna/model/operators/hyena/hyena.py:139,159,168-175: left pad K-1, F.conv1d with one group per
+    channel, first L samples), in float64, stored channel-last as (bs, L, D, 1) / (D, 1, K)."""
+    import torch.nn.functional as F
+
+    bs, L, D, K, dtype = 2, 150, 24, 3, torch.bfloat16
+    gen = torch.Generator().manual_seed(0)
+    x = torch.randn(bs, D, L, generator=gen).to(dtype).double().requires_grad_(True)
+    dy = torch.randn(bs, D, L, generator=gen).to(dtype).double()
+    w = (torch.randn(D, 1, K, generator=gen) / K ** 0.5).to(dtype).double().requires_grad_(True)
+    y = F.conv1d(F.pad(x, (K - 1, 0)), w, bias=None, stride=1, padding=0, groups=D)[..., :L]
+    y.backward(dy)
+    cl = lambda t: t.detach().permute(0, 2, 1).unsqueeze(-1).contiguous()   # (bs, L, D, 1)
+    np.savez_compressed(
+        os.path.join(HERE, "featurizer_bf16_small.npz"),
+        x=cl(x).float().numpy(), dy=cl(dy).float().numpy(), w=w.detach().float().numpy(),
+        y=cl(y).numpy(), dx=cl(x.grad).numpy(), dw=w.grad.numpy(), dtype=np.array(str(dtype)),
+    )
+    print("featurizer_bf16_small written")
+
+
 def main():
+    featurizer_case()
     for name, (bs, L, g, dg, hl, dtype) in CASES.items():
         gen = torch.Generator().manual_seed(0)
         x, B, C, dy = (torch.randn(bs, L, g, dg, generator=gen).to(dtype).double() for _ in range(4))

@@ -14,7 +14,9 @@ from helpers import TOL, TOL_DH, assert_close
 from savanna_amd import _lib
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-FILES = sorted(glob.glob(os.path.join(HERE, "golden", "*.npz")))
+ALL = sorted(glob.glob(os.path.join(HERE, "golden", "*.npz")))
+FILES = [f for f in ALL if not os.path.basename(f).startswith("featurizer")]      # the gated operator
+FEAT = [f for f in ALL if os.path.basename(f).startswith("featurizer")]           # the ungated featurizer conv
 DT = {"torch.float32": torch.float32, "torch.bfloat16": torch.bfloat16, "torch.float16": torch.float16}
 
 
@@ -25,7 +27,7 @@ def load(path):
 
 
 def test_fixtures_present():
-    assert len(FILES) >= 4
+    assert len(FILES) >= 4 and len(FEAT) >= 1
 
 
 @pytest.mark.parametrize("path", FILES, ids=[os.path.basename(f) for f in FILES])
@@ -56,3 +58,42 @@ def test_hip_reproduces_golden(gcg_lib, path, algo):
     grads = _lib.bwd(dev["dy"], dev["x"], dev["B"], dev["C"], dev["h"], algo=algo)
     for got, name in zip(grads, ("dx", "dB", "dC", "dh")):
         assert_close(got, t[name], TOL_DH[dtype] if name == "dh" else TOL[dtype], f"{name} [{algo}]")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("algo", ["auto", "direct"])
+@pytest.mark.parametrize("path", FILES, ids=[os.path.basename(f) for f in FILES])
+def test_hip_interleaved_reproduces_golden(gcg_lib, path, algo):
+    """The same vectors through the interleaved entry points: x, B, C packed into one
+    (bs, L, g, dg, 3) tensor, the three input gradients read back from one."""
+    t, dtype = load(path)
+    dev = {k: v.to(dtype).to("cuda:0") for k, v in t.items()}
+    feat = torch.stack([dev["C"], dev["B"], dev["x"]], dim=-1).contiguous()
+    y = _lib.fwd_interleaved(feat, dev["h"], algo=algo)
+    assert_close(y, t["y"], TOL[dtype], f"y [{algo}]")
+    dfeat, dh = _lib.bwd_interleaved(dev["dy"], feat, dev["h"], algo=algo)
+    for i, name in enumerate(("dC", "dB", "dx")):
+        assert_close(dfeat[..., i], t[name], TOL[dtype], f"{name} [{algo}]")
+    assert_close(dh, t["dh"], TOL_DH[dtype], f"dh [{algo}]")
+
+
+@pytest.mark.parametrize("path", FEAT, ids=[os.path.basename(f) for f in FEAT])
+def test_c_oracle_reproduces_featurizer_golden(path):
+    """The featurizer is the gated operator with both gates at one."""
+    t, _ = load(path)
+    one = torch.ones_like(t["x"])
+    assert_close(oracle.gcg_fwd_oracle(t["x"], one, one, t["w"]), t["y"], 2e-6, "y")
+    dx, _, _, dw = oracle.gcg_bwd_oracle(t["dy"], t["x"], one, one, t["w"])
+    assert_close(dx, t["dx"], 2e-6, "dx")
+    assert_close(dw, t["dw"], 2e-6, "dw")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", FEAT, ids=[os.path.basename(f) for f in FEAT])
+def test_hip_featurizer_reproduces_golden(gcg_lib, path):
+    t, dtype = load(path)
+    dev = {k: v.to(dtype).to("cuda:0") for k, v in t.items()}
+    assert_close(_lib.dwconv_fwd(dev["x"], dev["w"]), t["y"], TOL[dtype], "y")
+    dx, dw = _lib.dwconv_bwd(dev["dy"], dev["x"], dev["w"])
+    assert_close(dx, t["dx"], TOL[dtype], "dx")
+    assert_close(dw, t["dw"], TOL_DH[dtype], "dw")
