@@ -26,7 +26,7 @@ import torch
 import torch.nn as nn
 
 from .. import _lib
-from ..kernels.cgcg.interface import two_pass_chunked_gate_conv_gate
+from ..kernels.cgcg.interface import two_pass_chunked_gate_conv_gate, two_pass_chunked_gate_conv_gate_interleaved
 from ..kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
 
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
@@ -132,6 +132,7 @@ class _CgcgOperatorBase(nn.Module):
             x, B, C, h = (t.to(self.cgcg_dtype) for t in (v, x2, x1, h))
         else:
             x, B, C = v, x2, x1
+            h = h.to(dtype)             # parameters kept in another precision than the activations
         bs, seqlen, g, dg = x.shape
         z = self.cgcg_fn(
             x=x, B=B, C=C, h=h, bs=bs, seqlen=seqlen, g=g, dg=dg,
@@ -141,6 +142,21 @@ class _CgcgOperatorBase(nn.Module):
             fwd_kernel_cfg=self.cgcg_fwd_config,
             bwd_kernel_cfg=None if self.cfg.cgcg_bwd_autotune else self.cgcg_bwd_config,
         )
+        z = z.reshape(bs, seqlen, g * dg)
+        return z.to(dtype) if self.cgcg_dtype != dtype else z
+
+    def forward_features(self, features: torch.Tensor) -> torch.Tensor:
+        """The same on the projected features before their split: (b, l, 3*g*dg) laid out
+        "(g dg p)" with p = (x1, x2, v) fastest (block.py:886-888) -> z: (b, l, g*dg).  The kernels
+        read the tensor as it is and the backward writes its gradient in the same layout."""
+        dtype = features.dtype
+        bs, seqlen, d3 = features.shape
+        g, dg = self.num_groups, self.group_dim
+        assert d3 == 3 * g * dg
+        h = self._filter(seqlen)
+        if self.cgcg_dtype != dtype:
+            features = features.to(self.cgcg_dtype)
+        z = two_pass_chunked_gate_conv_gate_interleaved(features, h.to(self.cgcg_dtype), bs, seqlen, g, dg)
         z = z.reshape(bs, seqlen, g * dg)
         return z.to(dtype) if self.cgcg_dtype != dtype else z
 
@@ -221,3 +237,18 @@ class CausalDepthwiseConv1d(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.forward_bld(x.permute(0, 2, 1)).permute(0, 2, 1)
+
+
+class HyenaMixer(nn.Module):
+    """The convolutional part of ParallelSequenceMixer.forward for the hyena operators
+    (savanna/model/block.py:865-890): featurizer conv on the projected features, interleaved split,
+    gated convolution.  Input (b, l, 3*hidden) -- what the dense projection writes -- output
+    (b, l, hidden) for the output projection; no permute, gather or split copy in between."""
+
+    def __init__(self, operator: _CgcgOperatorBase, short_conv_L: int = 3, dtype=torch.float32, device=None):
+        super().__init__()
+        self.mixer = operator
+        self.hyena_proj_conv = CausalDepthwiseConv1d(3 * operator.hidden_size, short_conv_L, dtype=dtype, device=device)
+
+    def forward(self, features: torch.Tensor) -> torch.Tensor:
+        return self.mixer.forward_features(self.hyena_proj_conv.forward_bld(features))

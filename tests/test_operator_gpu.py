@@ -154,3 +154,32 @@ def test_graph_capture_and_replay(gcg_lib, hl, dtype):
         assert torch.equal(y_g, y_e), f"replay {it}: y"
         for a, b, n in zip(grads_g, grads_e, ("dx", "dB", "dC", "dh")):
             assert torch.equal(a, b), f"replay {it}: {n}"
+
+
+@pytest.mark.parametrize("kind", ["mr", "se"])
+def test_mixer_on_projected_features(gcg_lib, kind):
+    """HyenaMixer (featurizer conv -> interleaved split -> operator) against the reference's chain
+    written with torch ops: permute, F.pad + F.conv1d on (B, 3D, L), permute, the interleaved
+    rearrange / unbind of block.py:886-888, and the operator on the three views."""
+    import torch.nn.functional as F
+    from einops import rearrange
+
+    from savanna_amd.operators.hyena import CgcgConfig, HyenaMixer, HyenaMROperator, HyenaSEOperator
+
+    torch.manual_seed(21)
+    bs, L, hidden, groups = 2, 320, 128, 8
+    cfg = CgcgConfig(cgcg_dtype="bfloat16")
+    op = (HyenaMROperator(hidden, groups, 128, cfg, small_init=False, device=DEV) if kind == "mr"
+          else HyenaSEOperator(hidden, groups, 7, cfg, device=DEV))
+    mixer = HyenaMixer(op, 3, dtype=torch.bfloat16, device=DEV)
+    feats = torch.randn(bs, L, 3 * hidden, device=DEV).to(torch.bfloat16)
+    z = mixer(feats)
+    assert z.shape == (bs, L, hidden)
+
+    w = mixer.hyena_proj_conv.short_conv_weight.detach()
+    f = F.conv1d(F.pad(feats.permute(0, 2, 1).float(), (2, 0)), w.float(), groups=3 * hidden)[..., :L]
+    f = f.to(torch.bfloat16).permute(0, 2, 1)
+    x1, x2, v = rearrange(f, "b l (g dg p) -> b l g p dg", p=3, g=groups).unbind(dim=3)
+    z_ref = op(x1, x2, v)                       # the operator on the split views (checked against the oracle above)
+    torch.cuda.synchronize()
+    assert_close(z, z_ref, 1e-2, "z")
