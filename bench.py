@@ -58,16 +58,55 @@ class Op:
                                 with_dy=wl.backward)
             if wl.layout == "dwconv":
                 t = {"x": t["k"], "h": t["h"], "dy": t.get("dy")}
+            elif wl.layout.startswith("mixer"):
+                raw = torch.stack([t.pop("v"), t.pop("q"), t.pop("k")], dim=-1).reshape(wl.bs, wl.L, 3 * wl.d)
+                wf = (torch.randn(3 * wl.d, 1, 3, generator=torch.Generator().manual_seed(i)) / 3 ** 0.5)
+                t["raw"] = raw.contiguous().requires_grad_(True)
+                t["wf"] = wf.to(wl.dtype).to(device).requires_grad_(True)
+                t["h"] = t["h"].requires_grad_(True)
             elif wl.layout != "separate":
                 # kernel names: C = v, B = q, x = k
                 t["feat"] = torch.stack([t.pop("v"), t.pop("q"), t.pop("k")], dim=-1).contiguous()
             self.sets.append(t)
         self.layout = wl.layout
+        self.wl = wl
         self.hl = hl
         self.backward = wl.backward
         self.i = 0
         n = wl.bs * wl.L * wl.d * wl.elem_bytes
         self.fwd_bytes, self.bwd_bytes = (2 * n, 3 * n) if wl.layout == "dwconv" else (4 * n, 7 * n)
+
+    def run_mixer(self, t, ev):
+        """Featurizer conv + operator through autograd, ours or with the reference's data flow."""
+        import torch.nn.functional as F
+        from einops import rearrange
+
+        from savanna_amd.kernels.cgcg.interface import (two_pass_chunked_gate_conv_gate,
+                                                        two_pass_chunked_gate_conv_gate_interleaved)
+        from savanna_amd.kernels.cgcg.src.kernel_utils import FwdKernelConfigRefactor
+        from savanna_amd.operators.hyena import _CausalDepthwiseConv
+
+        wl = self.wl
+        raw, wf, h = t["raw"], t["wf"], t["h"]
+        raw.grad = wf.grad = h.grad = None
+        if ev is not None:
+            ev[0].record()
+        if self.layout == "mixer":
+            f = _CausalDepthwiseConv.apply(raw.reshape(wl.bs, wl.L, 3 * wl.d, 1), wf)
+            y = two_pass_chunked_gate_conv_gate_interleaved(f, h, wl.bs, wl.L, wl.g, wl.dg)
+        else:
+            u = raw.permute(0, 2, 1)                                               # block.py:867
+            f = F.conv1d(F.pad(u, (2, 0)), wf, groups=3 * wl.d)[..., :wl.L]        # hyena.py:139, :168-175
+            f = f.permute(0, 2, 1)                                                 # block.py:875
+            x1, x2, v = rearrange(f, "b l (g dg p) -> b l g p dg", p=3, g=wl.g).unbind(dim=3)
+            y = two_pass_chunked_gate_conv_gate(v.contiguous(), x2.contiguous(), x1.contiguous(), h, wl.bs, wl.L,
+                                                wl.g, wl.dg, fwd_kernel_cfg=FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row"),
+                                                bwd_autotune=True)
+        if self.backward:
+            y.backward(t["dy"])
+        if ev is not None:
+            ev[1].record()
+        return y
 
     def run_features(self, t, ev):
         """Workloads whose inputs are one interleaved features tensor.  The whole op is bracketed:
@@ -101,6 +140,8 @@ class Op:
     def run(self, ev=None):
         t = self.sets[self.i % self.nsets]
         self.i += 1
+        if self.layout.startswith("mixer"):
+            return self.run_mixer(t, ev)
         if self.layout != "separate":
             return self.run_features(t, ev)
         # kernel names: B = q, x = k, C = v

@@ -32,6 +32,10 @@ class Workload:
     # features tensor, handled the way the reference does (three strided gathers before the forward,
     # re-assembly of the feature gradient after the backward) around the separate-tensor kernels.
     # "dwconv": the ungated featurizer conv on one (bs, L, g, dg) tensor.
+    # "mixer": featurizer conv then the operator on the interleaved features, all on (bs, L, 3d);
+    # "mixer_reference_flow": the same chain as block.py:865-890 runs it -- permute to (B, 3D, L),
+    # F.pad + F.conv1d, permute back, interleaved split, three gathers -- around the separate-tensor
+    # kernels, with autograd doing the backward of the torch part.
     layout: str = "separate"
 
     @property
@@ -47,6 +51,9 @@ class Workload:
         return torch.empty((), dtype=self.dtype).element_size()
 
     def algorithmic_bytes(self) -> int:
+        if self.layout.startswith("mixer"):
+            # forward: read raw features 3N, write y N; backward: read dy N and raw features 3N, write d features 3N
+            return 11 * self.bs * self.L * self.d * self.elem_bytes * len(self.filters)
         if self.layout == "dwconv":      # ungated: forward reads x, writes y; backward reads dy, x, writes dx
             return (5 if self.backward else 2) * self.bs * self.L * self.d * self.elem_bytes * len(self.filters)
         return self._gated_bytes()
@@ -98,6 +105,14 @@ WORKLOADS = {
     "featurizer_fwdbwd_7b": Workload("featurizer_fwdbwd_7b", 2, 8192, 12288, 1, (3,), torch.bfloat16, True,
                                      "featurizer conv forward+backward, bf16, B=2 L=8192 channels=12288, one 3-tap "
                                      "filter per channel", layout="dwconv"),
+    "mixer_fwdbwd_7b": Workload("mixer_fwdbwd_7b", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
+                                "featurizer conv + Hyena-MR on interleaved features, forward+backward, bf16, B=2 L=8192 "
+                                "D=4096 G=256 hl=128", layout="mixer"),
+    "mixer_fwdbwd_7b_reference_flow": Workload("mixer_fwdbwd_7b_reference_flow", 2, 8192, 256, 16, (128,),
+                                               torch.bfloat16, True,
+                                               "the same chain with the reference's data flow (permutes, F.conv1d on "
+                                               "(B, 3D, L), gathers) around the separate-tensor kernels",
+                                               layout="mixer_reference_flow"),
 }
 # the order in which the benchmark reports them
 WORKLOAD_ORDER = ("se_fwd_fp32", "mr_fwd_7b", "mr_fwdbwd_7b", "se_mr_fwdbwd_40b", "mr_fwd_1m")
