@@ -494,7 +494,8 @@ int fwd_t(const void *x, const void *B, const void *C, const void *h, void *y, v
 bool mfma_supported(int dtype, const Dims &dm)
 {
     (void)dtype;   // bf16, f16 and fp32 all have a matrix-core form
-    return dm.hl <= 128 && dm.dg % 16 == 0;
+    // the shortest segment with its lead-in and look-ahead must fit one tensor window
+    return dm.hl <= 128 && dm.dg % 16 == 0 && (int64_t)(1 + 2 * 5) * STEP * 3 * dm.d * 4 <= WIN_MAX_BYTES;
 }
 
 int mfma_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h, void *y,
