@@ -139,6 +139,20 @@ __device__ __forceinline__ void win_store(win_t w, uint32_t off, const u32x4 &v)
     __builtin_amdgcn_raw_buffer_store_b128(v, w, (int)off, 0, WIN_NT_ST);
 }
 
+#ifndef GCG_XCD_SWIZZLE
+#define GCG_XCD_SWIZZLE 1
+#endif
+// Workgroups are dealt to the 8 XCDs round-robin by index.  Re-labelling them so that each XCD
+// receives a contiguous run of (batch, segment, channel-block) triples makes the workgroups of
+// one XCD cover whole tensor rows between them, which its L2 and the memory channels prefer.
+__device__ __forceinline__ int64_t xcd_contiguous_id(int64_t id, int64_t n)
+{
+#if GCG_XCD_SWIZZLE
+    if ((n & 7) == 0) return (id & 7) * (n >> 3) + (id >> 3);
+#endif
+    return id;
+}
+
 // ---- launch descriptors shared by host dispatch and kernels --------------------------
 struct Dims {
     int64_t bs, L;

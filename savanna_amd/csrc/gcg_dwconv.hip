@@ -107,7 +107,9 @@ __global__ __launch_bounds__(256) void dwconv_bwd_kernel(const T *__restrict__ d
 {
     typedef typename Vec<T, V>::raw raw_t;
     constexpr int ES = sizeof(T), NF = PCF ? V : 1;
-    int64_t wg = blockIdx.x;
+    // workgroups of one XCD take adjacent channel blocks of the same rows (measured +3-5 % in the
+    // backward kernels, -3 % in the forward ones, which keep the plain order)
+    int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
     const int seg = (int)(wg % pl.nseg);
     const int64_t b = wg / pl.nseg;
@@ -219,6 +221,8 @@ DwPlan plan(const Dims &dm, int V)
     p.nvec = (int)(dm.d / V);
     p.ts = 128;
     while (p.ts > 8 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
+    static const char *env = getenv("GCG_DWCONV_ROWS");     // tuning override: rows per lane, a multiple of 8
+    if (env && atoi(env) >= 8 && atoi(env) % 8 == 0) p.ts = atoi(env);
     while (p.ts > 8 && (int64_t)(p.ts + 2 * RING) * dm.d * 4 > WIN_MAX_BYTES) p.ts >>= 1;
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);
     p.nrows = dm.bs * p.nseg;

@@ -223,10 +223,6 @@ template <typename T> __device__ __forceinline__ Row<T> lds_load_row(const unsig
     return r;
 }
 
-#ifndef GCG_XCD_SWIZZLE
-#define GCG_XCD_SWIZZLE 1
-#endif
-
 // 16-, 12- and 4-byte accesses of a tensor window (gcg_common.h)
 __device__ __forceinline__ uint4 ldw16(win_t w, uint32_t off)
 {
@@ -252,17 +248,6 @@ template <typename T> __device__ __forceinline__ void stw_row(win_t w, uint32_t 
 {
 #pragma unroll
     for (int i = 0; i < MT<T>::RW; ++i) stw16(w, off + 16 * i, r.w[i]);
-}
-
-// Workgroups are dealt to the 8 XCDs round-robin by index.  Re-labelling them so that each XCD
-// receives a contiguous run of (batch, segment, channel-block) triples makes the workgroups of
-// one XCD cover whole tensor rows between them, which its L2 and the memory channels prefer.
-__device__ __forceinline__ int64_t xcd_contiguous_id(int64_t id, int64_t n)
-{
-#if GCG_XCD_SWIZZLE
-    if ((n & 7) == 0) return (id & 7) * (n >> 3) + (id >> 3);
-#endif
-    return id;
 }
 
 struct MfmaPlan { int ncb, nseg, steps_per_seg, nw; int64_t nsteps, nwg; };

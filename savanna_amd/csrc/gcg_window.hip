@@ -205,7 +205,9 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 {
     typedef typename Vec<T, V>::raw raw_t;
     constexpr int ES = sizeof(T), IS = PK ? 3 : 1;
-    int64_t wg = blockIdx.x;
+    // workgroups of one XCD take adjacent channel blocks of the same rows (measured +3-5 % in the
+    // backward kernels, -3 % in the forward ones, which keep the plain order)
+    int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
     const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
     const int seg = (int)(wg % pl.nseg);
     const int64_t b = wg / pl.nseg;
