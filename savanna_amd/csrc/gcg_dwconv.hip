@@ -321,6 +321,7 @@ size_t dwconv_bwd_workspace(const Dims &dm)
 {
     size_t n = 0;
     for (int v : {4, 8}) {
+        if (dm.d % v) continue;
         const DwPlan p = plan(dm, v);
         const int64_t nslot = dm.dg % v == 0 ? p.nvec : dm.d;
         const size_t need = (size_t)dm.hl * p.nrows * nslot * sizeof(float);

@@ -499,6 +499,7 @@ size_t window_bwd_workspace(const Dims &dm)
 {
     int64_t n = 0;
     for (int v : {1, 2, BWD_V}) {
+        if (dm.d % v) continue;
         const WinPlan p = plan(dm, v);
         if (p.nthreads > n) n = p.nthreads;
     }

@@ -193,3 +193,21 @@ def test_interleaved_views_are_recognised_on_the_host():
     b1, b2, bv = rearrange(big[1:], "b l (g dg p) -> b l g p dg", p=3, g=g).unbind(dim=3)
     src = interleaved_source(x=bv, B=b2, C=b1)
     assert src is not None and src.data_ptr() == big[1:].data_ptr()
+
+
+def test_workspace_sizing_runs_on_the_host_for_any_shape(gcg_lib):
+    """The *_workspace_bytes entry points are host arithmetic (launch plans): every shape, also a
+    tensor narrower than a lane's vector, must give a 256-byte multiple or 0 -- never trap."""
+    import itertools
+
+    for bs, L, g, dg, hl, dt in itertools.product((1, 3), (1, 7, 4096), (1, 2, 4, 12288), (1, 2, 4, 16), (1, 3, 7, 128, 200),
+                                                 (0, 1, 2)):
+        for algo in (0, 1, 2, 3):
+            n = gcg_lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dt, algo)
+            assert n % 256 == 0
+            if algo in (0, 1):
+                assert n > 0, (bs, L, g, dg, hl, dt, algo)      # the direct family takes everything
+        n = gcg_lib.gcg_dwconv_bwd_workspace_bytes(bs, L, g, dg, hl, dt)
+        supported = hl <= 8 and (g * dg) % 4 == 0 and (dg == 1 or dg % 4 == 0)
+        assert n % 256 == 0 and (n > 0) == supported, (bs, L, g, dg, hl, dt)
+        assert gcg_lib.gcg_select_algo(bs, L, g, dg, hl, dt, 1) in (1, 2, 3)
