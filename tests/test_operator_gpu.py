@@ -183,3 +183,39 @@ def test_mixer_on_projected_features(gcg_lib, kind):
     z_ref = op(x1, x2, v)                       # the operator on the split views (checked against the oracle above)
     torch.cuda.synchronize()
     assert_close(z, z_ref, 1e-2, "z")
+
+
+@pytest.mark.parametrize("repeat_interleave", [True, False])
+def test_run_short_hyena_layout(gcg_lib, repeat_interleave):
+    """run_short_hyena on (seqlen, bs, g, dg) inputs against the reference's own statement of that
+    operator (short_hyena/utils.py:36-66: rearrange to (bs, d, seqlen), F.conv1d with padding K-1 on
+    both sides trimmed to seqlen, times q, rearranged to (bs, g, seqlen, dg)), with gradients."""
+    import torch.nn.functional as F
+    from einops import rearrange
+
+    from savanna_amd.kernels.short_hyena import run_short_hyena
+
+    seqlen, bs, g, dg, hl = 96, 2, 4, 16, 3
+    gen = torch.Generator().manual_seed(31)
+    q, k, v = (torch.randn(seqlen, bs, g, dg, generator=gen) for _ in range(3))
+    w = torch.randn(g if repeat_interleave else g * dg, 1, hl, generator=gen) / hl ** 0.5
+    dy = 0.1 * torch.randn(bs, g, seqlen, dg, generator=gen)
+
+    dev = [t.to(DEV).requires_grad_(True) for t in (q, k, v, w)]
+    out = run_short_hyena(*dev, repeat_interleave=repeat_interleave, autotune=True)
+    assert out.shape == (bs, g, seqlen, dg)
+    out.backward(dy.to(DEV))
+
+    ref_in = [t.double().requires_grad_(True) for t in (q, k, v, w)]
+    rq, rk, rv, rw = ref_in
+    wd = rw.repeat_interleave(dg, dim=0) if repeat_interleave else rw
+    kv = rearrange(rk * rv, "s b g d -> b (g d) s")
+    conv = F.conv1d(kv, wd, bias=None, stride=1, padding=hl - 1, groups=g * dg)[..., :seqlen]
+    ref = rearrange(conv * rearrange(rq, "s b g d -> b (g d) s"), "b (g d) s -> b g s d", g=g)
+    ref.backward(dy.double())
+    torch.cuda.synchronize()
+    assert_close(out, ref, TOL[torch.float32], "out")
+    for a, r, n in zip(dev, ref_in, ("dq", "dk", "dv", "dw")):
+        assert_close(a.grad, r.grad, TOL_DH[torch.float32] if n == "dw" else TOL[torch.float32], n)
+    with pytest.raises(AssertionError, match="Must specify"):
+        run_short_hyena(*dev)
