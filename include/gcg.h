@@ -181,6 +181,26 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
             int32_t dtype, void *stream);
 
+/*
+ * Explicit decayed filter of Hyena-MR, ready for gcg_fwd, in one launch.
+ * Replaces ExplicitSingleDecayFilter.filter (savanna/model/operators/hyena/parametrization/
+ * explicit.py:68-75: h = self.h[:, :L] * self.decay[:, :L]) with L = min(hyena_mr_len, seq_len),
+ * the [:, None] of hyena.py:440-441 and the cast to cgcg_dtype of hyena.py:499-503.
+ *
+ *   w, decay   (g, l_cache) fp32: the parameter and the decay buffer
+ *   h          out, (g, 1, hl) of element type `dtype`:  h[g, 0, k] = dtype(w[g, k] * decay[g, k])
+ */
+GCG_API int gcg_filter_decay_fwd(const float *w, const float *decay, void *h,
+            int32_t g, int32_t l_cache, int32_t hl, int32_t dtype, void *stream);
+
+/*
+ * Its backward, what autograd derives for the cast, product and slice above:
+ *   dh   (g, 1, hl) of element type `dtype`, as gcg_bwd writes it
+ *   dw   out, (g, l_cache) fp32:  dw[g, k] = float(dh[g, 0, k]) * decay[g, k] for k < hl, else 0
+ */
+GCG_API int gcg_filter_decay_bwd(const void *dh, const float *decay, float *dw,
+            int32_t g, int32_t l_cache, int32_t hl, int32_t dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

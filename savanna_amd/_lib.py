@@ -27,6 +27,7 @@ EXPORTS = (
     "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_select_algo",
     "gcg_fwd_interleaved", "gcg_bwd_interleaved",
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
+    "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
 )
 
 _lock = threading.Lock()
@@ -74,6 +75,10 @@ def load() -> ctypes.CDLL:
         lib.gcg_dwconv_bwd_workspace_bytes.restype = sz
         lib.gcg_dwconv_bwd.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, vp]
         lib.gcg_dwconv_bwd.restype = ctypes.c_int
+        lib.gcg_filter_decay_fwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
+        lib.gcg_filter_decay_fwd.restype = ctypes.c_int
+        lib.gcg_filter_decay_bwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
+        lib.gcg_filter_decay_bwd.restype = ctypes.c_int
         _lib = lib
         return lib
 
@@ -265,6 +270,47 @@ def dwconv_bwd(dy, x, w):
                                 ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, st)
     check(rc, "gcg_dwconv_bwd")
     return dx, dw
+
+
+def _check_filter_params(w, decay):
+    for t in (w, decay):
+        if t.dim() != 2 or t.dtype != torch.float32 or not t.is_contiguous():
+            raise ValueError("w and decay must be contiguous fp32 (g, L_cache) tensors")
+    if w.shape != decay.shape or w.device != decay.device:
+        raise ValueError("w and decay must share shape and device")
+
+
+def filter_decay_fwd(w, decay, hl: int, dtype: torch.dtype):
+    """h (g, 1, hl) in ``dtype`` = w[:, :hl] * decay[:, :hl]."""
+    lib = load()
+    _require_gpu(w)
+    _check_filter_params(w, decay)
+    g, l_cache = w.shape
+    if not 0 < hl <= l_cache:
+        raise ValueError("hl must be in 1..L_cache")
+    h = torch.empty(g, 1, hl, dtype=dtype, device=w.device)
+    with torch.cuda.device(w.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_filter_decay_fwd(w.data_ptr(), decay.data_ptr(), h.data_ptr(), g, l_cache, hl, dtype_code(dtype), st)
+    check(rc, "gcg_filter_decay_fwd")
+    return h
+
+
+def filter_decay_bwd(dh, decay):
+    """dw (g, L_cache) fp32 from dh (g, 1, hl)."""
+    lib = load()
+    _require_gpu(dh)
+    _check_filter_params(decay, decay)
+    g, l_cache = decay.shape
+    if dh.dim() != 3 or dh.shape[0] != g or dh.shape[1] != 1 or dh.shape[2] > l_cache or not dh.is_contiguous():
+        raise ValueError("dh must be a contiguous (g, 1, hl) tensor with hl <= L_cache")
+    dw = torch.empty(g, l_cache, dtype=torch.float32, device=dh.device)
+    with torch.cuda.device(dh.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_filter_decay_bwd(dh.data_ptr(), decay.data_ptr(), dw.data_ptr(), g, l_cache, dh.shape[2],
+                                      dtype_code(dh.dtype), st)
+    check(rc, "gcg_filter_decay_bwd")
+    return dw
 
 
 def select_algo(bs, L, g, dg, hl, dtype: torch.dtype, backward=False) -> str:

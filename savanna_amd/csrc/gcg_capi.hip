@@ -95,7 +95,7 @@ GCG_API const char *gcg_strerror(int code)
 
 GCG_API int gcg_last_hip_error(void) { return tls_hip_error; }
 
-GCG_API int gcg_version(void) { return 102; }
+GCG_API int gcg_version(void) { return 103; }
 
 GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t backward)
 {
@@ -259,6 +259,28 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
     rc = check_device();
     if (rc) return rc;
     return finish(gcg::dwconv_bwd_launch(dtype, dy, x, w, dx, dw, workspace, dm, (hipStream_t)stream));
+}
+
+// ---- explicit decayed filter (Hyena-MR parametrization)
+
+GCG_API int gcg_filter_decay_fwd(const float *w, const float *decay, void *h, int32_t g, int32_t l_cache, int32_t hl,
+                                 int32_t dtype, void *stream)
+{
+    if (!w || !decay || !h || g <= 0 || hl <= 0 || l_cache < hl) return GCG_ERR_BAD_ARG;
+    if (dtype != GCG_F32 && dtype != GCG_BF16 && dtype != GCG_F16) return GCG_ERR_BAD_ARG;
+    const int rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::filter_fwd_launch(dtype, w, decay, h, g, l_cache, hl, (hipStream_t)stream));
+}
+
+GCG_API int gcg_filter_decay_bwd(const void *dh, const float *decay, float *dw, int32_t g, int32_t l_cache, int32_t hl,
+                                 int32_t dtype, void *stream)
+{
+    if (!dh || !decay || !dw || g <= 0 || hl <= 0 || l_cache < hl) return GCG_ERR_BAD_ARG;
+    if (dtype != GCG_F32 && dtype != GCG_BF16 && dtype != GCG_F16) return GCG_ERR_BAD_ARG;
+    const int rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::filter_bwd_launch(dtype, dh, decay, dw, g, l_cache, hl, (hipStream_t)stream));
 }
 
 } // extern "C"

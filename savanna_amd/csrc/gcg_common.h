@@ -221,4 +221,10 @@ size_t dwconv_bwd_workspace(const Dims &dm);
 int dwconv_bwd_launch(int dtype, const void *dy, const void *x, const void *w, void *dx, void *dw, void *ws,
                       const Dims &dm, hipStream_t st);
 
+// explicit decayed filter: h = T(w * decay) cut to hl taps, and its backward
+int filter_fwd_launch(int dtype, const float *w, const float *decay, void *h, int g, int l_cache, int hl,
+                      hipStream_t st);
+int filter_bwd_launch(int dtype, const void *dh, const float *decay, float *dw, int g, int l_cache, int hl,
+                      hipStream_t st);
+
 } // namespace gcg

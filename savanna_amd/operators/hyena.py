@@ -110,6 +110,23 @@ class ExplicitSingleDecayFilter(nn.Module):
     def forward(self, L: int) -> torch.Tensor:
         return self.h[:, :L] * self.decay[:, :L]
 
+    def fused(self, L: int, dtype: torch.dtype) -> torch.Tensor:
+        """(g, 1, L) filter in ``dtype`` for the convolution kernels: slice, product and cast in one
+        launch, and one launch for their backward (fp32 parameters on the GPU)."""
+        return _DecayedFilter.apply(self.h, self.decay, L, dtype)
+
+
+class _DecayedFilter(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, w, decay, hl, dtype):
+        ctx.save_for_backward(decay)
+        return _lib.filter_decay_fwd(w.contiguous(), decay.contiguous(), hl, dtype)
+
+    @staticmethod
+    def backward(ctx, dh):
+        (decay,) = ctx.saved_tensors
+        return _lib.filter_decay_bwd(dh.contiguous(), decay.contiguous()), None, None, None
+
 
 class _CgcgOperatorBase(nn.Module):
     def __init__(self, hidden_size: int, num_groups: int, cfg: Optional[CgcgConfig]):
@@ -172,7 +189,10 @@ class HyenaMROperator(_CgcgOperatorBase):
                                                 small_init=small_init, device=device)
 
     def _filter(self, L: int) -> torch.Tensor:
-        return self.filter(min(self.hyena_mr_len, L))[:, None]      # hyena.py:440-441, :503
+        hl = min(self.hyena_mr_len, L)                              # hyena.py:440-441, :503
+        if self.filter.h.is_cuda and self.filter.h.dtype == torch.float32:
+            return self.filter.fused(hl, self.cgcg_dtype)
+        return self.filter(hl)[:, None]
 
 
 class HyenaSEOperator(_CgcgOperatorBase):

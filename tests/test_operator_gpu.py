@@ -219,3 +219,25 @@ def test_run_short_hyena_layout(gcg_lib, repeat_interleave):
         assert_close(a.grad, r.grad, TOL_DH[torch.float32] if n == "dw" else TOL[torch.float32], n)
     with pytest.raises(AssertionError, match="Must specify"):
         run_short_hyena(*dev)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
+def test_decayed_filter_in_one_launch(gcg_lib, dtype):
+    """gcg_filter_decay_fwd / _bwd against the expression of explicit.py:68-75 followed by the
+    [:, None] and cast of hyena.py:440-441, :499-503, with autograd for the backward."""
+    from savanna_amd.operators.hyena import ExplicitSingleDecayFilter
+
+    g, l_cache, hl = 24, 160, 128
+    torch.manual_seed(41)
+    f = ExplicitSingleDecayFilter(g, l_cache, small_init=False, device=DEV)
+    h = f.fused(hl, dtype)
+    assert h.shape == (g, 1, hl) and h.dtype == dtype
+    dh = torch.randn(g, 1, hl, device=DEV).to(dtype)
+    h.backward(dh)
+    got_dw = f.h.grad.clone()
+    f.h.grad = None
+    h_ref = (f.h[:, :hl] * f.decay[:, :hl])[:, None].to(dtype)
+    h_ref.backward(dh)
+    assert torch.equal(h, h_ref)
+    assert_close(got_dw, f.h.grad, 1e-6, "dw")
+    assert not got_dw[:, hl:].any()
