@@ -241,3 +241,44 @@ def test_decayed_filter_in_one_launch(gcg_lib, dtype):
     assert torch.equal(h, h_ref)
     assert_close(got_dw, f.h.grad, 1e-6, "dw")
     assert not got_dw[:, hl:].any()
+
+
+@pytest.mark.parametrize("hl,dtype", [(7, torch.float32), (128, torch.bfloat16)])
+def test_graph_capture_of_the_feature_chain(gcg_lib, hl, dtype):
+    """Featurizer conv, interleaved operator and their backwards captured in one HIP graph and
+    replayed with new contents; every replay must equal the eager result."""
+    from savanna_amd import _lib
+
+    bs, L, g, dg = 1, 1024, 8, 16
+    raw = torch.randn(bs, L, 3 * g * dg, 1, device=DEV).to(dtype)
+    dy = torch.randn(bs, L, g, dg, device=DEV).to(dtype)
+    wf = (torch.randn(3 * g * dg, 1, 3, device=DEV) / 3 ** 0.5).to(dtype)
+    h = (torch.randn(g, 1, hl, device=DEV) / hl ** 0.5).to(dtype)
+
+    def chain(raw_t, dy_t):
+        f = _lib.dwconv_fwd(raw_t, wf)
+        feat = f.view(bs, L, g, dg, 3)
+        y = _lib.fwd_interleaved(feat, h)
+        dfeat, dh = _lib.bwd_interleaved(dy_t, feat, h)
+        draw, dwf = _lib.dwconv_bwd(dfeat.view(bs, L, 3 * g * dg, 1), raw_t, wf)
+        return y, dh, draw, dwf
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        chain(raw, dy)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs_g = chain(raw, dy)
+    for it in range(3):
+        fresh_raw, fresh_dy = torch.randn_like(raw), torch.randn_like(dy)
+        raw.copy_(fresh_raw)
+        dy.copy_(fresh_dy)
+        graph.replay()
+        torch.cuda.synchronize()
+        outs_e = chain(fresh_raw, fresh_dy)
+        torch.cuda.synchronize()
+        for a, b, n in zip(outs_g, outs_e, ("y", "dh", "d raw", "dw featurizer")):
+            assert torch.equal(a, b), f"replay {it}: {n}"
