@@ -1,0 +1,87 @@
+"""Seeded random shapes through every entry point with the kernel family chosen by the library,
+against the CPU oracle: ragged lengths, odd group widths, filters from one tap to beyond the
+matrix-core limit -- the combinations the hand-picked lists do not enumerate."""
+import random
+
+import pytest
+import torch
+
+import oracle
+from helpers import TOL, TOL_DH, assert_close
+from savanna_amd import _lib
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def _shapes(n, seed, dgs, max_hl):
+    rnd = random.Random(seed)
+    out = []
+    for _ in range(n):
+        bs, L = rnd.randint(1, 3), rnd.choice([1, 2, 7, 31, 32, 33, 64, 127, 129, 200, 511, 700])
+        g, dg = rnd.randint(1, 6), rnd.choice(dgs)
+        hl = rnd.choice([1, 2, 3, 4, 5, 7, 8, 9, 16, 31, 32, 33, 64, 100, 128, 129, 140])
+        out.append((bs, L, g, dg, min(hl, max_hl), DTYPES[rnd.randrange(3)]))
+    return out
+
+
+def _id(p):
+    bs, L, g, dg, hl, dtype = p
+    return f"{bs}x{L}x{g}x{dg}-hl{hl}-{str(dtype)[6:]}"
+
+
+def _inputs(bs, L, g, dg, hl, dtype, seed):
+    gen = torch.Generator().manual_seed(seed)
+    x, B, C = (torch.randn(bs, L, g, dg, generator=gen).to(dtype) for _ in range(3))
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen)).to(dtype)
+    h = (torch.randn(g, 1, hl, generator=gen) / hl ** 0.5).to(dtype)
+    return x, B, C, dy, h
+
+
+GATED = _shapes(48, 1, [1, 2, 4, 8, 16, 20, 32, 48], 140)
+
+
+@pytest.mark.parametrize("p", GATED, ids=[_id(p) for p in GATED])
+def test_gated_operator_random(gcg_lib, p):
+    bs, L, g, dg, hl, dtype = p
+    x, B, C, dy, h = _inputs(bs, L, g, dg, hl, dtype, seed=hash(p[:5]) & 0xffff)
+    y_ref = oracle.gcg_fwd_oracle(x.float(), B.float(), C.float(), h.float())
+    ref = oracle.gcg_bwd_oracle(dy.float(), x.float(), B.float(), C.float(), h.float())
+    xd, Bd, Cd, dyd, hd = (t.to(DEV) for t in (x, B, C, dy, h))
+    _, _, y = _lib.fwd(xd, Bd, Cd, hd)
+    got = _lib.bwd(dyd, xd, Bd, Cd, hd)
+    feat = torch.stack([Cd, Bd, xd], dim=-1).contiguous()
+    y_i = _lib.fwd_interleaved(feat, hd)
+    dfeat, dh_i = _lib.bwd_interleaved(dyd, feat, hd)
+    torch.cuda.synchronize()
+    few = bs * L * dg < 256          # a tap summed from a handful of rounded products can cancel
+    assert_close(y, y_ref, TOL[dtype], "y")
+    assert_close(y_i, y_ref, TOL[dtype], "y interleaved")
+    for o, oi, r, n in zip(got[:3], (dfeat[..., 2], dfeat[..., 1], dfeat[..., 0]), ref[:3], ("dx", "dB", "dC")):
+        assert_close(o, r, TOL[dtype], n)
+        assert_close(oi, r, TOL[dtype], n + " interleaved")
+    if not few or dtype == torch.float32:
+        assert_close(got[3], ref[3], TOL_DH[dtype], "dh")
+        assert_close(dh_i, ref[3], TOL_DH[dtype], "dh interleaved")
+
+
+FEAT = _shapes(24, 2, [1, 4, 8, 16], 8)
+
+
+@pytest.mark.parametrize("p", FEAT, ids=[_id(p) for p in FEAT])
+def test_featurizer_random(gcg_lib, p):
+    bs, L, g, dg, hl, dtype = p
+    if (g * dg) % 4:
+        g *= 4                        # the featurizer kernels take channel counts that are multiples of 4
+    x, _, _, dy, w = _inputs(bs, L, g, dg, hl, dtype, seed=hash(p[:5]) & 0xffff)
+    one = torch.ones(bs, L, g, dg)
+    y_ref = oracle.gcg_fwd_oracle(x.float(), one, one, w.float())
+    dx_ref, _, _, dw_ref = oracle.gcg_bwd_oracle(dy.float(), x.float(), one, one, w.float())
+    y = _lib.dwconv_fwd(x.to(DEV), w.to(DEV))
+    dx, dw = _lib.dwconv_bwd(dy.to(DEV), x.to(DEV), w.to(DEV))
+    torch.cuda.synchronize()
+    assert_close(y, y_ref, TOL[dtype], "y")
+    assert_close(dx, dx_ref, TOL[dtype], "dx")
+    if bs * L * dg >= 256 or dtype == torch.float32:
+        assert_close(dw, dw_ref, TOL_DH[dtype], "dw")
