@@ -103,6 +103,25 @@ def check(rc: int, what: str) -> None:
         raise GcgError(f"{what}: {msg} (code {rc}, hipError {lib.gcg_last_hip_error()})")
 
 
+class _on_device:
+    """``torch.cuda.device`` that does nothing when the tensor's device is already current (the
+    usual case): the context manager costs several microseconds, which shows at small shapes."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, device):
+        self.ctx = None if device.index == torch.cuda.current_device() else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
+
+
 def _require_gpu(t: torch.Tensor) -> None:
     if not t.is_cuda:
         raise RuntimeError(
@@ -126,7 +145,7 @@ def fwd(x, B, C, h, return_bx=False, return_y2=False, algo=ALGO_AUTO, out=None):
     bx = torch.empty_like(x) if return_bx else None
     if x.numel() == 0:
         return bx, y2, y
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_fwd(
             x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), y.data_ptr(),
@@ -152,7 +171,7 @@ def bwd(dy, x, B, C, h, algo=ALGO_AUTO):
     nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, a)
     if nbytes == 0:
         raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_bwd(
@@ -187,7 +206,7 @@ def fwd_interleaved(feat, h, algo=ALGO_AUTO, out=None):
     y = out if out is not None else torch.empty(feat.shape[:4], dtype=feat.dtype, device=feat.device)
     if y.numel() == 0:
         return y
-    with torch.cuda.device(feat.device):
+    with _on_device(feat.device):
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_fwd_interleaved(feat.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg, hl,
                                      dtype_code(feat.dtype), algo_code(algo), st)
@@ -212,7 +231,7 @@ def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO):
     nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, a)
     if nbytes == 0:
         raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")
-    with torch.cuda.device(feat.device):
+    with _on_device(feat.device):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=feat.device)
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_bwd_interleaved(dy.data_ptr(), feat.data_ptr(), h.data_ptr(), dfeat.data_ptr(), dh.data_ptr(),
@@ -239,7 +258,7 @@ def dwconv_fwd(x, w):
     y = torch.empty_like(x)
     if x.numel() == 0:
         return y
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_dwconv_fwd(x.data_ptr(), w.data_ptr(), y.data_ptr(), bs, L, g, dg, w.shape[-1],
                                 dtype_code(x.dtype), st)
@@ -263,7 +282,7 @@ def dwconv_bwd(dy, x, w):
     nbytes = lib.gcg_dwconv_bwd_workspace_bytes(bs, L, g, dg, hl, code)
     if nbytes == 0:
         check(-2, "gcg_dwconv_bwd_workspace_bytes")     # GCG_ERR_UNSUPPORTED
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_dwconv_bwd(dy.data_ptr(), x.data_ptr(), w.data_ptr(), dx.data_ptr(), dw.data_ptr(),
@@ -289,7 +308,7 @@ def filter_decay_fwd(w, decay, hl: int, dtype: torch.dtype):
     if not 0 < hl <= l_cache:
         raise ValueError("hl must be in 1..L_cache")
     h = torch.empty(g, 1, hl, dtype=dtype, device=w.device)
-    with torch.cuda.device(w.device):
+    with _on_device(w.device):
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_filter_decay_fwd(w.data_ptr(), decay.data_ptr(), h.data_ptr(), g, l_cache, hl, dtype_code(dtype), st)
     check(rc, "gcg_filter_decay_fwd")
@@ -305,7 +324,7 @@ def filter_decay_bwd(dh, decay):
     if dh.dim() != 3 or dh.shape[0] != g or dh.shape[1] != 1 or dh.shape[2] > l_cache or not dh.is_contiguous():
         raise ValueError("dh must be a contiguous (g, 1, hl) tensor with hl <= L_cache")
     dw = torch.empty(g, l_cache, dtype=torch.float32, device=dh.device)
-    with torch.cuda.device(dh.device):
+    with _on_device(dh.device):
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_filter_decay_bwd(dh.data_ptr(), decay.data_ptr(), dw.data_ptr(), g, l_cache, dh.shape[2],
                                       dtype_code(dh.dtype), st)
