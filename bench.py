@@ -337,6 +337,13 @@ def main():
             small = w.algorithmic_bytes() < (64 << 20)       # launch-bound: also report graph replay
             others[name] = time_workload(w, device, k, max(2, args.warmup // 2), graph=small)
         line["all_configs"] = others
+        # the rows next to the hot path: the operator fed from the interleaved projected features, the
+        # featurizer conv, and the two chained through autograd
+        extra = {}
+        for name in ("mr_fwdbwd_7b_interleaved", "se_fwdbwd_40b_interleaved", "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b"):
+            r = time_workload(WORKLOADS[name], device, max(5, args.steps // 3), 3)
+            extra[name] = {k: r[k] for k in ("ms_per_step", "tokens_per_s", "step_gbs", "step_hbm_frac")}
+        line["next_rows"] = extra
     if args.copy_calibration:
         src = torch.ones(256 << 20, dtype=torch.uint8, device=device)
         dst = torch.empty_like(src)
