@@ -182,6 +182,50 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
             int32_t dtype, void *stream);
 
 /*
+ * Featurizer convolution and short gated convolution in one pass: gcg_dwconv_fwd on the
+ * (bs, L, 3 * g * dg) projected features followed by gcg_fwd_interleaved on its result, without
+ * the featurized tensor ever going to memory.
+ * Replaces, for the Hyena-SE layers, the chain of ParallelSequenceMixer.forward
+ * (savanna/model/block.py:867-890: permute, ParallelCausalDepthwiseConv1d, permute, interleaved
+ * split) and ParallelShortHyenaOperator.forward with use_cgcg_short
+ * (savanna/model/operators/hyena/hyena.py:825-840 -> two_pass_chunked_gate_conv_gate).
+ *
+ *   raw    (bs, L, g, dg, 3) contiguous, i.e. (bs, L, 3 * g * dg): the dense projection's output
+ *   wf     (3 * g * dg, 1, kf): one featurizer filter per feature channel, kf <= 4
+ *   h      (g, 1, hl), hl <= 8
+ *   y      out, (bs, L, g, dg)
+ *
+ *   f[b, t, j] = dtype( sum_k wf[j, 0, k] * raw[b, t - (kf-1) + k, j] )       (fp32 accumulation)
+ *   y          = gcg_fwd_interleaved(f, h)
+ *
+ * Where the two calls it replaces run the register-window kernels (short filters at layer sizes),
+ * the result equals theirs bit for bit in fp32 and bf16.
+ * Supported: hl <= 8, kf <= 4, dg even, 16-byte aligned tensors; otherwise GCG_ERR_UNSUPPORTED.
+ */
+GCG_API int gcg_mixer_se_fwd(const void *raw, const void *wf, const void *h, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+
+/* Workspace of gcg_mixer_se_bwd (per-run partial sums of dh and dwf); 0 on invalid or unsupported arguments. */
+GCG_API size_t gcg_mixer_se_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t kf, int32_t dtype);
+
+/*
+ * Backward of gcg_mixer_se_fwd: gcg_bwd_interleaved (recomputing f from raw) followed by
+ * gcg_dwconv_bwd, in one pass; the gradient of f is rounded to `dtype` in between as when the two
+ * run separately.
+ *   dy     (bs, L, g, dg)
+ *   draw   out, (bs, L, g, dg, 3)
+ *   dwf    out, (3 * g * dg, 1, kf);  dh  out, (g, 1, hl); both overwritten, bit-reproducible
+ *   workspace  at least gcg_mixer_se_bwd_workspace_bytes(...) bytes, 256-byte aligned
+ */
+GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, const void *h,
+            void *draw, void *dwf, void *dh,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+
+/*
  * Explicit decayed filter of Hyena-MR, ready for gcg_fwd, in one launch.
  * Replaces ExplicitSingleDecayFilter.filter (savanna/model/operators/hyena/parametrization/
  * explicit.py:68-75: h = self.h[:, :L] * self.decay[:, :L]) with L = min(hyena_mr_len, seq_len),

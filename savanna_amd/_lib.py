@@ -27,6 +27,7 @@ EXPORTS = (
     "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_select_algo",
     "gcg_fwd_interleaved", "gcg_bwd_interleaved",
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
+    "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
 )
 
@@ -75,6 +76,12 @@ def load() -> ctypes.CDLL:
         lib.gcg_dwconv_bwd_workspace_bytes.restype = sz
         lib.gcg_dwconv_bwd.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, vp]
         lib.gcg_dwconv_bwd.restype = ctypes.c_int
+        lib.gcg_mixer_se_fwd.argtypes = [vp] * 4 + [i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_mixer_se_fwd.restype = ctypes.c_int
+        lib.gcg_mixer_se_bwd_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32, i32]
+        lib.gcg_mixer_se_bwd_workspace_bytes.restype = sz
+        lib.gcg_mixer_se_bwd.argtypes = [vp] * 8 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_mixer_se_bwd.restype = ctypes.c_int
         lib.gcg_filter_decay_fwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
         lib.gcg_filter_decay_fwd.restype = ctypes.c_int
         lib.gcg_filter_decay_bwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
@@ -289,6 +296,62 @@ def dwconv_bwd(dy, x, w):
                                 ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, st)
     check(rc, "gcg_dwconv_bwd")
     return dx, dw
+
+
+def _check_mixer_se(raw, wf, h):
+    if raw.dim() != 5 or raw.shape[-1] != 3 or not raw.is_contiguous():
+        raise ValueError("raw must be a contiguous (bs, L, g, dg, 3) tensor")
+    bs, L, g, dg, _ = raw.shape
+    if wf.dim() != 3 or wf.shape[0] != 3 * g * dg or wf.shape[1] != 1 or not wf.is_contiguous():
+        raise ValueError("wf must be a contiguous (3 * g * dg, 1, kf) tensor")
+    if h.dim() != 3 or h.shape[0] != g or h.shape[1] != 1 or not h.is_contiguous():
+        raise ValueError("h must be a contiguous (g, 1, hl) tensor")
+    for t in (wf, h):
+        if t.dtype != raw.dtype or t.device != raw.device:
+            raise ValueError("raw, wf and h must share dtype and device")
+
+
+def mixer_se_fwd(raw, wf, h):
+    """y (bs, L, g, dg) = fwd_interleaved(dwconv_fwd(raw, wf), h) in one pass over raw (bs, L, g, dg, 3)."""
+    lib = load()
+    _require_gpu(raw)
+    _check_mixer_se(raw, wf, h)
+    bs, L, g, dg, _ = raw.shape
+    y = torch.empty(bs, L, g, dg, dtype=raw.dtype, device=raw.device)
+    if y.numel() == 0:
+        return y
+    with _on_device(raw.device):
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_mixer_se_fwd(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg,
+                                  h.shape[-1], wf.shape[-1], dtype_code(raw.dtype), st)
+    check(rc, "gcg_mixer_se_fwd")
+    return y
+
+
+def mixer_se_bwd(dy, raw, wf, h):
+    """(draw, dwf, dh) of mixer_se_fwd."""
+    lib = load()
+    _require_gpu(raw)
+    _check_mixer_se(raw, wf, h)
+    bs, L, g, dg, _ = raw.shape
+    if dy.shape != (bs, L, g, dg) or dy.dtype != raw.dtype or not dy.is_contiguous() or dy.device != raw.device:
+        raise ValueError("dy must be a contiguous (bs, L, g, dg) tensor of raw's dtype and device")
+    hl, kf = h.shape[-1], wf.shape[-1]
+    draw, dwf, dh = torch.empty_like(raw), torch.empty_like(wf), torch.empty_like(h)
+    if raw.numel() == 0:
+        return draw, dwf.zero_(), dh.zero_()
+    code = dtype_code(raw.dtype)
+    nbytes = lib.gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code)
+    if nbytes == 0:
+        check(-2, "gcg_mixer_se_bwd_workspace_bytes")     # GCG_ERR_UNSUPPORTED
+    with _on_device(raw.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
+        st = torch.cuda.current_stream().cuda_stream
+        rc = lib.gcg_mixer_se_bwd(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
+                                  dwf.data_ptr(), dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl, kf,
+                                  code, st)
+    check(rc, "gcg_mixer_se_bwd")
+    return draw, dwf, dh
 
 
 def _check_filter_params(w, decay):

@@ -95,7 +95,7 @@ GCG_API const char *gcg_strerror(int code)
 
 GCG_API int gcg_last_hip_error(void) { return tls_hip_error; }
 
-GCG_API int gcg_version(void) { return 103; }
+GCG_API int gcg_version(void) { return 104; }
 
 GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t backward)
 {
@@ -259,6 +259,47 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
     rc = check_device();
     if (rc) return rc;
     return finish(gcg::dwconv_bwd_launch(dtype, dy, x, w, dx, dw, workspace, dm, (hipStream_t)stream));
+}
+
+// ---- featurizer + Hyena-SE operator in one pass
+
+GCG_API int gcg_mixer_se_fwd(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L, int32_t g,
+                             int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    if (!raw || !wf || !h || !y) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    if (kf <= 0) return GCG_ERR_BAD_ARG;
+    if (!gcg::mixer_se_supported(dm, kf) || !all_aligned16({raw, y})) return GCG_ERR_UNSUPPORTED;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::mixer_se_fwd_launch(dtype, raw, wf, h, y, dm, kf, (hipStream_t)stream));
+}
+
+GCG_API size_t gcg_mixer_se_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+                                                int32_t dtype)
+{
+    gcg::Dims dm;
+    if (make_dims(bs, L, g, dg, hl, dtype, &dm) || kf <= 0 || !gcg::mixer_se_supported(dm, kf)) return 0;
+    return (gcg::mixer_se_bwd_workspace(dtype, dm, kf) + 255) & ~(size_t)255;
+}
+
+GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf,
+                             void *dh, void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g,
+                             int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    if (!dy || !raw || !wf || !h || !draw || !dwf || !dh) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    if (kf <= 0) return GCG_ERR_BAD_ARG;
+    if (!gcg::mixer_se_supported(dm, kf) || !all_aligned16({dy, raw, draw})) return GCG_ERR_UNSUPPORTED;
+    const size_t need = gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, dtype);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::mixer_se_bwd_launch(dtype, dy, raw, wf, h, draw, dwf, dh, workspace, dm, kf, (hipStream_t)stream));
 }
 
 // ---- explicit decayed filter (Hyena-MR parametrization)

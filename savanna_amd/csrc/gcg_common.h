@@ -167,12 +167,6 @@ struct Dims {
 
 constexpr int kWave = 64;
 
-
-// interleaved operands: feat / dfeat are (bs, L, g, dg, 3) with [..., 0] = C, [..., 1] = B, [..., 2] = x
-int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st);
-int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
-                       void *ws, const Dims &dm, hipStream_t st);
-
 } // namespace gcg
 
 // Host-side launchers, one translation unit per kernel family.  Each returns a
@@ -203,12 +197,6 @@ int mfma_bwd_launch(int dtype, const void *dy, const void *x, const void *B, con
                     const void *h, void *dx, void *dB, void *dC, void *dh, void *ws,
                     const Dims &dm, hipStream_t st);
 
-
-// interleaved operands: feat / dfeat are (bs, L, g, dg, 3) with [..., 0] = C, [..., 1] = B, [..., 2] = x
-int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st);
-int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
-                       void *ws, const Dims &dm, hipStream_t st);
-
 // interleaved operands: feat / dfeat are (bs, L, g, dg, 3) with [..., 0] = C, [..., 1] = B, [..., 2] = x
 int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st);
 int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
@@ -220,6 +208,14 @@ int dwconv_fwd_launch(int dtype, const void *x, const void *w, void *y, const Di
 size_t dwconv_bwd_workspace(const Dims &dm);
 int dwconv_bwd_launch(int dtype, const void *dy, const void *x, const void *w, void *dx, void *dw, void *ws,
                       const Dims &dm, hipStream_t st);
+
+// featurizer and Hyena-SE operator in one pass: raw / draw are (bs, L, g, dg, 3), wf (3 * g * dg, 1, kf)
+bool mixer_se_supported(const Dims &dm, int kf);
+int mixer_se_fwd_launch(int dtype, const void *raw, const void *wf, const void *h, void *y, const Dims &dm, int kf,
+                        hipStream_t st);
+size_t mixer_se_bwd_workspace(int dtype, const Dims &dm, int kf);
+int mixer_se_bwd_launch(int dtype, const void *dy, const void *raw, const void *wf, const void *h, void *draw,
+                        void *dwf, void *dh, void *ws, const Dims &dm, int kf, hipStream_t st);
 
 // explicit decayed filter: h = T(w * decay) cut to hl taps, and its backward
 int filter_fwd_launch(int dtype, const float *w, const float *decay, void *h, int g, int l_cache, int hl,

@@ -1,0 +1,133 @@
+"""Featurizer conv + short gated convolution in one pass (gcg_mixer_se_fwd / gcg_mixer_se_bwd) through the
+C ABI: against the chain of entry points it replaces (gcg_dwconv_* and gcg_*_interleaved, bit for bit
+where the arithmetic is the same) and against the CPU oracle applied twice, which follows
+block.py:867-890 and hyena.py:825-840 of the reference."""
+import pytest
+import torch
+
+import oracle
+from helpers import TOL, TOL_DH, assert_close
+from savanna_amd import _lib
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+# (bs, L, g, dg, hl, kf)
+SHAPES = [
+    (2, 64, 4, 16, 7, 3),        # Hyena-SE: 7 taps after a 3-tap featurizer
+    (1, 300, 3, 8, 7, 3),        # ragged length, three runs
+    (2, 77, 2, 2, 4, 4),
+    (1, 1, 8, 2, 7, 3),          # a single row
+    (1, 5, 1, 4, 8, 4),
+    (1, 513, 2, 16, 3, 2),
+    (3, 129, 5, 6, 7, 1),        # featurizer of one tap: a per-channel scale
+    (1, 1000, 6, 10, 5, 3),
+    (2, 256, 130, 4, 7, 3),      # more lanes than one workgroup
+    (1, 40, 2, 6, 1, 3),         # operator of one tap
+]
+
+
+def data(bs, L, g, dg, hl, kf, dtype, seed):
+    gen = torch.Generator().manual_seed(seed)
+    raw = torch.randn(bs, L, g, dg, 3, generator=gen).to(dtype)
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen)).to(dtype)
+    wf = (torch.randn(3 * g * dg, 1, kf, generator=gen) / kf ** 0.5).to(dtype)
+    h = (torch.randn(g, 1, hl, generator=gen) / hl ** 0.5).to(dtype)
+    return raw, dy, wf, h
+
+
+def oracle_chain(raw, dy, wf, h, dtype):
+    """fp32 oracle of featurizer -> round to dtype -> gated convolution, and its backward with the
+    gradient of the features rounded to dtype in between, as the chain of kernels stores it."""
+    bs, L, g, dg, _ = raw.shape
+    r4 = raw.float().reshape(bs, L, 3 * g * dg, 1)
+    one = torch.ones_like(r4)
+    f = oracle.gcg_fwd_oracle(r4, one, one, wf.float()).to(dtype).float().reshape(bs, L, g, dg, 3)
+    C, B, x = f[..., 0].contiguous(), f[..., 1].contiguous(), f[..., 2].contiguous()
+    y = oracle.gcg_fwd_oracle(x, B, C, h.float())
+    dx, dB, dC, dh = oracle.gcg_bwd_oracle(dy.float(), x, B, C, h.float())
+    df = torch.stack([dC, dB, dx], dim=-1).to(dtype).float().reshape(bs, L, 3 * g * dg, 1)
+    draw, _, _, dwf = oracle.gcg_bwd_oracle(df, r4, one, one, wf.float())
+    return y, draw.reshape(raw.shape), dwf, dh
+
+
+def kernel_chain(raw, dy, wf, h):
+    bs, L, g, dg, _ = raw.shape
+    r4 = raw.view(bs, L, 3 * g * dg, 1)
+    f = _lib.dwconv_fwd(r4, wf).view(bs, L, g, dg, 3)
+    y = _lib.fwd_interleaved(f, h)
+    df, dh = _lib.bwd_interleaved(dy, f, h)
+    draw, dwf = _lib.dwconv_bwd(df.view(bs, L, 3 * g * dg, 1), r4, wf)
+    return y, draw.view(raw.shape), dwf, dh
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
+@pytest.mark.parametrize("bs,L,g,dg,hl,kf", SHAPES)
+def test_mixer_se_fwd_bwd(gcg_lib, bs, L, g, dg, hl, kf, dtype):
+    raw, dy, wf, h = data(bs, L, g, dg, hl, kf, dtype, seed=L + hl)
+    ref = oracle_chain(raw, dy, wf, h, dtype)
+    rawd, dyd, wfd, hd = (t.to(DEV) for t in (raw, dy, wf, h))
+    y = _lib.mixer_se_fwd(rawd, wfd, hd)
+    draw, dwf, dh = _lib.mixer_se_bwd(dyd, rawd, wfd, hd)
+    torch.cuda.synchronize()
+    assert y.shape == (bs, L, g, dg) and draw.shape == raw.shape and dwf.shape == wf.shape and dh.shape == h.shape
+    # two rounded stages back to back: the gradient's tolerance is twice the single-stage one
+    assert_close(y, ref[0], TOL[dtype], "y")
+    assert_close(draw, ref[1], 2 * TOL[dtype], "d raw")
+    if bs * L * dg >= 256 or dtype == torch.float32:      # a tap summed from a handful of rounded terms can cancel
+        assert_close(dwf, ref[2], 2 * TOL_DH[dtype], "dwf")
+        assert_close(dh, ref[3], TOL_DH[dtype], "dh")
+    if (3 * g * dg) % 4 == 0:                              # the stand-alone featurizer takes multiples of 4 channels
+        y_c, draw_c, dwf_c, dh_c = kernel_chain(rawd, dyd, wfd, hd)
+        torch.cuda.synchronize()
+        # the chain may run another kernel family for this shape (another summation order), so bitwise
+        # equality is asserted only at the layer shape below, where both walk rows in registers
+        assert_close(y, y_c, 1e-5 if dtype == torch.float32 else TOL[dtype], "y vs chain")
+        assert_close(draw, draw_c, 1e-5 if dtype == torch.float32 else TOL[dtype], "d raw vs chain")
+        if bs * L * dg >= 256 or dtype == torch.float32:
+            assert_close(dwf, dwf_c, TOL_DH[dtype], "dwf vs chain")
+            assert_close(dh, dh_c, TOL_DH[dtype], "dh vs chain")
+
+
+def test_mixer_se_is_deterministic_and_rejects_what_it_cannot_run(gcg_lib):
+    raw, dy, wf, h = (t.to(DEV) for t in data(2, 512, 8, 16, 7, 3, torch.bfloat16, seed=1))
+    a, b = _lib.mixer_se_bwd(dy, raw, wf, h), _lib.mixer_se_bwd(dy, raw, wf, h)
+    assert all(torch.equal(p, q) for p, q in zip(a, b))
+    raw9, dy9, wf9, h9 = (t.to(DEV) for t in data(1, 64, 8, 2, 9, 3, torch.float32, seed=2))      # 9 taps
+    with pytest.raises(_lib.GcgError, match="not supported"):
+        _lib.mixer_se_fwd(raw9, wf9, h9)
+    raw5, dy5, wf5, h5 = (t.to(DEV) for t in data(1, 64, 8, 2, 7, 5, torch.float32, seed=2))      # 5 featurizer taps
+    with pytest.raises(_lib.GcgError, match="not supported"):
+        _lib.mixer_se_bwd(dy5, raw5, wf5, h5)
+    raw3, _, wf3, h3 = (t.to(DEV) for t in data(1, 64, 8, 3, 7, 3, torch.float32, seed=2))        # odd group width
+    with pytest.raises(_lib.GcgError, match="not supported"):
+        _lib.mixer_se_fwd(raw3, wf3, h3)
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        _lib.mixer_se_fwd(raw.cpu(), wf.cpu(), h.cpu())
+
+
+def test_mixer_se_shape_of_a_40b_layer(gcg_lib):
+    """B=1, L=8192, 8192 channels in 256 groups, 7 taps after 3, bf16: equal to the chain of kernels
+    bit for bit, and a shift featurizer with a one-tap operator reproduces products of the input."""
+    bs, L, g, dg, hl, kf, dtype = 1, 8192, 256, 32, 7, 3, torch.bfloat16
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    raw = torch.randn(bs, L, g, dg, 3, generator=gen, device=DEV).to(dtype)
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen, device=DEV)).to(dtype)
+    wf = (torch.randn(3 * g * dg, 1, kf, generator=gen, device=DEV) / kf ** 0.5).to(dtype)
+    h = (torch.randn(g, 1, hl, generator=gen, device=DEV) / hl ** 0.5).to(dtype)
+    y = _lib.mixer_se_fwd(raw, wf, h)
+    draw, dwf, dh = _lib.mixer_se_bwd(dy, raw, wf, h)
+    y_c, draw_c, dwf_c, dh_c = kernel_chain(raw, dy, wf, h)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_c) and torch.equal(draw, draw_c)
+    assert_close(dwf, dwf_c, TOL_DH[dtype], "dwf")
+    assert_close(dh, dh_c, TOL_DH[dtype], "dh")
+    # featurizer = delay by one row, operator = delay by two: y[t] = C[t-1] * (B * x)[t-3]
+    wf.zero_(); wf[:, 0, 1] = 1.0
+    h.zero_(); h[:, 0, hl - 3] = 1.0
+    y = _lib.mixer_se_fwd(raw, wf, h)
+    torch.cuda.synchronize()
+    C, B, x = raw[..., 0].float(), raw[..., 1].float(), raw[..., 2].float()
+    want = (C[:, 2:-1] * (B[:, :-3] * x[:, :-3])).to(dtype)
+    assert torch.equal(y[:, 3:], want) and not y[:, :3].any()
