@@ -198,8 +198,8 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
  *   f[b, t, j] = dtype( sum_k wf[j, 0, k] * raw[b, t - (kf-1) + k, j] )       (fp32 accumulation)
  *   y          = gcg_fwd_interleaved(f, h)
  *
- * Where the two calls it replaces run the register-window kernels (short filters at layer sizes),
- * the result equals theirs bit for bit in fp32 and bf16.
+ * The result equals that of the two calls it replaces up to the rounding of the fp32 sums (the
+ * taps are added in another order).
  * Supported: hl <= 8, kf <= 4, dg even, 16-byte aligned tensors; otherwise GCG_ERR_UNSUPPORTED.
  */
 GCG_API int gcg_mixer_se_fwd(const void *raw, const void *wf, const void *h, void *y,

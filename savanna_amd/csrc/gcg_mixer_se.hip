@@ -23,7 +23,17 @@ namespace {
 #define MIXER_WPE 2               // waves per SIMD the backward is compiled for (its register budget)
 #endif
 constexpr int BATCH = 4;          // rows fetched together
+#ifndef MIXER_BATCH16
+#define MIXER_BATCH16 2
+#endif
+constexpr int BATCH16 = MIXER_BATCH16;   // the same in the 16-bit backward, whose registers are scarce
 constexpr int KF_MAX = 4;         // featurizer taps: kernels are built for 3 and 4 (shorter filters are zero-padded)
+
+// x if the wave-uniform condition holds, else +0: as a bit mask, which stays one VALU operation with a
+// scalar operand (written as a select, the compiler may turn a uniform condition into a branch
+// around the row's work, and a branch costs the exact wait counts of the straight-line walk)
+__device__ __forceinline__ uint32_t keep_mask(bool uniform_cond) { return uniform_cond ? 0xffffffffu : 0u; }
+__device__ __forceinline__ float keep(float x, uint32_t m) { return __uint_as_float(__float_as_uint(x) & m); }
 
 struct MixPlan { int ch, nvec, nseg, ts, ncvb, threads; int64_t nrows, nwg; };
 
@@ -49,15 +59,6 @@ template <typename T> struct Piece {
             const u32x3 p = pack(f);
             unpack(p, f);
         }
-    }
-    // The same words, but as values the compiler cannot trace back: a second unpack of a row kept in
-    // a ring is then done where it is written, instead of the first unpack's floats being kept
-    // alive for as many rows as the ring is deep (which costs twice the registers at 16 bits).
-    static __device__ __forceinline__ u32x3 reread(const u32x3 &p)
-    {
-        uint32_t a = p[0], b = p[1], c = p[2];
-        asm volatile("" : "+v"(a), "+v"(b), "+v"(c));
-        return u32x3{a, b, c};
     }
     static __device__ __forceinline__ uint32_t pack_unit(const float (&f)[CH]) { return Word<T>::pack(f); }
     static __device__ __forceinline__ void unpack_unit(uint32_t w, float (&f)[CH]) { Word<T>::unpack(w, f); }
@@ -105,7 +106,7 @@ __device__ __forceinline__ void featurize_packed(const float (&wfr)[KF][Piece<T>
 #pragma unroll
     for (int j = KF - 1; j >= 0; --j) {
         float r[Piece<T>::E];
-        Piece<T>::unpack(j ? Piece<T>::reread(rp[(s - j) & 15]) : rp[(s - j) & 15], r);
+        Piece<T>::unpack(rp[(s - j) & 15], r);
 #pragma unroll
         for (int e = 0; e < Piece<T>::E; ++e) f[e] = fmaf(wfr[j][e], r[e], f[e]);
     }
@@ -300,14 +301,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
                     rp[k & 15] = in[kk];
                     featurize_packed<T, KF>(wfr, rp, k & 15, f);
                     P::unpack_unit(dyr[kk], dyf);
-                    const bool live = t < t_df;         // rows whose d f is wanted (uniform)
-                    const bool in_run = t < t_end;      // rows whose filter-gradient terms are ours
+                    const uint32_t live = keep_mask(t < t_df);       // rows whose d f is wanted
+                    const uint32_t in_run = keep_mask(t < t_end);    // rows whose filter-gradient terms are ours
 #pragma unroll
                     for (int ch = 0; ch < CH; ++ch) {
                         xv[ch] = f[3 * ch + 2];
                         Bv[ch] = f[3 * ch + 1];
                         gr[k & 7][ch] = dyf[ch] * f[3 * ch];
-                        ur[k & 7][ch] = live ? Bv[ch] * xv[ch] : 0.f;
+                        ur[k & 7][ch] = keep(Bv[ch] * xv[ch], live);
                     }
                     xs[k & 7] = P::pack_unit(xv);
                     Bs[k & 7] = P::pack_unit(Bv);
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
                         for (int ch = 0; ch < CH; ++ch) {
                             const float u = ur[(k - j) & 7][ch];
                             y2v[ch] = fmaf(hr[j], u, y2v[ch]);
-                            sacc = fmaf(in_run ? gr[k & 7][ch] : 0.f, u, sacc);
+                            sacc = fmaf(keep(gr[k & 7][ch], in_run), u, sacc);
                         }
                         dha[j] += sacc;
                     }
@@ -343,23 +344,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
                     P::unpack_unit(xs[k1 & 7], xo);
                     P::unpack_unit(Bs[k1 & 7], Bo);
                     P::unpack_unit(dCs[k1 & 7], dCo);
-                    const bool have = t1 >= t_start && t1 < t_df;          // uniform; outside, d f counts as zero
+                    const uint32_t have = keep_mask(t1 >= t_start && t1 < t_df);     // outside, d f counts as zero
 #pragma unroll
                     for (int ch = 0; ch < CH; ++ch) {
-                        df[3 * ch] = have ? dCo[ch] : 0.f;
-                        df[3 * ch + 1] = have ? du[ch] * xo[ch] : 0.f;
-                        df[3 * ch + 2] = have ? du[ch] * Bo[ch] : 0.f;
+                        const float duv = keep(du[ch], have);
+                        df[3 * ch] = keep(dCo[ch], have);
+                        df[3 * ch + 1] = duv * xo[ch];
+                        df[3 * ch + 2] = duv * Bo[ch];
                     }
                     const u32x3 dfp = P::pack(df);
                     P::unpack(dfp, df);
                     // featurizer filter gradient: dwf[.., KF-1-j] += d f[t1] * raw[t1 - j], rows of the run only
-                    const bool mine = t1 >= t_start && t1 < t_end;
+                    const uint32_t mine = keep_mask(t1 >= t_start && t1 < t_end);
                     float rj[E];
 #pragma unroll
                     for (int j = 0; j < KF; ++j) {
-                        P::unpack(P::reread(rp[(k1 - j) & 15]), rj);
+                        P::unpack(rp[(k1 - j) & 15], rj);
 #pragma unroll
-                        for (int e = 0; e < E; ++e) dwa[j][e] = fmaf(mine ? df[e] : 0.f, rj[e], dwa[j][e]);
+                        for (int e = 0; e < E; ++e) dwa[j][e] = fmaf(keep(df[e], mine), rj[e], dwa[j][e]);
                     }
                     dfr[k1 & 3] = dfp;
                 }
@@ -372,12 +374,405 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
 #pragma unroll
                     for (int j = 0; j < KF; ++j) {
                         float dfj[E];
-                        P::unpack(P::reread(dfr[(k2 + j) & 3]), dfj);
+                        P::unpack(dfr[(k2 + j) & 3], dfj);
 #pragma unroll
                         for (int e = 0; e < E; ++e) dr[e] = fmaf(wfr[j][e], dfj[e], dr[e]);
                     }
                     win_store(wdr, lane_i + (uint32_t)(t - D1 - D2 - t_start) * irow, P::pack(dr));
                 }
+            }
+        }
+    }
+    // partials: ws_h[tap][(batch, run)][lane], ws_w[tap][(batch, run)][feature channel]
+    const int64_t prow = b * pl.nseg + seg;
+#pragma unroll
+    for (int j = 0; j < HL; ++j)
+        if (j < hl) ws_h[((size_t)(hl - 1 - j) * pl.nrows + prow) * pl.nvec + cv] = dha[j];
+#pragma unroll
+    for (int j = 0; j < KF; ++j)
+        if (j < kf) {
+            float *dst = ws_w + ((size_t)(kf - 1 - j) * pl.nrows + prow) * (3 * d) + 3 * c;
+#pragma unroll
+            for (int e = 0; e < E; ++e) dst[e] = dwa[j][e];
+        }
+}
+
+// ------------------------------------------------------------- 16-bit elements: taps two at a time
+// At 16 bits a lane's 12-byte piece holds six feature channels, and unpacking them to floats for
+// every tap makes the walk arithmetic-bound.  v_dot2c_f32_{bf16,f16} takes two 16-bit products
+// per operand word and adds them to an fp32 accumulator, so the featurizer's sums along time are
+// done on words that hold one channel's samples of two consecutive rows: v_perm_b32 builds such a
+// word from the words of the two rows, and the packed taps (Wa: taps 0 and 1 rows back, Wb: 2 and 3)
+// stay in 12 registers.  The same words serve the three sums along time of the backward (f, d raw, dwf).
+template <typename T> struct Pair;
+template <> struct Pair<bf16_t> {
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c)
+    {
+        typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+        v2 x, y;
+        __builtin_memcpy(&x, &a, 4);
+        __builtin_memcpy(&y, &b, 4);
+        return __builtin_amdgcn_fdot2_f32_bf16(x, y, c, false);
+    }
+    // Both floats converted as one vector: written as two scalar casts put into a vector, the
+    // compiler keeps the two bf16 apart, one 32-bit register each, wherever the word is later
+    // assembled into another by halves, and every ring of such words then costs twice its registers.
+    // (Not inline assembly: the compiler must see which instructions read the result of a dot
+    // product, because it has to space them from it.)
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi)
+    {
+        typedef __bf16 bv2 __attribute__((ext_vector_type(2)));
+        typedef float fv2 __attribute__((ext_vector_type(2)));
+        const bv2 r = __builtin_convertvector(fv2{lo, hi}, bv2);
+        uint32_t u;
+        __builtin_memcpy(&u, &r, 4);
+        return u;
+    }
+};
+template <> struct Pair<f16_t> {
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c)
+    {
+        typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+        v2 x, y;
+        __builtin_memcpy(&x, &a, 4);
+        __builtin_memcpy(&y, &b, 4);
+        return __builtin_amdgcn_fdot2(x, y, c, false);
+    }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
+};
+// a row of six floats / a pair of floats as elements of T
+template <typename T> __device__ __forceinline__ u32x3 pack6(const float (&f)[6])
+{
+    return u32x3{Pair<T>::pack2(f[0], f[1]), Pair<T>::pack2(f[2], f[3]), Pair<T>::pack2(f[4], f[5])};
+}
+// p[e] = (low half: row `lo`'s sample of feature channel e, high half: row `hi`'s)
+__device__ __forceinline__ void pair_rows(const u32x3 &lo, const u32x3 &hi, uint32_t (&p)[6])
+{
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+        p[2 * i] = __builtin_amdgcn_perm(hi[i], lo[i], 0x05040100u);
+        p[2 * i + 1] = __builtin_amdgcn_perm(hi[i], lo[i], 0x07060302u);
+    }
+}
+// word whose low half is half hx of x and whose high half is half hy of y
+template <int HX, int HY> __device__ __forceinline__ uint32_t halves(uint32_t x, uint32_t y)
+{
+    constexpr uint32_t sel = (2u * HX) | ((2u * HX + 1u) << 8) | ((4u + 2u * HY) << 16) | ((5u + 2u * HY) << 24);
+    return __builtin_amdgcn_perm(y, x, sel);
+}
+// packed taps of a lane: Wa[e] = (tap 0 rows back, tap 1 row back), Wb[e] = (2 back, 3 back); hr as above
+template <typename T, int HL>
+__device__ __forceinline__ void load_taps16(const T *wf, const T *h, int64_t c, const Dims &dm, int kf,
+                                            uint32_t (&Wa)[6], uint32_t (&Wb)[6], float (&hr)[HL])
+{
+#pragma unroll
+    for (int e = 0; e < 6; ++e) {
+        const T *wp = wf + (3 * c + e) * kf;
+        float w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) w[j] = (j < kf) ? Elem<T>::load(wp + kf - 1 - j) : 0.f;
+        Wa[e] = Word<T>::pack(&w[0]);
+        Wb[e] = Word<T>::pack(&w[2]);
+    }
+    const T *hg = h + (c / dm.dg) * dm.hl;
+#pragma unroll
+    for (int j = 0; j < HL; ++j) hr[j] = (j < dm.hl) ? Elem<T>::load(hg + dm.hl - 1 - j) : 0.f;
+}
+// f of row t from pe_t = pair_rows(raw[t], raw[t-1]) and pe_t2 = pair_rows(raw[t-2], raw[t-3]), rounded to T
+// (fp: the same row as elements of T)
+template <typename T>
+__device__ __forceinline__ void featurize16(const uint32_t (&Wa)[6], const uint32_t (&Wb)[6], const uint32_t (&pe_t)[6],
+                                            const uint32_t (&pe_t2)[6], float (&f)[6], u32x3 &fp)
+{
+#pragma unroll
+    for (int e = 0; e < 6; ++e) f[e] = Pair<T>::dot2(pe_t[e], Wa[e], Pair<T>::dot2(pe_t2[e], Wb[e], 0.f));
+    fp = pack6<T>(f);
+    Piece<T>::unpack(fp, f);
+}
+template <typename T>
+__device__ __forceinline__ void featurize16(const uint32_t (&Wa)[6], const uint32_t (&Wb)[6], const uint32_t (&pe_t)[6],
+                                            const uint32_t (&pe_t2)[6], float (&f)[6])
+{
+    u32x3 fp;
+    featurize16<T>(Wa, Wb, pe_t, pe_t2, f, fp);
+}
+
+template <typename T, int HL>
+__global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict__ raw, const T *__restrict__ wf,
+                                                             const T *__restrict__ h, T *__restrict__ y, Dims dm,
+                                                             int kf, MixPlan pl)
+{
+    typedef Piece<T> P;
+    constexpr int ES = 2, CH = 2, NH = HL - 1 + 3;
+    int64_t wg = blockIdx.x;
+    const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
+    const int seg = (int)(wg % pl.nseg);
+    const int64_t b = wg / pl.nseg;
+    const int cv = cvb * (int)blockDim.x + (int)threadIdx.x;
+    if (cv >= pl.nvec) return;
+    const int64_t L = dm.L, d = dm.d, c = (int64_t)cv * CH;
+
+    uint32_t Wa[6], Wb[6];
+    float hr[HL];
+    load_taps16<T, HL>(wf, h, c, dm, kf, Wa, Wb, hr);
+
+    const int64_t t_start = (int64_t)seg * pl.ts;
+    const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
+    const int64_t t0 = t_start - NH > 0 ? t_start - NH : 0;
+    const uint32_t orow = (uint32_t)(d * ES), irow = 3 * orow;
+    const win_t wr = make_window(raw + 3 * (b * L + t0) * d, (t_end - t0) * irow);
+    const win_t wy = make_window(y + (b * L + t_start) * d, (t_end - t_start) * orow);
+    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = 3 * lane_o;
+    auto load_raw = [&](int64_t t) { return win_load<u32x3>(wr, lane_i + (uint32_t)(t - t0) * irow); };
+
+    // pe[row & 3] = pair_rows(raw[row], raw[row - 1]); ur[row & 7] = u of the row
+    uint32_t pe[4][6];
+    float ur[8][CH];
+    u32x3 prev = u32x3{0u, 0u, 0u};
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int e = 0; e < 6; ++e) pe[s][e] = 0u;
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) ur[s][ch] = 0.f;
+
+    // halo: HL-1 rows of u before the run, and three more rows of raw before those for their f
+    {
+        u32x3 hp[NH];
+#pragma unroll
+        for (int i = 1; i <= NH; ++i) hp[i - 1] = load_raw(t_start - i);
+#pragma unroll
+        for (int i = NH; i >= 1; --i) {
+            pair_rows(hp[i - 1], prev, pe[(-i) & 3]);
+            prev = hp[i - 1];
+            if (i <= HL - 1) {
+                float f[6];
+                featurize16<T>(Wa, Wb, pe[(-i) & 3], pe[(-i - 2) & 3], f);
+#pragma unroll
+                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+            }
+        }
+    }
+
+    u32x3 in[2][BATCH];
+#pragma unroll
+    for (int kk = 0; kk < BATCH; ++kk) in[0][kk] = load_raw(t_start + kk);
+    for (int64_t tb = t_start; tb < t_end; tb += 8) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int cur = half, nxt = half ^ 1;
+#pragma unroll
+            for (int kk = 0; kk < BATCH; ++kk) in[nxt][kk] = load_raw(tb + (half + 1) * BATCH + kk);
+#pragma unroll
+            for (int kk = 0; kk < BATCH; ++kk) {
+                const int k = half * BATCH + kk;
+                float f[6], out[CH];
+                pair_rows(in[cur][kk], prev, pe[k & 3]);
+                prev = in[cur][kk];
+                featurize16<T>(Wa, Wb, pe[k & 3], pe[(k - 2) & 3], f);
+#pragma unroll
+                for (int ch = 0; ch < CH; ++ch) {
+                    ur[k][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                    float acc = 0.f;
+#pragma unroll
+                    for (int j = HL - 1; j >= 0; --j) acc = fmaf(hr[j], ur[(k - j) & 7][ch], acc);
+                    out[ch] = f[3 * ch] * acc;
+                }
+                win_store(wy, lane_o + (uint32_t)(tb + k - t_start) * orow, Pair<T>::pack2(out[0], out[1]));
+            }
+        }
+    }
+}
+
+// The backward walk above with the featurizer's three sums done two taps (or two rows) at a time.
+// d raw lags d f by three rows whatever the filter length (the fourth tap is zero for shorter filters).
+template <typename T, int HL, int KF>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE)))
+void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, const T *__restrict__ wf,
+                           const T *__restrict__ h, T *__restrict__ draw, float *__restrict__ ws_h,
+                           float *__restrict__ ws_w, Dims dm, int kf, MixPlan pl)
+{
+    typedef Piece<T> P;
+    constexpr int ES = 2, CH = 2, E = 6, D1 = HL - 1, D2 = 3, NH = D1 + D2;
+    int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;
+    const int seg = (int)(wg % pl.nseg);
+    const int64_t b = wg / pl.nseg;
+    const int cv = cvb * (int)blockDim.x + (int)threadIdx.x;
+    if (cv >= pl.nvec) return;
+    const int64_t L = dm.L, d = dm.d, c = (int64_t)cv * CH;
+    const int hl = dm.hl;
+
+    uint32_t Wa[6], Wb[6];
+    float hr[HL];
+    load_taps16<T, HL>(wf, h, c, dm, kf, Wa, Wb, hr);
+
+    const int64_t t_start = (int64_t)seg * pl.ts;
+    const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
+    const int64_t t_stop = t_end + NH;
+    const int64_t t0 = t_start - NH > 0 ? t_start - NH : 0;
+    const int64_t t_far = t_stop < L ? t_stop : L;
+    const uint32_t orow = (uint32_t)(d * ES), irow = 3 * orow;
+    const win_t wr = make_window(raw + 3 * (b * L + t0) * d, (t_far - t0) * irow);
+    const win_t wdy = make_window(dy + (b * L + t0) * d, (t_far - t0) * orow);
+    const win_t wdr = make_window(draw + 3 * (b * L + t_start) * d, (t_end - t_start) * irow);
+    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = 3 * lane_o;
+
+    // rings, slot = row & (size-1): rp raw rows as loaded; pe = pair_rows(raw[row], raw[row-1]);
+    // ur u; gr g2; xs / Bs / dCs f's x, B and dC as elements of T; pd = pair_rows(d f[row-1], d f[row])
+    float ur[8][CH], gr[8][CH], dha[HL], dwa[KF][E];
+    u32x3 rp[16], dfprev = u32x3{0u, 0u, 0u};
+    uint32_t pe[4][6], pd[4][6], xs[8], Bs[8], dCs[8];
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int e = 0; e < 6; ++e) { pe[s][e] = 0u; pd[s][e] = 0u; }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        xs[s] = 0u; Bs[s] = 0u; dCs[s] = 0u;
+#pragma unroll
+        for (int ch = 0; ch < CH; ++ch) { ur[s][ch] = 0.f; gr[s][ch] = 0.f; }
+    }
+#pragma unroll
+    for (int s = 0; s < 16; ++s) rp[s] = u32x3{0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < HL; ++j) dha[j] = 0.f;
+#pragma unroll
+    for (int j = 0; j < KF; ++j)
+#pragma unroll
+        for (int e = 0; e < E; ++e) dwa[j][e] = 0.f;
+
+    // halo on the left (t_start is a multiple of 16)
+    {
+        u32x3 hp[NH];
+#pragma unroll
+        for (int i = 1; i <= NH; ++i) hp[i - 1] = win_load<u32x3>(wr, lane_i + (uint32_t)(t_start - i - t0) * irow);
+#pragma unroll
+        for (int i = NH; i >= 1; --i) {
+            rp[(-i) & 15] = hp[i - 1];
+            pair_rows(rp[(-i) & 15], rp[(-i - 1) & 15], pe[(-i) & 3]);
+            if (i <= D1) {
+                float f[E];
+                featurize16<T>(Wa, Wb, pe[(-i) & 3], pe[(-i - 2) & 3], f);
+#pragma unroll
+                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+            }
+        }
+    }
+
+    // rows are counted from the run's start in the walk: 32-bit scalars for offsets and bounds
+    const int n_run = (int)(t_end - t_start), n_df = n_run + D2, n_stop = n_run + NH;
+    const uint32_t in0 = lane_i + (uint32_t)(t_start - t0) * irow, dy0 = lane_o + (uint32_t)(t_start - t0) * orow;
+    // the next batch of rows is in flight while the current one is worked on
+    u32x3 in[2][BATCH16];
+    uint32_t dyr[2][BATCH16];
+    uint32_t vin = in0, vdy = dy0, vout = lane_i - (uint32_t)NH * irow;      // offsets of the next row to load / store
+    auto fetch = [&](int slot) {
+#pragma unroll
+        for (int kk = 0; kk < BATCH16; ++kk) {
+            in[slot][kk] = win_load<u32x3>(wr, vin);          // zero past t_far
+            dyr[slot][kk] = win_load<uint32_t>(wdy, vdy);
+            vin += irow;
+            vdy += orow;
+        }
+    };
+    fetch(0);
+    for (int tb = 0; tb < n_stop; tb += 16) {
+#pragma unroll
+        for (int q = 0; q < 16 / BATCH16; ++q) {
+            const int cur = q & 1;
+            fetch(cur ^ 1);
+#pragma unroll
+            for (int kk = 0; kk < BATCH16; ++kk) {
+                const int k = q * BATCH16 + kk;
+                const int t = tb + k;                     // row t_start + t
+                // ---- stage 1: row t
+                {
+                    float f[E], dyf[CH], dCv[CH], gd[CH];
+                    u32x3 fp;
+                    rp[k & 15] = in[cur][kk];
+                    pair_rows(rp[k & 15], rp[(k - 1) & 15], pe[k & 3]);
+                    featurize16<T>(Wa, Wb, pe[k & 3], pe[(k - 2) & 3], f, fp);
+                    P::unpack_unit(dyr[cur][kk], dyf);
+                    const uint32_t live = keep_mask(t < n_df);       // rows whose d f is wanted
+                    const uint32_t in_run = keep_mask(t < n_run);   // rows whose filter-gradient terms are ours
+#pragma unroll
+                    for (int ch = 0; ch < CH; ++ch) {
+                        gr[k & 7][ch] = dyf[ch] * f[3 * ch];
+                        gd[ch] = keep(gr[k & 7][ch], in_run);
+                        ur[k & 7][ch] = keep(f[3 * ch + 1] * f[3 * ch + 2], live);
+                    }
+                    xs[k & 7] = halves<0, 1>(fp[1], fp[2]);          // (x of channel 0, x of channel 1)
+                    Bs[k & 7] = halves<1, 0>(fp[0], fp[2]);          // (B, B)
+                    float y2v[CH];
+#pragma unroll
+                    for (int ch = 0; ch < CH; ++ch) y2v[ch] = 0.f;
+#pragma unroll
+                    for (int j = HL - 1; j >= 0; --j) {
+#pragma unroll
+                        for (int ch = 0; ch < CH; ++ch) y2v[ch] = fmaf(hr[j], ur[(k - j) & 7][ch], y2v[ch]);
+                        dha[j] = fmaf(gd[0], ur[(k - j) & 7][0], fmaf(gd[1], ur[(k - j) & 7][1], dha[j]));
+                    }
+#pragma unroll
+                    for (int ch = 0; ch < CH; ++ch) dCv[ch] = dyf[ch] * y2v[ch];
+                    dCs[k & 7] = Pair<T>::pack2(dCv[0], dCv[1]);
+                }
+                // ---- stage 2: d f of row t1 = t - D1, as elements of T
+                {
+                    const int k1 = k - D1;
+                    const int t1 = t - D1;
+                    float du[CH], xo[CH], Bo[CH], dBv[CH], dxv[CH];
+                    const uint32_t have = keep_mask(t1 >= 0 && t1 < n_df);    // outside, d f counts as zero
+#pragma unroll
+                    for (int ch = 0; ch < CH; ++ch) du[ch] = 0.f;
+#pragma unroll
+                    for (int j = 0; j < HL; ++j)
+#pragma unroll
+                        for (int ch = 0; ch < CH; ++ch) du[ch] = fmaf(hr[j], gr[(k1 + j) & 7][ch], du[ch]);
+                    P::unpack_unit(xs[k1 & 7], xo);
+                    P::unpack_unit(Bs[k1 & 7], Bo);
+#pragma unroll
+                    for (int ch = 0; ch < CH; ++ch) {
+                        const float duv = keep(du[ch], have);
+                        dBv[ch] = duv * xo[ch];
+                        dxv[ch] = duv * Bo[ch];
+                    }
+                    // the row (dC, dB, dx) x 2 channels, assembled from words of two channels each
+                    const uint32_t pC = dCs[k1 & 7] & have, pB = Pair<T>::pack2(dBv[0], dBv[1]), pX = Pair<T>::pack2(dxv[0], dxv[1]);
+                    const u32x3 dfp = u32x3{halves<0, 0>(pC, pB), halves<0, 1>(pX, pC), halves<1, 1>(pB, pX)};
+                    pair_rows(dfprev, dfp, pd[k1 & 3]);
+                    dfprev = dfp;
+                    // dwf[.., kf-1-j] += d f[t1-1] * raw[t1-1-j] + d f[t1] * raw[t1-j], every second row;
+                    // runs start on even rows, so a pair lies in the run when its first row does
+                    if ((k1 & 1) != 0) {
+                        const uint32_t mine = keep_mask(t1 - 1 >= 0 && t1 - 1 < n_run);
+                        uint32_t pm[6];
+#pragma unroll
+                        for (int e = 0; e < E; ++e) pm[e] = pd[k1 & 3][e] & mine;
+#pragma unroll
+                        for (int j = 0; j < KF; ++j) {
+                            uint32_t qr[6];
+                            pair_rows(rp[(k1 - 1 - j) & 15], rp[(k1 - j) & 15], qr);
+#pragma unroll
+                            for (int e = 0; e < E; ++e) dwa[j][e] = Pair<T>::dot2(pm[e], qr[e], dwa[j][e]);
+                        }
+                    }
+                }
+                // ---- stage 3: d raw of row t2 = t1 - 3 from d f of rows t2 .. t2 + 3
+                {
+                    const int k1 = k - D1;
+                    float dr[E];
+#pragma unroll
+                    for (int e = 0; e < E; ++e)
+                        dr[e] = Pair<T>::dot2(pd[(k1 - 2) & 3][e], Wa[e], Pair<T>::dot2(pd[k1 & 3][e], Wb[e], 0.f));
+                    win_store(wdr, vout, pack6<T>(dr));
+                    vout += irow;
+                }
+                // rows are scheduled one after the other: interleaved, their temporaries overlap and the
+                // walk no longer fits the register budget
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
@@ -422,8 +817,12 @@ int fwd_launch(const void *raw, const void *wf, const void *h, void *y, const Di
 {
     const MixPlan p = plan(dm, Piece<T>::CH);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((mixer_se_fwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st, (const T *)raw,
-                       (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+    if constexpr (sizeof(T) == 2)
+        hipLaunchKernelGGL((mixer_se_fwd16_kernel<T, HL>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st, (const T *)raw,
+                           (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+    else
+        hipLaunchKernelGGL((mixer_se_fwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+                           (const T *)raw, (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
     return (int)hipGetLastError();
 }
 
@@ -435,8 +834,12 @@ int bwd_launch(const void *dy, const void *raw, const void *wf, const void *h, v
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     float *ws_h = (float *)ws;
     float *ws_w = ws_h + (size_t)dm.hl * p.nrows * p.nvec;
-    hipLaunchKernelGGL((mixer_se_bwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st, (const T *)dy,
-                       (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+    if constexpr (sizeof(T) == 2)
+        hipLaunchKernelGGL((mixer_se_bwd16_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+                           (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+    else
+        hipLaunchKernelGGL((mixer_se_bwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+                           (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
     int e = (int)hipGetLastError();
     if (e) return e;
     e = launch_colsum_reduce<T>(ws_h, (T *)dh, p.nrows, p.nvec, dm.dg / p.ch, dm.g, dm.hl, st);

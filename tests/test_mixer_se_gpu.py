@@ -1,6 +1,6 @@
 """Featurizer conv + short gated convolution in one pass (gcg_mixer_se_fwd / gcg_mixer_se_bwd) through the
-C ABI: against the chain of entry points it replaces (gcg_dwconv_* and gcg_*_interleaved, bit for bit
-where the arithmetic is the same) and against the CPU oracle applied twice, which follows
+C ABI: against the chain of entry points it replaces (gcg_dwconv_* and gcg_*_interleaved) and against
+the CPU oracle applied twice, which follows
 block.py:867-890 and hyena.py:825-840 of the reference."""
 import pytest
 import torch
@@ -81,8 +81,7 @@ def test_mixer_se_fwd_bwd(gcg_lib, bs, L, g, dg, hl, kf, dtype):
     if (3 * g * dg) % 4 == 0:                              # the stand-alone featurizer takes multiples of 4 channels
         y_c, draw_c, dwf_c, dh_c = kernel_chain(rawd, dyd, wfd, hd)
         torch.cuda.synchronize()
-        # the chain may run another kernel family for this shape (another summation order), so bitwise
-        # equality is asserted only at the layer shape below, where both walk rows in registers
+        # same products, other summation orders: equal up to rounding
         assert_close(y, y_c, 1e-5 if dtype == torch.float32 else TOL[dtype], "y vs chain")
         assert_close(draw, draw_c, 1e-5 if dtype == torch.float32 else TOL[dtype], "d raw vs chain")
         if bs * L * dg >= 256 or dtype == torch.float32:
@@ -108,8 +107,8 @@ def test_mixer_se_is_deterministic_and_rejects_what_it_cannot_run(gcg_lib):
 
 
 def test_mixer_se_shape_of_a_40b_layer(gcg_lib):
-    """B=1, L=8192, 8192 channels in 256 groups, 7 taps after 3, bf16: equal to the chain of kernels
-    bit for bit, and a shift featurizer with a one-tap operator reproduces products of the input."""
+    """B=1, L=8192, 8192 channels in 256 groups, 7 taps after 3, bf16: against the chain of kernels,
+    and a shift featurizer with a one-tap operator must reproduce products of the input bit for bit."""
     bs, L, g, dg, hl, kf, dtype = 1, 8192, 256, 32, 7, 3, torch.bfloat16
     gen = torch.Generator(device=DEV).manual_seed(7)
     raw = torch.randn(bs, L, g, dg, 3, generator=gen, device=DEV).to(dtype)
@@ -120,7 +119,11 @@ def test_mixer_se_shape_of_a_40b_layer(gcg_lib):
     draw, dwf, dh = _lib.mixer_se_bwd(dy, raw, wf, h)
     y_c, draw_c, dwf_c, dh_c = kernel_chain(raw, dy, wf, h)
     torch.cuda.synchronize()
-    assert torch.equal(y, y_c) and torch.equal(draw, draw_c)
+    # the featurizer's taps are summed two at a time here and one at a time in the chain: the same
+    # products, another rounding of their sum
+    assert_close(y, y_c, TOL[dtype], "y")
+    assert_close(draw, draw_c, TOL[dtype], "d raw")
+    assert (y != y_c).float().mean() < 0.02, "more than rounding separates y from the chain of kernels"
     assert_close(dwf, dwf_c, TOL_DH[dtype], "dwf")
     assert_close(dh, dh_c, TOL_DH[dtype], "dh")
     # featurizer = delay by one row, operator = delay by two: y[t] = C[t-1] * (B * x)[t-3]
