@@ -84,14 +84,16 @@ class Op:
         from savanna_amd.kernels.cgcg.interface import (two_pass_chunked_gate_conv_gate,
                                                         two_pass_chunked_gate_conv_gate_interleaved)
         from savanna_amd.kernels.cgcg.src.kernel_utils import FwdKernelConfigRefactor
-        from savanna_amd.operators.hyena import _CausalDepthwiseConv
+        from savanna_amd.operators.hyena import _CausalDepthwiseConv, _FeaturizedShortGateConvGate
 
         wl = self.wl
         raw, wf, h = t["raw"], t["wf"], t["h"]
         raw.grad = wf.grad = h.grad = None
         if ev is not None:
             ev[0].record()
-        if self.layout == "mixer":
+        if self.layout == "mixer_fused":
+            y = _FeaturizedShortGateConvGate.apply(raw.reshape(wl.bs, wl.L, wl.g, wl.dg, 3), wf, h)
+        elif self.layout == "mixer":
             f = _CausalDepthwiseConv.apply(raw.reshape(wl.bs, wl.L, 3 * wl.d, 1), wf)
             y = two_pass_chunked_gate_conv_gate_interleaved(f, h, wl.bs, wl.L, wl.g, wl.dg)
         else:
@@ -340,7 +342,8 @@ def main():
         # the rows next to the hot path: the operator fed from the interleaved projected features, the
         # featurizer conv, and the two chained through autograd
         extra = {}
-        for name in ("mr_fwdbwd_7b_interleaved", "se_fwdbwd_40b_interleaved", "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b"):
+        for name in ("mr_fwdbwd_7b_interleaved", "se_fwdbwd_40b_interleaved", "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b",
+                     "mixer_se_fwdbwd_40b", "mixer_se_fwdbwd_40b_fused"):
             r = time_workload(WORKLOADS[name], device, max(5, args.steps // 3), 3)
             extra[name] = {k: r[k] for k in ("ms_per_step", "tokens_per_s", "step_gbs", "step_hbm_frac")}
         line["next_rows"] = extra

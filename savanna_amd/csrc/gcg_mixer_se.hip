@@ -502,7 +502,6 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
                                                              const T *__restrict__ h, T *__restrict__ y, Dims dm,
                                                              int kf, MixPlan pl)
 {
-    typedef Piece<T> P;
     constexpr int ES = 2, CH = 2, NH = HL - 1 + 3;
     int64_t wg = blockIdx.x;
     const int cvb = (int)(wg % pl.ncvb); wg /= pl.ncvb;

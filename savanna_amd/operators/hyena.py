@@ -259,16 +259,57 @@ class CausalDepthwiseConv1d(nn.Module):
         return self.forward_bld(x.permute(0, 2, 1)).permute(0, 2, 1)
 
 
+class _FeaturizedShortGateConvGate(torch.autograd.Function):
+    """z = gated short convolution of the featurized projection, raw (b, l, g, dg, 3) -> (b, l, g, dg),
+    in one kernel each way; the featurized tensor exists in registers only."""
+
+    @staticmethod
+    def forward(ctx, raw, wf, h):
+        raw, wf, h = (t if t.is_contiguous() else t.contiguous() for t in (raw, wf, h))
+        ctx.save_for_backward(raw, wf, h)
+        return _lib.mixer_se_fwd(raw, wf, h)
+
+    @staticmethod
+    def backward(ctx, dz):
+        raw, wf, h = ctx.saved_tensors
+        return _lib.mixer_se_bwd(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, h)
+
+
 class HyenaMixer(nn.Module):
     """The convolutional part of ParallelSequenceMixer.forward for the hyena operators
     (savanna/model/block.py:865-890): featurizer conv on the projected features, interleaved split,
     gated convolution.  Input (b, l, 3*hidden) -- what the dense projection writes -- output
-    (b, l, hidden) for the output projection; no permute, gather or split copy in between."""
+    (b, l, hidden) for the output projection; no permute, gather or split copy in between.
 
-    def __init__(self, operator: _CgcgOperatorBase, short_conv_L: int = 3, dtype=torch.float32, device=None):
+    With a short operator filter (Hyena-SE: at most 8 taps, featurizer of at most 4, one filter per
+    feature channel) the two convolutions run as one kernel each way (``fuse_short``); the result
+    differs from the two-kernel chain by the rounding of fp32 sums only."""
+
+    def __init__(self, operator: _CgcgOperatorBase, short_conv_L: int = 3, dtype=torch.float32, device=None,
+                 fuse_short: bool = True):
         super().__init__()
         self.mixer = operator
+        self.fuse_short = fuse_short
         self.hyena_proj_conv = CausalDepthwiseConv1d(3 * operator.hidden_size, short_conv_L, dtype=dtype, device=device)
 
+    def _fusable(self, features: torch.Tensor, hl: int) -> bool:
+        conv, op = self.hyena_proj_conv, self.mixer
+        return (self.fuse_short and features.is_cuda and hl <= 8 and conv.kernel_size <= 4 and conv.group_dim == 1
+                and op.group_dim % 2 == 0)
+
     def forward(self, features: torch.Tensor) -> torch.Tensor:
-        return self.mixer.forward_features(self.hyena_proj_conv.forward_bld(features))
+        op = self.mixer
+        bs, seqlen, d3 = features.shape
+        h = op._filter(seqlen)
+        if not self._fusable(features, h.shape[-1]):
+            return op.forward_features(self.hyena_proj_conv.forward_bld(features))
+        dtype = features.dtype
+        if op.cgcg_dtype != dtype:
+            features = features.to(op.cgcg_dtype)
+        g, dg = op.num_groups, op.group_dim
+        assert d3 == 3 * g * dg
+        z = _FeaturizedShortGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3),
+                                               self.hyena_proj_conv.short_conv_weight.to(op.cgcg_dtype),
+                                               h.to(op.cgcg_dtype))
+        z = z.reshape(bs, seqlen, g * dg)
+        return z.to(dtype) if op.cgcg_dtype != dtype else z

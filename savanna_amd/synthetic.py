@@ -33,6 +33,7 @@ class Workload:
     # re-assembly of the feature gradient after the backward) around the separate-tensor kernels.
     # "dwconv": the ungated featurizer conv on one (bs, L, g, dg) tensor.
     # "mixer": featurizer conv then the operator on the interleaved features, all on (bs, L, 3d);
+    # "mixer_fused": the same result from the one-pass kernels (short operator filters only);
     # "mixer_reference_flow": the same chain as block.py:865-890 runs it -- permute to (B, 3D, L),
     # F.pad + F.conv1d, permute back, interleaved split, three gathers -- around the separate-tensor
     # kernels, with autograd doing the backward of the torch part.
@@ -113,6 +114,13 @@ WORKLOADS = {
                                                "the same chain with the reference's data flow (permutes, F.conv1d on "
                                                "(B, 3D, L), gathers) around the separate-tensor kernels",
                                                layout="mixer_reference_flow"),
+    # the Hyena-SE layer of the 40B shape from the dense projection's output to the operator's output
+    "mixer_se_fwdbwd_40b": Workload("mixer_se_fwdbwd_40b", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
+                                    "featurizer conv + Hyena-SE on interleaved features as two kernels each way, "
+                                    "forward+backward, bf16, B=1 L=32768 D=8192 G=512 hl=7", layout="mixer"),
+    "mixer_se_fwdbwd_40b_fused": Workload("mixer_se_fwdbwd_40b_fused", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
+                                          "the same as one kernel each way (the featurized tensor stays in "
+                                          "registers)", layout="mixer_fused"),
 }
 # the order in which the benchmark reports them
 WORKLOAD_ORDER = ("se_fwd_fp32", "mr_fwd_7b", "mr_fwdbwd_7b", "se_mr_fwdbwd_40b", "mr_fwd_1m")

@@ -134,3 +134,39 @@ def test_mixer_se_shape_of_a_40b_layer(gcg_lib):
     C, B, x = raw[..., 0].float(), raw[..., 1].float(), raw[..., 2].float()
     want = (C[:, 2:-1] * (B[:, :-3] * x[:, :-3])).to(dtype)
     assert torch.equal(y[:, 3:], want) and not y[:, :3].any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "f32"])
+def test_hyena_mixer_routes_short_operators_through_the_fused_kernels(gcg_lib, dtype):
+    """HyenaMixer with a Hyena-SE operator: the fused path (one kernel each way) against the same
+    module with fuse_short=False (featurizer kernel, then interleaved operator), output and all
+    gradients; activations in bf16 or fp32 with fp32 parameters, as the block holds them."""
+    import copy
+
+    from savanna_amd.operators.hyena import CgcgConfig, HyenaMixer, HyenaSEOperator, _FeaturizedShortGateConvGate
+
+    torch.manual_seed(5)
+    bs, L, hidden, groups = 2, 300, 192, 12
+    cfg = CgcgConfig(cgcg_dtype="bfloat16" if dtype == torch.bfloat16 else "float32")
+    fused = HyenaMixer(HyenaSEOperator(hidden, groups, 7, cfg, device=DEV), 3, device=DEV)
+    chain = copy.deepcopy(fused)
+    chain.fuse_short = False
+    feats = torch.randn(bs, L, 3 * hidden, device=DEV).to(dtype)
+    dz = (0.1 * torch.randn(bs, L, hidden, device=DEV)).to(dtype)
+    assert fused._fusable(feats, 7) and not chain._fusable(feats, 7)
+    out = []
+    for m in (fused, chain):
+        x = feats.clone().requires_grad_(True)
+        z = m(x)
+        z.backward(dz)
+        out.append((z, x.grad, m.hyena_proj_conv.short_conv_weight.grad, m.mixer.short_conv_weight.grad))
+    torch.cuda.synchronize()
+    tol = TOL[dtype] if dtype != torch.float32 else 1e-5
+    assert_close(out[0][0], out[1][0], tol, "z")
+    assert_close(out[0][1], out[1][1], tol, "d features")
+    assert_close(out[0][2], out[1][2], TOL_DH[dtype], "d featurizer weight")
+    assert_close(out[0][3], out[1][3], TOL_DH[dtype], "d operator weight")
+    # the fused path really is the one that ran
+    x = feats.clone().requires_grad_(True)
+    producer = fused(x).grad_fn.next_functions[0][0]            # below the reshape to (b, l, hidden)
+    assert type(producer).__name__.startswith(_FeaturizedShortGateConvGate.__name__)
