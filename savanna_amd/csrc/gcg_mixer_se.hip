@@ -794,9 +794,10 @@ MixPlan plan(const Dims &dm, int ch)
     MixPlan p;
     p.ch = ch;
     p.nvec = (int)(dm.d / ch);
-    p.ts = 128;
-    // runs of 128 rows unless that leaves fewer than two workgroups per CU; multiples of 16 (the
-    // backward's longest ring) down to 16
+    p.ts = 512;
+    // runs of 512 rows (the halo of up to 10 rows each side and the filter-gradient partials cost 4 %
+    // of the traffic there, 9 % at 128) unless that leaves fewer than two workgroups per CU;
+    // multiples of 16 (the backward's longest ring) down to 16
     while (p.ts > 16 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
     static const char *env = getenv("GCG_MIXER_ROWS");      // tuning override: rows per lane, a multiple of 16
     if (env && atoi(env) >= 16 && atoi(env) % 16 == 0) p.ts = atoi(env);
