@@ -24,7 +24,7 @@ namespace {
 #endif
 constexpr int BATCH = 4;          // rows fetched together
 #ifndef MIXER_BATCH16
-#define MIXER_BATCH16 2
+#define MIXER_BATCH16 4
 #endif
 constexpr int BATCH16 = MIXER_BATCH16;   // the same in the 16-bit backward, whose registers are scarce
 constexpr int KF_MAX = 4;         // featurizer taps: kernels are built for 3 and 4 (shorter filters are zero-padded)
@@ -769,9 +769,6 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
                     win_store(wdr, vout, pack6<T>(dr));
                     vout += irow;
                 }
-                // rows are scheduled one after the other: interleaved, their temporaries overlap and the
-                // walk no longer fits the register budget
-                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
