@@ -211,3 +211,6 @@ def test_workspace_sizing_runs_on_the_host_for_any_shape(gcg_lib):
         supported = hl <= 8 and (g * dg) % 4 == 0 and (dg == 1 or dg % 4 == 0)
         assert n % 256 == 0 and (n > 0) == supported, (bs, L, g, dg, hl, dt)
         assert gcg_lib.gcg_select_algo(bs, L, g, dg, hl, dt, 1) in (1, 2, 3)
+        for kf in (1, 3, 4, 5):
+            n = gcg_lib.gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, dt)
+            assert n % 256 == 0 and (n > 0) == (hl <= 8 and kf <= 4 and dg % 2 == 0), (bs, L, g, dg, hl, kf, dt)

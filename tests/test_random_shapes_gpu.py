@@ -85,3 +85,25 @@ def test_featurizer_random(gcg_lib, p):
     assert_close(dx, dx_ref, TOL[dtype], "dx")
     if bs * L * dg >= 256 or dtype == torch.float32:
         assert_close(dw, dw_ref, TOL_DH[dtype], "dw")
+
+
+MIX = _shapes(24, 3, [2, 4, 6, 8, 16, 20, 32], 8)
+
+
+@pytest.mark.parametrize("p", MIX, ids=[_id(p) for p in MIX])
+def test_fused_mixer_random(gcg_lib, p):
+    from test_mixer_se_gpu import data, oracle_chain
+
+    bs, L, g, dg, hl, dtype = p
+    kf = 1 + (hash(p[:5]) % 4)
+    raw, dy, wf, h = data(bs, L, g, dg, hl, kf, dtype, seed=hash(p[:5]) & 0xffff)
+    ref = oracle_chain(raw, dy, wf, h, dtype)
+    rawd, dyd, wfd, hd = (t.to(DEV) for t in (raw, dy, wf, h))
+    y = _lib.mixer_se_fwd(rawd, wfd, hd)
+    draw, dwf, dh = _lib.mixer_se_bwd(dyd, rawd, wfd, hd)
+    torch.cuda.synchronize()
+    assert_close(y, ref[0], TOL[dtype], "y")
+    assert_close(draw, ref[1], 2 * TOL[dtype], "d raw")
+    if bs * L * dg >= 256 or dtype == torch.float32:
+        assert_close(dwf, ref[2], 2 * TOL_DH[dtype], "dwf")
+        assert_close(dh, ref[3], TOL_DH[dtype], "dh")
