@@ -15,6 +15,7 @@
 #include "gcg_rowvec.h"
 
 #include <cstdlib>
+#include <type_traits>
 
 namespace gcg {
 namespace {
@@ -661,8 +662,13 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
         }
     }
 
-    // rows are counted from the run's start in the walk: 32-bit scalars for offsets and bounds
-    const int n_run = (int)(t_end - t_start), n_df = n_run + D2, n_stop = n_run + NH;
+    // Rows are counted from the run's start.  No row of the walk needs a run-time mask:
+    //  * before the run, d f comes out zero by itself, because the rings of x, B and dC start at zero;
+    //  * a run cut short by the end of the sequence reads zeros there (dy = 0 gives g2 = du = dC = 0);
+    //  * a full run ends at row ts, a multiple of 16, so the rows past it are the last iteration of the
+    //    walk, and what they may contribute is known when the kernel is compiled (`past` below):
+    //    nothing to dh, d f only for 3 rows, dwf only from pairs of rows inside the run.
+    const int ts = pl.ts, n_stop = (int)(t_end - t_start) + NH;
     const uint32_t in0 = lane_i + (uint32_t)(t_start - t0) * irow, dy0 = lane_o + (uint32_t)(t_start - t0) * orow;
     // the next batch of rows is in flight while the current one is worked on
     u32x3 in[2][BATCH16];
@@ -677,99 +683,101 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
             vdy += orow;
         }
     };
-    fetch(0);
-    for (int tb = 0; tb < n_stop; tb += 16) {
+    // one row of the walk: k = its place in the iteration of 16 (ring slots), past = the iteration after a full run
+    auto row = [&](auto past_tag, int k, const u32x3 &inrow, uint32_t dyrow) {
+        constexpr bool past = decltype(past_tag)::value;
+        const int k1 = k - D1;                                 // the row whose d f completes now
+        if (past && k >= NH) return;                           // nothing of these rows reaches the run
+        // ---- stage 1: row t
+        {
+            float f[E], dyf[CH], dCv[CH];
+            u32x3 fp;
+            rp[k & 15] = inrow;
+            pair_rows(rp[k & 15], rp[(k - 1) & 15], pe[k & 3]);
+            featurize16<T>(Wa, Wb, pe[k & 3], pe[(k - 2) & 3], f, fp);
+            P::unpack_unit(dyrow, dyf);
 #pragma unroll
-        for (int q = 0; q < 16 / BATCH16; ++q) {
-            const int cur = q & 1;
-            fetch(cur ^ 1);
+            for (int ch = 0; ch < CH; ++ch) {
+                gr[k & 7][ch] = dyf[ch] * f[3 * ch];
+                ur[k & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+            }
+            xs[k & 7] = halves<0, 1>(fp[1], fp[2]);          // (x of channel 0, x of channel 1)
+            Bs[k & 7] = halves<1, 0>(fp[0], fp[2]);          // (B, B)
+            float y2v[CH];
 #pragma unroll
-            for (int kk = 0; kk < BATCH16; ++kk) {
-                const int k = q * BATCH16 + kk;
-                const int t = tb + k;                     // row t_start + t
-                // ---- stage 1: row t
-                {
-                    float f[E], dyf[CH], dCv[CH], gd[CH];
-                    u32x3 fp;
-                    rp[k & 15] = in[cur][kk];
-                    pair_rows(rp[k & 15], rp[(k - 1) & 15], pe[k & 3]);
-                    featurize16<T>(Wa, Wb, pe[k & 3], pe[(k - 2) & 3], f, fp);
-                    P::unpack_unit(dyr[cur][kk], dyf);
-                    const uint32_t live = keep_mask(t < n_df);       // rows whose d f is wanted
-                    const uint32_t in_run = keep_mask(t < n_run);   // rows whose filter-gradient terms are ours
+            for (int ch = 0; ch < CH; ++ch) y2v[ch] = 0.f;
 #pragma unroll
-                    for (int ch = 0; ch < CH; ++ch) {
-                        gr[k & 7][ch] = dyf[ch] * f[3 * ch];
-                        gd[ch] = keep(gr[k & 7][ch], in_run);
-                        ur[k & 7][ch] = keep(f[3 * ch + 1] * f[3 * ch + 2], live);
-                    }
-                    xs[k & 7] = halves<0, 1>(fp[1], fp[2]);          // (x of channel 0, x of channel 1)
-                    Bs[k & 7] = halves<1, 0>(fp[0], fp[2]);          // (B, B)
-                    float y2v[CH];
+            for (int j = HL - 1; j >= 0; --j) {
 #pragma unroll
-                    for (int ch = 0; ch < CH; ++ch) y2v[ch] = 0.f;
+                for (int ch = 0; ch < CH; ++ch) y2v[ch] = fmaf(hr[j], ur[(k - j) & 7][ch], y2v[ch]);
+                if (!past)                                   // rows past the run belong to the next run's dh
+                    dha[j] = fmaf(gr[k & 7][0], ur[(k - j) & 7][0], fmaf(gr[k & 7][1], ur[(k - j) & 7][1], dha[j]));
+            }
 #pragma unroll
-                    for (int j = HL - 1; j >= 0; --j) {
+            for (int ch = 0; ch < CH; ++ch) dCv[ch] = dyf[ch] * y2v[ch];
+            dCs[k & 7] = Pair<T>::pack2(dCv[0], dCv[1]);
+        }
+        // ---- stage 2: d f of row t1 = t - D1, as elements of T; past the run it is wanted for 3 rows
+        {
+            u32x3 dfp = u32x3{0u, 0u, 0u};
+            if (!past || k1 < D2) {
+                float du[CH], xo[CH], Bo[CH], dBv[CH], dxv[CH];
 #pragma unroll
-                        for (int ch = 0; ch < CH; ++ch) y2v[ch] = fmaf(hr[j], ur[(k - j) & 7][ch], y2v[ch]);
-                        dha[j] = fmaf(gd[0], ur[(k - j) & 7][0], fmaf(gd[1], ur[(k - j) & 7][1], dha[j]));
-                    }
+                for (int ch = 0; ch < CH; ++ch) du[ch] = 0.f;
 #pragma unroll
-                    for (int ch = 0; ch < CH; ++ch) dCv[ch] = dyf[ch] * y2v[ch];
-                    dCs[k & 7] = Pair<T>::pack2(dCv[0], dCv[1]);
+                for (int j = 0; j < HL; ++j)
+#pragma unroll
+                    for (int ch = 0; ch < CH; ++ch) du[ch] = fmaf(hr[j], gr[(k1 + j) & 7][ch], du[ch]);
+                P::unpack_unit(xs[k1 & 7], xo);
+                P::unpack_unit(Bs[k1 & 7], Bo);
+#pragma unroll
+                for (int ch = 0; ch < CH; ++ch) {
+                    dBv[ch] = du[ch] * xo[ch];
+                    dxv[ch] = du[ch] * Bo[ch];
                 }
-                // ---- stage 2: d f of row t1 = t - D1, as elements of T
-                {
-                    const int k1 = k - D1;
-                    const int t1 = t - D1;
-                    float du[CH], xo[CH], Bo[CH], dBv[CH], dxv[CH];
-                    const uint32_t have = keep_mask(t1 >= 0 && t1 < n_df);    // outside, d f counts as zero
+                // the row (dC, dB, dx) x 2 channels, assembled from words of two channels each
+                const uint32_t pC = dCs[k1 & 7], pB = Pair<T>::pack2(dBv[0], dBv[1]), pX = Pair<T>::pack2(dxv[0], dxv[1]);
+                dfp = u32x3{halves<0, 0>(pC, pB), halves<0, 1>(pX, pC), halves<1, 1>(pB, pX)};
+            }
+            pair_rows(dfprev, dfp, pd[k1 & 3]);
+            dfprev = dfp;
+            // dwf[.., kf-1-j] += d f[t1-1] * raw[t1-1-j] + d f[t1] * raw[t1-j], every second row; runs start
+            // and end on even rows, so a pair lies in the run when its first row does
+            if ((k1 & 1) != 0 && (!past || k1 - 1 < 0)) {
 #pragma unroll
-                    for (int ch = 0; ch < CH; ++ch) du[ch] = 0.f;
+                for (int j = 0; j < KF; ++j) {
+                    uint32_t qr[6];
+                    pair_rows(rp[(k1 - 1 - j) & 15], rp[(k1 - j) & 15], qr);
 #pragma unroll
-                    for (int j = 0; j < HL; ++j)
-#pragma unroll
-                        for (int ch = 0; ch < CH; ++ch) du[ch] = fmaf(hr[j], gr[(k1 + j) & 7][ch], du[ch]);
-                    P::unpack_unit(xs[k1 & 7], xo);
-                    P::unpack_unit(Bs[k1 & 7], Bo);
-#pragma unroll
-                    for (int ch = 0; ch < CH; ++ch) {
-                        const float duv = keep(du[ch], have);
-                        dBv[ch] = duv * xo[ch];
-                        dxv[ch] = duv * Bo[ch];
-                    }
-                    // the row (dC, dB, dx) x 2 channels, assembled from words of two channels each
-                    const uint32_t pC = dCs[k1 & 7] & have, pB = Pair<T>::pack2(dBv[0], dBv[1]), pX = Pair<T>::pack2(dxv[0], dxv[1]);
-                    const u32x3 dfp = u32x3{halves<0, 0>(pC, pB), halves<0, 1>(pX, pC), halves<1, 1>(pB, pX)};
-                    pair_rows(dfprev, dfp, pd[k1 & 3]);
-                    dfprev = dfp;
-                    // dwf[.., kf-1-j] += d f[t1-1] * raw[t1-1-j] + d f[t1] * raw[t1-j], every second row;
-                    // runs start on even rows, so a pair lies in the run when its first row does
-                    if ((k1 & 1) != 0) {
-                        const uint32_t mine = keep_mask(t1 - 1 >= 0 && t1 - 1 < n_run);
-                        uint32_t pm[6];
-#pragma unroll
-                        for (int e = 0; e < E; ++e) pm[e] = pd[k1 & 3][e] & mine;
-#pragma unroll
-                        for (int j = 0; j < KF; ++j) {
-                            uint32_t qr[6];
-                            pair_rows(rp[(k1 - 1 - j) & 15], rp[(k1 - j) & 15], qr);
-#pragma unroll
-                            for (int e = 0; e < E; ++e) dwa[j][e] = Pair<T>::dot2(pm[e], qr[e], dwa[j][e]);
-                        }
-                    }
-                }
-                // ---- stage 3: d raw of row t2 = t1 - 3 from d f of rows t2 .. t2 + 3
-                {
-                    const int k1 = k - D1;
-                    float dr[E];
-#pragma unroll
-                    for (int e = 0; e < E; ++e)
-                        dr[e] = Pair<T>::dot2(pd[(k1 - 2) & 3][e], Wa[e], Pair<T>::dot2(pd[k1 & 3][e], Wb[e], 0.f));
-                    win_store(wdr, vout, pack6<T>(dr));
-                    vout += irow;
+                    for (int e = 0; e < E; ++e) dwa[j][e] = Pair<T>::dot2(pd[k1 & 3][e], qr[e], dwa[j][e]);
                 }
             }
+        }
+        // ---- stage 3: d raw of row t2 = t1 - 3 from d f of rows t2 .. t2 + 3
+        {
+            float dr[E];
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                dr[e] = Pair<T>::dot2(pd[(k1 - 2) & 3][e], Wa[e], Pair<T>::dot2(pd[k1 & 3][e], Wb[e], 0.f));
+            win_store(wdr, vout, pack6<T>(dr));
+            vout += irow;
+        }
+    };
+    fetch(0);
+    for (int tb = 0; tb < ts && tb < n_stop; tb += 16) {
+#pragma unroll
+        for (int q = 0; q < 16 / BATCH16; ++q) {
+            fetch((q & 1) ^ 1);
+#pragma unroll
+            for (int kk = 0; kk < BATCH16; ++kk) row(std::false_type{}, q * BATCH16 + kk, in[q & 1][kk], dyr[q & 1][kk]);
+        }
+    }
+    if (n_stop > ts) {
+#pragma unroll
+        for (int q = 0; q < (NH + BATCH16 - 1) / BATCH16; ++q) {
+            fetch((q & 1) ^ 1);
+#pragma unroll
+            for (int kk = 0; kk < BATCH16; ++kk) row(std::true_type{}, q * BATCH16 + kk, in[q & 1][kk], dyr[q & 1][kk]);
         }
     }
     // partials: ws_h[tap][(batch, run)][lane], ws_w[tap][(batch, run)][feature channel]
