@@ -12,6 +12,10 @@
 // rows: the featurizer's taps reach back over rows the lane has just seen, and in the backward
 // the two transposed convolutions are two delays of the same walk.  A lane takes one 12-byte piece
 // of the interleaved row per step -- (C, B, x) of two channels at 16 bits, of one at fp32.
+//
+// Two pairs of kernels: mixer_se_fwd_kernel / mixer_se_bwd_kernel in the plain form, one FMA per
+// tap (instantiated for fp32, where a word is an element and nothing has to be unpacked), and
+// mixer_se_fwd16_kernel / mixer_se_bwd16_kernel for bf16 and f16, further down.
 #include "gcg_rowvec.h"
 
 #include <cstdlib>
