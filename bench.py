@@ -94,8 +94,8 @@ class Op:
         if self.layout == "mixer_fused":
             y = _FeaturizedShortGateConvGate.apply(raw.reshape(wl.bs, wl.L, wl.g, wl.dg, 3), wf, h)
         elif self.layout == "mixer":
-            f = _CausalDepthwiseConv.apply(raw.reshape(wl.bs, wl.L, 3 * wl.d, 1), wf)
-            y = two_pass_chunked_gate_conv_gate_interleaved(f, h, wl.bs, wl.L, wl.g, wl.dg)
+            f = _CausalDepthwiseConv.apply(raw.reshape(wl.bs, wl.L, 3 * wl.d, 1), wf, True)
+            y = two_pass_chunked_gate_conv_gate_interleaved(f, h, wl.bs, wl.L, wl.g, wl.dg, keep_dfeatures=True)
         else:
             u = raw.permute(0, 2, 1)                                               # block.py:867
             f = F.conv1d(F.pad(u, (2, 0)), wf, groups=3 * wl.d)[..., :wl.L]        # hyena.py:139, :168-175

@@ -68,9 +68,9 @@ def load() -> ctypes.CDLL:
         lib.gcg_select_algo.restype = ctypes.c_int
         lib.gcg_fwd_interleaved.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_fwd_interleaved.restype = ctypes.c_int
-        lib.gcg_bwd_interleaved.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_bwd_interleaved.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, i32, i32, vp]
         lib.gcg_bwd_interleaved.restype = ctypes.c_int
-        lib.gcg_dwconv_fwd.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, vp]
+        lib.gcg_dwconv_fwd.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_dwconv_fwd.restype = ctypes.c_int
         lib.gcg_dwconv_bwd_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32]
         lib.gcg_dwconv_bwd_workspace_bytes.restype = sz
@@ -221,8 +221,12 @@ def fwd_interleaved(feat, h, algo=ALGO_AUTO, out=None):
     return y
 
 
-def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO):
-    """(dfeat, dh): dfeat has feat's layout, dfeat[..., 0] = dC, [..., 1] = dB, [..., 2] = dx."""
+KEEP_OUTPUT = 1       # GCG_KEEP_OUTPUT
+
+
+def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO, keep_output=False):
+    """(dfeat, dh): dfeat has feat's layout, dfeat[..., 0] = dC, [..., 1] = dB, [..., 2] = dx.
+    ``keep_output``: dfeat goes to dwconv_bwd next, store it through the cache."""
     lib = load()
     _require_gpu(feat)
     _check_feat(feat, h)
@@ -242,7 +246,8 @@ def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=feat.device)
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_bwd_interleaved(dy.data_ptr(), feat.data_ptr(), h.data_ptr(), dfeat.data_ptr(), dh.data_ptr(),
-                                     ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, a, st)
+                                     ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, a,
+                                     KEEP_OUTPUT if keep_output else 0, st)
     check(rc, "gcg_bwd_interleaved")
     return dfeat, dh
 
@@ -256,8 +261,9 @@ def _check_dwconv(x, w):
         raise ValueError("x and w must share dtype and device")
 
 
-def dwconv_fwd(x, w):
-    """y = causal depthwise convolution of x (bs, L, g, dg) with w (g, 1, hl), no gates."""
+def dwconv_fwd(x, w, keep_output=False):
+    """y = causal depthwise convolution of x (bs, L, g, dg) with w (g, 1, hl), no gates.
+    ``keep_output``: y goes to fwd_interleaved next, store it through the cache."""
     lib = load()
     _require_gpu(x)
     _check_dwconv(x, w)
@@ -268,7 +274,7 @@ def dwconv_fwd(x, w):
     with _on_device(x.device):
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_dwconv_fwd(x.data_ptr(), w.data_ptr(), y.data_ptr(), bs, L, g, dg, w.shape[-1],
-                                dtype_code(x.dtype), st)
+                                dtype_code(x.dtype), KEEP_OUTPUT if keep_output else 0, st)
     check(rc, "gcg_dwconv_fwd")
     return y
 

@@ -31,7 +31,7 @@ int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t 
 {
     if (bs <= 0 || L <= 0 || g <= 0 || dg <= 0 || hl <= 0) return GCG_ERR_BAD_ARG;
     if (dtype != GCG_F32 && dtype != GCG_BF16 && dtype != GCG_F16) return GCG_ERR_BAD_ARG;
-    dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg; dm->es = 1;
+    dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg; dm->es = 1; dm->keep_out = 0;
     return GCG_OK;
 }
 
@@ -95,7 +95,7 @@ GCG_API const char *gcg_strerror(int code)
 
 GCG_API int gcg_last_hip_error(void) { return tls_hip_error; }
 
-GCG_API int gcg_version(void) { return 104; }
+GCG_API int gcg_version(void) { return 105; }
 
 GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t backward)
 {
@@ -196,13 +196,14 @@ GCG_API int gcg_fwd_interleaved(const void *feat, const void *h, void *y, int64_
 
 GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *workspace,
                                 size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
-                                int32_t dtype, int32_t algo, void *stream)
+                                int32_t dtype, int32_t algo, int32_t flags, void *stream)
 {
-    if (!dy || !feat || !h || !dfeat || !dh) return GCG_ERR_BAD_ARG;
+    if (!dy || !feat || !h || !dfeat || !dh || (flags & ~GCG_KEEP_OUTPUT)) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
     if (rc) return rc;
     dm.es = 3;
+    dm.keep_out = flags & GCG_KEEP_OUTPUT;
     const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, feat, dfeat}));
     if (a < 0) return a;
     const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
@@ -226,12 +227,13 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
 // ---- ungated short causal depthwise convolution (featurizer)
 
 GCG_API int gcg_dwconv_fwd(const void *x, const void *w, void *y, int64_t bs, int64_t L, int32_t g, int32_t dg,
-                           int32_t hl, int32_t dtype, void *stream)
+                           int32_t hl, int32_t dtype, int32_t flags, void *stream)
 {
-    if (!x || !w || !y) return GCG_ERR_BAD_ARG;
+    if (!x || !w || !y || (flags & ~GCG_KEEP_OUTPUT)) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
     if (rc) return rc;
+    dm.keep_out = flags & GCG_KEEP_OUTPUT;
     if (!gcg::dwconv_supported(dm) || !all_aligned16({x, y})) return GCG_ERR_UNSUPPORTED;
     rc = check_device();
     if (rc) return rc;

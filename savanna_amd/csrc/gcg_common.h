@@ -138,6 +138,22 @@ __device__ __forceinline__ void win_store(win_t w, uint32_t off, const u32x4 &v)
 {
     __builtin_amdgcn_raw_buffer_store_b128(v, w, (int)off, 0, WIN_NT_ST);
 }
+// The same without the nontemporal hint, for an output the next kernel of a chain reads back at once
+// (the featurized tensor, the gradient of the features): stored through the cache it is still
+// partly there when that kernel starts.  A kernel timed alone loses a few percent this way, which
+// is why it is the caller's choice (GCG_KEEP_OUTPUT).
+template <bool KEEP> __device__ __forceinline__ void win_store_as(win_t w, uint32_t off, const u32x2 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b64(v, w, (int)off, 0, KEEP ? 0 : WIN_NT_ST);
+}
+template <bool KEEP> __device__ __forceinline__ void win_store_as(win_t w, uint32_t off, const u32x3 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b96(v, w, (int)off, 0, KEEP ? 0 : WIN_NT_ST);
+}
+template <bool KEEP> __device__ __forceinline__ void win_store_as(win_t w, uint32_t off, const u32x4 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(v, w, (int)off, 0, KEEP ? 0 : WIN_NT_ST);
+}
 
 #ifndef GCG_XCD_SWIZZLE
 #define GCG_XCD_SWIZZLE 1
@@ -163,6 +179,7 @@ struct Dims {
     // [..., 2] = x; the launchers then receive C = base, B = base + 1, x = base + 2 elements
     // (and dC, dB, dx likewise).  y, y2, bx and dy are always plain.
     int32_t es;
+    int32_t keep_out;   // GCG_KEEP_OUTPUT: store the main output through the cache (kernels that have the variant)
 };
 
 constexpr int kWave = 64;

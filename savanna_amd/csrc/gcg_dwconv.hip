@@ -31,7 +31,7 @@ __device__ __forceinline__ void load_taps(const T *w, int64_t c, int dg, int hl,
     }
 }
 
-template <typename T, int HL, int V, bool PCF>
+template <typename T, int HL, int V, bool PCF, bool KEEP>
 __global__ __launch_bounds__(256) void dwconv_fwd_kernel(const T *__restrict__ x, const T *__restrict__ w,
                                                          T *__restrict__ y, Dims dm, DwPlan pl)
 {
@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void dwconv_fwd_kernel(const T *__restrict__ x
 #pragma unroll
                     for (int v = 0; v < V; ++v)
                         acc[v] = fmaf(hr[j][PCF ? v : 0], ring[(k - j) & (RING - 1)][v], acc[v]);
-                win_store(wy, lane + (uint32_t)(tb + k - t0) * row, packv<T, V>(acc));
+                win_store_as<KEEP>(wy, lane + (uint32_t)(tb + k - t0) * row, packv<T, V>(acc));
             }
         }
     }
@@ -237,8 +237,12 @@ int fwd_launch(const void *x, const void *w, void *y, const Dims &dm, hipStream_
 {
     const DwPlan p = plan(dm, V);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((dwconv_fwd_kernel<T, HL, V, PCF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
-                       (const T *)x, (const T *)w, (T *)y, dm, p);
+    if (dm.keep_out)
+        hipLaunchKernelGGL((dwconv_fwd_kernel<T, HL, V, PCF, true>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+                           (const T *)x, (const T *)w, (T *)y, dm, p);
+    else
+        hipLaunchKernelGGL((dwconv_fwd_kernel<T, HL, V, PCF, false>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+                           (const T *)x, (const T *)w, (T *)y, dm, p);
     return (int)hipGetLastError();
 }
 

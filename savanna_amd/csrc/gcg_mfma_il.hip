@@ -229,7 +229,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 // iterations before those are used, and the outputs of a row leave as one interleaved row.
 // The early x, B values wait in LDS: each lane parks its own two row vectors in a ring of NK-1
 // slots and reads them back itself, so the ring needs no barrier.
-template <typename T, int NK, int NW>
+template <typename T, int NK, int NW, bool KEEP>
 __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ feat,
                                                           const T *__restrict__ h, T *__restrict__ dfeat,
                                                           float *__restrict__ ws, Dims dm, MfmaPlan pl)
@@ -481,7 +481,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
                     il_join<T, NR>(ox, oB, oC, po);
                     const uint32_t o = lane_off + step_off(s);
 #pragma unroll
-                    for (int k = 0; k < NR; ++k) stw12(wdf, 3 * (o + k * pass_off) + bad, po[k]);
+                    for (int k = 0; k < NR; ++k) win_store_as<KEEP>(wdf, 3 * (o + k * pass_off) + bad, po[k]);
                 }
 #pragma unroll
                 for (int k = 0; k < NR; ++k) in[k] = nx[k];
@@ -552,8 +552,12 @@ int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, voi
 {
     const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((mfma_il_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)dy,
-                       (const T *)feat, (const T *)h, (T *)dfeat, (float *)ws, dm, p);
+    if (dm.keep_out)
+        hipLaunchKernelGGL((mfma_il_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+                           (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (float *)ws, dm, p);
+    else
+        hipLaunchKernelGGL((mfma_il_bwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+                           (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (float *)ws, dm, p);
     int e = (int)hipGetLastError();
     if (e) return e;
     const int64_t n = (int64_t)dm.g * dm.hl;

@@ -29,6 +29,11 @@ __device__ __forceinline__ void store_piece(win_t w, uint32_t off, const u32x1 (
 {
     win_store(w, off, u32x3{p[0][0], p[1][0], p[2][0]});
 }
+// (with the choice of cache policy; the interleaved kernels' lanes are one word wide)
+template <bool KEEP> __device__ __forceinline__ void store_piece_as(win_t w, uint32_t off, const u32x1 (&p)[3])
+{
+    win_store_as<KEEP>(w, off, u32x3{p[0][0], p[1][0], p[2][0]});
+}
 template <typename R> __device__ __forceinline__ void load_piece(win_t w, uint32_t off, R (&p)[3])
 {
     constexpr int NB = sizeof(R);

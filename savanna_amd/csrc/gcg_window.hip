@@ -196,7 +196,7 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
 // every row outside reads as zero or is dropped, so the walk has no branch around an access.
 // (occupancy floor: three workgroups per CU at 16 bits, two at fp32, so that the scheduler
 // does not trade waves for longer load batches)
-template <typename T, int HL, int V, bool PK>
+template <typename T, int HL, int V, bool PK, bool KEEP>
 __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                          const T *__restrict__ B, const T *__restrict__ C,
                                                          const T *__restrict__ h, T *__restrict__ dx,
@@ -356,7 +356,8 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                         unpackv<T, V>(dCs[(k - (HL - 1)) & (RING - 1)], oC);
                         join3<T, V>(o, oB, oC, p);
                         const uint32_t q = lane_i + (uint32_t)(out_t - t_start) * irow;
-                        store_piece(wdC, q, p);
+                        if constexpr (KEEP) store_piece_as<true>(wdC, q, p);
+                        else store_piece(wdC, q, p);
                     } else {
                         const uint32_t q = lane_o + (uint32_t)(out_t - t_start) * orow;
 #pragma unroll
@@ -433,12 +434,16 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
     const WinPlan p = plan(dm, dm.es == 3 ? il_v<T>() : BWD_V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    if (dm.es == 3)
-        hipLaunchKernelGGL((window_bwd_kernel<T, HL, il_v<T>(), true>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
-                           (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
+    if (dm.es == 3 && dm.keep_out)
+        hipLaunchKernelGGL((window_bwd_kernel<T, HL, il_v<T>(), true, true>), dim3((unsigned)nwg), dim3(p.threads), 0,
+                           st, (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
+                           (T *)dC, (float *)ws, dm, p);
+    else if (dm.es == 3)
+        hipLaunchKernelGGL((window_bwd_kernel<T, HL, il_v<T>(), true, false>), dim3((unsigned)nwg), dim3(p.threads), 0,
+                           st, (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
     else
-        hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V, false>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+        hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V, false, false>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
                            (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
     int e = (int)hipGetLastError();

@@ -120,27 +120,31 @@ class InterleavedGateConvGate(torch.autograd.Function):
     produced in the features' layout and autograd has nothing to re-assemble."""
 
     @staticmethod
-    def forward(ctx, feat, h):
+    def forward(ctx, feat, h, keep_dfeatures=False):
         feat, h = _contig(feat), _contig(h)
         y = _lib.fwd_interleaved(feat, h)
         ctx.save_for_backward(feat, h)
+        ctx.keep_dfeatures = keep_dfeatures
         return y
 
     @staticmethod
     def backward(ctx, dy):
         feat, h = ctx.saved_tensors
-        dfeat, dh = _lib.bwd_interleaved(_contig(dy), feat, h)
-        return dfeat, dh
+        dfeat, dh = _lib.bwd_interleaved(_contig(dy), feat, h, keep_output=ctx.keep_dfeatures)
+        return dfeat, dh, None
 
 
 def two_pass_chunked_gate_conv_gate_interleaved(features: torch.Tensor, h: torch.Tensor,
-                                                bs: int, seqlen: int, g: int, dg: int) -> torch.Tensor:
+                                                bs: int, seqlen: int, g: int, dg: int,
+                                                keep_dfeatures: bool = False) -> torch.Tensor:
     """y = x1 * conv(x2 * v, h) for projected features laid out "(g dg p)" with p = (x1, x2, v)
     fastest, i.e. the tensor savanna/model/block.py:886-890 splits before calling the mixer.
 
     features: (bs, seqlen, 3*g*dg) or (bs, seqlen, g, dg, 3); h: (g, 1, hl).  Returns (bs, seqlen, g, dg).
     Equivalent to ``two_pass_chunked_gate_conv_gate(x=v, B=x2, C=x1, h=h, ...)`` on the split views.
+    ``keep_dfeatures``: the gradient of the features is read at once by the backward of the op that
+    produced them (the featurizer conv); it is then stored through the cache.  Same values either way.
     """
     assert features.numel() == bs * seqlen * g * dg * 3, "features must hold 3*g*dg values per position"
     assert h.dim() == 3 and h.shape[0] == g and h.shape[1] == 1, "h must be (g, 1, hl)"
-    return InterleavedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3), h)
+    return InterleavedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3), h, keep_dfeatures)

@@ -162,10 +162,11 @@ class _CgcgOperatorBase(nn.Module):
         z = z.reshape(bs, seqlen, g * dg)
         return z.to(dtype) if self.cgcg_dtype != dtype else z
 
-    def forward_features(self, features: torch.Tensor) -> torch.Tensor:
+    def forward_features(self, features: torch.Tensor, from_featurizer: bool = False) -> torch.Tensor:
         """The same on the projected features before their split: (b, l, 3*g*dg) laid out
         "(g dg p)" with p = (x1, x2, v) fastest (block.py:886-888) -> z: (b, l, g*dg).  The kernels
-        read the tensor as it is and the backward writes its gradient in the same layout."""
+        read the tensor as it is and the backward writes its gradient in the same layout.
+        ``from_featurizer``: the gradient goes straight into the featurizer's backward (cache hint)."""
         dtype = features.dtype
         bs, seqlen, d3 = features.shape
         g, dg = self.num_groups, self.group_dim
@@ -173,7 +174,8 @@ class _CgcgOperatorBase(nn.Module):
         h = self._filter(seqlen)
         if self.cgcg_dtype != dtype:
             features = features.to(self.cgcg_dtype)
-        z = two_pass_chunked_gate_conv_gate_interleaved(features, h.to(self.cgcg_dtype), bs, seqlen, g, dg)
+        z = two_pass_chunked_gate_conv_gate_interleaved(features, h.to(self.cgcg_dtype), bs, seqlen, g, dg,
+                                                        keep_dfeatures=from_featurizer)
         z = z.reshape(bs, seqlen, g * dg)
         return z.to(dtype) if self.cgcg_dtype != dtype else z
 
@@ -214,16 +216,16 @@ class _CausalDepthwiseConv(torch.autograd.Function):
     """y[b, t, c] = sum_k w[c / dg, 0, k] x[b, t - (K-1) + k, c] on (b, l, g, dg) tensors."""
 
     @staticmethod
-    def forward(ctx, x, w):
+    def forward(ctx, x, w, feeds_operator=False):
         x = x if x.is_contiguous() else x.contiguous()
         w = w if w.is_contiguous() else w.contiguous()
         ctx.save_for_backward(x, w)
-        return _lib.dwconv_fwd(x, w)
+        return _lib.dwconv_fwd(x, w, keep_output=feeds_operator)
 
     @staticmethod
     def backward(ctx, dy):
         x, w = ctx.saved_tensors
-        return _lib.dwconv_bwd(dy if dy.is_contiguous() else dy.contiguous(), x, w)
+        return _lib.dwconv_bwd(dy if dy.is_contiguous() else dy.contiguous(), x, w) + (None,)
 
 
 class CausalDepthwiseConv1d(nn.Module):
@@ -248,11 +250,13 @@ class CausalDepthwiseConv1d(nn.Module):
         w = torch.empty(self.num_groups, 1, kernel_size, dtype=dtype, device=device).uniform_(-bound, bound)
         self.short_conv_weight = nn.Parameter(w)
 
-    def forward_bld(self, x: torch.Tensor) -> torch.Tensor:
+    def forward_bld(self, x: torch.Tensor, feeds_operator: bool = False) -> torch.Tensor:
+        """``feeds_operator``: the result goes straight into the interleaved operator; it is then stored
+        through the cache, where part of it still is when that kernel starts (same values either way)."""
         b, l, d = x.shape
         assert d == self.d_model
         y = _CausalDepthwiseConv.apply(x.reshape(b, l, self.num_groups, self.group_dim),
-                                       self.short_conv_weight.to(x.dtype))
+                                       self.short_conv_weight.to(x.dtype), feeds_operator)
         return y.reshape(b, l, d)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
@@ -302,7 +306,8 @@ class HyenaMixer(nn.Module):
         bs, seqlen, d3 = features.shape
         h = op._filter(seqlen)
         if not self._fusable(features, h.shape[-1]):
-            return op.forward_features(self.hyena_proj_conv.forward_bld(features))
+            return op.forward_features(self.hyena_proj_conv.forward_bld(features, feeds_operator=True),
+                                       from_featurizer=True)
         dtype = features.dtype
         if op.cgcg_dtype != dtype:
             features = features.to(op.cgcg_dtype)

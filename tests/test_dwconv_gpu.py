@@ -161,3 +161,22 @@ def test_featurizer_shape_of_a_7b_layer(gcg_lib):
     assert_close(y.index_select(2, idx), y_ref, TOL[dtype], "y")
     assert_close(dx.index_select(2, idx), dx_ref, TOL[dtype], "dx")
     assert_close(dw.index_select(0, idx), dw_ref, TOL_DH[dtype], "dw")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=["f32", "bf16", "f16"])
+def test_keep_output_changes_the_cache_policy_not_the_values(gcg_lib, dtype):
+    """GCG_KEEP_OUTPUT on the two entry points that write a chain's intermediates: the featurized
+    tensor (gcg_dwconv_fwd) and the gradient of the features (gcg_bwd_interleaved, matrix-core and
+    register-window families); an unknown flag is refused."""
+    x, _, w = (t.to(DEV) for t in data(2, 300, 48, 1, 3, dtype, seed=4))
+    assert torch.equal(_lib.dwconv_fwd(x, w), _lib.dwconv_fwd(x, w, keep_output=True))
+    for (bs, L, g, dg, hl) in [(1, 300, 3, 16, 128), (2, 200, 4, 8, 7)]:
+        gen = torch.Generator().manual_seed(hl)
+        feat = torch.randn(bs, L, g, dg, 3, generator=gen).to(dtype).to(DEV)
+        dy = torch.randn(bs, L, g, dg, generator=gen).to(dtype).to(DEV)
+        h = (torch.randn(g, 1, hl, generator=gen) / hl ** 0.5).to(dtype).to(DEV)
+        a, b = _lib.bwd_interleaved(dy, feat, h), _lib.bwd_interleaved(dy, feat, h, keep_output=True)
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    lib = _lib.load()
+    p = x.data_ptr()
+    assert lib.gcg_dwconv_fwd(p, p, p, 1, 64, 16, 1, 3, 0, 2, None) == -1        # unknown flag
