@@ -39,6 +39,9 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
+KEEP_INTERMEDIATES = True      # mixer workloads: the chain's two intermediates stored through the cache (--no-keep-output)
+
+
 class Op:
     """One convolution of a workload with its resident inputs (rotated over `nsets` copies
     when a single copy would sit in the 256 MB last-level cache)."""
@@ -94,8 +97,9 @@ class Op:
         if self.layout == "mixer_fused":
             y = _FeaturizedShortGateConvGate.apply(raw.reshape(wl.bs, wl.L, wl.g, wl.dg, 3), wf, h)
         elif self.layout == "mixer":
-            f = _CausalDepthwiseConv.apply(raw.reshape(wl.bs, wl.L, 3 * wl.d, 1), wf, True)
-            y = two_pass_chunked_gate_conv_gate_interleaved(f, h, wl.bs, wl.L, wl.g, wl.dg, keep_dfeatures=True)
+            f = _CausalDepthwiseConv.apply(raw.reshape(wl.bs, wl.L, 3 * wl.d, 1), wf, KEEP_INTERMEDIATES)
+            y = two_pass_chunked_gate_conv_gate_interleaved(f, h, wl.bs, wl.L, wl.g, wl.dg,
+                                                            keep_dfeatures=KEEP_INTERMEDIATES)
         else:
             u = raw.permute(0, 2, 1)                                               # block.py:867
             f = F.conv1d(F.pad(u, (2, 0)), wf, groups=3 * wl.d)[..., :wl.L]        # hyena.py:139, :168-175
@@ -285,12 +289,16 @@ def main():
     ap.add_argument("--workload", default="mr_fwdbwd_7b", choices=list(WORKLOADS))
     ap.add_argument("--all", action="store_true", help="also time the other four configurations")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-keep-output", action="store_true",
+                    help="mixer workloads: store the chain's intermediates past the cache like every other output")
     ap.add_argument("--graph", action="store_true",
                     help="also time the step replayed from a captured HIP graph (launch-bound shapes)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, so a counter profile of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
+    global KEEP_INTERMEDIATES
+    KEEP_INTERMEDIATES = not args.no_keep_output
     if args.gpus != 1:
         print("bench.py: this build is single-GPU; the path has no collective or sharded variant, "
               "so --gpus must be 1", file=sys.stderr)
