@@ -37,8 +37,8 @@ constexpr int KF_MAX = 4;         // featurizer taps: kernels are built for 3 an
 // x if the wave-uniform condition holds, else +0: as a bit mask, which stays one VALU operation with a
 // scalar operand (written as a select, the compiler may turn a uniform condition into a branch
 // around the row's work, and a branch costs the exact wait counts of the straight-line walk)
-__device__ __forceinline__ uint32_t keep_mask(bool uniform_cond) { return uniform_cond ? 0xffffffffu : 0u; }
-__device__ __forceinline__ float keep(float x, uint32_t m) { return __uint_as_float(__float_as_uint(x) & m); }
+__device__ __forceinline__ uint32_t row_mask(bool uniform_cond) { return uniform_cond ? 0xffffffffu : 0u; }
+__device__ __forceinline__ float masked(float x, uint32_t m) { return __uint_as_float(__float_as_uint(x) & m); }
 
 struct MixPlan { int ch, nvec, nseg, ts, ncvb, threads; int64_t nrows, nwg; };
 
@@ -306,14 +306,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
                     rp[k & 15] = in[kk];
                     featurize_packed<T, KF>(wfr, rp, k & 15, f);
                     P::unpack_unit(dyr[kk], dyf);
-                    const uint32_t live = keep_mask(t < t_df);       // rows whose d f is wanted
-                    const uint32_t in_run = keep_mask(t < t_end);    // rows whose filter-gradient terms are ours
+                    const uint32_t live = row_mask(t < t_df);       // rows whose d f is wanted
+                    const uint32_t in_run = row_mask(t < t_end);    // rows whose filter-gradient terms are ours
 #pragma unroll
                     for (int ch = 0; ch < CH; ++ch) {
                         xv[ch] = f[3 * ch + 2];
                         Bv[ch] = f[3 * ch + 1];
                         gr[k & 7][ch] = dyf[ch] * f[3 * ch];
-                        ur[k & 7][ch] = keep(Bv[ch] * xv[ch], live);
+                        ur[k & 7][ch] = masked(Bv[ch] * xv[ch], live);
                     }
                     xs[k & 7] = P::pack_unit(xv);
                     Bs[k & 7] = P::pack_unit(Bv);
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
                         for (int ch = 0; ch < CH; ++ch) {
                             const float u = ur[(k - j) & 7][ch];
                             y2v[ch] = fmaf(hr[j], u, y2v[ch]);
-                            sacc = fmaf(keep(gr[k & 7][ch], in_run), u, sacc);
+                            sacc = fmaf(masked(gr[k & 7][ch], in_run), u, sacc);
                         }
                         dha[j] += sacc;
                     }
@@ -349,24 +349,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
                     P::unpack_unit(xs[k1 & 7], xo);
                     P::unpack_unit(Bs[k1 & 7], Bo);
                     P::unpack_unit(dCs[k1 & 7], dCo);
-                    const uint32_t have = keep_mask(t1 >= t_start && t1 < t_df);     // outside, d f counts as zero
+                    const uint32_t have = row_mask(t1 >= t_start && t1 < t_df);     // outside, d f counts as zero
 #pragma unroll
                     for (int ch = 0; ch < CH; ++ch) {
-                        const float duv = keep(du[ch], have);
-                        df[3 * ch] = keep(dCo[ch], have);
+                        const float duv = masked(du[ch], have);
+                        df[3 * ch] = masked(dCo[ch], have);
                         df[3 * ch + 1] = duv * xo[ch];
                         df[3 * ch + 2] = duv * Bo[ch];
                     }
                     const u32x3 dfp = P::pack(df);
                     P::unpack(dfp, df);
                     // featurizer filter gradient: dwf[.., KF-1-j] += d f[t1] * raw[t1 - j], rows of the run only
-                    const uint32_t mine = keep_mask(t1 >= t_start && t1 < t_end);
+                    const uint32_t mine = row_mask(t1 >= t_start && t1 < t_end);
                     float rj[E];
 #pragma unroll
                     for (int j = 0; j < KF; ++j) {
                         P::unpack(rp[(k1 - j) & 15], rj);
 #pragma unroll
-                        for (int e = 0; e < E; ++e) dwa[j][e] = fmaf(keep(df[e], mine), rj[e], dwa[j][e]);
+                        for (int e = 0; e < E; ++e) dwa[j][e] = fmaf(masked(df[e], mine), rj[e], dwa[j][e]);
                     }
                     dfr[k1 & 3] = dfp;
                 }
