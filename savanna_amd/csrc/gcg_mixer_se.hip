@@ -798,15 +798,17 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
         }
 }
 
-MixPlan plan(const Dims &dm, int ch)
+MixPlan plan(const Dims &dm, int ch, bool backward)
 {
     MixPlan p;
     p.ch = ch;
     p.nvec = (int)(dm.d / ch);
-    p.ts = 512;
-    // runs of 512 rows (the halo of up to 10 rows each side and the filter-gradient partials cost 4 %
-    // of the traffic there, 9 % at 128) unless that leaves fewer than two workgroups per CU;
-    // multiples of 16 (the backward's longest ring) down to 16
+    // The longest runs that still leave two workgroups per CU: the halo of up to 10 rows each side
+    // and the filter-gradient partials cost 9 % of the traffic at 128 rows, 4 % at 512.  The
+    // backward, which holds two workgroups per CU at a time, gains nothing beyond 512 rows; the
+    // forward does (measured at the 40B shape: 409 us at 512 rows, 383 at 1024).  Multiples of 16
+    // (the backward's longest ring) down to 16.
+    p.ts = backward ? 512 : 1024;
     while (p.ts > 16 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
     static const char *env = getenv("GCG_MIXER_ROWS");      // tuning override: rows per lane, a multiple of 16
     if (env && atoi(env) >= 16 && atoi(env) % 16 == 0) p.ts = atoi(env);
@@ -824,7 +826,7 @@ int lane_channels(int dtype) { return dtype == GCG_F32 ? 1 : 2; }
 template <typename T, int HL, int KF>
 int fwd_launch(const void *raw, const void *wf, const void *h, void *y, const Dims &dm, int kf, hipStream_t st)
 {
-    const MixPlan p = plan(dm, Piece<T>::CH);
+    const MixPlan p = plan(dm, Piece<T>::CH, false);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if constexpr (sizeof(T) == 2)
         hipLaunchKernelGGL((mixer_se_fwd16_kernel<T, HL>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st, (const T *)raw,
@@ -839,7 +841,7 @@ template <typename T, int HL, int KF>
 int bwd_launch(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf, void *dh,
                void *ws, const Dims &dm, int kf, hipStream_t st)
 {
-    const MixPlan p = plan(dm, Piece<T>::CH);
+    const MixPlan p = plan(dm, Piece<T>::CH, true);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     float *ws_h = (float *)ws;
     float *ws_w = ws_h + (size_t)dm.hl * p.nrows * p.nvec;
@@ -905,7 +907,7 @@ int mixer_se_fwd_launch(int dtype, const void *raw, const void *wf, const void *
 
 size_t mixer_se_bwd_workspace(int dtype, const Dims &dm, int kf)
 {
-    const MixPlan p = plan(dm, lane_channels(dtype));
+    const MixPlan p = plan(dm, lane_channels(dtype), true);
     return ((size_t)dm.hl * p.nrows * p.nvec + (size_t)kf * p.nrows * 3 * dm.d) * sizeof(float);
 }
 

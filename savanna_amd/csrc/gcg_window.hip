@@ -383,9 +383,10 @@ WinPlan plan(const Dims &dm, int v)
     WinPlan p;
     p.v = v;
     p.nvec = (int)(dm.d / v);
-    p.ts = 128;
-    // 128-row runs measured best (64 and 256 are both ~10 % slower at the 7B and 40B shapes);
-    // shorter runs only when 128 would leave fewer than two workgroups per CU
+    p.ts = 1024;
+    // the longest runs (up to 1024 rows) that still leave two workgroups per CU: measured best at the
+    // 7B and 40B shapes for either operand layout (fewer halo rows and filter-gradient partials;
+    // one step further and the machine is no longer covered)
     while (p.ts > 8 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
     static const char *env = getenv("GCG_WINDOW_ROWS");   // tuning override: rows per lane, a multiple of 8
     if (env && atoi(env) >= 8 && atoi(env) % 8 == 0) p.ts = atoi(env);
