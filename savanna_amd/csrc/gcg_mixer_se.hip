@@ -853,9 +853,10 @@ int bwd_launch(const void *dy, const void *raw, const void *wf, const void *h, v
                            (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
     int e = (int)hipGetLastError();
     if (e) return e;
-    e = launch_colsum_reduce<T>(ws_h, (T *)dh, p.nrows, p.nvec, dm.dg / p.ch, dm.g, dm.hl, st);
-    if (e) return e;
-    return launch_colsum_reduce<T>(ws_w, (T *)dwf, p.nrows, 3 * dm.d, 1, (int)(3 * dm.d), kf, st);
+    // both filter gradients in one launch
+    const ColsumJob jh{ws_h, dh, p.nrows, p.nvec, dm.dg / p.ch, dm.g, dm.hl};
+    const ColsumJob jw{ws_w, dwf, p.nrows, 3 * dm.d, 1, (int)(3 * dm.d), kf};
+    return launch_colsum_reduce2<T>(jh, jw, st);
 }
 
 template <typename T, int KF>

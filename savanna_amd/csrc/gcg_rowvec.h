@@ -102,14 +102,17 @@ template <typename T, int VV> __device__ __forceinline__ typename Vec<T, VV>::ra
 // filter if it is wider) and 4 row slices: its 64-lane rows read contiguous runs of a partial
 // row, every thread adds its terms in a fixed order, and the slices and columns of a filter are
 // then combined in a fixed order -- the result is bit-reproducible.
-template <typename T>
-__global__ __launch_bounds__(256) void colsum_reduce_kernel(const float *__restrict__ ws, T *__restrict__ out,
-                                                            int64_t nrow, int64_t ncol, int lpg, int nfilt, int ntap)
+struct ColsumJob { const float *ws; void *out; int64_t nrow, ncol; int lpg, nfilt, ntap; };
+
+template <typename T> __device__ __forceinline__ void colsum_reduce_block(const ColsumJob &jb, int bx, int tap)
 {
     __shared__ float red[4][64];
+    const float *__restrict__ ws = jb.ws;
+    T *__restrict__ out = (T *)jb.out;
+    const int64_t nrow = jb.nrow, ncol = jb.ncol;
+    const int lpg = jb.lpg, nfilt = jb.nfilt, ntap = jb.ntap;
     const int fpb = lpg >= 64 ? 1 : 64 / lpg;                 // filters per workgroup
-    const int tap = blockIdx.y;
-    const int64_t f0 = (int64_t)blockIdx.x * fpb;
+    const int64_t f0 = (int64_t)bx * fpb;
     const int nf = (int)((f0 + fpb <= nfilt) ? fpb : nfilt - f0);
     const int width = nf * lpg;                                // columns of the tile
     const int c = threadIdx.x & 63, slice = threadIdx.x >> 6;
@@ -138,13 +141,43 @@ __global__ __launch_bounds__(256) void colsum_reduce_kernel(const float *__restr
 }
 
 template <typename T>
+__global__ __launch_bounds__(256) void colsum_reduce_kernel(ColsumJob jb)
+{
+    colsum_reduce_block<T>(jb, blockIdx.x, blockIdx.y);
+}
+
+// two reductions in one launch (the filter gradients of two filters from one walk): the first
+// nb0 workgroups of a grid row belong to the first; grid rows beyond a job's tap count idle
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_reduce2_kernel(ColsumJob j0, ColsumJob j1, int nb0)
+{
+    const bool second = (int)blockIdx.x >= nb0;
+    const ColsumJob &jb = second ? j1 : j0;
+    if ((int)blockIdx.y >= jb.ntap) return;
+    colsum_reduce_block<T>(jb, second ? (int)blockIdx.x - nb0 : (int)blockIdx.x, blockIdx.y);
+}
+
+inline unsigned colsum_blocks(int lpg, int nfilt)
+{
+    const int fpb = lpg >= 64 ? 1 : 64 / lpg;
+    return (unsigned)((nfilt + fpb - 1) / fpb);
+}
+
+template <typename T>
 inline int launch_colsum_reduce(const float *ws, T *out, int64_t nrow, int64_t ncol, int lpg, int nfilt, int ntap,
                                 hipStream_t st)
 {
-    const int fpb = lpg >= 64 ? 1 : 64 / lpg;
-    const unsigned nbx = (unsigned)((nfilt + fpb - 1) / fpb);
-    hipLaunchKernelGGL(colsum_reduce_kernel<T>, dim3(nbx, (unsigned)ntap), dim3(256), 0, st, ws, out, nrow, ncol, lpg,
-                       nfilt, ntap);
+    const ColsumJob jb{ws, out, nrow, ncol, lpg, nfilt, ntap};
+    hipLaunchKernelGGL(colsum_reduce_kernel<T>, dim3(colsum_blocks(lpg, nfilt), (unsigned)ntap), dim3(256), 0, st, jb);
+    return (int)hipGetLastError();
+}
+
+template <typename T>
+inline int launch_colsum_reduce2(const ColsumJob &j0, const ColsumJob &j1, hipStream_t st)
+{
+    const unsigned nb0 = colsum_blocks(j0.lpg, j0.nfilt), nb1 = colsum_blocks(j1.lpg, j1.nfilt);
+    const unsigned ny = (unsigned)(j0.ntap > j1.ntap ? j0.ntap : j1.ntap);
+    hipLaunchKernelGGL(colsum_reduce2_kernel<T>, dim3(nb0 + nb1, ny), dim3(256), 0, st, j0, j1, (int)nb0);
     return (int)hipGetLastError();
 }
 
