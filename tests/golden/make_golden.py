@@ -51,8 +51,42 @@ def featurizer_case():
     print("featurizer_bf16_small written")
 
 
+def mixer_se_case():
+    """The convolutional part of a Hyena-SE layer as the reference chains it, in float64 with its
+    bf16 tensors emulated: permute, ParallelCausalDepthwiseConv1d on (B, 3D, L), permute
+    (savanna/model/block.py:867-876), the interleaved split (block.py:886-890), and
+    y = x1 * conv(x2 * v, h) (hyena.py:825-840 -> ref_fwd.py:109-129).  The featurized tensor is a
+    bf16 tensor there, so it is rounded on the way forward and its gradient on the way back."""
+    import torch.nn.functional as F
+    from einops import rearrange
+
+    bs, L, g, dg, hl, K, dtype = 2, 150, 3, 8, 7, 3, torch.bfloat16
+    D = g * dg
+    gen = torch.Generator().manual_seed(0)
+    raw = torch.randn(bs, L, 3 * D, generator=gen).to(dtype).double().requires_grad_(True)
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen)).to(dtype).double()
+    wf = (torch.randn(3 * D, 1, K, generator=gen) / K ** 0.5).to(dtype).double().requires_grad_(True)
+    h = (torch.randn(g, 1, hl, generator=gen) / hl ** 0.5).to(dtype).double().requires_grad_(True)
+    u = raw.permute(0, 2, 1)
+    f = F.conv1d(F.pad(u, (K - 1, 0)), wf, bias=None, stride=1, padding=0, groups=3 * D)[..., :L].permute(0, 2, 1)
+    f = f + (f.to(dtype).double() - f).detach()                  # stored as bf16
+    f.register_hook(lambda gr: gr.to(dtype).double())            # and so is its gradient
+    x1, x2, v = rearrange(f, "b l (g dg p) -> b l g p dg", p=3, g=g).unbind(dim=3)
+    y = oracle.gcg_fwd_ref_torch(v.contiguous(), x2.contiguous(), x1.contiguous(), h)
+    y.backward(dy)
+    np.savez_compressed(
+        os.path.join(HERE, "mixer_se_bf16_small.npz"),
+        raw=raw.detach().reshape(bs, L, g, dg, 3).float().numpy(), dy=dy.float().numpy(),
+        wf=wf.detach().float().numpy(), h=h.detach().float().numpy(), y=y.detach().numpy(),
+        draw=raw.grad.reshape(bs, L, g, dg, 3).numpy(), dwf=wf.grad.numpy(), dh=h.grad.numpy(),
+        dtype=np.array(str(dtype)),
+    )
+    print("mixer_se_bf16_small written")
+
+
 def main():
     featurizer_case()
+    mixer_se_case()
     for name, (bs, L, g, dg, hl, dtype) in CASES.items():
         gen = torch.Generator().manual_seed(0)
         x, B, C, dy = (torch.randn(bs, L, g, dg, generator=gen).to(dtype).double() for _ in range(4))

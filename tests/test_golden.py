@@ -15,8 +15,9 @@ from savanna_amd import _lib
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ALL = sorted(glob.glob(os.path.join(HERE, "golden", "*.npz")))
-FILES = [f for f in ALL if not os.path.basename(f).startswith("featurizer")]      # the gated operator
 FEAT = [f for f in ALL if os.path.basename(f).startswith("featurizer")]           # the ungated featurizer conv
+MIXER = [f for f in ALL if os.path.basename(f).startswith("mixer_se")]            # featurizer + Hyena-SE operator
+FILES = [f for f in ALL if f not in FEAT and f not in MIXER]                      # the gated operator
 DT = {"torch.float32": torch.float32, "torch.bfloat16": torch.bfloat16, "torch.float16": torch.float16}
 
 
@@ -27,7 +28,7 @@ def load(path):
 
 
 def test_fixtures_present():
-    assert len(FILES) >= 4 and len(FEAT) >= 1
+    assert len(FILES) >= 4 and len(FEAT) >= 1 and len(MIXER) >= 1
 
 
 @pytest.mark.parametrize("path", FILES, ids=[os.path.basename(f) for f in FILES])
@@ -97,3 +98,45 @@ def test_hip_featurizer_reproduces_golden(gcg_lib, path):
     dx, dw = _lib.dwconv_bwd(dev["dy"], dev["x"], dev["w"])
     assert_close(dx, t["dx"], TOL[dtype], "dx")
     assert_close(dw, t["dw"], TOL_DH[dtype], "dw")
+
+
+def _chain_with_oracle(t, dtype):
+    """The two C-oracle applications that make up the chain, with the tensors that the chain holds
+    in `dtype` rounded to it."""
+    bs, L, g, dg, _ = t["raw"].shape
+    r4 = t["raw"].reshape(bs, L, 3 * g * dg, 1)
+    one = torch.ones_like(r4)
+    f = oracle.gcg_fwd_oracle(r4, one, one, t["wf"]).to(dtype).float().reshape(bs, L, g, dg, 3)
+    C, B, x = (f[..., i].contiguous() for i in range(3))
+    y = oracle.gcg_fwd_oracle(x, B, C, t["h"])
+    dx, dB, dC, dh = oracle.gcg_bwd_oracle(t["dy"], x, B, C, t["h"])
+    df = torch.stack([dC, dB, dx], dim=-1).to(dtype).float().reshape(bs, L, 3 * g * dg, 1)
+    draw, _, _, dwf = oracle.gcg_bwd_oracle(df, r4, one, one, t["wf"])
+    return y, draw.reshape(t["raw"].shape), dwf, dh
+
+
+@pytest.mark.parametrize("path", MIXER, ids=[os.path.basename(f) for f in MIXER])
+def test_c_oracle_chain_reproduces_mixer_golden(path):
+    """The oracle applied twice (featurizer, then operator) against the reference's chain written
+    with F.conv1d, rearrange / unbind and autograd in float64.  Where the float64 value of the
+    featurized tensor sits next to a bf16 rounding boundary the fp32 oracle may round it the other
+    way (one bf16 ulp in that element), hence the tolerance of a rounded stage."""
+    t, dtype = load(path)
+    y, draw, dwf, dh = _chain_with_oracle(t, dtype)
+    assert_close(y, t["y"], TOL[dtype], "y")
+    assert_close(draw, t["draw"], TOL[dtype], "d raw")
+    assert_close(dwf, t["dwf"], TOL_DH[dtype], "dwf")
+    assert_close(dh, t["dh"], TOL_DH[dtype], "dh")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("path", MIXER, ids=[os.path.basename(f) for f in MIXER])
+def test_hip_mixer_reproduces_golden(gcg_lib, path):
+    t, dtype = load(path)
+    dev = {k: v.to(dtype).to("cuda:0") for k, v in t.items()}
+    y = _lib.mixer_se_fwd(dev["raw"], dev["wf"], dev["h"])
+    draw, dwf, dh = _lib.mixer_se_bwd(dev["dy"], dev["raw"], dev["wf"], dev["h"])
+    assert_close(y, t["y"], TOL[dtype], "y")
+    assert_close(draw, t["draw"], 2 * TOL[dtype], "d raw")
+    assert_close(dwf, t["dwf"], 2 * TOL_DH[dtype], "dwf")
+    assert_close(dh, t["dh"], TOL_DH[dtype], "dh")
