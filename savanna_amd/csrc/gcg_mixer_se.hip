@@ -31,6 +31,9 @@ constexpr int BATCH = 4;          // rows fetched together
 #ifndef MIXER_BATCH16
 #define MIXER_BATCH16 4
 #endif
+#ifndef MIXER_BATCH_FWD16
+#define MIXER_BATCH_FWD16 4
+#endif
 constexpr int BATCH16 = MIXER_BATCH16;   // the same in the 16-bit backward, whose registers are scarce
 constexpr int KF_MAX = 4;         // featurizer taps: kernels are built for 3 and 4 (shorter filters are zero-padded)
 
@@ -560,25 +563,27 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
         }
     }
 
-    u32x3 in[2][BATCH];
+    // FB rows are in flight while FB are worked on
+    constexpr int FB = MIXER_BATCH_FWD16;
+    u32x3 in[2][FB];
 #pragma unroll
-    for (int kk = 0; kk < BATCH; ++kk) in[0][kk] = load_raw(t_start + kk);
-    for (int64_t tb = t_start; tb < t_end; tb += 8) {
+    for (int kk = 0; kk < FB; ++kk) in[0][kk] = load_raw(t_start + kk);
+    for (int64_t tb = t_start; tb < t_end; tb += 2 * FB) {
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             const int cur = half, nxt = half ^ 1;
 #pragma unroll
-            for (int kk = 0; kk < BATCH; ++kk) in[nxt][kk] = load_raw(tb + (half + 1) * BATCH + kk);
+            for (int kk = 0; kk < FB; ++kk) in[nxt][kk] = load_raw(tb + (half + 1) * FB + kk);
 #pragma unroll
-            for (int kk = 0; kk < BATCH; ++kk) {
-                const int k = half * BATCH + kk;
+            for (int kk = 0; kk < FB; ++kk) {
+                const int k = half * FB + kk;
                 float f[6], out[CH];
                 pair_rows(in[cur][kk], prev, pe[k & 3]);
                 prev = in[cur][kk];
                 featurize16<T>(Wa, Wb, pe[k & 3], pe[(k - 2) & 3], f);
 #pragma unroll
                 for (int ch = 0; ch < CH; ++ch) {
-                    ur[k][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                    ur[k & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
                     float acc = 0.f;
 #pragma unroll
                     for (int j = HL - 1; j >= 0; --j) acc = fmaf(hr[j], ur[(k - j) & 7][ch], acc);
