@@ -352,7 +352,7 @@ def main():
         extra = {}
         for name in ("mr_fwdbwd_7b_interleaved", "se_fwdbwd_40b_interleaved", "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b",
                      "mixer_se_fwdbwd_40b", "mixer_se_fwdbwd_40b_fused"):
-            r = time_workload(WORKLOADS[name], device, max(5, args.steps // 3), 3)
+            r = time_workload(WORKLOADS[name], device, max(10, args.steps // 2), 4)
             extra[name] = {k: r[k] for k in ("ms_per_step", "tokens_per_s", "step_gbs", "step_hbm_frac")}
         line["next_rows"] = extra
     if args.copy_calibration:
