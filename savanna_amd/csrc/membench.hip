@@ -5,7 +5,8 @@
 // Prints the HBM rate of (a) flat streams with R reads and W writes per element, plain and
 // nontemporal, and (b) the tile walk the MFMA kernels perform -- a workgroup owns ROWB bytes of
 // every row of a (bs, L, d) bf16 tensor set and walks a run of 32-row steps with a one-step
-// prefetch -- for several row widths, read/write mixes and row strides.  These are the rates the
+// prefetch -- for several row widths, read/write mixes, run lengths and row strides, and with
+// neighbouring column blocks in or out of step.  These are the rates the
 // memory system gives the kernels' access pattern; the kernels are compared with them, not
 // only with the 8 TB/s nominal peak.
 #include <hip/hip_runtime.h>
@@ -37,7 +38,7 @@ __global__ __launch_bounds__(256) void flat_kernel(const u4 *a, const u4 *b, con
 // THREADS lanes cover (THREADS*16/ROWB) rows of ROWB bytes per step
 template <int THREADS, int ROWB, int R, int W>
 __global__ __launch_bounds__(THREADS) void tile_kernel(const char *a, const char *b, const char *c, const char *e, char *y, char *z, char *w,
-                                                       int64_t L, int64_t rowbytes, int ncb, int nseg, int steps)
+                                                       int64_t L, int64_t rowbytes, int ncb, int nseg, int steps, int skew)
 {
     int64_t id = blockIdx.x;
     const int cb = id % ncb; id /= ncb;
@@ -45,13 +46,16 @@ __global__ __launch_bounds__(THREADS) void tile_kernel(const char *a, const char
     const int64_t bb = id / nseg;
     constexpr int LPR = ROWB / 16, RPS = THREADS / LPR;
     const int r = threadIdx.x / LPR, l = threadIdx.x % LPR;
-    int64_t o = bb * L * rowbytes + (int64_t)cb * ROWB + l * 16 + ((int64_t)seg * steps * RPS + r) * rowbytes;
+    // skew > 0: column block cb starts its run skew*cb steps in and wraps round (same rows, other order)
+    const int64_t base = bb * L * rowbytes + (int64_t)cb * ROWB + l * 16 + ((int64_t)seg * steps * RPS + r) * rowbytes;
+    const int phi = (int)((int64_t)cb * skew % steps);
+    int64_t o = base + (int64_t)phi * RPS * rowbytes;
     u4 v0 = ld<1>((const u4 *)(a + o)), v1 = v0, v2 = v0, v3 = v0;
     if (R > 1) v1 = ld<1>((const u4 *)(b + o));
     if (R > 2) v2 = ld<1>((const u4 *)(c + o));
     if (R > 3) v3 = ld<1>((const u4 *)(e + o));
     for (int s = 0; s < steps; ++s) {
-        const int64_t on = o + (int64_t)RPS * rowbytes;
+        const int64_t on = base + (int64_t)((s + 1 + phi) % steps) * RPS * rowbytes;
         u4 n0 = v0, n1 = v1, n2 = v2, n3 = v3;
         if (s + 1 < steps) {
             n0 = ld<1>((const u4 *)(a + on));
@@ -104,10 +108,10 @@ int main()
             timeit("flat 3R1W nontemporal", 4 * n1, [&] { flat_kernel<3, 1, 1><<<8192, 256>>>(q[0], q[1], q[2], q[3], q[4], q[5], q[6], n16); });
             timeit("flat 4R3W nontemporal", 7 * n1, [&] { flat_kernel<4, 3, 1><<<8192, 256>>>(q[0], q[1], q[2], q[3], q[4], q[5], q[6], n16); });
         }
-        auto tile = [&](auto kern, int threads, int rowb, int rd, int wr, int steps) {
+        auto tile = [&](auto kern, int threads, int rowb, int rd, int wr, int steps, int skew = 0) {
             const int ncb = (int)(d * 2 / rowb), rps = threads * 16 / rowb, nseg = (int)(L / rps / steps);
-            snprintf(nm, sizeof nm, "tile %dR%dW rows of %3d B, %4d threads, %3d steps, stride %lld", rd, wr, rowb, threads, steps, (long long)rowbytes);
-            timeit(nm, (rd + wr) * n1, [&] { kern<<<(unsigned)(bs * nseg * ncb), threads>>>(p[0], p[1], p[2], p[3], p[4], p[5], p[6], L, rowbytes, ncb, nseg, steps); });
+            snprintf(nm, sizeof nm, "tile %dR%dW rows of %3d B, %4d threads, %3d steps%s, stride %lld", rd, wr, rowb, threads, steps, skew ? ", skewed" : "", (long long)rowbytes);
+            timeit(nm, (rd + wr) * n1, [&] { kern<<<(unsigned)(bs * nseg * ncb), threads>>>(p[0], p[1], p[2], p[3], p[4], p[5], p[6], L, rowbytes, ncb, nseg, steps, skew); });
         };
         tile(tile_kernel<256, 128, 3, 1>, 256, 128, 3, 1, 128);
         tile(tile_kernel<512, 256, 3, 1>, 512, 256, 3, 1, 64);
@@ -115,6 +119,14 @@ int main()
         tile(tile_kernel<256, 128, 4, 3>, 256, 128, 4, 3, 128);
         tile(tile_kernel<512, 256, 4, 3>, 512, 256, 4, 3, 64);
         tile(tile_kernel<1024, 512, 4, 3>, 1024, 512, 4, 3, 32);
+        // the same walks cut into shorter runs: 2 and 4 workgroups resident per CU instead of 1
+        tile(tile_kernel<512, 256, 4, 3>, 512, 256, 4, 3, 32);
+        tile(tile_kernel<512, 256, 4, 3>, 512, 256, 4, 3, 16);
+        tile(tile_kernel<256, 128, 4, 3>, 256, 128, 4, 3, 32);
+        tile(tile_kernel<256, 128, 4, 3>, 256, 128, 4, 3, 16);
+        // column blocks out of step with their neighbours
+        tile(tile_kernel<512, 256, 4, 3>, 512, 256, 4, 3, 64, 1);
+        tile(tile_kernel<512, 256, 4, 3>, 512, 256, 4, 3, 64, 5);
         for (int i = 0; i < 7; ++i) CK(hipFree(p[i]));
     }
     return 0;
