@@ -6,7 +6,8 @@
 // nontemporal, and (b) the tile walk the MFMA kernels perform -- a workgroup owns ROWB bytes of
 // every row of a (bs, L, d) bf16 tensor set and walks a run of 32-row steps with a one-step
 // prefetch -- for several row widths, read/write mixes, run lengths and row strides, and with
-// neighbouring column blocks in or out of step.  These are the rates the
+// neighbouring column blocks in or out of step, and (c) the row walk of the register-window
+// kernels (a lane owns a few bytes of every row of a run).  These are the rates the
 // memory system gives the kernels' access pattern; the kernels are compared with them, not
 // only with the 8 TB/s nominal peak.
 #include <hip/hip_runtime.h>
@@ -71,6 +72,56 @@ __global__ __launch_bounds__(THREADS) void tile_kernel(const char *a, const char
     }
 }
 
+// The register-window kernels' pattern: a lane owns VB bytes of every row and walks a run of ts rows,
+// four rows fetched together one batch ahead; a workgroup's 256 lanes cover 256*VB contiguous bytes.
+template <int VB, int R, int W>
+__global__ __launch_bounds__(256) void walk_kernel(const char *a, const char *b, const char *c, const char *e, char *y, char *z, char *w,
+                                                   int64_t L, int64_t rowbytes, int ncvb, int nseg, int ts)
+{
+    typedef uint32_t vec_t __attribute__((ext_vector_type(VB / 4)));
+    int64_t id = blockIdx.x;
+    const int cvb = id % ncvb; id /= ncvb;
+    const int seg = id % nseg;
+    const int64_t bb = id / nseg;
+    int64_t o = (bb * L + (int64_t)seg * ts) * rowbytes + ((int64_t)cvb * 256 + threadIdx.x) * VB;
+    if (((int64_t)cvb * 256 + threadIdx.x) * VB >= rowbytes) return;
+    vec_t v[2][4][4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        v[0][k][0] = __builtin_nontemporal_load((const vec_t *)(a + o + k * rowbytes));
+        if (R > 1) v[0][k][1] = __builtin_nontemporal_load((const vec_t *)(b + o + k * rowbytes));
+        if (R > 2) v[0][k][2] = __builtin_nontemporal_load((const vec_t *)(c + o + k * rowbytes));
+        if (R > 3) v[0][k][3] = __builtin_nontemporal_load((const vec_t *)(e + o + k * rowbytes));
+    }
+    for (int t = 0; t < ts; t += 8) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int cur = half, nxt = half ^ 1;
+            const int64_t on = o + 4 * rowbytes;
+            if (t + 4 * half + 4 < ts) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    v[nxt][k][0] = __builtin_nontemporal_load((const vec_t *)(a + on + k * rowbytes));
+                    if (R > 1) v[nxt][k][1] = __builtin_nontemporal_load((const vec_t *)(b + on + k * rowbytes));
+                    if (R > 2) v[nxt][k][2] = __builtin_nontemporal_load((const vec_t *)(c + on + k * rowbytes));
+                    if (R > 3) v[nxt][k][3] = __builtin_nontemporal_load((const vec_t *)(e + on + k * rowbytes));
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                vec_t r = v[cur][k][0];
+                if (R > 1) r ^= v[cur][k][1];
+                if (R > 2) r ^= v[cur][k][2];
+                if (R > 3) r ^= v[cur][k][3];
+                __builtin_nontemporal_store(r, (vec_t *)(y + o + k * rowbytes));
+                if (W > 1) __builtin_nontemporal_store(r ^ v[cur][k][0], (vec_t *)(z + o + k * rowbytes));
+                if (W > 2) __builtin_nontemporal_store(r ^ r, (vec_t *)(w + o + k * rowbytes));
+            }
+            o = on;
+        }
+    }
+}
+
 static hipEvent_t e0, e1;
 template <typename F> static void timeit(const char *name, double bytes, F launch)
 {
@@ -127,7 +178,42 @@ int main()
         // column blocks out of step with their neighbours
         tile(tile_kernel<512, 256, 4, 3>, 512, 256, 4, 3, 64, 1);
         tile(tile_kernel<512, 256, 4, 3>, 512, 256, 4, 3, 64, 5);
+        if (!pad) {
+            auto walk = [&](auto kern, int vb, int rd, int wr, int ts) {
+                const int ncvb = (int)((rowbytes / vb + 255) / 256), nseg = (int)(L / ts);
+                snprintf(nm, sizeof nm, "walk %dR%dW %2d B per lane, runs of %4d rows", rd, wr, vb, ts);
+                timeit(nm, (rd + wr) * n1, [&] { kern<<<(unsigned)(bs * nseg * ncvb), 256>>>(p[0], p[1], p[2], p[3], p[4], p[5], p[6], L, rowbytes, ncvb, nseg, ts); });
+            };
+            walk(walk_kernel<8, 3, 1>, 8, 3, 1, 128);
+            walk(walk_kernel<16, 3, 1>, 16, 3, 1, 128);
+            walk(walk_kernel<8, 4, 3>, 8, 4, 3, 128);
+            walk(walk_kernel<16, 4, 3>, 16, 4, 3, 128);
+        }
         for (int i = 0; i < 7; ++i) CK(hipFree(p[i]));
+    }
+    {   // the featurizer's tensors: (2, 8192, 12288) bf16, one read and one written (forward), two read and one written (backward)
+        const int64_t rowbytes = 3 * d * 2, bytes = bs * L * rowbytes;
+        char *p[3];
+        for (int i = 0; i < 3; ++i) { CK(hipMalloc(&p[i], bytes)); CK(hipMemset(p[i], i + 1, bytes)); }
+        const double n3 = (double)bytes;
+        char nm[128];
+        const int64_t n16 = bytes / 16;
+        u4 **q = (u4 **)p;
+        timeit("featurizer shape: flat 1R1W", 2 * n3, [&] { flat_kernel<1, 1, 0><<<8192, 256>>>(q[0], q[1], q[1], q[1], q[2], q[2], q[2], n16); });
+        timeit("featurizer shape: flat 1R1W nontemporal", 2 * n3, [&] { flat_kernel<1, 1, 1><<<8192, 256>>>(q[0], q[1], q[1], q[1], q[2], q[2], q[2], n16); });
+        timeit("featurizer shape: flat 2R1W nontemporal", 3 * n3, [&] { flat_kernel<2, 1, 1><<<8192, 256>>>(q[0], q[1], q[1], q[1], q[2], q[2], q[2], n16); });
+        auto walk = [&](auto kern, int vb, int rd, int wr, int ts) {
+            const int ncvb = (int)((rowbytes / vb + 255) / 256), nseg = (int)(L / ts);
+            snprintf(nm, sizeof nm, "featurizer shape: walk %dR%dW %2d B per lane, runs of %4d rows", rd, wr, vb, ts);
+            timeit(nm, (rd + wr) * n3, [&] { kern<<<(unsigned)(bs * nseg * ncvb), 256>>>(p[0], p[1], p[1], p[1], p[2], p[2], p[2], L, rowbytes, ncvb, nseg, ts); });
+        };
+        walk(walk_kernel<8, 1, 1>, 8, 1, 1, 128);
+        walk(walk_kernel<16, 1, 1>, 16, 1, 1, 128);
+        walk(walk_kernel<8, 2, 1>, 8, 2, 1, 128);
+        walk(walk_kernel<16, 2, 1>, 16, 2, 1, 128);
+        walk(walk_kernel<8, 1, 1>, 8, 1, 1, 1024);
+        walk(walk_kernel<8, 2, 1>, 8, 2, 1, 1024);
+        for (int i = 0; i < 3; ++i) CK(hipFree(p[i]));
     }
     return 0;
 }
