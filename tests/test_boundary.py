@@ -214,3 +214,25 @@ def test_workspace_sizing_runs_on_the_host_for_any_shape(gcg_lib):
         for kf in (1, 3, 4, 5):
             n = gcg_lib.gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, dt)
             assert n % 256 == 0 and (n > 0) == (hl <= 8 and kf <= 4 and dg % 2 == 0), (bs, L, g, dg, hl, kf, dt)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark measures one GPU: asking for more ends with a message, before any device is touched."""
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=300)
+    assert r.returncode != 0
+    assert "--gpus must be 1" in r.stderr + r.stdout
+    assert "{" not in r.stdout                       # no result line
+
+
+@pytest.mark.skipif(torch.cuda.is_available(), reason="checks the behaviour on a machine without a GPU")
+def test_bench_has_no_cpu_path():
+    import sys
+
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--steps", "1", "--warmup", "0"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0
+    assert "no GPU" in r.stderr + r.stdout
+    assert "{" not in r.stdout
