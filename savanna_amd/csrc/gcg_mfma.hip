@@ -223,7 +223,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     constexpr int OFF_H = OFF_D + STEP * YROW;              // filter tables
     constexpr int LDS_MAIN = OFF_H + NW * HTAB * (int)sizeof(hraw_t);
     constexpr int LDS_TAIL = NW * ND * 256 * 4;             // P tiles at the end
-    constexpr int LDS_BYTES = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
+    // A 4-wave workgroup at 16 bits asks for more than half of the CU's 160 KB, so that a CU holds one
+    // (two on a CU, two waves per SIMD, are a third slower than one).
+    constexpr int LDS_NEED = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
+    constexpr int LDS_ALONE = (NW == 4 && ES == 2) ? 82 * 1024 : 0;
+    constexpr int LDS_BYTES = LDS_NEED > LDS_ALONE ? LDS_NEED : LDS_ALONE;
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
     unsigned char *u_rm = smem + OFF_U, *g_rm = smem + OFF_G, *y_st = smem + OFF_Y, *d_st = smem + OFF_D;
     hraw_t *htab = (hraw_t *)(smem + OFF_H);
@@ -516,7 +520,7 @@ template <typename T, int NK, int NW>
 int bwd_launch(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
                void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
+    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4, false);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     hipLaunchKernelGGL((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
@@ -534,7 +538,7 @@ int bwd_nk(const void *dy, const void *x, const void *B, const void *C, const vo
            void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
     if constexpr (sizeof(T) == 2) {
-        if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+        if (choose_nw_bwd(dm, false, false) == 8) return bwd_launch<T, NK, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     }
     return bwd_launch<T, NK, 4>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
 }
@@ -556,8 +560,14 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
 
 size_t mfma_bwd_workspace(int dtype, const Dims &dm)
 {
-    const MfmaPlan p = plan_bwd(dm, dtype == GCG_F32);
-    return (size_t)p.nwg * p.nw * 128 * sizeof(float);
+    // one figure for gcg_bwd and gcg_bwd_interleaved, whose geometries differ
+    size_t n = 0;
+    for (bool il : {false, true}) {
+        const MfmaPlan p = plan_bwd(dm, dtype == GCG_F32, il);
+        const size_t need = (size_t)p.nwg * p.nw * 128 * sizeof(float);
+        if (need > n) n = need;
+    }
+    return n;
 }
 
 int mfma_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C, const void *h,

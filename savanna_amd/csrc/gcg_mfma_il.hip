@@ -3,7 +3,8 @@
 // dC, dB, dx in the same interleaved layout.
 //
 // The product side is the one of gcg_mfma.hip (same operand tiles, same order of operations,
-// so results agree bit for bit with the separate-tensor kernels).  The memory side differs: a
+// so y, dC, dB, dx agree bit for bit with the separate-tensor kernels, and dh up to the order in
+// which the runs' partial sums are added).  The memory side differs: a
 // row of the workgroup's 16*NW channels is 48*NW elements of (C, B, x) triples, and a lane
 // takes 12 bytes of it per row -- two channels at 16 bits, one at fp32 -- so that the 64 lanes
 // of a load or store cover one contiguous 768-byte run.  (Eight channels per lane, as in the
@@ -550,7 +551,7 @@ template <typename T, int NK, int NW>
 int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *ws, const Dims &dm,
                hipStream_t st)
 {
-    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
+    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4, true);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (dm.keep_out)
         hipLaunchKernelGGL((mfma_il_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
@@ -571,7 +572,7 @@ int bwd_nk(const void *dy, const void *feat, const void *h, void *dfeat, void *d
            hipStream_t st)
 {
     if constexpr (sizeof(T) == 2) {
-        if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, feat, h, dfeat, dh, ws, dm, st);
+        if (choose_nw_bwd(dm, false, true) == 8) return bwd_launch<T, NK, 8>(dy, feat, h, dfeat, dh, ws, dm, st);
     }
     return bwd_launch<T, NK, 4>(dy, feat, h, dfeat, dh, ws, dm, st);
 }

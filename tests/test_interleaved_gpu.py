@@ -162,8 +162,8 @@ def test_features_entry_point(gcg_lib):
     (1, 4096, 512, 16, 7, torch.float32),
 ], ids=["mr-7b-bf16", "se-40b-bf16", "mr-f32", "se-f32"])
 def test_benchmark_shapes_match_separate_tensors(gcg_lib, bs, L, g, dg, hl, dtype):
-    """Every element of y, d features and dh equals what the separate-tensor entry points give
-    (those are checked against the oracle at these shapes in test_fullsize_gpu.py)."""
+    """Every element of y and d features equals what the separate-tensor entry points give, and dh agrees
+    to its summation order (those are checked against the oracle at these shapes in test_fullsize_gpu.py)."""
     gen = torch.Generator(device=DEV).manual_seed(13)
     feat = torch.randn(bs, L, g, dg, 3, generator=gen, device=DEV).to(dtype)
     dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen, device=DEV)).to(dtype)
@@ -176,10 +176,9 @@ def test_benchmark_shapes_match_separate_tensors(gcg_lib, bs, L, g, dg, hl, dtyp
     torch.cuda.synchronize()
     assert torch.equal(y, y_p)
     assert torch.equal(dfeat[..., 0], dC) and torch.equal(dfeat[..., 1], dB) and torch.equal(dfeat[..., 2], dx)
-    if hl > 8:
-        assert torch.equal(dh, dh_p)
-    else:       # register-window kernels: lanes of another width sum dh in another order
-        assert_close(dh, dh_p, TOL_DH[dtype], "dh")
+    # dh: same terms, summed in another order -- the register-window kernels give a lane another width,
+    # and the two matrix-core backward kernels cut the sequence into runs of different length
+    assert_close(dh, dh_p, TOL_DH[dtype], "dh")
 
 
 def test_interleaved_64bit_offsets(gcg_lib):
