@@ -34,12 +34,57 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 # this script scaled by a 256 MiB copy in the same run (the repository keeps the profiler summary).
 # Counters cannot be read from inside the process; configurations without a profile report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("mr_fwdbwd_7b", "gcg_bwd hl=128 mfma"): 943801 * 1024,
-    ("mr_fwd_7b", "gcg_fwd hl=128 mfma"): 546674 * 1024,
+    ("mr_fwdbwd_7b", "gcg_bwd hl=128 mfma"): 926656 * 1024,
+    ("mr_fwd_7b", "gcg_fwd hl=128 mfma"): 547250 * 1024,
 }
 
 
 KEEP_INTERMEDIATES = True      # mixer workloads: the chain's two intermediates stored through the cache (--no-keep-output)
+
+
+class KernelEvents:
+    """Pairs of hipEvent_t for gcg_time_next_kernel: the runtime stamps a pair at the start and the end of one
+    kernel, so the elapsed time is that kernel's launch duration (what a profiler's kernel trace reports),
+    without the small reduction kernel and the dispatch gap that a bracket around the whole call also holds."""
+
+    def __init__(self, n):
+        import ctypes
+
+        path = None
+        with open("/proc/self/maps") as f:          # the HIP runtime this process already uses
+            for line in f:
+                if "libamdhip64" in line:
+                    path = line.split()[-1]
+                    break
+        if path is None:
+            raise RuntimeError("HIP runtime not loaded")
+        self.ct = ctypes
+        self.hip = ctypes.CDLL(path)
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+        self.pairs = []
+        for _ in range(n):
+            a, b = ctypes.c_void_p(), ctypes.c_void_p()
+            if self.hip.hipEventCreate(ctypes.byref(a)) or self.hip.hipEventCreate(ctypes.byref(b)):
+                raise RuntimeError("hipEventCreate failed")
+            self.pairs.append((a, b))
+
+    def mean_ms(self):
+        """Mean over the pairs, or None if one of them was never stamped."""
+        tot = 0.0
+        for a, b in self.pairs:
+            ms = self.ct.c_float()
+            if self.hip.hipEventElapsedTime(self.ct.byref(ms), a, b):
+                return None
+            tot += ms.value
+        return tot / len(self.pairs)
+
+    def close(self):
+        for a, b in self.pairs:
+            self.hip.hipEventDestroy(a)
+            self.hip.hipEventDestroy(b)
+        self.pairs = []
 
 
 class Op:
@@ -143,7 +188,8 @@ class Op:
             ev[1].record()
         return y
 
-    def run(self, ev=None):
+    def run(self, ev=None, kev=None):
+        """ev: torch events recorded around the dominant call; kev: a hipEvent_t pair armed for its main kernel."""
         t = self.sets[self.i % self.nsets]
         self.i += 1
         if self.layout.startswith("mixer"):
@@ -153,12 +199,16 @@ class Op:
         # kernel names: B = q, x = k, C = v
         if ev is not None and not self.backward:
             ev[0].record()
+        if kev is not None and not self.backward:
+            _lib.time_next_kernel(kev[0], kev[1])
         _, _, y = _lib.fwd(t["k"], t["q"], t["v"], t["h"])
         if ev is not None and not self.backward:
             ev[1].record()
         if self.backward:
             if ev is not None:
                 ev[0].record()
+            if kev is not None:
+                _lib.time_next_kernel(kev[0], kev[1])
             _lib.bwd(t["dy"], t["k"], t["q"], t["v"], t["h"])
             if ev is not None:
                 ev[1].record()
@@ -201,15 +251,24 @@ def time_workload(wl, device, steps, warmup, graph=False):
             op.run()
     torch.cuda.synchronize()
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    kevents = KernelEvents(steps) if wl.layout == "separate" else None
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(steps):
         for i, op in enumerate(ops):
-            op.run(events[k] if i == dom else None)
+            if i == dom:
+                op.run(events[k], kevents.pairs[k] if kevents else None)
+            else:
+                op.run()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / steps
-    kern_ms = sum(a.elapsed_time(b) for a, b in events) / steps
+    call_ms = sum(a.elapsed_time(b) for a, b in events) / steps      # bracket around the whole entry point
+    kern_ms = kevents.mean_ms() if kevents else None                 # the main kernel alone
+    if kevents:
+        kevents.close()
+    if kern_ms is None:
+        kern_ms = call_ms
     op = ops[dom]
     kern_bytes = op.bwd_bytes if op.backward else op.fwd_bytes
     kern_name = ("gcg_bwd" if op.backward else "gcg_fwd") + f" hl={op.hl} " + _lib.select_algo(
@@ -227,6 +286,7 @@ def time_workload(wl, device, steps, warmup, graph=False):
         "step_tflops": wl.algorithmic_flops() / (ms_per_step * 1e-3) / 1e12,
         "kernel": kern_name,
         "kernel_ms": kern_ms,
+        "call_ms": call_ms,
         "kernel_bytes": kern_bytes,
         "kernel_gbs": achieved,
         "kernel_hbm_frac": achieved / HBM_PEAK_GBS,
@@ -332,7 +392,7 @@ def main():
                    "step_mfma_frac": res["step_tflops"] / MFMA_BF16_PEAK_TFLOPS},
         "roofline": {"bound": "hbm", "kernel": res["kernel"], "achieved": res["kernel_gbs"],
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": res["kernel_hbm_frac"],
-                     "kernel_ms": res["kernel_ms"], "algorithmic_bytes": res["kernel_bytes"],
+                     "kernel_ms": res["kernel_ms"], "call_ms": res["call_ms"], "algorithmic_bytes": res["kernel_bytes"],
                      "traffic": MEASURED_TRAFFIC_BYTES.get((wl.name, res["kernel"]))},
     }
     if args.graph:

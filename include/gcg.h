@@ -67,6 +67,19 @@ GCG_API const char *gcg_strerror(int code);
  * thread (0 when none). */
 GCG_API int gcg_last_hip_error(void);
 
+/*
+ * Measurement hook; it has no counterpart in the reference.  Arms a pair of HIP events
+ * (hipEvent_t, created with timing enabled) on the calling thread.  The next gcg_fwd, gcg_bwd,
+ * gcg_fwd_interleaved or gcg_bwd_interleaved call on this thread that runs the register-window
+ * or matrix-core kernels has the runtime stamp the two events at the start and at the end of
+ * its main kernel -- not of the small filter-gradient reduction that follows a backward -- so
+ * that hipEventElapsedTime(start, stop) is that kernel's own duration, as a profiler reports
+ * it.  The arming lasts for one entry-point call: every entry point clears it on return,
+ * whether its launcher used the events or not.  Two null pointers disarm; one null pointer is
+ * GCG_ERR_BAD_ARG.
+ */
+GCG_API int gcg_time_next_kernel(void *start_event, void *stop_event);
+
 /* Library version, e.g. 100 for 0.1.0. */
 GCG_API int gcg_version(void);
 

@@ -23,7 +23,7 @@ _DTYPES = {torch.float32: GCG_F32, torch.bfloat16: GCG_BF16, torch.float16: GCG_
 
 # every symbol include/gcg.h declares
 EXPORTS = (
-    "gcg_strerror", "gcg_last_hip_error", "gcg_version", "gcg_fwd",
+    "gcg_strerror", "gcg_last_hip_error", "gcg_time_next_kernel", "gcg_version", "gcg_fwd",
     "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_select_algo",
     "gcg_fwd_interleaved", "gcg_bwd_interleaved",
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
@@ -56,6 +56,8 @@ def load() -> ctypes.CDLL:
         lib.gcg_strerror.restype = ctypes.c_char_p
         lib.gcg_last_hip_error.argtypes = []
         lib.gcg_last_hip_error.restype = ctypes.c_int
+        lib.gcg_time_next_kernel.argtypes = [vp, vp]
+        lib.gcg_time_next_kernel.restype = ctypes.c_int
         lib.gcg_version.argtypes = []
         lib.gcg_version.restype = ctypes.c_int
         lib.gcg_fwd.argtypes = [vp] * 7 + [i64, i64, i32, i32, i32, i32, i32, vp]
@@ -101,6 +103,12 @@ def algo_code(algo) -> int:
     if isinstance(algo, str):
         return ALGO_NAMES[algo]
     return int(algo)
+
+
+def time_next_kernel(start_event, stop_event) -> None:
+    """Arm two hipEvent_t handles (integers; timing enabled) for the next fwd / bwd / *_interleaved call on
+    this thread: the runtime stamps them at the start and the end of that call's main kernel."""
+    check(load().gcg_time_next_kernel(start_event, stop_event), "gcg_time_next_kernel")
 
 
 def check(rc: int, what: str) -> None:

@@ -7,6 +7,7 @@
 namespace {
 
 thread_local int tls_hip_error = 0;
+thread_local gcg::KernelTimer tls_timer = {nullptr, nullptr};
 
 // gfx950 check, cached per device ordinal.
 int check_device()
@@ -63,6 +64,7 @@ bool all_aligned16(std::initializer_list<const void *> ps)
 
 int finish(int hip_rc)
 {
+    tls_timer = {nullptr, nullptr};   // one entry point per arming, whether its launcher took the events or not
     if (hip_rc == 0) return GCG_OK;
     tls_hip_error = hip_rc;
     return GCG_ERR_LAUNCH;
@@ -77,6 +79,15 @@ template <typename P> P *at(P *p, size_t elems, int dtype)
 }
 
 } // namespace
+
+namespace gcg {
+KernelTimer take_kernel_timer()
+{
+    const KernelTimer t = tls_timer;
+    tls_timer = {nullptr, nullptr};
+    return t;
+}
+} // namespace gcg
 
 extern "C" {
 
@@ -95,7 +106,14 @@ GCG_API const char *gcg_strerror(int code)
 
 GCG_API int gcg_last_hip_error(void) { return tls_hip_error; }
 
-GCG_API int gcg_version(void) { return 105; }
+GCG_API int gcg_time_next_kernel(void *start_event, void *stop_event)
+{
+    if ((start_event == nullptr) != (stop_event == nullptr)) return GCG_ERR_BAD_ARG;
+    tls_timer = {(hipEvent_t)start_event, (hipEvent_t)stop_event};
+    return GCG_OK;
+}
+
+GCG_API int gcg_version(void) { return 106; }
 
 GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t backward)
 {

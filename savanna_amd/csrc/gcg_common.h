@@ -1,6 +1,7 @@
 // Shared device helpers for the gated chunked causal convolution kernels (gfx950).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "../../include/gcg.h"
@@ -189,6 +190,22 @@ constexpr int kWave = 64;
 // Host-side launchers, one translation unit per kernel family.  Each returns a
 // hipError_t as int; none of them allocates or synchronises.
 namespace gcg {
+
+// gcg_time_next_kernel: a pair of events the caller armed on this thread.  The launcher of an entry
+// point's main kernel takes them (once) and has the runtime stamp them at that kernel's own start
+// and end, so the elapsed time is the kernel's duration without the launches around it.
+struct KernelTimer { hipEvent_t start, stop; };
+KernelTimer take_kernel_timer();
+
+template <typename... KArgs, typename... Args>
+inline void launch_main(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t st, Args... args)
+{
+    const KernelTimer t = take_kernel_timer();
+    if (t.start && t.stop)
+        hipExtLaunchKernelGGL(kernel, grid, block, 0, st, t.start, t.stop, 0, static_cast<KArgs>(args)...);
+    else
+        hipLaunchKernelGGL(kernel, grid, block, 0, st, static_cast<KArgs>(args)...);
+}
 
 int direct_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h,
                       void *y, void *y2, void *bx, const Dims &dm, hipStream_t st);

@@ -520,7 +520,7 @@ int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStre
 {
     const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((mfma_il_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st, (const T *)feat,
+    launch_main((mfma_il_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)feat,
                        (const T *)h, (T *)y, dm, p);
     return (int)hipGetLastError();
 }
@@ -554,10 +554,10 @@ int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, voi
     const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4, true);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (dm.keep_out)
-        hipLaunchKernelGGL((mfma_il_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+        launch_main((mfma_il_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (float *)ws, dm, p);
     else
-        hipLaunchKernelGGL((mfma_il_bwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), 0, st,
+        launch_main((mfma_il_bwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (float *)ws, dm, p);
     int e = (int)hipGetLastError();
     if (e) return e;

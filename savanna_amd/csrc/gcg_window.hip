@@ -412,7 +412,7 @@ int fwd_v(const void *x, const void *B, const void *C, const void *h, void *y, v
         constexpr int VI = il_v<T>();
         const WinPlan p = plan(dm, VI);
         if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-        hipLaunchKernelGGL((window_fwd_kernel<T, HL, VI, true, false>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+        launch_main((window_fwd_kernel<T, HL, VI, true, false>), dim3((unsigned)p.nwg), dim3(p.threads), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
         return (int)hipGetLastError();
     }
@@ -420,10 +420,10 @@ int fwd_v(const void *x, const void *B, const void *C, const void *h, void *y, v
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (y2 || bx)
-        hipLaunchKernelGGL((window_fwd_kernel<T, HL, V, false, true>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+        launch_main((window_fwd_kernel<T, HL, V, false, true>), dim3((unsigned)nwg), dim3(p.threads), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     else
-        hipLaunchKernelGGL((window_fwd_kernel<T, HL, V, false, false>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+        launch_main((window_fwd_kernel<T, HL, V, false, false>), dim3((unsigned)nwg), dim3(p.threads), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     return (int)hipGetLastError();
 }
@@ -436,15 +436,15 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (dm.es == 3 && dm.keep_out)
-        hipLaunchKernelGGL((window_bwd_kernel<T, HL, il_v<T>(), true, true>), dim3((unsigned)nwg), dim3(p.threads), 0,
+        launch_main((window_bwd_kernel<T, HL, il_v<T>(), true, true>), dim3((unsigned)nwg), dim3(p.threads),
                            st, (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
     else if (dm.es == 3)
-        hipLaunchKernelGGL((window_bwd_kernel<T, HL, il_v<T>(), true, false>), dim3((unsigned)nwg), dim3(p.threads), 0,
+        launch_main((window_bwd_kernel<T, HL, il_v<T>(), true, false>), dim3((unsigned)nwg), dim3(p.threads),
                            st, (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
     else
-        hipLaunchKernelGGL((window_bwd_kernel<T, HL, BWD_V, false, false>), dim3((unsigned)nwg), dim3(p.threads), 0, st,
+        launch_main((window_bwd_kernel<T, HL, BWD_V, false, false>), dim3((unsigned)nwg), dim3(p.threads), st,
                            (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
     int e = (int)hipGetLastError();

@@ -149,3 +149,47 @@ def test_misaligned_tensors_take_the_direct_kernels(gcg_lib, dtype, hl):
     forced = "mfma" if hl > 8 else "window"
     with pytest.raises(_lib.GcgError, match="not supported"):
         _lib.fwd(xs, Bs, Cs, hd, algo=forced)
+
+
+def test_kernel_timer_hook(gcg_lib):
+    """gcg_time_next_kernel: the armed events are stamped by the next call's main kernel only, the arming lasts
+    one call, and results are what they are without it."""
+    import ctypes
+
+    hip = None
+    with open("/proc/self/maps") as f:
+        for line in f:
+            if "libamdhip64" in line:
+                hip = ctypes.CDLL(line.split()[-1])
+                break
+    assert hip is not None
+    hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+    hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+    hip.hipEventDestroy.argtypes = [ctypes.c_void_p]
+    a, b = ctypes.c_void_p(), ctypes.c_void_p()
+    assert hip.hipEventCreate(ctypes.byref(a)) == 0 and hip.hipEventCreate(ctypes.byref(b)) == 0
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(2, 2048, 16, 16, 128, torch.bfloat16, seed=3, dy_scale=0.1))
+    want = _lib.bwd(dy, x, B, C, h)
+    t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    assert gcg_lib.gcg_time_next_kernel(a, None) == -1             # one null pointer
+    _lib.time_next_kernel(a, b)
+    t0.record()
+    got = _lib.bwd(dy, x, B, C, h)
+    t1.record()
+    torch.cuda.synchronize()
+    ms = ctypes.c_float()
+    assert hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0
+    assert 0.0 < ms.value <= t0.elapsed_time(t1)                   # inside the bracket around the whole call
+    for g_, w_ in zip(got, want):
+        assert torch.equal(g_, w_)
+    # one call per arming: the next call leaves the events alone, and a forward takes them when armed again
+    before = ms.value
+    _lib.bwd(dy, x, B, C, h)
+    torch.cuda.synchronize()
+    assert hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0 and ms.value == before
+    _lib.time_next_kernel(a, b)
+    _lib.fwd(x, B, C, h)
+    torch.cuda.synchronize()
+    assert hip.hipEventElapsedTime(ctypes.byref(ms), a, b) == 0 and ms.value > 0.0
+    hip.hipEventDestroy(a)
+    hip.hipEventDestroy(b)
