@@ -88,13 +88,14 @@ class KernelEvents:
 
 
 class Op:
-    """One convolution of a workload with its resident inputs (rotated over `nsets` copies
-    when a single copy would sit in the 256 MB last-level cache)."""
+    """One convolution of a workload with its resident inputs, rotated over `nsets` copies so that
+    no step finds its inputs in the 256 MB last-level cache."""
 
     def __init__(self, wl, hl, device, rotate_bytes=512 << 20):
         n_in = 5 if wl.backward else 3
         set_bytes = n_in * wl.bs * wl.L * wl.d * wl.elem_bytes
-        self.nsets = int(max(1, min(64, -(-rotate_bytes // set_bytes))))
+        # at least two sets (up to 4 GB each): part of a single one is still in the last-level cache a step later
+        self.nsets = int(max(2 if set_bytes <= (4 << 30) else 1, min(64, -(-rotate_bytes // set_bytes))))
         self.sets = []
         big = wl.bs * wl.L * wl.d >= (1 << 31)
         for i in range(self.nsets):

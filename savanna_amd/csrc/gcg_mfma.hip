@@ -520,7 +520,7 @@ template <typename T, int NK, int NW>
 int bwd_launch(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
                void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4, false);
+    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     launch_main((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
@@ -538,7 +538,7 @@ int bwd_nk(const void *dy, const void *x, const void *B, const void *C, const vo
            void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
     if constexpr (sizeof(T) == 2) {
-        if (choose_nw_bwd(dm, false, false) == 8) return bwd_launch<T, NK, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+        if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     }
     return bwd_launch<T, NK, 4>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
 }
@@ -560,14 +560,8 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
 
 size_t mfma_bwd_workspace(int dtype, const Dims &dm)
 {
-    // one figure for gcg_bwd and gcg_bwd_interleaved, whose geometries differ
-    size_t n = 0;
-    for (bool il : {false, true}) {
-        const MfmaPlan p = plan_bwd(dm, dtype == GCG_F32, il);
-        const size_t need = (size_t)p.nwg * p.nw * 128 * sizeof(float);
-        if (need > n) n = need;
-    }
-    return n;
+    const MfmaPlan p = plan_bwd(dm, dtype == GCG_F32);
+    return (size_t)p.nwg * p.nw * 128 * sizeof(float);
 }
 
 int mfma_bwd_launch(int dtype, const void *dy, const void *x, const void *B, const void *C, const void *h,

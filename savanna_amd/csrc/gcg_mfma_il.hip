@@ -254,7 +254,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     constexpr int XB_VEC = G::NT * 16 * M::RW;              // one row vector of every lane
     constexpr int LDS_MAIN = OFF_XB + XB_SLOTS * 2 * XB_VEC;
     constexpr int LDS_TAIL = NW * ND * 256 * 4;             // P tiles at the end
-    constexpr int LDS_BYTES = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
+    // a 4-wave workgroup at 16 bits asks for more than half of the CU's 160 KB, so that a CU holds one
+    constexpr int LDS_NEED = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
+    constexpr int LDS_ALONE = (NW == 4 && M::ES == 2) ? 82 * 1024 : 0;
+    constexpr int LDS_BYTES = LDS_NEED > LDS_ALONE ? LDS_NEED : LDS_ALONE;
     static_assert(LDS_BYTES <= 160 * 1024, "workgroup exceeds the 160 KB of LDS");
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
     unsigned char *u_rm = smem + OFF_U, *g_rm = smem + OFF_G, *y_st = smem + OFF_Y, *d_st = smem + OFF_D;
@@ -551,7 +554,7 @@ template <typename T, int NK, int NW>
 int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *ws, const Dims &dm,
                hipStream_t st)
 {
-    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4, true);
+    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (dm.keep_out)
         launch_main((mfma_il_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
@@ -572,7 +575,7 @@ int bwd_nk(const void *dy, const void *feat, const void *h, void *dfeat, void *d
            hipStream_t st)
 {
     if constexpr (sizeof(T) == 2) {
-        if (choose_nw_bwd(dm, false, true) == 8) return bwd_launch<T, NK, 8>(dy, feat, h, dfeat, dh, ws, dm, st);
+        if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, feat, h, dfeat, dh, ws, dm, st);
     }
     return bwd_launch<T, NK, 4>(dy, feat, h, dfeat, dh, ws, dm, st);
 }

@@ -338,22 +338,23 @@ MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu, int elem_
 int nk_for(int hl) { const int n = (hl + 30) / 32 + 1; return n > 5 ? 5 : n; }
 
 // The backward holds about twice the forward's register state per wave (two waves per SIMD at
-// most).  Separate tensors: one wave per SIMD measured best -- 4-wave workgroups, one per CU,
-// with runs twice as long (half the lead-in) take 182 us where 8-wave workgroups take 206 at
-// (2, 8192, 4096), 686 against 755 at (1, 32768, 8192); two 4-wave workgroups sharing a CU are
-// slower than either (237 us), so the kernel's LDS request keeps a CU to one.  The
-// interleaved backward gains nothing from it and stays at 8 waves (128 channels, 768-byte rows).
-int choose_nw_bwd(const Dims &dm, bool fp32, bool interleaved)
+// most), and one wave per SIMD measured best: 4-wave workgroups, one per CU, with runs twice as
+// long (half the lead-in) take 176 us where 8-wave workgroups take 201 at (2, 8192, 4096) and 660
+// against 749 at (1, 32768, 8192); on interleaved operands 173 against 196 and 641 against 754.
+// Two 4-wave workgroups sharing a CU are slower than either (237 us), so the kernels' LDS
+// request keeps a CU to one.
+int choose_nw_bwd(const Dims &dm, bool fp32)
 {
+    (void)dm;
     static const int forced = env_int("GCG_MFMA_BWD_NW", 0);   // tuning override: 4 or 8
     if (forced == 4 || (forced == 8 && !fp32)) return forced;
-    return (interleaved && dm.d >= 128 && !fp32) ? 8 : 4;
+    return 4;
 }
 
-// one workgroup per CU in either geometry (fp32: one wave per SIMD as well, by its registers)
-MfmaPlan plan_bwd(const Dims &dm, bool fp32, bool interleaved)
+// one workgroup per CU in either geometry (fp32: one wave per SIMD by its registers alone)
+MfmaPlan plan_bwd(const Dims &dm, bool fp32)
 {
-    const int nw = choose_nw_bwd(dm, fp32, interleaved);
+    const int nw = choose_nw_bwd(dm, fp32);
     return plan(dm, nw, 16, nw, fp32 ? 4 : 2);
 }
 
