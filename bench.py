@@ -36,6 +36,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 MEASURED_TRAFFIC_BYTES = {
     ("mr_fwdbwd_7b", "gcg_bwd hl=128 mfma"): 926656 * 1024,
     ("mr_fwd_7b", "gcg_fwd hl=128 mfma"): 547250 * 1024,
+    ("se_mr_fwdbwd_40b", "gcg_bwd hl=128 mfma"): 3679015 * 1024,
 }
 
 
