@@ -74,9 +74,9 @@ GCG_API int gcg_last_hip_error(void);
  * or matrix-core kernels has the runtime stamp the two events at the start and at the end of
  * its main kernel -- not of the small filter-gradient reduction that follows a backward -- so
  * that hipEventElapsedTime(start, stop) is that kernel's own duration, as a profiler reports
- * it.  The arming lasts for one entry-point call: every entry point clears it on return,
- * whether its launcher used the events or not.  Two null pointers disarm; one null pointer is
- * GCG_ERR_BAD_ARG.
+ * it.  The arming lasts for one call: every entry point that launches kernels clears it on
+ * return, whatever it returns and whether its launcher used the events or not.  Two null
+ * pointers disarm; one null pointer is GCG_ERR_BAD_ARG.
  */
 GCG_API int gcg_time_next_kernel(void *start_event, void *stop_event);
 

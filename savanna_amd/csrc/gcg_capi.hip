@@ -9,6 +9,9 @@ namespace {
 thread_local int tls_hip_error = 0;
 thread_local gcg::KernelTimer tls_timer = {nullptr, nullptr};
 
+// an armed kernel timer lasts for one launching entry point, however that call ends
+struct TimerScope { ~TimerScope() { tls_timer = {nullptr, nullptr}; } };
+
 // gfx950 check, cached per device ordinal.
 int check_device()
 {
@@ -64,7 +67,6 @@ bool all_aligned16(std::initializer_list<const void *> ps)
 
 int finish(int hip_rc)
 {
-    tls_timer = {nullptr, nullptr};   // one entry point per arming, whether its launcher took the events or not
     if (hip_rc == 0) return GCG_OK;
     tls_hip_error = hip_rc;
     return GCG_ERR_LAUNCH;
@@ -127,6 +129,7 @@ GCG_API int gcg_fwd(const void *x, const void *B, const void *C, const void *h, 
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t algo,
             void *stream)
 {
+    TimerScope timer_scope;
     if (!x || !B || !C || !h || !y) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
@@ -166,6 +169,7 @@ GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C,
             void *dC, void *dh, void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g,
             int32_t dg, int32_t hl, int32_t dtype, int32_t algo, void *stream)
 {
+    TimerScope timer_scope;
     if (!dy || !x || !B || !C || !h || !dx || !dB || !dC || !dh) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
@@ -193,6 +197,7 @@ GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C,
 GCG_API int gcg_fwd_interleaved(const void *feat, const void *h, void *y, int64_t bs, int64_t L, int32_t g, int32_t dg,
                                 int32_t hl, int32_t dtype, int32_t algo, void *stream)
 {
+    TimerScope timer_scope;
     if (!feat || !h || !y) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
@@ -216,6 +221,7 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
                                 size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
                                 int32_t dtype, int32_t algo, int32_t flags, void *stream)
 {
+    TimerScope timer_scope;
     if (!dy || !feat || !h || !dfeat || !dh || (flags & ~GCG_KEEP_OUTPUT)) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
@@ -247,6 +253,7 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
 GCG_API int gcg_dwconv_fwd(const void *x, const void *w, void *y, int64_t bs, int64_t L, int32_t g, int32_t dg,
                            int32_t hl, int32_t dtype, int32_t flags, void *stream)
 {
+    TimerScope timer_scope;
     if (!x || !w || !y || (flags & ~GCG_KEEP_OUTPUT)) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
@@ -269,6 +276,7 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
                            size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
                            int32_t dtype, void *stream)
 {
+    TimerScope timer_scope;
     if (!dy || !x || !w || !dx || !dw) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
@@ -286,6 +294,7 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
 GCG_API int gcg_mixer_se_fwd(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L, int32_t g,
                              int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
 {
+    TimerScope timer_scope;
     if (!raw || !wf || !h || !y) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
@@ -309,6 +318,7 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
                              void *dh, void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g,
                              int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
 {
+    TimerScope timer_scope;
     if (!dy || !raw || !wf || !h || !draw || !dwf || !dh) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
@@ -327,6 +337,7 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
 GCG_API int gcg_filter_decay_fwd(const float *w, const float *decay, void *h, int32_t g, int32_t l_cache, int32_t hl,
                                  int32_t dtype, void *stream)
 {
+    TimerScope timer_scope;
     if (!w || !decay || !h || g <= 0 || hl <= 0 || l_cache < hl) return GCG_ERR_BAD_ARG;
     if (dtype != GCG_F32 && dtype != GCG_BF16 && dtype != GCG_F16) return GCG_ERR_BAD_ARG;
     const int rc = check_device();
@@ -337,6 +348,7 @@ GCG_API int gcg_filter_decay_fwd(const float *w, const float *decay, void *h, in
 GCG_API int gcg_filter_decay_bwd(const void *dh, const float *decay, float *dw, int32_t g, int32_t l_cache, int32_t hl,
                                  int32_t dtype, void *stream)
 {
+    TimerScope timer_scope;
     if (!dh || !decay || !dw || g <= 0 || hl <= 0 || l_cache < hl) return GCG_ERR_BAD_ARG;
     if (dtype != GCG_F32 && dtype != GCG_BF16 && dtype != GCG_F16) return GCG_ERR_BAD_ARG;
     const int rc = check_device();
