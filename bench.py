@@ -252,22 +252,23 @@ def time_workload(wl, device, steps, warmup, graph=False):
         for op in ops:
             op.run()
     torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    # the kernel-only events cost a few microseconds of launch time each: every fifth step carries a pair
+    # events cost a few microseconds of launch time and of GPU time each: every fifth step carries them
     stride = 5 if steps >= 25 else 2 if steps >= 4 else 1
-    kevents = KernelEvents(-(-steps // stride)) if wl.layout == "separate" else None
+    nsamp = -(-steps // stride)
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nsamp)]
+    kevents = KernelEvents(nsamp) if wl.layout == "separate" else None
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(steps):
         for i, op in enumerate(ops):
-            if i == dom:
-                op.run(events[k], kevents.pairs[k // stride] if kevents and k % stride == 0 else None)
+            if i == dom and k % stride == 0:
+                op.run(events[k // stride], kevents.pairs[k // stride] if kevents else None)
             else:
                 op.run()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / steps
-    call_ms = sum(a.elapsed_time(b) for a, b in events) / steps      # bracket around the whole entry point
+    call_ms = sum(a.elapsed_time(b) for a, b in events) / nsamp      # bracket around the whole entry point
     kern_ms = kevents.mean_ms() if kevents else None                 # the main kernel alone
     if kevents:
         kevents.close()
