@@ -317,17 +317,27 @@ MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu, int elem_
     p.ncb = (int)((dm.d + cb - 1) / cb);
     p.nsteps = (dm.L + STEP - 1) / STEP;
     const int wg_per_cu = waves_per_cu / nw > 0 ? waves_per_cu / nw : 1;
-    int64_t cols = dm.bs * p.ncb;
-    int64_t want = ((int64_t)cu_count() * wg_per_cu + cols - 1) / cols;   // segments to fill the chip
+    // Segments per (batch row, channel block): the count that needs the fewest step times.  With
+    // `slots` workgroups running at once the launch takes ceil(workgroups / slots) rounds of a run's
+    // steps plus its lead-in; e.g. 192 columns on 256 slots are better cut in 4 (3 rounds of 68
+    // steps) than in 2 (2 rounds of 132), and 128 columns in 2 (one round of 132).
+    const int64_t cols = dm.bs * p.ncb, slots = (int64_t)cu_count() * wg_per_cu;
     int64_t max_seg = p.nsteps / min_steps;
     if (max_seg < 1) max_seg = 1;
-    if (want > max_seg) want = max_seg;
-    if (want < 1) want = 1;
+    const int64_t lead = (dm.hl + 30) / 32 < 4 ? (dm.hl + 30) / 32 : 4;     // NK - 1 steps replayed by a later segment
+    int64_t cap = WIN_MAX_BYTES / (STEP * 3 * dm.d * elem_bytes) - 2 * 5;   // a run, with NK-1 steps either side, fits a window
+    if (cap < 1) cap = 1;
+    const int64_t n_min = (p.nsteps + cap - 1) / cap;                       // fewest segments the windows allow
+    int64_t want = n_min, best = -1;
+    for (int64_t n = n_min; (n <= max_seg || n == n_min) && n <= n_min + 4 * (slots / cols + 1); ++n) {
+        const int64_t rounds = (cols * n + slots - 1) / slots;
+        const int64_t cost = rounds * ((p.nsteps + n - 1) / n + (n > 1 ? lead : 0));
+        if (best < 0 || cost < best) { best = cost; want = n; }
+    }
     static const int forced = env_int("GCG_MFMA_STEPS_PER_SEG", 0);        // tuning override
     int64_t sps = (p.nsteps + want - 1) / want;
     if (forced > 0) sps = forced;
-    const int64_t cap = WIN_MAX_BYTES / (STEP * 3 * dm.d * elem_bytes) - 2 * 5;   // rows of NK-1 steps either side
-    if (sps > cap) sps = cap > 1 ? cap : 1;
+    if (sps > cap) sps = cap;
     p.steps_per_seg = (int)sps;
     p.nseg = (int)((p.nsteps + sps - 1) / sps);
     p.nwg = dm.bs * p.nseg * p.ncb;
