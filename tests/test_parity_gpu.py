@@ -46,6 +46,8 @@ SMALL = [
     (2, 5, 2, 16, 128),      # sequence shorter than one step and than the filter
     (1, 1, 1, 16, 7),        # a single row
     (1, 2049, 20, 16, 97),   # odd length, odd filter, d = 320
+    (3, 2500, 10, 16, 128),  # odd batch, ragged length: several runs per column and more than one round of workgroups
+    (5, 1111, 3, 16, 65),
 ]
 
 
