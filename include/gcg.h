@@ -76,7 +76,8 @@ GCG_API int gcg_last_hip_error(void);
  * that hipEventElapsedTime(start, stop) is that kernel's own duration, as a profiler reports
  * it.  The arming lasts for one call: every entry point that launches kernels clears it on
  * return, whatever it returns and whether its launcher used the events or not.  Two null
- * pointers disarm; one null pointer is GCG_ERR_BAD_ARG.
+ * pointers disarm; one null pointer is GCG_ERR_BAD_ARG.  Not for a stream that is being
+ * captured into a graph: a timed launch is not a plain kernel node.
  */
 GCG_API int gcg_time_next_kernel(void *start_event, void *stop_event);
 
