@@ -57,6 +57,26 @@ def test_wide_groups(gcg_lib, g, hl):
         check_groups_against_oracle(inp, y, grads, list(range(g)), dtype)
 
 
+@pytest.mark.parametrize("bs,L", [(3, 8192), (5, 4000)], ids=["b3", "b5-ragged"])
+def test_more_workgroups_than_fit_at_once(gcg_lib, bs, L):
+    """Batch sizes whose columns do not divide the CU count: the matrix-core kernels then cut the sequence so
+    that the launch takes several rounds of workgroups (768 and 1280 in the backward here).  Separate and
+    interleaved operands, groups against the oracle and dx against the other kernel family on every element."""
+    g, dg, hl, dtype = 256, 16, 128, torch.bfloat16
+    inp = make_inputs(bs, L, g, dg, hl, dtype, seed=bs, device=DEV)
+    _, _, y = _lib.fwd(inp["k"], inp["q"], inp["v"], inp["h"])
+    grads = _lib.bwd(inp["dy"], inp["k"], inp["q"], inp["v"], inp["h"])
+    check_groups_against_oracle(inp, y, grads, [0, 77, 255], dtype)
+    feat = torch.stack([inp["v"], inp["q"], inp["k"]], dim=-1).contiguous()
+    y_i = _lib.fwd_interleaved(feat, inp["h"])
+    dfeat, dh_i = _lib.bwd_interleaved(inp["dy"], feat, inp["h"])
+    assert torch.equal(y_i, y)
+    assert torch.equal(dfeat[..., 2], grads[0]) and torch.equal(dfeat[..., 1], grads[1]) and torch.equal(dfeat[..., 0], grads[2])
+    assert_close(dh_i, grads[3], TOL_DH[dtype], "dh interleaved")
+    direct = _lib.bwd(inp["dy"], inp["k"], inp["q"], inp["v"], inp["h"], algo="direct")
+    assert_close(grads[0], direct[0], TOL[dtype], "dx, matrix cores against vector ALUs")
+
+
 # ---- the benchmark configurations ------------------------------------------------------------------
 def test_mr_7b_delta_filter_bit_exact(gcg_lib):
     """h = e_{hl-1-s}: y[t] = C[t] * bf16(B*x)[t-s], every bit, at B=2 L=8192 D=4096."""
