@@ -90,7 +90,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     __shared__ __attribute__((aligned(16))) unsigned char y_st[STEP * YROW];
     __shared__ hraw_t htab[NW][HTAB];
 
-    int64_t wg = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    int64_t wg = pl.xcd ? xcd_contiguous_id(blockIdx.x, gridDim.x) : (int64_t)blockIdx.x;
     const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
     const int seg = (int)(wg % pl.nseg);
     const int64_t b = wg / pl.nseg;
@@ -521,8 +521,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
 template <typename T, int NK, int NW>
 int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
 {
-    const MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
+    MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    static const int order = env_int("GCG_MFMA_FWD_ORDER", -1);   // tuning override: 0 round-robin, 1 XCD-contiguous
+    p.xcd = order >= 0 ? (order != 0) : 1;
     launch_main((mfma_il_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)feat,
                        (const T *)h, (T *)y, dm, p);
     return (int)hipGetLastError();

@@ -250,7 +250,7 @@ template <typename T> __device__ __forceinline__ void stw_row(win_t w, uint32_t 
     for (int i = 0; i < MT<T>::RW; ++i) stw16(w, off + 16 * i, r.w[i]);
 }
 
-struct MfmaPlan { int ncb, nseg, steps_per_seg, nw; int64_t nsteps, nwg; };
+struct MfmaPlan { int ncb, nseg, steps_per_seg, nw, xcd; int64_t nsteps, nwg; };
 
 // Operand tile of the banded Toeplitz matrix at row offset doff = (out time) - (in time) of the
 // tile origins: element e of lane (j, q) is the tap for lag doff + j - kmap(q, e)  (MT<T>::toeplitz).
@@ -341,6 +341,7 @@ MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu, int elem_
     p.steps_per_seg = (int)sps;
     p.nseg = (int)((p.nsteps + sps - 1) / sps);
     p.nwg = dm.bs * p.nseg * p.ncb;
+    p.xcd = 1;
     return p;
 }
 
