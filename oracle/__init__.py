@@ -9,7 +9,6 @@ from .gcg_ref import (  # noqa: F401
     correction_toeplitz,
     gcg_bwd_oracle,
     gcg_bwd_ref_torch,
-    gcg_fwd_cpu_port_f32,
     gcg_fwd_oracle,
     gcg_fwd_ref_torch,
     gcg_two_pass_chunked_bwd,

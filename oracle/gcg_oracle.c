@@ -27,7 +27,8 @@
  * Pinned by tests/test_oracle.py against F.conv1d (the library routine the
  * reference calls), closed forms (delta taps, all-ones inputs), a brute-force
  * Python loop on tiny shapes, finite differences / the adjoint identity for the
- * gradients, and the two-pass Toeplitz form (oracle/two_pass.py).
+ * gradients, and the two-pass Toeplitz form
+ * (gcg_two_pass_chunked_fwd / _bwd in oracle/gcg_ref.py).
  *
  * Build: make -C oracle   (gcc -O2 -fopenmp -shared -fPIC)
  */
@@ -137,32 +138,6 @@ int gcg_oracle_bwd_f32(const float *dy, const float *x, const float *B, const fl
             dh[(size_t)gi * hl + k] = (float)s;
         }
     free(dh_col);
-    return 0;
-}
-
-/* ---- float I/O, float accumulation: the timed CPU port --------------------- */
-/* Same sums with single-precision accumulators, the arithmetic a CPU user of the
- * reference gets from F.conv1d in fp32.  Used only as a timing baseline. */
-int gcg_oracle_fwd_f32acc(const float *x, const float *B, const float *C, const float *h,
-                          float *y, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl)
-{
-    if (bs < 0 || L < 0 || g <= 0 || dg <= 0 || hl <= 0) return -1;
-    const int64_t d = (int64_t)g * dg;
-    const int64_t rows = bs * L;
-#pragma omp parallel for schedule(static)
-    for (int64_t r = 0; r < rows; ++r) {
-        const int64_t b = r / L, t = r % L;
-        const int64_t jmax = (t < hl - 1) ? t : hl - 1;
-        float *yr = y + IDX(b, t, 0);
-        for (int64_t c = 0; c < d; ++c) yr[c] = 0.f;
-        for (int64_t j = 0; j <= jmax; ++j) {
-            const float *xr = x + IDX(b, t - j, 0), *Br = B + IDX(b, t - j, 0);
-            for (int64_t c = 0; c < d; ++c)
-                yr[c] += h[(size_t)(c / dg) * hl + (hl - 1 - j)] * (Br[c] * xr[c]);
-        }
-        const float *Cr = C + IDX(b, t, 0);
-        for (int64_t c = 0; c < d; ++c) yr[c] *= Cr[c];
-    }
     return 0;
 }
 

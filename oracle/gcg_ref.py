@@ -44,8 +44,6 @@ def load_c_oracle() -> ctypes.CDLL:
     lib.gcg_oracle_fwd_f32.restype = ctypes.c_int
     lib.gcg_oracle_bwd_f32.argtypes = [f32p] * 9 + [i64, i64, i32, i32, i32]
     lib.gcg_oracle_bwd_f32.restype = ctypes.c_int
-    lib.gcg_oracle_fwd_f32acc.argtypes = [f32p] * 5 + [i64, i64, i32, i32, i32]
-    lib.gcg_oracle_fwd_f32acc.restype = ctypes.c_int
     lib.gcg_oracle_toeplitz_f64.argtypes = [f32p, i32, i32, f32p, f32p]
     lib.gcg_oracle_toeplitz_f64.restype = ctypes.c_int
     _LIB = lib
@@ -101,18 +99,6 @@ def gcg_bwd_oracle(dy, x, B, C, h):
     )
     assert rc == 0, rc
     return dx, dB, dC, dh
-
-
-def gcg_fwd_cpu_port_f32(x, B, C, h):
-    """Single-precision-accumulate forward (timing baseline only)."""
-    lib = load_c_oracle()
-    bs, L, g, dg, hl = _dims(x, h)
-    x_, B_, C_, h_ = _f32c(x), _f32c(B), _f32c(C), _f32c(h)
-    y = torch.empty_like(x_)
-    rc = lib.gcg_oracle_fwd_f32acc(x_.data_ptr(), B_.data_ptr(), C_.data_ptr(), h_.data_ptr(),
-                                   y.data_ptr(), bs, L, g, dg, hl)
-    assert rc == 0, rc
-    return y
 
 
 # ------------------------------------------------------------------- library formulation

@@ -4,6 +4,9 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
+#include <tuple>
+#include <utility>
+
 #include "../../include/gcg.h"
 
 namespace gcg {
@@ -197,14 +200,35 @@ namespace gcg {
 struct KernelTimer { hipEvent_t start, stop; };
 KernelTimer take_kernel_timer();
 
-template <typename... KArgs, typename... Args>
-inline void launch_main(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t st, Args... args)
+// Every launch returns the runtime's own code for that launch (hipLaunchKernel / hipExtLaunchKernel)
+// rather than the thread's sticky last error, so an error left behind by other code on the thread is
+// neither reported as this library's nor cleared from under its owner.
+template <typename... KArgs, size_t... I>
+inline int launch_packed(const void *fn, dim3 grid, dim3 block, hipStream_t st, const KernelTimer &t,
+                         std::tuple<KArgs...> &vals, std::index_sequence<I...>)
 {
-    const KernelTimer t = take_kernel_timer();
+    void *ptrs[] = {(void *)&std::get<I>(vals)...};
     if (t.start && t.stop)
-        hipExtLaunchKernelGGL(kernel, grid, block, 0, st, t.start, t.stop, 0, static_cast<KArgs>(args)...);
-    else
-        hipLaunchKernelGGL(kernel, grid, block, 0, st, static_cast<KArgs>(args)...);
+        return (int)hipExtLaunchKernel(fn, grid, block, ptrs, 0, st, t.start, t.stop, 0);
+    return (int)hipLaunchKernel(fn, grid, block, ptrs, 0, st);
+}
+
+// a small kernel beside the main one (reductions, filter generation): never timed
+template <typename... KArgs, typename... Args>
+inline int launch_plain(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t st, Args... args)
+{
+    std::tuple<KArgs...> vals{static_cast<KArgs>(args)...};
+    return launch_packed((const void *)kernel, grid, block, st, KernelTimer{nullptr, nullptr}, vals,
+                         std::index_sequence_for<KArgs...>{});
+}
+
+// an entry point's main kernel: carries the caller's event pair when one is armed
+template <typename... KArgs, typename... Args>
+inline int launch_main(void (*kernel)(KArgs...), dim3 grid, dim3 block, hipStream_t st, Args... args)
+{
+    std::tuple<KArgs...> vals{static_cast<KArgs>(args)...};
+    return launch_packed((const void *)kernel, grid, block, st, take_kernel_timer(), vals,
+                         std::index_sequence_for<KArgs...>{});
 }
 
 int direct_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h,

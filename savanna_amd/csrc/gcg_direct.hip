@@ -278,29 +278,30 @@ template <typename T>
 int fwd_t(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
           const Dims &dm, hipStream_t st)
 {
+    int e = 0;
     const int nct = (int)((dm.d + CT - 1) / CT), ntt = (int)((dm.L + TT - 1) / TT);
     const int64_t nwg = dm.bs * ntt * nct;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL(direct_fwd_kernel<T>, dim3((unsigned)nwg), dim3(256), 0, st, (const T *)x, (const T *)B,
+    e = launch_plain(direct_fwd_kernel<T>, dim3((unsigned)nwg), dim3(256), st, (const T *)x, (const T *)B,
                        (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, nct, ntt);
-    return (int)hipGetLastError();
+    return e;
 }
 
 template <typename T>
 int bwd_t(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
           void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
+    int e = 0;
     const BwdPlan p = plan_bwd(dm);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL(direct_bwd_kernel<T>, dim3((unsigned)p.nwg), dim3(256), 0, st, (const T *)dy,
+    e = launch_plain(direct_bwd_kernel<T>, dim3((unsigned)p.nwg), dim3(256), st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
                        (float *)ws, dm, p.nct, p.ntt, p.nseg, p.tps, p.gpt);
-    int e = (int)hipGetLastError();
     if (e) return e;
     const int64_t n = (int64_t)dm.g * dm.hl;
-    hipLaunchKernelGGL(direct_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+    e = launch_plain(direct_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
                        (const float *)ws, (T *)dh, dm, p.nct, p.nseg, p.gpt);
-    return (int)hipGetLastError();
+    return e;
 }
 
 } // namespace

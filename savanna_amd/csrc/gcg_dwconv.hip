@@ -235,26 +235,27 @@ DwPlan plan(const Dims &dm, int V)
 template <typename T, int HL, int V, bool PCF>
 int fwd_launch(const void *x, const void *w, void *y, const Dims &dm, hipStream_t st)
 {
+    int e = 0;
     const DwPlan p = plan(dm, V);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (dm.keep_out)
-        hipLaunchKernelGGL((dwconv_fwd_kernel<T, HL, V, PCF, true>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+        e = launch_plain((dwconv_fwd_kernel<T, HL, V, PCF, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
                            (const T *)x, (const T *)w, (T *)y, dm, p);
     else
-        hipLaunchKernelGGL((dwconv_fwd_kernel<T, HL, V, PCF, false>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+        e = launch_plain((dwconv_fwd_kernel<T, HL, V, PCF, false>), dim3((unsigned)p.nwg), dim3(p.threads), st,
                            (const T *)x, (const T *)w, (T *)y, dm, p);
-    return (int)hipGetLastError();
+    return e;
 }
 
 template <typename T, int HL, int V, bool PCF>
 int bwd_launch(const void *dy, const void *x, const void *w, void *dx, void *dw, void *ws, const Dims &dm,
                hipStream_t st)
 {
+    int e = 0;
     const DwPlan p = plan(dm, V);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL((dwconv_bwd_kernel<T, HL, V, PCF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+    e = launch_plain((dwconv_bwd_kernel<T, HL, V, PCF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
                        (const T *)dy, (const T *)x, (const T *)w, (T *)dx, (float *)ws, dm, p);
-    int e = (int)hipGetLastError();
     if (e) return e;
     // partials are ws[tap][(batch, run)][slot], slot = channel (per-channel filters) or lane
     return launch_colsum_reduce<T>((const float *)ws, (T *)dw, p.nrows, PCF ? dm.d : p.nvec, PCF ? dm.dg : dm.dg / V,

@@ -34,27 +34,29 @@ __global__ __launch_bounds__(256) void filter_bwd_kernel(const T *__restrict__ d
 int filter_fwd_launch(int dtype, const float *w, const float *decay, void *h, int g, int l_cache, int hl,
                       hipStream_t st)
 {
+    int e = 0;
     const unsigned nb = (unsigned)(((int64_t)g * hl + 255) / 256);
     switch (dtype) {
-    case GCG_F32:  hipLaunchKernelGGL(filter_fwd_kernel<float>, dim3(nb), dim3(256), 0, st, w, decay, (float *)h, g, l_cache, hl); break;
-    case GCG_BF16: hipLaunchKernelGGL(filter_fwd_kernel<bf16_t>, dim3(nb), dim3(256), 0, st, w, decay, (bf16_t *)h, g, l_cache, hl); break;
-    case GCG_F16:  hipLaunchKernelGGL(filter_fwd_kernel<f16_t>, dim3(nb), dim3(256), 0, st, w, decay, (f16_t *)h, g, l_cache, hl); break;
+    case GCG_F32:  e = launch_plain(filter_fwd_kernel<float>, dim3(nb), dim3(256), st, w, decay, (float *)h, g, l_cache, hl); break;
+    case GCG_BF16: e = launch_plain(filter_fwd_kernel<bf16_t>, dim3(nb), dim3(256), st, w, decay, (bf16_t *)h, g, l_cache, hl); break;
+    case GCG_F16:  e = launch_plain(filter_fwd_kernel<f16_t>, dim3(nb), dim3(256), st, w, decay, (f16_t *)h, g, l_cache, hl); break;
     default: return (int)hipErrorInvalidValue;
     }
-    return (int)hipGetLastError();
+    return e;
 }
 
 int filter_bwd_launch(int dtype, const void *dh, const float *decay, float *dw, int g, int l_cache, int hl,
                       hipStream_t st)
 {
+    int e = 0;
     const unsigned nb = (unsigned)(((int64_t)g * l_cache + 255) / 256);
     switch (dtype) {
-    case GCG_F32:  hipLaunchKernelGGL(filter_bwd_kernel<float>, dim3(nb), dim3(256), 0, st, (const float *)dh, decay, dw, g, l_cache, hl); break;
-    case GCG_BF16: hipLaunchKernelGGL(filter_bwd_kernel<bf16_t>, dim3(nb), dim3(256), 0, st, (const bf16_t *)dh, decay, dw, g, l_cache, hl); break;
-    case GCG_F16:  hipLaunchKernelGGL(filter_bwd_kernel<f16_t>, dim3(nb), dim3(256), 0, st, (const f16_t *)dh, decay, dw, g, l_cache, hl); break;
+    case GCG_F32:  e = launch_plain(filter_bwd_kernel<float>, dim3(nb), dim3(256), st, (const float *)dh, decay, dw, g, l_cache, hl); break;
+    case GCG_BF16: e = launch_plain(filter_bwd_kernel<bf16_t>, dim3(nb), dim3(256), st, (const bf16_t *)dh, decay, dw, g, l_cache, hl); break;
+    case GCG_F16:  e = launch_plain(filter_bwd_kernel<f16_t>, dim3(nb), dim3(256), st, (const f16_t *)dh, decay, dw, g, l_cache, hl); break;
     default: return (int)hipErrorInvalidValue;
     }
-    return (int)hipGetLastError();
+    return e;
 }
 
 } // namespace gcg

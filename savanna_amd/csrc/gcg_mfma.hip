@@ -456,6 +456,7 @@ template <typename T, int NK, int NW>
 int fwd_launch(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
                const Dims &dm, hipStream_t st)
 {
+    int e = 0;
     // 16-bit: ~112 registers, 4 waves per SIMD; fp32: ~200 registers, 2 waves per SIMD
     MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
@@ -465,12 +466,12 @@ int fwd_launch(const void *x, const void *B, const void *C, const void *h, void 
     static const int order = env_int("GCG_MFMA_FWD_ORDER", -1);   // tuning override: 0 round-robin, 1 XCD-contiguous
     p.xcd = order >= 0 ? (order != 0) : (p.ncb >= 32);
     if (y2 || bx)
-        launch_main((mfma_fwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+        e = launch_main((mfma_fwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     else
-        launch_main((mfma_fwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+        e = launch_main((mfma_fwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
-    return (int)hipGetLastError();
+    return e;
 }
 
 template <typename T, int NK>
@@ -525,17 +526,17 @@ template <typename T, int NK, int NW>
 int bwd_launch(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
                void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
+    int e = 0;
     const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    launch_main((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
+    e = launch_main((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
                        (float *)ws, dm, p);
-    int e = (int)hipGetLastError();
     if (e) return e;
     const int64_t n = (int64_t)dm.g * dm.hl;
-    hipLaunchKernelGGL(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+    e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
                        (const float *)ws, (T *)dh, dm, p);
-    return (int)hipGetLastError();
+    return e;
 }
 
 template <typename T, int NK>

@@ -521,13 +521,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
 template <typename T, int NK, int NW>
 int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
 {
+    int e = 0;
     MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     static const int order = env_int("GCG_MFMA_FWD_ORDER", -1);   // tuning override: 0 round-robin, 1 XCD-contiguous
     p.xcd = order >= 0 ? (order != 0) : 1;
-    launch_main((mfma_il_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)feat,
+    e = launch_main((mfma_il_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)feat,
                        (const T *)h, (T *)y, dm, p);
-    return (int)hipGetLastError();
+    return e;
 }
 
 template <typename T, int NK> int fwd_nk(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
@@ -556,20 +557,20 @@ template <typename T, int NK, int NW>
 int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *ws, const Dims &dm,
                hipStream_t st)
 {
+    int e = 0;
     const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (dm.keep_out)
-        launch_main((mfma_il_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+        e = launch_main((mfma_il_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (float *)ws, dm, p);
     else
-        launch_main((mfma_il_bwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+        e = launch_main((mfma_il_bwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (float *)ws, dm, p);
-    int e = (int)hipGetLastError();
     if (e) return e;
     const int64_t n = (int64_t)dm.g * dm.hl;
-    hipLaunchKernelGGL(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+    e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
                        (const float *)ws, (T *)dh, dm, p);
-    return (int)hipGetLastError();
+    return e;
 }
 
 template <typename T, int NK>

@@ -288,10 +288,14 @@ int cu_count()
     return n;
 }
 
+// tuning overrides from the environment: unset or empty -> dflt; any integer, 0 included, is taken
 int env_int(const char *name, int dflt)
 {
     const char *v = getenv(name);
-    return (v && atoi(v) > 0) ? atoi(v) : dflt;
+    if (!v || !*v) return dflt;
+    char *end = nullptr;
+    const long n = strtol(v, &end, 10);
+    return (end == v) ? dflt : (int)n;
 }
 
 // Waves per workgroup: wider workgroups read wider rows (16*NW channels, 32*NW bytes), which

@@ -831,32 +831,33 @@ int lane_channels(int dtype) { return dtype == GCG_F32 ? 1 : 2; }
 template <typename T, int HL, int KF>
 int fwd_launch(const void *raw, const void *wf, const void *h, void *y, const Dims &dm, int kf, hipStream_t st)
 {
+    int e = 0;
     const MixPlan p = plan(dm, Piece<T>::CH, false);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if constexpr (sizeof(T) == 2)
-        hipLaunchKernelGGL((mixer_se_fwd16_kernel<T, HL>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st, (const T *)raw,
+        e = launch_plain((mixer_se_fwd16_kernel<T, HL>), dim3((unsigned)p.nwg), dim3(p.threads), st, (const T *)raw,
                            (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
     else
-        hipLaunchKernelGGL((mixer_se_fwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+        e = launch_plain((mixer_se_fwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
                            (const T *)raw, (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
-    return (int)hipGetLastError();
+    return e;
 }
 
 template <typename T, int HL, int KF>
 int bwd_launch(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf, void *dh,
                void *ws, const Dims &dm, int kf, hipStream_t st)
 {
+    int e = 0;
     const MixPlan p = plan(dm, Piece<T>::CH, true);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     float *ws_h = (float *)ws;
     float *ws_w = ws_h + (size_t)dm.hl * p.nrows * p.nvec;
     if constexpr (sizeof(T) == 2)
-        hipLaunchKernelGGL((mixer_se_bwd16_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+        e = launch_plain((mixer_se_bwd16_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
                            (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
     else
-        hipLaunchKernelGGL((mixer_se_bwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), 0, st,
+        e = launch_plain((mixer_se_bwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
                            (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
-    int e = (int)hipGetLastError();
     if (e) return e;
     // both filter gradients in one launch
     const ColsumJob jh{ws_h, dh, p.nrows, p.nvec, dm.dg / p.ch, dm.g, dm.hl};

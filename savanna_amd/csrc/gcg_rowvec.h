@@ -167,18 +167,20 @@ template <typename T>
 inline int launch_colsum_reduce(const float *ws, T *out, int64_t nrow, int64_t ncol, int lpg, int nfilt, int ntap,
                                 hipStream_t st)
 {
+    int e = 0;
     const ColsumJob jb{ws, out, nrow, ncol, lpg, nfilt, ntap};
-    hipLaunchKernelGGL(colsum_reduce_kernel<T>, dim3(colsum_blocks(lpg, nfilt), (unsigned)ntap), dim3(256), 0, st, jb);
-    return (int)hipGetLastError();
+    e = launch_plain(colsum_reduce_kernel<T>, dim3(colsum_blocks(lpg, nfilt), (unsigned)ntap), dim3(256), st, jb);
+    return e;
 }
 
 template <typename T>
 inline int launch_colsum_reduce2(const ColsumJob &j0, const ColsumJob &j1, hipStream_t st)
 {
+    int e = 0;
     const unsigned nb0 = colsum_blocks(j0.lpg, j0.nfilt), nb1 = colsum_blocks(j1.lpg, j1.nfilt);
     const unsigned ny = (unsigned)(j0.ntap > j1.ntap ? j0.ntap : j1.ntap);
-    hipLaunchKernelGGL(colsum_reduce2_kernel<T>, dim3(nb0 + nb1, ny), dim3(256), 0, st, j0, j1, (int)nb0);
-    return (int)hipGetLastError();
+    e = launch_plain(colsum_reduce2_kernel<T>, dim3(nb0 + nb1, ny), dim3(256), st, j0, j1, (int)nb0);
+    return e;
 }
 
 } // namespace

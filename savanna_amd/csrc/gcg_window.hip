@@ -408,46 +408,47 @@ template <typename T, int HL, int V>
 int fwd_v(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
           const Dims &dm, hipStream_t st)
 {
+    int e = 0;
     if (dm.es == 3) {
         constexpr int VI = il_v<T>();
         const WinPlan p = plan(dm, VI);
         if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-        launch_main((window_fwd_kernel<T, HL, VI, true, false>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+        e = launch_main((window_fwd_kernel<T, HL, VI, true, false>), dim3((unsigned)p.nwg), dim3(p.threads), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
-        return (int)hipGetLastError();
+        return e;
     }
     const WinPlan p = plan(dm, V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (y2 || bx)
-        launch_main((window_fwd_kernel<T, HL, V, false, true>), dim3((unsigned)nwg), dim3(p.threads), st,
+        e = launch_main((window_fwd_kernel<T, HL, V, false, true>), dim3((unsigned)nwg), dim3(p.threads), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
     else
-        launch_main((window_fwd_kernel<T, HL, V, false, false>), dim3((unsigned)nwg), dim3(p.threads), st,
+        e = launch_main((window_fwd_kernel<T, HL, V, false, false>), dim3((unsigned)nwg), dim3(p.threads), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
-    return (int)hipGetLastError();
+    return e;
 }
 
 template <typename T, int HL>
 int bwd_t(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
           void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
+    int e = 0;
     const WinPlan p = plan(dm, dm.es == 3 ? il_v<T>() : BWD_V);
     const int64_t nwg = p.nwg;
     if (nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (dm.es == 3 && dm.keep_out)
-        launch_main((window_bwd_kernel<T, HL, il_v<T>(), true, true>), dim3((unsigned)nwg), dim3(p.threads),
+        e = launch_main((window_bwd_kernel<T, HL, il_v<T>(), true, true>), dim3((unsigned)nwg), dim3(p.threads),
                            st, (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
     else if (dm.es == 3)
-        launch_main((window_bwd_kernel<T, HL, il_v<T>(), true, false>), dim3((unsigned)nwg), dim3(p.threads),
+        e = launch_main((window_bwd_kernel<T, HL, il_v<T>(), true, false>), dim3((unsigned)nwg), dim3(p.threads),
                            st, (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
     else
-        launch_main((window_bwd_kernel<T, HL, BWD_V, false, false>), dim3((unsigned)nwg), dim3(p.threads), st,
+        e = launch_main((window_bwd_kernel<T, HL, BWD_V, false, false>), dim3((unsigned)nwg), dim3(p.threads), st,
                            (const T *)dy, (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB,
                            (T *)dC, (float *)ws, dm, p);
-    int e = (int)hipGetLastError();
     if (e) return e;
     // partials are ws[tap][(batch, run)][lane]; a filter owns dg / v adjacent lanes
     return launch_colsum_reduce<T>((const float *)ws, (T *)dh, dm.bs * p.nseg, p.nvec, dm.dg / p.v, dm.g, dm.hl, st);

@@ -196,7 +196,8 @@ def test_c_bwd_matches_autograd(bs, L, g, dg, hl):
 
 
 def test_c_bwd_matches_finite_differences():
-    """Central differences of <dy, y> in fp64 through the C forward (not autograd)."""
+    """The C backward against central differences of <dy, y>, y from the library-form forward evaluated in fp64
+    (plain function values: autograd is not involved)."""
     bs, L, g, dg, hl = 1, 12, 2, 2, 5
     x, B, C, h, dy = rand(bs, L, g, dg, hl, dtype=torch.float64)
     dx, dB, dC, dh = oracle.gcg_bwd_oracle(dy, x, B, C, h)
@@ -245,3 +246,8 @@ def test_bf16_rounding_helper():
     x, B, C, h, _ = rand(1, 20, 1, 2, 3, dtype=torch.float32)
     bx, _, _ = oracle.gcg_fwd_oracle(x, B, C, h, round_bx_bf16=True, return_intermediates=True)
     torch.testing.assert_close(bx, oracle.bf16_round(B * x))
+    # the rounded product also enters the sums: same y2, y as the plain oracle fed the rounded product as x with B = 1
+    _, y2r, yr = oracle.gcg_fwd_oracle(x, B, C, h, round_bx_bf16=True, return_intermediates=True)
+    _, y2p, yp = oracle.gcg_fwd_oracle(oracle.bf16_round(B * x), torch.ones_like(B), C, h, return_intermediates=True)
+    assert torch.equal(y2r, y2p) and torch.equal(yr, yp)
+    assert not torch.equal(y2r, oracle.gcg_fwd_oracle(x, B, C, h, return_intermediates=True)[1])
