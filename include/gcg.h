@@ -57,7 +57,8 @@ enum {
     GCG_ERR_UNSUPPORTED = -2, /* shape outside what the forced algo handles          */
     GCG_ERR_WORKSPACE   = -3, /* workspace missing or smaller than *_workspace_bytes */
     GCG_ERR_LAUNCH      = -4, /* hipLaunchKernel / stream error; see gcg_last_hip_error */
-    GCG_ERR_DEVICE      = -5  /* current device is not gfx950                        */
+    GCG_ERR_DEVICE      = -5, /* current device is not gfx950                        */
+    GCG_ERR_STATIC_SCRATCH = -6 /* gcg_bwd_static: sizes need more scratch than it holds */
 };
 
 /* Human-readable text for a code above. */
@@ -124,6 +125,29 @@ GCG_API size_t gcg_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t
 GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C, const void *h,
             void *dx, void *dB, void *dC, void *dh,
             void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, int32_t algo, void *stream);
+
+/*
+ * Backward for callers that cannot allocate.  It has no counterpart in the reference: it is
+ * gcg_bwd for code that runs where device memory cannot be obtained -- under HIP graph capture,
+ * in a tight serving loop, in a harness that forbids hipMalloc -- and so has no workspace to
+ * hand over.  The per-workgroup partial sums of dh go to a device array that is part of the
+ * library image (GCG_BWD_STATIC_SCRATCH_BYTES per GPU, held from the first call on that GPU until
+ * the process ends); the call itself allocates and frees nothing.  Same kernels, same order of
+ * summation, hence the same bits as gcg_bwd.
+ *
+ * Sizes whose gcg_bwd_workspace_bytes(...) exceeds GCG_BWD_STATIC_SCRATCH_BYTES are rejected with
+ * GCG_ERR_STATIC_SCRATCH (the Evo2-7B and 40B layer shapes need 0.5 MB on the matrix-core kernels and
+ * 3.5 and 7 MB on the register-window kernels).  All calls on one GPU share the one array: two calls that
+ * may overlap in time (different streams, different threads) race on it and must be ordered by the
+ * caller.  Nothing in it has to start at zero and nothing of a call's result stays in it.
+ * The first call on a GPU looks the array's address up, which may load the library's code onto that
+ * GPU; make that call before, not during, a graph capture.
+ */
+#define GCG_BWD_STATIC_SCRATCH_BYTES (8u << 20)
+GCG_API int gcg_bwd_static(const void *dy, const void *x, const void *B, const void *C, const void *h,
+            void *dx, void *dB, void *dC, void *dh,
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
             int32_t dtype, int32_t algo, void *stream);
 

@@ -24,7 +24,7 @@ _DTYPES = {torch.float32: GCG_F32, torch.bfloat16: GCG_BF16, torch.float16: GCG_
 # every symbol include/gcg.h declares
 EXPORTS = (
     "gcg_strerror", "gcg_last_hip_error", "gcg_time_next_kernel", "gcg_version", "gcg_fwd",
-    "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_select_algo",
+    "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_bwd_static", "gcg_select_algo",
     "gcg_fwd_interleaved", "gcg_bwd_interleaved",
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
@@ -66,6 +66,8 @@ def load() -> ctypes.CDLL:
         lib.gcg_bwd_workspace_bytes.restype = sz
         lib.gcg_bwd.argtypes = [vp] * 10 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_bwd.restype = ctypes.c_int
+        lib.gcg_bwd_static.argtypes = [vp] * 9 + [i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_bwd_static.restype = ctypes.c_int
         lib.gcg_select_algo.argtypes = [i64, i64, i32, i32, i32, i32, i32]
         lib.gcg_select_algo.restype = ctypes.c_int
         lib.gcg_fwd_interleaved.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, i32, vp]
@@ -196,6 +198,26 @@ def bwd(dy, x, B, C, h, algo=ALGO_AUTO):
         )
     check(rc, "gcg_bwd")
     return dx, dB, dC, dh
+
+
+STATIC_SCRATCH_BYTES = 8 << 20      # GCG_BWD_STATIC_SCRATCH_BYTES
+
+
+def bwd_static(dy, x, B, C, h, dx, dB, dC, dh, algo=ALGO_AUTO):
+    """gcg_bwd_static: the backward into the caller's output tensors with the library's built-in scratch
+    array instead of a workspace; nothing is allocated by the call (for callers under graph capture).
+    Calls that overlap on one GPU share the array and must be ordered by the caller."""
+    lib = load()
+    _require_gpu(x)
+    bs, L, g, dg = x.shape
+    with _on_device(x.device):
+        rc = lib.gcg_bwd_static(
+            dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(),
+            dx.data_ptr(), dB.data_ptr(), dC.data_ptr(), dh.data_ptr(),
+            bs, L, g, dg, h.shape[-1], dtype_code(x.dtype), algo_code(algo),
+            torch.cuda.current_stream().cuda_stream,
+        )
+    check(rc, "gcg_bwd_static")
 
 
 def _check_feat(feat, h):

@@ -74,6 +74,31 @@ int finish(int hip_rc)
 
 size_t elem_bytes(int dtype) { return dtype == GCG_F32 ? 4 : 2; }
 
+// Scratch of gcg_bwd_static: the filter-gradient partials live in this file-scope device array
+// instead of a caller's workspace.  Every GPU the library runs on holds its own copy from the
+// first use until the process ends.  `scratch` itself is only the host-side handle of the
+// symbol; the device address is looked up once per device and kernels are given that address.
+static __device__ __align__(256) unsigned char scratch[GCG_BWD_STATIC_SCRATCH_BYTES];
+
+int static_scratch(void **out)
+{
+    static std::mutex mu;
+    static void *ptr[64];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { tls_hip_error = (int)e; return GCG_ERR_LAUNCH; }
+    if (dev < 0 || dev >= 64) return GCG_ERR_DEVICE;
+    std::lock_guard<std::mutex> lk(mu);
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) { tls_hip_error = (int)e; return GCG_ERR_LAUNCH; }
+        ptr[dev] = p;
+    }
+    *out = ptr[dev];
+    return GCG_OK;
+}
+
 // pointer `elems` elements of `dtype` past p
 template <typename P> P *at(P *p, size_t elems, int dtype)
 {
@@ -102,6 +127,9 @@ GCG_API const char *gcg_strerror(int code)
     case GCG_ERR_WORKSPACE:   return "workspace missing, misaligned or too small";
     case GCG_ERR_LAUNCH:      return "HIP launch failed (see gcg_last_hip_error)";
     case GCG_ERR_DEVICE:      return "current device is not gfx950";
+    case GCG_ERR_STATIC_SCRATCH:
+        return "sizes need more filter-gradient scratch than gcg_bwd_static holds (GCG_BWD_STATIC_SCRATCH_BYTES); "
+               "use gcg_bwd with a workspace";
     }
     return "unknown error";
 }
@@ -188,6 +216,37 @@ GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C,
         return finish(gcg::window_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
     case GCG_ALGO_MFMA:
         return finish(gcg::mfma_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
+GCG_API int gcg_bwd_static(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx,
+                           void *dB, void *dC, void *dh, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                           int32_t dtype, int32_t algo, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !x || !B || !C || !h || !dx || !dB || !dC || !dh) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, x, B, C, dx, dB, dC}));
+    if (a < 0) return a;
+    const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
+    if (need == 0) return GCG_ERR_BAD_ARG;
+    if (need > (size_t)GCG_BWD_STATIC_SCRATCH_BYTES) return GCG_ERR_STATIC_SCRATCH;
+    rc = check_device();
+    if (rc) return rc;
+    void *ws = nullptr;
+    rc = static_scratch(&ws);
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (a) {
+    case GCG_ALGO_DIRECT:
+        return finish(gcg::direct_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st));
+    case GCG_ALGO_WINDOW:
+        return finish(gcg::window_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st));
+    case GCG_ALGO_MFMA:
+        return finish(gcg::mfma_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st));
     }
     return GCG_ERR_BAD_ARG;
 }

@@ -35,7 +35,7 @@ def test_header_and_library_agree(gcg_lib):
 def test_version_and_error_text(gcg_lib):
     assert gcg_lib.gcg_version() >= 100
     assert gcg_lib.gcg_strerror(0) == b"ok"
-    for code in (-1, -2, -3, -4, -5):
+    for code in (-1, -2, -3, -4, -5, -6):
         assert len(gcg_lib.gcg_strerror(code)) > 5
     assert gcg_lib.gcg_strerror(-99) == b"unknown error"
 
