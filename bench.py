@@ -1,14 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the gated chunked causal convolution on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--all]
 
 A step is one pass of the hot path over one batch of synthetic input that is already
 resident in HBM: forward, plus backward for the forward+backward workloads.  The default
 workload is the one the headline metric is quoted on (Hyena-MR forward+backward at the
 Evo2-7B layer shape).  One JSON line is printed; it carries the whole-job throughput in
 tokens/s, the roofline position of the dominant kernel (algorithmic bytes over the HIP-event
-duration of that launch) and a CPU baseline timed on the host cores in the same run.
+duration of that launch), the same figures for the other four configurations (`all_configs`;
+`--only` leaves them out) and a CPU baseline timed on the host cores in the same run.
 """
 from __future__ import annotations
 
@@ -25,19 +26,26 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 from savanna_amd import _lib  # noqa: E402
-from savanna_amd.synthetic import WORKLOAD_ORDER, WORKLOADS, make_inputs, make_inputs_device  # noqa: E402
+from savanna_amd.synthetic import WORKLOAD_ORDER, WORKLOADS, make_inputs, make_inputs_device  # noqa: E402,F401
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # dense bf16, published
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this script scaled by a 256 MiB copy in the same run (the repository keeps the profiler summary).
-# Counters cannot be read from inside the process; configurations without a profile report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("mr_fwdbwd_7b", "gcg_bwd hl=128 mfma"): 926656 * 1024,
-    ("mr_fwd_7b", "gcg_fwd hl=128 mfma"): 547250 * 1024,
-    ("se_mr_fwdbwd_40b", "gcg_bwd hl=128 mfma"): 3679015 * 1024,
-}
+# HBM bytes per launch of the dominant kernel as counted by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script (scaled by a plain copy of known size in the same run).  Counters cannot be read from inside the process, so
+# the figures are kept in a data file that is rewritten whenever the counter profile is; a workload without an
+# entry (or a checkout without the file) reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+
+
+def measured_traffic(workload, kernel):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        return None
+    entry = table.get(workload, {}).get(kernel)
+    return entry["bytes"] if entry else None
 
 
 KEEP_INTERMEDIATES = True      # mixer workloads: the chain's two intermediates stored through the cache (--no-keep-output)
@@ -71,15 +79,16 @@ class KernelEvents:
                 raise RuntimeError("hipEventCreate failed")
             self.pairs.append((a, b))
 
-    def mean_ms(self):
-        """Mean over the pairs, or None if one of them was never stamped."""
+    def mean_ms(self, which=None):
+        """Mean over the pairs (or those with the given indices), or None if one of them was never stamped."""
+        pairs = self.pairs if which is None else [self.pairs[i] for i in which]
         tot = 0.0
-        for a, b in self.pairs:
+        for a, b in pairs:
             ms = self.ct.c_float()
             if self.hip.hipEventElapsedTime(self.ct.byref(ms), a, b):
                 return None
             tot += ms.value
-        return tot / len(self.pairs)
+        return tot / len(pairs)
 
     def close(self):
         for a, b in self.pairs:
@@ -98,14 +107,9 @@ class Op:
         # at least two sets (up to 4 GB each): part of a single one is still in the last-level cache a step later
         self.nsets = int(max(2 if set_bytes <= (4 << 30) else 1, min(64, -(-rotate_bytes // set_bytes))))
         self.sets = []
-        big = wl.bs * wl.L * wl.d >= (1 << 31)
         for i in range(self.nsets):
-            if big:
-                t = make_inputs_device(wl.bs, wl.L, wl.g, wl.dg, hl, wl.dtype, device, seed=i,
-                                       with_dy=wl.backward)
-            else:
-                t = make_inputs(wl.bs, wl.L, wl.g, wl.dg, hl, wl.dtype, seed=i, device=device,
-                                with_dy=wl.backward)
+            # drawn on the device (same distributions as the CPU recipe; the values are not compared here)
+            t = make_inputs_device(wl.bs, wl.L, wl.g, wl.dg, hl, wl.dtype, device, seed=i, with_dy=wl.backward)
             if wl.layout == "dwconv":
                 t = {"x": t["k"], "h": t["h"], "dy": t.get("dy")}
             elif wl.layout.startswith("mixer"):
@@ -252,24 +256,37 @@ def time_workload(wl, device, steps, warmup, graph=False):
         for op in ops:
             op.run()
     torch.cuda.synchronize()
-    # events cost a few microseconds of launch time and of GPU time each: every fifth step carries them
-    stride = 5 if steps >= 25 else 2 if steps >= 4 else 1
-    nsamp = -(-steps // stride)
+    # A step that carries events costs 10-15 us more than a plain one (two event records, and a timed launch is
+    # more than a kernel packet), so only a few steps of the timed region carry them; the same instrumented step
+    # is then repeated after the timed region for a steadier mean.  Both sample sets are reported.
+    n_in = min(4, steps)
+    marks = {(steps * (2 * j + 1)) // (2 * n_in): j for j in range(n_in)}       # spread over the region, not step 0
+    n_after = min(16, max(4, steps))
+    nsamp = n_in + n_after
     events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nsamp)]
     kevents = KernelEvents(nsamp) if wl.layout == "separate" else None
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(steps):
+        j = marks.get(k)
         for i, op in enumerate(ops):
-            if i == dom and k % stride == 0:
-                op.run(events[k // stride], kevents.pairs[k // stride] if kevents else None)
+            if i == dom and j is not None:
+                op.run(events[j], kevents.pairs[j] if kevents else None)
             else:
                 op.run()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / steps
+    for j in range(n_in, nsamp):
+        for i, op in enumerate(ops):
+            if i == dom:
+                op.run(events[j], kevents.pairs[j] if kevents else None)
+            else:
+                op.run()
+    torch.cuda.synchronize()
     call_ms = sum(a.elapsed_time(b) for a, b in events) / nsamp      # bracket around the whole entry point
     kern_ms = kevents.mean_ms() if kevents else None                 # the main kernel alone
+    kern_ms_in = kevents.mean_ms(range(n_in)) if kevents else None
     if kevents:
         kevents.close()
     if kern_ms is None:
@@ -291,6 +308,8 @@ def time_workload(wl, device, steps, warmup, graph=False):
         "step_tflops": wl.algorithmic_flops() / (ms_per_step * 1e-3) / 1e12,
         "kernel": kern_name,
         "kernel_ms": kern_ms,
+        "kernel_ms_timed_region": kern_ms_in,
+        "kernel_samples": {"timed_region": n_in, "after": n_after},
         "call_ms": call_ms,
         "kernel_bytes": kern_bytes,
         "kernel_gbs": achieved,
@@ -329,11 +348,12 @@ def cpu_baseline(wl, budget_s=20.0):
 
     once(g_s)                                   # warm-up (thread pool, mkldnn primitives)
     dt = once(g_s)
-    # grow the sample towards the budget, keep at least two timed runs
-    while g_s * 2 <= wl.g and dt * 2 * 3 < budget_s:
+    # grow the sample until three timed runs of it fill the budget
+    while g_s * 2 <= wl.g and dt * 2 * 4 < budget_s:
         g_s *= 2
         dt = once(g_s)
-    dt = min(dt, once(g_s))
+    runs = sorted([dt, once(g_s), once(g_s)])
+    dt = runs[1]                                # median of three
     tokens_per_s = L / dt * (g_s / wl.g) / len(wl.filters)
     return {
         "value": tokens_per_s,
@@ -341,7 +361,7 @@ def cpu_baseline(wl, budget_s=20.0):
         "cores": threads,
         "kind": "port",
         "sample": f"1 batch row x {L} tokens x {g_s * wl.dg} of {wl.d} channels, hl={hl}, fp32, "
-                  f"{'fwd+bwd' if wl.backward else 'fwd'}; best of 2; scaled linearly to {wl.d} channels"
+                  f"{'fwd+bwd' if wl.backward else 'fwd'}; median of 3 runs; scaled linearly to {wl.d} channels"
                   + (f" and {len(wl.filters)} ops" if len(wl.filters) > 1 else ""),
     }
 
@@ -352,7 +372,9 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="mr_fwdbwd_7b", choices=list(WORKLOADS))
-    ap.add_argument("--all", action="store_true", help="also time the other four configurations")
+    ap.add_argument("--only", action="store_true", help="time the chosen workload alone (no all_configs block)")
+    ap.add_argument("--all", action="store_true", help="also time the rows next to the hot path (interleaved "
+                                                       "features, featurizer conv, mixer chains)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-keep-output", action="store_true",
                     help="mixer workloads: store the chain's intermediates past the cache like every other output")
@@ -398,20 +420,28 @@ def main():
         "roofline": {"bound": "hbm", "kernel": res["kernel"], "achieved": res["kernel_gbs"],
                      "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": res["kernel_hbm_frac"],
                      "kernel_ms": res["kernel_ms"], "call_ms": res["call_ms"], "algorithmic_bytes": res["kernel_bytes"],
-                     "traffic": MEASURED_TRAFFIC_BYTES.get((wl.name, res["kernel"]))},
+                     "kernel_ms_timed_region": res["kernel_ms_timed_region"], "kernel_samples": res["kernel_samples"],
+                     "traffic": measured_traffic(wl.name, res["kernel"])},
     }
     if args.graph:
         line["graph"] = {k: res[k] for k in ("graph_ms_per_step", "graph_tokens_per_s", "graph_hbm_frac")}
-    if args.all:
+    if not args.only:
+        # the other four configurations, each with its own roofline position (fewer steps where a step is long)
         others = {}
         for name in WORKLOAD_ORDER:
             if name == wl.name:
                 continue
             w = WORKLOADS[name]
-            k = args.steps if w.bs * w.L * w.d < (1 << 30) else max(3, args.steps // 10)
+            n = w.bs * w.L * w.d
+            k = max(100, args.steps) if n < (1 << 22) else args.steps if n < (1 << 28) else \
+                max(5, args.steps // 2) if n < (1 << 30) else 3
             small = w.algorithmic_bytes() < (64 << 20)       # launch-bound: also report graph replay
-            others[name] = time_workload(w, device, k, max(2, args.warmup // 2), graph=small)
+            r = time_workload(w, device, k, max(2, min(args.warmup, k // 2)), graph=small)
+            r["steps"] = k
+            r["traffic"] = measured_traffic(w.name, r["kernel"])
+            others[name] = r
         line["all_configs"] = others
+    if args.all:
         # the rows next to the hot path: the operator fed from the interleaved projected features, the
         # featurizer conv, and the two chained through autograd
         extra = {}

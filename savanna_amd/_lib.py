@@ -1,7 +1,10 @@
-"""ctypes binding of libgcg_hip.so (C ABI: include/gcg.h).
+"""Python entry points of the kernels in libgcg_hip.so (C ABI: include/gcg.h).
 
-There is no CPU or PyTorch fallback: if the library is missing, or a call fails,
-an exception is raised.
+Two bindings of the same library: the ``torch.ops.gcg`` operators of the PyTorch extension
+(``_ops``; used whenever it is built, traceable by ``torch.compile``) and a plain ctypes binding
+(``load()``; host-side queries, the entry points that take caller-owned outputs, and every call
+when the extension is absent).  There is no CPU or PyTorch fallback: if the library is missing,
+or a call fails, an exception is raised.
 """
 from __future__ import annotations
 
@@ -10,6 +13,8 @@ import os
 import threading
 
 import torch
+
+from . import _ops
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 # GCG_HIP_LIB points at another build of the same library (e.g. a tuning variant)
@@ -33,10 +38,12 @@ EXPORTS = (
 
 _lock = threading.Lock()
 _lib = None
+TORCH_OPS = _ops.AVAILABLE          # calls go through torch.ops.gcg (else through ctypes)
 
 
 class GcgError(RuntimeError):
-    """A gcg_* entry point returned a negative code."""
+    """A gcg_* entry point returned a negative code (ctypes binding; the torch operators raise a plain
+    RuntimeError with the same text)."""
 
 
 def load() -> ctypes.CDLL:
@@ -150,13 +157,24 @@ def _require_gpu(t: torch.Tensor) -> None:
 def fwd(x, B, C, h, return_bx=False, return_y2=False, algo=ALGO_AUTO, out=None):
     """y (and optionally bx, y2) for contiguous (bs, L, g, dg) inputs and (g, 1, hl) filter.
     ``out``: optional pre-allocated contiguous tensor of x's shape, dtype and device for y."""
-    lib = load()
     _require_gpu(x)
-    bs, L, g, dg = x.shape
-    hl = h.shape[-1]
     if out is not None:
         if out.shape != x.shape or out.dtype != x.dtype or out.device != x.device or not out.is_contiguous():
             raise ValueError("out must be a contiguous tensor with the shape, dtype and device of x")
+    if TORCH_OPS:
+        a = algo_code(algo)
+        if out is not None and not (return_bx or return_y2):
+            torch.ops.gcg.fwd_out(x, B, C, h, out, a)
+            return None, None, out
+        if not (return_bx or return_y2):
+            return None, None, torch.ops.gcg.fwd(x, B, C, h, a)
+        bx, y2, y = torch.ops.gcg.fwd_full(x, B, C, h, return_bx, return_y2, a)
+        if out is not None:
+            y = out.copy_(y)
+        return (bx if return_bx else None), (y2 if return_y2 else None), y
+    lib = load()
+    bs, L, g, dg = x.shape
+    hl = h.shape[-1]
     y = out if out is not None else torch.empty_like(x)
     y2 = torch.empty_like(x) if return_y2 else None
     bx = torch.empty_like(x) if return_bx else None
@@ -176,8 +194,10 @@ def fwd(x, B, C, h, return_bx=False, return_y2=False, algo=ALGO_AUTO, out=None):
 
 def bwd(dy, x, B, C, h, algo=ALGO_AUTO):
     """(dx, dB, dC, dh) for contiguous inputs; dh has h's shape and dtype."""
-    lib = load()
     _require_gpu(x)
+    if TORCH_OPS:
+        return torch.ops.gcg.bwd(dy, x, B, C, h, algo_code(algo))
+    lib = load()
     bs, L, g, dg = x.shape
     hl = h.shape[-1]
     dx, dB, dC = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
@@ -231,8 +251,10 @@ def _check_feat(feat, h):
 
 def fwd_interleaved(feat, h, algo=ALGO_AUTO, out=None):
     """y (bs, L, g, dg) for feat (bs, L, g, dg, 3) with feat[..., 0] = C, [..., 1] = B, [..., 2] = x."""
-    lib = load()
     _require_gpu(feat)
+    if TORCH_OPS and out is None:
+        return torch.ops.gcg.fwd_interleaved(feat, h, algo_code(algo))
+    lib = load()
     _check_feat(feat, h)
     bs, L, g, dg, _ = feat.shape
     hl = h.shape[-1]
@@ -257,8 +279,10 @@ KEEP_OUTPUT = 1       # GCG_KEEP_OUTPUT
 def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO, keep_output=False):
     """(dfeat, dh): dfeat has feat's layout, dfeat[..., 0] = dC, [..., 1] = dB, [..., 2] = dx.
     ``keep_output``: dfeat goes to dwconv_bwd next, store it through the cache."""
-    lib = load()
     _require_gpu(feat)
+    if TORCH_OPS:
+        return torch.ops.gcg.bwd_interleaved(dy, feat, h, algo_code(algo), bool(keep_output))
+    lib = load()
     _check_feat(feat, h)
     bs, L, g, dg, _ = feat.shape
     hl = h.shape[-1]
@@ -294,8 +318,10 @@ def _check_dwconv(x, w):
 def dwconv_fwd(x, w, keep_output=False):
     """y = causal depthwise convolution of x (bs, L, g, dg) with w (g, 1, hl), no gates.
     ``keep_output``: y goes to fwd_interleaved next, store it through the cache."""
-    lib = load()
     _require_gpu(x)
+    if TORCH_OPS:
+        return torch.ops.gcg.dwconv_fwd(x, w, bool(keep_output))
+    lib = load()
     _check_dwconv(x, w)
     bs, L, g, dg = x.shape
     y = torch.empty_like(x)
@@ -311,8 +337,10 @@ def dwconv_fwd(x, w, keep_output=False):
 
 def dwconv_bwd(dy, x, w):
     """(dx, dw) of dwconv_fwd."""
-    lib = load()
     _require_gpu(x)
+    if TORCH_OPS:
+        return torch.ops.gcg.dwconv_bwd(dy, x, w)
+    lib = load()
     _check_dwconv(x, w)
     if dy.shape != x.shape or dy.dtype != x.dtype or not dy.is_contiguous():
         raise ValueError("dy must be a contiguous tensor of x's shape and dtype")
@@ -349,8 +377,10 @@ def _check_mixer_se(raw, wf, h):
 
 def mixer_se_fwd(raw, wf, h):
     """y (bs, L, g, dg) = fwd_interleaved(dwconv_fwd(raw, wf), h) in one pass over raw (bs, L, g, dg, 3)."""
-    lib = load()
     _require_gpu(raw)
+    if TORCH_OPS:
+        return torch.ops.gcg.mixer_se_fwd(raw, wf, h)
+    lib = load()
     _check_mixer_se(raw, wf, h)
     bs, L, g, dg, _ = raw.shape
     y = torch.empty(bs, L, g, dg, dtype=raw.dtype, device=raw.device)
@@ -366,8 +396,10 @@ def mixer_se_fwd(raw, wf, h):
 
 def mixer_se_bwd(dy, raw, wf, h):
     """(draw, dwf, dh) of mixer_se_fwd."""
-    lib = load()
     _require_gpu(raw)
+    if TORCH_OPS:
+        return torch.ops.gcg.mixer_se_bwd(dy, raw, wf, h)
+    lib = load()
     _check_mixer_se(raw, wf, h)
     bs, L, g, dg, _ = raw.shape
     if dy.shape != (bs, L, g, dg) or dy.dtype != raw.dtype or not dy.is_contiguous() or dy.device != raw.device:
@@ -400,8 +432,10 @@ def _check_filter_params(w, decay):
 
 def filter_decay_fwd(w, decay, hl: int, dtype: torch.dtype):
     """h (g, 1, hl) in ``dtype`` = w[:, :hl] * decay[:, :hl]."""
-    lib = load()
     _require_gpu(w)
+    if TORCH_OPS:
+        return torch.ops.gcg.filter_decay_fwd(w, decay, hl, dtype)
+    lib = load()
     _check_filter_params(w, decay)
     g, l_cache = w.shape
     if not 0 < hl <= l_cache:
@@ -416,8 +450,10 @@ def filter_decay_fwd(w, decay, hl: int, dtype: torch.dtype):
 
 def filter_decay_bwd(dh, decay):
     """dw (g, L_cache) fp32 from dh (g, 1, hl)."""
-    lib = load()
     _require_gpu(dh)
+    if TORCH_OPS:
+        return torch.ops.gcg.filter_decay_bwd(dh, decay)
+    lib = load()
     _check_filter_params(decay, decay)
     g, l_cache = decay.shape
     if dh.dim() != 3 or dh.shape[0] != g or dh.shape[1] != 1 or dh.shape[2] > l_cache or not dh.is_contiguous():

@@ -207,7 +207,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                                                        const T *__restrict__ B, const T *__restrict__ C,
                                                        const T *__restrict__ h, T *__restrict__ dx,
                                                        T *__restrict__ dB, T *__restrict__ dC,
-                                                       float *__restrict__ ws, Dims dm, MfmaPlan pl)
+                                                       T *__restrict__ dh, float *__restrict__ ws, Dims dm,
+                                                       MfmaPlan pl)
 {
     typedef MT<T> M;
     typedef typename M::op_t op_t;
@@ -430,26 +431,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         }
     }
 
-    // diagonal sums of the P tiles -> per-wave filter-gradient partials
-    __syncthreads();
-    float *pt = (float *)smem + w * ND * 256;
-#pragma unroll
-    for (int dl = 0; dl < ND; ++dl)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) pt[dl * 256 + (4 * q + v) * 16 + j] = P[dl][v];
-    __syncthreads();
-    if (wave_valid) {
-        float *out = ws + ((size_t)wg_id * NW + w) * 128;
-        for (int lag = l; lag < 128; lag += 64) {
-            const int d0 = lag >> 4, rr = lag & 15;
-            float sum = 0.f;
-            if (d0 < ND)
-                for (int jj = 0; jj + rr < 16; ++jj) sum += pt[d0 * 256 + (jj + rr) * 16 + jj];
-            if (d0 + 1 < ND)
-                for (int ii = 0; ii < rr; ++ii) sum += pt[(d0 + 1) * 256 + ii * 16 + ii + 16 - rr];
-            out[lag] = sum;
-        }
-    }
+    dh_finish<T, NW, ND>(P, smem, ws, dh, dm, pl, wg_id, cb, wave_valid);
 }
 
 template <typename T, int NK, int NW>
@@ -527,12 +509,13 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
                void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
     int e = 0;
-    const MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
+    MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    if (p.fuse_dh) p.slot = next_dh_slot();
     e = launch_main((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
-                       (float *)ws, dm, p);
-    if (e) return e;
+                       (T *)dh, (float *)ws, dm, p);
+    if (e || p.fuse_dh) return e;
     const int64_t n = (int64_t)dm.g * dm.hl;
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
                        (const float *)ws, (T *)dh, dm, p);

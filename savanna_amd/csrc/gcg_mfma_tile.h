@@ -5,6 +5,7 @@
 #pragma once
 #include "gcg_common.h"
 
+#include <atomic>
 #include <cstdlib>
 
 namespace gcg {
@@ -250,7 +251,7 @@ template <typename T> __device__ __forceinline__ void stw_row(win_t w, uint32_t 
     for (int i = 0; i < MT<T>::RW; ++i) stw16(w, off + 16 * i, r.w[i]);
 }
 
-struct MfmaPlan { int ncb, nseg, steps_per_seg, nw, xcd; int64_t nsteps, nwg; };
+struct MfmaPlan { int ncb, nseg, steps_per_seg, nw, xcd; int64_t nsteps, nwg; int fuse_dh, slot; };
 
 // Operand tile of the banded Toeplitz matrix at row offset doff = (out time) - (in time) of the
 // tile origins: element e of lane (j, q) is the tap for lag doff + j - kmap(q, e)  (MT<T>::toeplitz).
@@ -272,6 +273,89 @@ __global__ __launch_bounds__(256) void mfma_dh_reduce_kernel(const float *__rest
         for (int k = 0; k < bpg; ++k)
             sum += ws[(p * slots + grp * bpg + k) * 128 + lag];
     Elem<T>::store(dh + i, sum);
+}
+
+// ---- filter-gradient reduction at the end of the backward kernel itself ----------------------
+// The workgroups that share a channel block -- one per (batch row, segment) -- each leave a partial
+// sum per wave in the workspace.  Instead of a second launch, the last of them to finish adds the
+// partials of its channel block, in the same fixed order whoever that is, so dh stays
+// bit-reproducible.  "Last" is decided by a ticket per channel block.  The tickets live in the
+// library image (zero when the code is loaded; the last arrival puts its ticket back to zero), in
+// DH_SLOTS sets that launches take in turn, so that launches which run at the same time on
+// different streams do not share one: a GPU executes at most one kernel per hardware queue at a
+// time and a process has at most 32 of those.
+//
+// Visibility across the XCDs' separate L2 caches comes from the accesses themselves, not from
+// fences: partials are written and read with device-scope atomic stores and loads, which go
+// through to memory, and a workgroup takes its ticket only after its own partials have completed.
+// A device-scope fence instead writes back and invalidates the whole L2 of the XCD, and one per
+// workgroup cost 45 us at the end of a 175 us kernel.
+constexpr int DH_SLOTS = 64, DH_UNITS = 1024;
+static __device__ unsigned int dh_tickets[DH_SLOTS * DH_UNITS];
+
+int next_dh_slot()
+{
+    static std::atomic<unsigned> n{0};
+    return (int)(n.fetch_add(1, std::memory_order_relaxed) % DH_SLOTS);
+}
+
+// Tail of both backward kernels.  P: the wave's ND accumulator tiles, P[dl][v] = element
+// (row 4q+v, column j) of tile dl; smem: at least NW*ND*1 KB of LDS that is no longer in use.
+template <typename T, int NW, int ND>
+__device__ __forceinline__ void dh_finish(const f32x4 (&P)[ND], unsigned char *smem, float *__restrict__ ws,
+                                          T *__restrict__ dh, const Dims &dm, const MfmaPlan &pl, int64_t wg_id,
+                                          int cb, bool wave_valid)
+{
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, j = l & 15, q = l >> 4;
+    // diagonal sums of the P tiles -> per-wave partials, lag = 16*tile + row - column
+    __syncthreads();
+    float *pt = (float *)smem + w * ND * 256;
+#pragma unroll
+    for (int dl = 0; dl < ND; ++dl)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) pt[dl * 256 + (4 * q + v) * 16 + j] = P[dl][v];
+    __syncthreads();
+    if (wave_valid) {
+        float *out = ws + ((size_t)wg_id * NW + w) * 128;
+        for (int lag = l; lag < 128; lag += 64) {
+            const int d0 = lag >> 4, rr = lag & 15;
+            float sum = 0.f;
+            if (d0 < ND)
+                for (int jj = 0; jj + rr < 16; ++jj) sum += pt[d0 * 256 + (jj + rr) * 16 + jj];
+            if (d0 + 1 < ND)
+                for (int ii = 0; ii < rr; ++ii) sum += pt[(d0 + 1) * 256 + ii * 16 + ii + 16 - rr];
+            __hip_atomic_store(out + lag, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (!pl.fuse_dh) return;       // a second launch adds the partials
+
+    __shared__ unsigned int is_last;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // every wave's partials have completed ...
+    __syncthreads();                                         // ... before thread 0 takes the ticket
+    if (tid == 0) {
+        unsigned int *tk = dh_tickets + pl.slot * DH_UNITS + cb;
+        const unsigned int arrivals = (unsigned int)(dm.bs * pl.nseg);
+        const unsigned int mine = atomicAdd(tk, 1u) + 1u;
+        is_last = (mine == arrivals);
+        if (mine == arrivals) __hip_atomic_store(tk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    constexpr int CB = 16 * NW;
+    const int gpc = CB / dm.dg, bpg = dm.dg / 16;      // filter groups per channel block, 16-channel blocks per group
+    const int64_t np = dm.bs * pl.nseg;
+    for (int idx = tid; idx < gpc * dm.hl; idx += 64 * NW) {
+        const int gl = idx / dm.hl, k = idx % dm.hl;
+        const int64_t grp = (int64_t)cb * gpc + gl;
+        if (grp >= dm.g) continue;
+        const int lag = dm.hl - 1 - k;
+        float sum = 0.f;
+        for (int64_t p = 0; p < np; ++p)
+            for (int kk = 0; kk < bpg; ++kk)
+                sum += __hip_atomic_load(ws + ((p * pl.ncb + cb) * NW + gl * bpg + kk) * 128 + lag, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+        Elem<T>::store(dh + grp * dm.hl + k, sum);
+    }
 }
 
 int cu_count()
@@ -346,6 +430,8 @@ MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu, int elem_
     p.nseg = (int)((p.nsteps + sps - 1) / sps);
     p.nwg = dm.bs * p.nseg * p.ncb;
     p.xcd = 1;
+    p.fuse_dh = 0;
+    p.slot = 0;
     return p;
 }
 
@@ -370,7 +456,11 @@ int choose_nw_bwd(const Dims &dm, bool fp32)
 MfmaPlan plan_bwd(const Dims &dm, bool fp32)
 {
     const int nw = choose_nw_bwd(dm, fp32);
-    return plan(dm, nw, 16, nw, fp32 ? 4 : 2);
+    MfmaPlan p = plan(dm, nw, 16, nw, fp32 ? 4 : 2);
+    // the kernel adds the partials itself when a filter group lies within one channel block
+    static const int fuse = env_int("GCG_MFMA_FUSE_DH", 1);    // tuning override: 0 = always a second launch
+    p.fuse_dh = fuse && (16 * nw) % dm.dg == 0 && p.ncb <= DH_UNITS;
+    return p;
 }
 
 } // namespace

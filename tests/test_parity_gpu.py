@@ -111,9 +111,9 @@ def test_bwd_is_deterministic(gcg_lib, algo):
 
 def test_error_codes(gcg_lib):
     x, B, C, h, dy = (t.to(DEV) for t in inputs(1, 64, 2, 16, 200, torch.bfloat16))
-    with pytest.raises(_lib.GcgError, match="not supported"):
+    with pytest.raises(RuntimeError, match="not supported"):
         _lib.fwd(x, B, C, h, algo="mfma")        # hl > 128
-    with pytest.raises(_lib.GcgError, match="not supported"):
+    with pytest.raises(RuntimeError, match="not supported"):
         _lib.fwd(x, B, C, h, algo="window")      # hl > 8
     with pytest.raises(RuntimeError, match="no CPU path"):
         _lib.fwd(x.cpu(), B.cpu(), C.cpu(), h.cpu())
@@ -149,7 +149,7 @@ def test_misaligned_tensors_take_the_direct_kernels(gcg_lib, dtype, hl):
     for o, r_, n_ in zip(got, oracle_bwd(dy, x, B, C, h), ("dx", "dB", "dC", "dh")):
         assert_close(o, r_, TOL_DH[dtype] if n_ == "dh" else TOL[dtype], n_)
     forced = "mfma" if hl > 8 else "window"
-    with pytest.raises(_lib.GcgError, match="not supported"):
+    with pytest.raises(RuntimeError, match="not supported"):
         _lib.fwd(xs, Bs, Cs, hd, algo=forced)
 
 

@@ -1,0 +1,110 @@
+"""The torch.ops.gcg operators on the GPU: results against the oracle, agreement of the two bindings of the library
+(torch operators and ctypes), torch.library's own operator checks, and torch.compile(fullgraph=True) of the
+reference-compatible entry point against eager (the reference compiles its filter, explicit.py:71, so callers of
+this path are traced)."""
+import pytest
+import torch
+
+from helpers import TOL, TOL_DH, assert_close, inputs, oracle_bwd, oracle_fwd
+from savanna_amd import _lib, _ops, two_pass_chunked_gate_conv_gate
+from savanna_amd.kernels.cgcg.interface import two_pass_chunked_gate_conv_gate_interleaved
+from savanna_amd.kernels.cgcg.src.kernel_utils import FwdKernelConfigRefactor
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+CFG = FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row")
+
+
+@pytest.mark.parametrize("shape,dtype", [((2, 300, 3, 16, 128), torch.bfloat16), ((1, 200, 4, 16, 7), torch.float32),
+                                         ((1, 700, 2, 16, 200), torch.float16)])
+def test_ops_against_oracle(gcg_lib, shape, dtype):
+    assert _ops.AVAILABLE, _ops.LOAD_ERROR
+    x, B, C, h, dy = inputs(*shape, dtype)
+    xd, Bd, Cd, hd, dyd = (t.to(DEV) for t in (x, B, C, h, dy))
+    bx, y2, y = torch.ops.gcg.fwd_full(xd, Bd, Cd, hd, True, True)
+    rbx, ry2, ry = oracle_fwd(x, B, C, h)
+    for name, got, ref in (("bx", bx, rbx), ("y2", y2, ry2), ("y", y, ry)):
+        assert_close(got, ref, TOL[dtype], name)
+    assert torch.equal(torch.ops.gcg.fwd(xd, Bd, Cd, hd), y)
+    out = torch.full_like(xd, float("nan"))
+    torch.ops.gcg.fwd_out(xd, Bd, Cd, hd, out)
+    assert torch.equal(out, y)
+    got = torch.ops.gcg.bwd(dyd, xd, Bd, Cd, hd)
+    for name, g_, r_ in zip(("dx", "dB", "dC", "dh"), got, oracle_bwd(dy, x, B, C, h)):
+        assert_close(g_, r_, TOL_DH[dtype] if name == "dh" else TOL[dtype], name)
+
+
+def test_both_bindings_give_the_same_bits(gcg_lib, monkeypatch):
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(2, 1000, 5, 16, 100, torch.bfloat16, seed=3))
+    feat = torch.stack([C, B, x], dim=-1).contiguous()
+    via_ops = (_lib.fwd(x, B, C, h)[2], *_lib.bwd(dy, x, B, C, h), _lib.fwd_interleaved(feat, h),
+               *_lib.bwd_interleaved(dy, feat, h))
+    monkeypatch.setattr(_lib, "TORCH_OPS", False)
+    via_ctypes = (_lib.fwd(x, B, C, h)[2], *_lib.bwd(dy, x, B, C, h), _lib.fwd_interleaved(feat, h),
+                  *_lib.bwd_interleaved(dy, feat, h))
+    for a, b in zip(via_ops, via_ctypes):
+        assert torch.equal(a, b)
+
+
+def test_ops_run_on_the_current_stream_and_device(gcg_lib):
+    """Enqueued on torch's current stream: a side stream's result is complete once that stream is waited on."""
+    x, B, C, h, _ = (t.to(DEV) for t in inputs(1, 4096, 16, 16, 128, torch.bfloat16, seed=5))
+    ref = torch.ops.gcg.fwd(x, B, C, h)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            y = torch.ops.gcg.fwd(x, B, C, h)
+    torch.cuda.current_stream().wait_stream(side)
+    assert torch.equal(y, ref)
+
+
+def test_library_opcheck(gcg_lib):
+    """torch.library.opcheck: schema (no undeclared mutation or aliasing) and meta implementation vs device result."""
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(1, 130, 2, 16, 33, torch.bfloat16))
+    feat = torch.stack([C, B, x], dim=-1).contiguous()
+    checks = ("test_schema", "test_faketensor")
+    torch.library.opcheck(torch.ops.gcg.fwd, (x, B, C, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.fwd_full, (x, B, C, h, True, True), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.bwd, (dy, x, B, C, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.fwd_interleaved, (feat, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.bwd_interleaved, (dy, feat, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.fwd_out, (x, B, C, h, torch.empty_like(x)), test_utils=checks)
+
+
+def _grads(fn, tensors, dy):
+    leaves = [t.detach().clone().requires_grad_(True) for t in tensors]
+    y = fn(*leaves)
+    y.backward(dy)
+    return [y.detach()] + [t.grad for t in leaves]
+
+
+@pytest.mark.parametrize("shape,dtype", [((2, 512, 4, 16, 128), torch.bfloat16), ((1, 256, 8, 16, 7), torch.float32)])
+def test_compile_fullgraph_matches_eager(gcg_lib, shape, dtype):
+    bs, L, g, dg, hl = shape
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(*shape, dtype, seed=7))
+
+    def op(x, B, C, h):
+        return two_pass_chunked_gate_conv_gate(x, B, C, h, bs, L, g, dg, fwd_kernel_cfg=CFG)
+
+    eager = _grads(op, (x, B, C, h), dy)
+    torch._dynamo.reset()
+    compiled = _grads(torch.compile(op, fullgraph=True, backend="aot_eager"), (x, B, C, h), dy)
+    for name, a, b in zip(("y", "dx", "dB", "dC", "dh"), eager, compiled):
+        assert torch.equal(a, b), name
+
+
+def test_compile_fullgraph_interleaved(gcg_lib):
+    bs, L, g, dg, hl = 1, 384, 4, 16, 128
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(bs, L, g, dg, hl, torch.bfloat16, seed=9))
+    feat = torch.stack([C, B, x], dim=-1).reshape(bs, L, 3 * g * dg).contiguous()
+
+    def op(feat, h):
+        return two_pass_chunked_gate_conv_gate_interleaved(feat, h, bs, L, g, dg)
+
+    eager = _grads(op, (feat, h), dy)
+    torch._dynamo.reset()
+    compiled = _grads(torch.compile(op, fullgraph=True, backend="aot_eager"), (feat, h), dy)
+    for name, a, b in zip(("y", "dfeat", "dh"), eager, compiled):
+        assert torch.equal(a, b), name
