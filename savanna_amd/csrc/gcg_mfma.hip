@@ -16,10 +16,11 @@
 // fp32 and stored with full rows.
 //
 // Element types.  bf16 / f16: v_mfma_f32_16x16x32; the operand (8 consecutive time samples of
-// one channel per lane) comes from the transposing LDS read ds_read_b64_tr_b16.  fp32: the
-// same 32-deep product is eight v_mfma_f32_16x16x4_f32 (exact fp32 multiply-add, so the fp32
-// path keeps fp32 accuracy); a lane's eight operand values are time samples q, q+4, ... of one
-// channel, read straight from the row-major tile.
+// one channel per lane) comes from the transposing LDS read ds_read_b64_tr_b16.  fp32: every
+// operand is split into three bf16 planes whose sum is the fp32 value, the planes sit side by
+// side in the LDS tiles, and the same 32-deep product is six bf16 matrix instructions (the
+// plane pairs that matter to 2^-24), accumulated in fp32: fp32 accuracy at 3/8 of the matrix
+// time of the fp32 instructions.  Memory traffic stays fp32.
 #include "gcg_mfma_tile.h"
 
 namespace gcg {
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 #pragma unroll
     for (int i = 0; i < NK; ++i) A[i] = M::zero_op();
 
-    unsigned char *u_wr = u_rm + r * UROW + 8 * ES * a;
+    unsigned char *u_wr = u_rm + r * UROW + 8 * M::LES * a;
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
 
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
             unpack8<T>(lB[i - 1], Bf);
 #pragma unroll
             for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
-            lds_store_row<T>(u_wr, pack8<T>(uf));
+            store_operand_row<T>(u_wr, UROW, pack8<T>(uf));
             __syncthreads();
             A[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
             __syncthreads();
@@ -150,7 +151,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 #pragma unroll
                 for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
                 const Row<T> up = pack8<T>(uf);
-                lds_store_row<T>(u_wr, up);
+                store_operand_row<T>(u_wr, UROW, up);
                 const uint32_t o = lane_off + step_off(s);
                 if constexpr (EXTRA) stw_row<T>(wbx, o, up);
                 __syncthreads();
@@ -279,7 +280,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // LDS addresses of this lane
-    const int rm_off = r * UROW + 8 * ES * a;                                 // row layout, 8 channels
+    const int rm_off = r * UROW + 8 * M::LES * a;                                // row layout, 8 channels
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
     unsigned char *d_wr = d_st + (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
@@ -332,13 +333,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
             unpack8<T>(wB_[i - 1], f1);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
-            lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
+            store_operand_row<T>(u_rm + rm_off, UROW, pack8<T>(pf));
             unpack8<T>(wdy_[i - 1], f0);
             unpack8<T>(wC_[i - 1], f1);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
             unsigned char *g_slot = g_rm + (NK - 1 - i) * STEP * UROW;
-            lds_store_row<T>(g_slot + rm_off, pack8<T>(pf));
+            store_operand_row<T>(g_slot + rm_off, UROW, pack8<T>(pf));
             dyq[NK - 1 - i] = wdy_[i - 1];
             __syncthreads();
             Au[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
@@ -362,13 +363,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                 unpack8<T>(Br, Bf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[e] = xf[e] * Bf[e];
-                lds_store_row<T>(u_rm + rm_off, pack8<T>(pf));
+                store_operand_row<T>(u_rm + rm_off, UROW, pack8<T>(pf));
                 unpack8<T>(dyr, tf);
                 unpack8<T>(Cr, cf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[e] = tf[e] * cf[e];
                 unsigned char *g_slot = g_rm + slot_new * STEP * UROW;
-                lds_store_row<T>(g_slot + rm_off, pack8<T>(pf));
+                store_operand_row<T>(g_slot + rm_off, UROW, pack8<T>(pf));
                 dyq[slot_new] = dyr;
                 __syncthreads();
                 Au[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
@@ -388,14 +389,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                     *(f32x4 *)d_wr = dac0;
                     *(f32x4 *)(d_wr + 16 * YROW) = dac1;
                     // filter-gradient tiles: natural-layout operands (rows j and 16+j of a 32-row window)
-                    const op_t un = M::load_natural(u_rm + j * UROW, u_rm + (16 + j) * UROW, w, q);
+                    const op_t un = M::load_natural(u_rm + j * UROW, u_rm + (16 + j) * UROW, UROW, w, q);
 #pragma unroll
                     for (int dl = 0; dl < ND; ++dl) {
                         int row0 = STEP * ph + 16 * dl + j;              // ring rows of the window's two halves
                         int row1 = row0 + 16;
                         row0 = (row0 >= RING_ROWS) ? row0 - RING_ROWS : row0;
                         row1 = (row1 >= RING_ROWS) ? row1 - RING_ROWS : row1;
-                        const op_t gn = M::load_natural(g_rm + row0 * UROW, g_rm + row1 * UROW, w, q);
+                        const op_t gn = M::load_natural(g_rm + row0 * UROW, g_rm + row1 * UROW, UROW, w, q);
                         P[dl] = M::mfma(gn, un, P[dl]);
                     }
                 }

@@ -65,6 +65,18 @@ template <typename T> __device__ __forceinline__ uint32_t pack_unit(const float 
     if constexpr (MT<T>::ES == 4) return __float_as_uint(f[0]);
     else return MT<T>::pack2(f[0], f[1]);
 }
+// one lane's unit of a row (CH channels) into a matrix-operand tile, in the tile's own element format
+template <typename T> __device__ __forceinline__ void store_operand_unit(unsigned char *p, int urow, const float *f)
+{
+    if constexpr (MT<T>::ES == 4) {
+        uint16_t v[3];
+        MT<T>::split(f[0], v[0], v[1], v[2]);
+#pragma unroll
+        for (int m = 0; m < 3; ++m) *(uint16_t *)(p + m * MT<T>::plane(urow)) = v[m];
+    } else {
+        *(uint32_t *)p = MT<T>::pack2(f[0], f[1]);
+    }
+}
 // NR units in a row vector: unpack8 then yields them in element order e = k * CH + c
 template <typename T, int NR> __device__ __forceinline__ Row<T> units_row(const uint32_t (&u)[NR])
 {
@@ -122,7 +134,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 #pragma unroll
     for (int i = 0; i < NK; ++i) A[i] = M::zero_op();
 
-    unsigned char *u_wr = u_rm + rr * UROW + 4 * a;
+    unsigned char *u_wr = u_rm + rr * UROW + M::LES * CH * a;
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
     const unsigned char *y_rd = y_st + rr * YROW + 4 * CH * a;
 
@@ -133,7 +145,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     };
     auto store_u = [&](const float (&uf)[8]) {
 #pragma unroll
-        for (int k = 0; k < NR; ++k) *(uint32_t *)(u_wr + RP * k * UROW) = pack_unit<T>(&uf[CH * k]);
+        for (int k = 0; k < NR; ++k) store_operand_unit<T>(u_wr + RP * k * UROW, UROW, &uf[CH * k]);
     };
     u32x3 in[NR];
     fetch(s_lo, in);
@@ -249,11 +261,12 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     constexpr int OFF_G = OFF_U + STEP * UROW;              // g2 ring, NK steps, row-major
     constexpr int OFF_Y = OFF_G + RING_ROWS * UROW;         // y2 tile, fp32, row-major
     constexpr int OFF_D = OFF_Y + STEP * YROW;              // du tile, fp32, row-major
-    constexpr int OFF_H = OFF_D + STEP * YROW;              // filter tables
-    constexpr int OFF_XB = (OFF_H + NW * HTAB * (int)sizeof(hraw_t) + 15) & ~15;   // waiting x, B values
+    constexpr int OFF_H = OFF_D + STEP * YROW;              // filter tables: dead once the Toeplitz tiles are built,
+    constexpr int OFF_XB = OFF_H;                           // so the waiting x, B values take the same place
     constexpr int XB_SLOTS = NK > 1 ? NK - 1 : 0;
     constexpr int XB_VEC = G::NT * 16 * M::RW;              // one row vector of every lane
-    constexpr int LDS_MAIN = OFF_XB + XB_SLOTS * 2 * XB_VEC;
+    constexpr int XB_BYTES = XB_SLOTS * 2 * XB_VEC, H_BYTES = NW * HTAB * (int)sizeof(hraw_t);
+    constexpr int LDS_MAIN = OFF_XB + (XB_BYTES > H_BYTES ? XB_BYTES : H_BYTES);
     constexpr int LDS_TAIL = NW * ND * 256 * 4;             // P tiles at the end
     // a 4-wave workgroup at 16 bits asks for more than half of the CU's 160 KB, so that a CU holds one
     constexpr int LDS_NEED = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
@@ -310,7 +323,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // LDS addresses of this lane
-    const int rm_off = rr * UROW + 4 * a;                                     // memory layout, row rr
+    const int rm_off = rr * UROW + M::LES * CH * a;                                    // memory layout, row rr
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
     unsigned char *d_wr = d_st + (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
     const unsigned char *y_rd = y_st + rr * YROW + 4 * CH * a;
@@ -332,7 +345,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     };
     auto store_rows = [&](unsigned char *tile, const float (&f)[8]) {
 #pragma unroll
-        for (int k = 0; k < NR; ++k) *(uint32_t *)(tile + rm_off + RP * k * UROW) = pack_unit<T>(&f[CH * k]);
+        for (int k = 0; k < NR; ++k) store_operand_unit<T>(tile + rm_off + RP * k * UROW, UROW, &f[CH * k]);
     };
 
     // iteration sigma brings the interleaved rows and dy of step sigma+NK-1
@@ -372,6 +385,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
         W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
         W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
     }
+    __syncthreads();      // the filter tables have been read: their place now holds the waiting x, B values
 
     if constexpr (NK > 1) {
 #pragma unroll
@@ -456,14 +470,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
                     *(f32x4 *)d_wr = dac0;
                     *(f32x4 *)(d_wr + 16 * YROW) = dac1;
                     // filter-gradient tiles: natural-layout operands (rows j and 16+j of a 32-row window)
-                    const op_t un = M::load_natural(u_rm + j * UROW, u_rm + (16 + j) * UROW, w, q);
+                    const op_t un = M::load_natural(u_rm + j * UROW, u_rm + (16 + j) * UROW, UROW, w, q);
 #pragma unroll
                     for (int dl = 0; dl < ND; ++dl) {
                         int row0 = STEP * ph + 16 * dl + j;              // ring rows of the window's two halves
                         int row1 = row0 + 16;
                         row0 = (row0 >= RING_ROWS) ? row0 - RING_ROWS : row0;
                         row1 = (row1 >= RING_ROWS) ? row1 - RING_ROWS : row1;
-                        const op_t gn = M::load_natural(g_rm + row0 * UROW, g_rm + row1 * UROW, w, q);
+                        const op_t gn = M::load_natural(g_rm + row0 * UROW, g_rm + row1 * UROW, UROW, w, q);
                         P[dl] = M::mfma(gn, un, P[dl]);
                     }
                 }

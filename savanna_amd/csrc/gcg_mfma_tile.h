@@ -32,10 +32,27 @@ __device__ __forceinline__ s16x4 lds_read_tr(const unsigned char *p)
 // quad q stands for contraction index kmap(q, e); both factors of a product use the same map.
 template <typename T> struct MT;
 
+// The transposed operand of the 32-deep product from a row-major LDS tile of 16-bit elements: time samples
+// 8q .. 8q+7 of channel 16w+j from rows 0..31 (reversed: 31-k).
+__device__ __forceinline__ uint4 tr_operand16(const unsigned char *tile, int urow, int w, int j, int q, bool reversed)
+{
+    const int col = (16 * w + 4 * (j & 3)) * 2;
+    const int r0 = reversed ? 31 - 8 * q - (j >> 2) : 8 * q + (j >> 2);
+    const int r1 = reversed ? r0 - 4 : r0 + 4;
+    const s16x4 lo = lds_read_tr(tile + r0 * urow + col);
+    const s16x4 hi = lds_read_tr(tile + r1 * urow + col);
+    const short v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+    uint4 r;
+    __builtin_memcpy(&r, v, 16);
+    return r;
+}
+
 template <typename OP> struct MT16 {
-    static constexpr int ES = 2;                 // bytes per element
+    static constexpr int ES = 2;                 // bytes per element in memory
     static constexpr int RW = 1;                 // 16-byte words per 8-channel row vector
-    static constexpr int UPAD = 32;              // row padding: consecutive rows start 8 banks apart
+    static constexpr int LES = 2;                // bytes per element of the operand tiles in LDS
+    // bytes per LDS row of an operand tile of cb channels; the padding makes consecutive rows start 8 banks apart
+    static constexpr int urow(int cb) { return cb * 2 + 32; }
     typedef OP op_t;
     typedef uint16_t hraw_t;
     static __device__ __forceinline__ int kmap(int q, int e) { return 8 * q + e; }
@@ -50,26 +67,28 @@ template <typename OP> struct MT16 {
     static __device__ __forceinline__ op_t load_operand(const unsigned char *tile, int urow, int w, int j, int q,
                                                         bool reversed)
     {
-        const int col = (16 * w + 4 * (j & 3)) * 2;
-        const int r0 = reversed ? 31 - 8 * q - (j >> 2) : 8 * q + (j >> 2);
-        const int r1 = reversed ? r0 - 4 : r0 + 4;
-        const s16x4 lo = lds_read_tr(tile + r0 * urow + col);
-        const s16x4 hi = lds_read_tr(tile + r1 * urow + col);
-        const short v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        const uint4 t4 = tr_operand16(tile, urow, w, j, q, reversed);
         op_t r;
-        __builtin_memcpy(&r, v, 16);
+        __builtin_memcpy(&r, &t4, 16);
         return r;
     }
     // natural-layout operand of the filter-gradient product: 8 channels of one of two rows;
     // lane quad q takes row half q>>1 and channels 8*(q&1)..+7 of the wave's 16
     static __device__ __forceinline__ op_t load_natural(const unsigned char *row_half0,
-                                                        const unsigned char *row_half1, int w, int q)
+                                                        const unsigned char *row_half1, int urow, int w, int q)
     {
+        (void)urow;
         const unsigned char *p = ((q >> 1) ? row_half1 : row_half0) + (16 * w + 8 * (q & 1)) * 2;
         const uint4 t4 = *(const uint4 *)p;
         op_t r;
         __builtin_memcpy(&r, &t4, 16);
         return r;
+    }
+    // a lane's 8 channels of one row (already packed to 16 bits) into an operand tile
+    static __device__ __forceinline__ void store_u8(unsigned char *p, int urow, const uint4 &packed)
+    {
+        (void)urow;
+        *(uint4 *)p = packed;
     }
     static __device__ __forceinline__ op_t toeplitz(const hraw_t *htab, int doff, int j, int q)
     {
@@ -110,66 +129,108 @@ template <> struct MT<f16_t> : MT16<f16x8> {
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
 };
 
-struct F32x8 { float v[8]; };
+// fp32 on the bf16 matrix cores.  An fp32 value is the exact sum of three bf16 values (8 significant bits each:
+// v1 = bf16(v), v2 = bf16(v - v1), v3 = bf16(v - v1 - v2)), and the product of two bf16 values is exact in the
+// fp32 accumulator, so  a * b  =  sum of a_m * b_n  over the planes; the six terms with m + n <= 4 carry it to
+// 2^-24 relative to |a b| (the three left out are below that), i.e. to fp32 accuracy, at 6 matrix instructions of 16
+// cycles instead of the 8 fp32 ones of 32 cycles that the same 32-deep product costs on the fp32 matrix path.
+// Operand tiles in LDS hold the three planes of a row side by side (plane m at byte offset m * plane(urow)), each
+// laid out like a 16-bit tile, so operands come from the same transposing reads.
+struct Split3 { bf16x8 p[3]; };
 template <> struct MT<float> {
     static constexpr int ES = 4;
     static constexpr int RW = 2;
-    static constexpr int UPAD = 64;              // consecutive rows start 16 banks apart
-    typedef F32x8 op_t;
+    static constexpr int LES = 2;
+    static constexpr int NP = 3;
+    static constexpr int RPAD = 32;              // with it consecutive rows start an odd multiple of 8 banks apart
+    static constexpr int urow(int cb) { return NP * cb * 2 + RPAD; }
+    static __device__ __forceinline__ int plane(int urow) { return (urow - RPAD) / NP; }   // bytes between planes
+    typedef Split3 op_t;
     typedef float hraw_t;
-    // instruction e of the eight contracts time samples 4e .. 4e+3, one per lane quad
-    static __device__ __forceinline__ int kmap(int q, int e) { return 4 * e + q; }
+    static __device__ __forceinline__ int kmap(int q, int e) { return 8 * q + e; }
+    static __device__ __forceinline__ void split(float v, uint16_t &v1, uint16_t &v2, uint16_t &v3)
+    {
+        v1 = (uint16_t)float_to_bf16_bits(v);
+        const float r1 = v - bf16_bits_to_float(v1);
+        v2 = (uint16_t)float_to_bf16_bits(r1);
+        const float r2 = r1 - bf16_bits_to_float(v2);
+        v3 = (uint16_t)float_to_bf16_bits(r2);
+    }
     static __device__ __forceinline__ op_t zero_op()
     {
         op_t r;
+        const uint4 z = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) r.v[e] = 0.f;
+        for (int m = 0; m < NP; ++m) __builtin_memcpy(&r.p[m], &z, 16);
         return r;
     }
     static __device__ __forceinline__ op_t load_operand(const unsigned char *tile, int urow, int w, int j, int q,
                                                         bool reversed)
     {
         op_t r;
-        const int col = (16 * w + j) * 4;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            const int k = kmap(q, e);
-            r.v[e] = *(const float *)(tile + (reversed ? 31 - k : k) * urow + col);
+        for (int m = 0; m < NP; ++m) {
+            const uint4 t4 = tr_operand16(tile + m * plane(urow), urow, w, j, q, reversed);
+            __builtin_memcpy(&r.p[m], &t4, 16);
         }
         return r;
     }
-    // element e: row half e>>2, channel 4q + (e&3) of the wave's 16
     static __device__ __forceinline__ op_t load_natural(const unsigned char *row_half0,
-                                                        const unsigned char *row_half1, int w, int q)
+                                                        const unsigned char *row_half1, int urow, int w, int q)
     {
-        const int col = (16 * w + 4 * q) * 4;
-        const f32x4 a = *(const f32x4 *)(row_half0 + col), b = *(const f32x4 *)(row_half1 + col);
+        const unsigned char *p = ((q >> 1) ? row_half1 : row_half0) + (16 * w + 8 * (q & 1)) * 2;
         op_t r;
-        r.v[0] = a[0]; r.v[1] = a[1]; r.v[2] = a[2]; r.v[3] = a[3];
-        r.v[4] = b[0]; r.v[5] = b[1]; r.v[6] = b[2]; r.v[7] = b[3];
+#pragma unroll
+        for (int m = 0; m < NP; ++m) {
+            const uint4 t4 = *(const uint4 *)(p + m * plane(urow));
+            __builtin_memcpy(&r.p[m], &t4, 16);
+        }
         return r;
     }
     static __device__ __forceinline__ op_t toeplitz(const hraw_t *htab, int doff, int j, int q)
     {
+        uint16_t v[NP][8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) split(htab[doff + j - kmap(q, e) + HPAD], v[0][e], v[1][e], v[2][e]);
         op_t r;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) r.v[e] = htab[doff + j - kmap(q, e) + HPAD];
+        for (int m = 0; m < NP; ++m) __builtin_memcpy(&r.p[m], v[m], 16);
         return r;
     }
+    // smallest terms first
     static __device__ __forceinline__ f32x4 mfma(const op_t &a, const op_t &b, f32x4 c)
     {
-#pragma unroll
-        for (int e = 0; e < 8; ++e) c = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v[e], b.v[e], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[2], b.p[0], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[1], b.p[1], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[0], b.p[2], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[1], b.p[0], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[0], b.p[1], c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[0], b.p[0], c, 0, 0, 0);
         return c;
+    }
+    // a lane's 8 fp32 channels of one row (two 16-byte words) into the three planes of an operand tile
+    static __device__ __forceinline__ void store_u8(unsigned char *p, int urow, const uint4 &w0, const uint4 &w1)
+    {
+        const float f[8] = {__uint_as_float(w0.x), __uint_as_float(w0.y), __uint_as_float(w0.z), __uint_as_float(w0.w),
+                            __uint_as_float(w1.x), __uint_as_float(w1.y), __uint_as_float(w1.z), __uint_as_float(w1.w)};
+        uint16_t v[NP][8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) split(f[e], v[0][e], v[1][e], v[2][e]);
+#pragma unroll
+        for (int m = 0; m < NP; ++m) {
+            uint4 t4;
+            __builtin_memcpy(&t4, v[m], 16);
+            *(uint4 *)(p + m * plane(urow)) = t4;
+        }
     }
 };
 
-// A workgroup of NW waves owns CB = 16*NW adjacent channels; LDS rows are padded (see UPAD;
+// A workgroup of NW waves owns CB = 16*NW adjacent channels; LDS rows are padded (see MT<T>::urow;
 // the fp32 result tile: consecutive rows start 4 banks apart).
 template <typename T, int NW> struct Geo {
     static constexpr int CB = 16 * NW;                          // channels per workgroup
     static constexpr int LPR = CB / 8;                          // lanes per row in the row layout (8 channels each)
-    static constexpr int UROW = CB * MT<T>::ES + MT<T>::UPAD;   // bytes per LDS row of u / g2
+    static constexpr int UROW = MT<T>::urow(CB);                // bytes per LDS row of u / g2
     static constexpr int YROW = CB * 4 + 16;                    // bytes per LDS row of y2 / du
     static constexpr int NT = 64 * NW;                          // threads
 };
@@ -214,6 +275,13 @@ template <typename T> __device__ __forceinline__ void lds_store_row(unsigned cha
 {
 #pragma unroll
     for (int i = 0; i < MT<T>::RW; ++i) *(uint4 *)(p + 16 * i) = r.w[i];
+}
+
+// a lane's 8 channels of one row into a matrix-operand tile (in the tile's own element format)
+template <typename T> __device__ __forceinline__ void store_operand_row(unsigned char *p, int urow, const Row<T> &r)
+{
+    if constexpr (MT<T>::ES == 4) MT<T>::store_u8(p, urow, r.w[0], r.w[1]);
+    else MT<T>::store_u8(p, urow, r.w[0]);
 }
 
 template <typename T> __device__ __forceinline__ Row<T> lds_load_row(const unsigned char *p)
