@@ -39,9 +39,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     typedef typename M::hraw_t hraw_t;
     typedef Geo<T, NW> G;
     constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW, ES = M::ES;
-    __shared__ __attribute__((aligned(16))) unsigned char u_rm[STEP * UROW];
-    __shared__ __attribute__((aligned(16))) unsigned char y_st[STEP * YROW];
-    __shared__ hraw_t htab[NW][HTAB];
+    // LDS: filter tables | u tile of the current step | fp32 result tile.  Before the walk the NK-1
+    // lead-in tiles of u lie side by side from the u tile on (over the result tile, not yet in use).
+    constexpr int NLEAD_T = NK > 1 ? NK - 1 : 0;
+    constexpr int OFF_U = (NW * HTAB * (int)sizeof(hraw_t) + 15) & ~15, OFF_Y = OFF_U + STEP * UROW;
+    constexpr int LDS_WALK = STEP * UROW + STEP * YROW, LDS_LEAD = NLEAD_T * STEP * UROW;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[OFF_U + (LDS_WALK > LDS_LEAD ? LDS_WALK : LDS_LEAD)];
+    unsigned char *u_rm = smem + OFF_U, *y_st = smem + OFF_Y;
+    hraw_t (*htab)[HTAB] = (hraw_t (*)[HTAB])smem;
 
     int64_t wg = pl.xcd ? xcd_contiguous_id(blockIdx.x, gridDim.x) : (int64_t)blockIdx.x;
     const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
@@ -78,19 +83,28 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
 
-    Row<T> xr, Br, Cr;
-    auto fetch = [&](int64_t s, Row<T> &xo, Row<T> &Bo, Row<T> &Co) {
-        const uint32_t o = lane_off + step_off(s);
-        xo = ldw_row<T>(wx, o);
-        Bo = ldw_row<T>(wB, o);
-        Co = ldw_row<T>(wC, o);
-    };
-    fetch(s_lo, xr, Br, Cr);
+    // The filter taps of this wave's group are requested before any row: the filter table and the
+    // Toeplitz operand tiles are then built while the rows are in flight (loads complete in the
+    // order of issue, so taps requested after the rows would arrive after all of them).
+    // htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0.
+    hraw_t hv[HTAB / 64];
+    {
+        const int64_t cw = c0 + 16 * w;
+        const int64_t grp = (cw < d) ? cw / dm.dg : 0;
+        const hraw_t *hg = (const hraw_t *)h + grp * hl;
+#pragma unroll
+        for (int k = 0; k < HTAB / 64; ++k) {
+            const int lag = l + 64 * k - HPAD;
+            const bool in = lag >= 0 && lag < hl;
+            const hraw_t v = hg[in ? hl - 1 - lag : 0];          // no branch around the load
+            hv[k] = in ? v : (hraw_t)0;
+        }
+    }
 
     // The operands of the NK-1 steps before the segment are rebuilt first (zero before the
     // start of the sequence).  Their rows are requested together, so the replay costs one
     // memory latency instead of NK-1; step s_lo-i lands in ring slot NK-i, where phase 0
-    // expects it.
+    // expects it.  The rows of the first step follow them: they are needed last.
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
     Row<T> lx[NLEAD], lB[NLEAD];
     if constexpr (NK > 1) {
@@ -101,18 +115,17 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
             lB[i - 1] = ldw_row<T>(wB, o);
         }
     }
+    Row<T> xr, Br, Cr;
+    auto fetch = [&](int64_t s, Row<T> &xo, Row<T> &Bo, Row<T> &Co) {
+        const uint32_t o = lane_off + step_off(s);
+        xo = ldw_row<T>(wx, o);
+        Bo = ldw_row<T>(wB, o);
+        Co = ldw_row<T>(wC, o);
+    };
+    fetch(s_lo, xr, Br, Cr);
 
-    // While those rows are in flight: filter table of this wave's group,
-    // htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0, and the Toeplitz operand tiles.
-    {
-        const int64_t cw = c0 + 16 * w;
-        const int64_t grp = (cw < d) ? cw / dm.dg : 0;
-        const hraw_t *hg = (const hraw_t *)h + grp * hl;
-        for (int i = l; i < HTAB; i += 64) {
-            const int lag = i - HPAD;
-            htab[w][i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
-        }
-    }
+#pragma unroll
+    for (int k = 0; k < HTAB / 64; ++k) htab[w][l + 64 * k] = hv[k];
     __syncthreads();
     op_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
 #pragma unroll
@@ -122,6 +135,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     }
 
     if constexpr (NK > 1) {
+        // all lead-in tiles go to LDS together: one pair of barriers instead of NK-1
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
             float xf[8], Bf[8], uf[8];
@@ -129,11 +143,12 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
             unpack8<T>(lB[i - 1], Bf);
 #pragma unroll
             for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
-            store_operand_row<T>(u_wr, UROW, pack8<T>(uf));
-            __syncthreads();
-            A[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
-            __syncthreads();
+            store_operand_row<T>(u_wr + (i - 1) * STEP * UROW, UROW, pack8<T>(uf));
         }
+        __syncthreads();
+#pragma unroll
+        for (int i = 1; i < NK; ++i) A[NK - i] = M::load_operand(u_rm + (i - 1) * STEP * UROW, UROW, w, j, q, false);
+        __syncthreads();
     }
 
     int64_t s = s_lo;
@@ -286,6 +301,21 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     const unsigned char *y_rd = y_st + r * YROW + 32 * a;
     const unsigned char *d_rd = d_st + r * YROW + 32 * a;
 
+    // The filter taps of this wave's group are requested before any row, so that the filter table
+    // and the Toeplitz tiles are built while the rows are in flight (loads complete in order of issue).
+    hraw_t hv[HTAB / 64];
+    {
+        const int64_t grp = wave_valid ? (c0 + 16 * w) / dm.dg : 0;
+        const hraw_t *hg = (const hraw_t *)h + grp * hl;
+#pragma unroll
+        for (int k = 0; k < HTAB / 64; ++k) {
+            const int lag = l + 64 * k - HPAD;
+            const bool in = lag >= 0 && lag < hl;
+            const hraw_t v = hg[in ? hl - 1 - lag : 0];          // no branch around the load
+            hv[k] = in ? v : (hraw_t)0;
+        }
+    }
+
     // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the windows)
     auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
         const uint32_t o = lane_off + step_off(sg), o2 = lane_off + step_off(sg + NK - 1);
@@ -294,28 +324,22 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         dyo = ldw_row<T>(wdy, o2);
         Co = ldw_row<T>(wC, o2);
     };
-    Row<T> xr, Br, dyr, Cr;
-    fetch(s_lo, xr, Br, dyr, Cr);
 
     // Lead-in: u of the NK-1 steps before the segment and g2 of its first NK-1 steps, i.e. the
     // rows iterations s_lo-NK+1 .. s_lo-1 would have brought.  They are requested together,
-    // so the lead-in costs one memory latency instead of NK-1.
+    // so the lead-in costs one memory latency instead of NK-1; the rows of the first iteration
+    // follow them (needed last).
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
     Row<T> wx_[NLEAD], wB_[NLEAD], wdy_[NLEAD], wC_[NLEAD];
     if constexpr (NK > 1) {
 #pragma unroll
         for (int i = 1; i < NK; ++i) fetch(s_lo - i, wx_[i - 1], wB_[i - 1], wdy_[i - 1], wC_[i - 1]);
     }
+    Row<T> xr, Br, dyr, Cr;
+    fetch(s_lo, xr, Br, dyr, Cr);
 
-    // While those rows are in flight: the filter table of this wave's group and the Toeplitz tiles.
-    {
-        const int64_t grp = wave_valid ? (c0 + 16 * w) / dm.dg : 0;
-        const hraw_t *hg = (const hraw_t *)h + grp * hl;
-        for (int i = l; i < HTAB; i += 64) {
-            const int lag = i - HPAD;
-            htab[w * HTAB + i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
-        }
-    }
+#pragma unroll
+    for (int k = 0; k < HTAB / 64; ++k) htab[w * HTAB + l + 64 * k] = hv[k];
     __syncthreads();
     op_t W0[NK], W1[NK];
 #pragma unroll
