@@ -30,8 +30,17 @@ extern "C" {
 #define GCG_API
 #endif
 
-/* Element types (the reference's `cgcg_dtype`, savanna/arguments/global_config.py:404). */
-enum { GCG_F32 = 0, GCG_BF16 = 1, GCG_F16 = 2 };
+/* Element types (the reference's `cgcg_dtype`, savanna/arguments/global_config.py:404).
+ *
+ * GCG_BF16_F32 and GCG_F16_F32 replace the casts the reference's operators put around the
+ * call when `cgcg_dtype` ("float32", the default) differs from the activations' dtype
+ * (savanna/model/operators/hyena/hyena.py:499-503 and :533-534, :805-817): the tensors
+ * x, B, C, y, dy, dx, dB, dC are 16-bit, the filter h and its gradient dh are fp32, and
+ * nothing is rounded to 16 bits between a load and a store -- the values are those of
+ * `op(x.float(), B.float(), C.float(), h).to(bf16)` and of its autograd backward.
+ * gcg_fwd, gcg_bwd, gcg_bwd_static, gcg_fwd_interleaved, gcg_bwd_interleaved take them
+ * (every kernel family); the featurizer entry points do not (GCG_ERR_BAD_ARG). */
+enum { GCG_F32 = 0, GCG_BF16 = 1, GCG_F16 = 2, GCG_BF16_F32 = 3, GCG_F16_F32 = 4 };
 
 /* Kernel families.  GCG_ALGO_AUTO picks by (dtype, hl, dg); the others force one
  * family and fail with GCG_ERR_UNSUPPORTED when the shape does not fit it. */

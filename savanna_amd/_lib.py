@@ -25,6 +25,7 @@ ALGO_AUTO, ALGO_DIRECT, ALGO_WINDOW, ALGO_MFMA = 0, 1, 2, 3
 ALGO_NAMES = {"auto": ALGO_AUTO, "direct": ALGO_DIRECT, "window": ALGO_WINDOW, "mfma": ALGO_MFMA}
 
 _DTYPES = {torch.float32: GCG_F32, torch.bfloat16: GCG_BF16, torch.float16: GCG_F16}
+GCG_BF16_F32, GCG_F16_F32 = 3, 4       # 16-bit tensors, fp32 filter and arithmetic
 
 # every symbol include/gcg.h declares
 EXPORTS = (
@@ -108,6 +109,17 @@ def dtype_code(dtype: torch.dtype) -> int:
         raise TypeError(f"unsupported dtype {dtype}; expected float32, bfloat16 or float16") from None
 
 
+def gated_code(x: torch.Tensor, h: torch.Tensor) -> int:
+    """dtype code of the gated operator: the tensors' dtype, or 16-bit tensors with a float32 filter
+    (GCG_BF16_F32 / GCG_F16_F32: fp32 arithmetic and an fp32 filter gradient, no casts around the call)."""
+    if h.dtype == x.dtype:
+        return dtype_code(x.dtype)
+    if h.dtype == torch.float32 and x.dtype in (torch.bfloat16, torch.float16):
+        return GCG_BF16_F32 if x.dtype == torch.bfloat16 else GCG_F16_F32
+    raise TypeError(f"the filter must have the tensors' dtype, or be float32 with bfloat16 / float16 tensors; "
+                    f"got {x.dtype} tensors and a {h.dtype} filter")
+
+
 def algo_code(algo) -> int:
     if isinstance(algo, str):
         return ALGO_NAMES[algo]
@@ -186,7 +198,7 @@ def fwd(x, B, C, h, return_bx=False, return_y2=False, algo=ALGO_AUTO, out=None):
             x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), y.data_ptr(),
             y2.data_ptr() if y2 is not None else None,
             bx.data_ptr() if bx is not None else None,
-            bs, L, g, dg, hl, dtype_code(x.dtype), algo_code(algo), st,
+            bs, L, g, dg, hl, gated_code(x, h), algo_code(algo), st,
         )
     check(rc, "gcg_fwd")
     return bx, y2, y
@@ -204,7 +216,7 @@ def bwd(dy, x, B, C, h, algo=ALGO_AUTO):
     dh = torch.empty_like(h)
     if x.numel() == 0:
         return dx, dB, dC, dh.zero_()
-    code, a = dtype_code(x.dtype), algo_code(algo)
+    code, a = gated_code(x, h), algo_code(algo)
     nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, a)
     if nbytes == 0:
         raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")
@@ -234,7 +246,7 @@ def bwd_static(dy, x, B, C, h, dx, dB, dC, dh, algo=ALGO_AUTO):
         rc = lib.gcg_bwd_static(
             dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(),
             dx.data_ptr(), dB.data_ptr(), dC.data_ptr(), dh.data_ptr(),
-            bs, L, g, dg, h.shape[-1], dtype_code(x.dtype), algo_code(algo),
+            bs, L, g, dg, h.shape[-1], gated_code(x, h), algo_code(algo),
             torch.cuda.current_stream().cuda_stream,
         )
     check(rc, "gcg_bwd_static")
@@ -245,7 +257,8 @@ def _check_feat(feat, h):
         raise ValueError("feat must be a contiguous (bs, L, g, dg, 3) tensor")
     if h.dim() != 3 or h.shape[0] != feat.shape[2] or h.shape[1] != 1 or not h.is_contiguous():
         raise ValueError("h must be a contiguous (g, 1, hl) tensor")
-    if h.dtype != feat.dtype or h.device != feat.device:
+    gated_code(feat, h)
+    if h.device != feat.device:
         raise ValueError("feat and h must share dtype and device")
 
 
@@ -268,7 +281,7 @@ def fwd_interleaved(feat, h, algo=ALGO_AUTO, out=None):
     with _on_device(feat.device):
         st = torch.cuda.current_stream().cuda_stream
         rc = lib.gcg_fwd_interleaved(feat.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg, hl,
-                                     dtype_code(feat.dtype), algo_code(algo), st)
+                                     gated_code(feat, h), algo_code(algo), st)
     check(rc, "gcg_fwd_interleaved")
     return y
 
@@ -292,7 +305,7 @@ def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO, keep_output=False):
     dh = torch.empty_like(h)
     if dy.numel() == 0:
         return dfeat, dh.zero_()
-    code, a = dtype_code(feat.dtype), algo_code(algo)
+    code, a = gated_code(feat, h), algo_code(algo)
     nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, a)
     if nbytes == 0:
         raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")

@@ -31,10 +31,14 @@ int check_device()
     return ok[dev] == 1 ? GCG_OK : GCG_ERR_DEVICE;
 }
 
-int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, gcg::Dims *dm)
+// mixed_ok: the entry point takes GCG_BF16_F32 / GCG_F16_F32 (the gated operator does, the featurizer does not)
+int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, gcg::Dims *dm,
+              bool mixed_ok = false)
 {
     if (bs <= 0 || L <= 0 || g <= 0 || dg <= 0 || hl <= 0) return GCG_ERR_BAD_ARG;
-    if (dtype != GCG_F32 && dtype != GCG_BF16 && dtype != GCG_F16) return GCG_ERR_BAD_ARG;
+    const bool plain = dtype == GCG_F32 || dtype == GCG_BF16 || dtype == GCG_F16;
+    const bool mixed = dtype == GCG_BF16_F32 || dtype == GCG_F16_F32;
+    if (!plain && !(mixed && mixed_ok)) return GCG_ERR_BAD_ARG;
     dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg; dm->es = 1; dm->keep_out = 0;
     return GCG_OK;
 }
@@ -148,7 +152,7 @@ GCG_API int gcg_version(void) { return 106; }
 GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t backward)
 {
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     return resolve_algo(GCG_ALGO_AUTO, dtype, dm, backward != 0);
 }
@@ -160,7 +164,7 @@ GCG_API int gcg_fwd(const void *x, const void *B, const void *C, const void *h, 
     TimerScope timer_scope;
     if (!x || !B || !C || !h || !y) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     const int a = resolve_algo(algo, dtype, dm, false, all_aligned16({x, B, C, y, y2, bx}));
     if (a < 0) return a;
@@ -179,7 +183,7 @@ GCG_API size_t gcg_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t
                                int32_t algo)
 {
     gcg::Dims dm;
-    if (make_dims(bs, L, g, dg, hl, dtype, &dm)) return 0;
+    if (make_dims(bs, L, g, dg, hl, dtype, &dm, true)) return 0;
     const int a = resolve_algo(algo, dtype, dm, true);
     size_t n = 0;
     switch (a) {
@@ -200,7 +204,7 @@ GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C,
     TimerScope timer_scope;
     if (!dy || !x || !B || !C || !h || !dx || !dB || !dC || !dh) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, x, B, C, dx, dB, dC}));
     if (a < 0) return a;
@@ -227,7 +231,7 @@ GCG_API int gcg_bwd_static(const void *dy, const void *x, const void *B, const v
     TimerScope timer_scope;
     if (!dy || !x || !B || !C || !h || !dx || !dB || !dC || !dh) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, x, B, C, dx, dB, dC}));
     if (a < 0) return a;
@@ -259,7 +263,7 @@ GCG_API int gcg_fwd_interleaved(const void *feat, const void *h, void *y, int64_
     TimerScope timer_scope;
     if (!feat || !h || !y) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     dm.es = 3;
     const int a = resolve_algo(algo, dtype, dm, false, all_aligned16({feat, y}));
@@ -283,7 +287,7 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
     TimerScope timer_scope;
     if (!dy || !feat || !h || !dfeat || !dh || (flags & ~GCG_KEEP_OUTPUT)) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     dm.es = 3;
     dm.keep_out = flags & GCG_KEEP_OUTPUT;

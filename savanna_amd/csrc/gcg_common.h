@@ -15,6 +15,14 @@ namespace gcg {
 // bf16 and f16 travel as raw 16-bit patterns; arithmetic is always fp32.
 struct bf16_t { uint16_t v; };
 struct f16_t  { uint16_t v; };
+// GCG_BF16_F32 / GCG_F16_F32: 16-bit tensors with an fp32 filter, fp32 filter gradient and nothing rounded to
+// 16 bits between load and store -- the operator "run in fp32" on a 16-bit model without the casts around it.
+struct bf16w_t { uint16_t v; };
+struct f16w_t  { uint16_t v; };
+// element type of h and dh for tensors of type T
+template <typename T> struct Filt { typedef T type; };
+template <> struct Filt<bf16w_t> { typedef float type; };
+template <> struct Filt<f16w_t> { typedef float type; };
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t lo16)
 {
@@ -60,6 +68,10 @@ template <> struct Elem<bf16_t> {
     static __device__ __forceinline__ float load(const bf16_t *p) { return bf16_bits_to_float(p->v); }
     static __device__ __forceinline__ void store(bf16_t *p, float v) { p->v = (uint16_t)float_to_bf16_bits(v); }
 };
+template <> struct Elem<bf16w_t> {
+    static __device__ __forceinline__ float load(const bf16w_t *p) { return bf16_bits_to_float(p->v); }
+    static __device__ __forceinline__ void store(bf16w_t *p, float v) { p->v = (uint16_t)float_to_bf16_bits(v); }
+};
 template <> struct Elem<f16_t> {
     static __device__ __forceinline__ float load(const f16_t *p)
     {
@@ -72,6 +84,11 @@ template <> struct Elem<f16_t> {
         _Float16 hv = (_Float16)v;
         __builtin_memcpy(&p->v, &hv, 2);
     }
+};
+
+template <> struct Elem<f16w_t> {
+    static __device__ __forceinline__ float load(const f16w_t *p) { return Elem<f16_t>::load((const f16_t *)p); }
+    static __device__ __forceinline__ void store(f16w_t *p, float v) { Elem<f16_t>::store((f16_t *)p, v); }
 };
 
 // ---- tensor windows --------------------------------------------------------------------

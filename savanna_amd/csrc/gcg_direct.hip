@@ -40,7 +40,8 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(const T *__restrict__ x
     const int hl = dm.hl;
     const int64_t es = dm.es;   // element stride of x, B, C (3 when they are interleaved in one tensor)
     const int64_t t0 = tt * TT;
-    const T *hg = h + (cvalid ? (c / dm.dg) : 0) * hl;
+    typedef typename Filt<T>::type FT;           // element type of the filter
+    const FT *hg = (const FT *)h + (cvalid ? (c / dm.dg) : 0) * hl;
 
     float acc[RB];
 #pragma unroll
@@ -126,7 +127,8 @@ __global__ __launch_bounds__(256) void direct_bwd_kernel(const T *__restrict__ d
     const bool cvalid = c < d;
     const int hl = dm.hl, dg = dm.dg;
     const int64_t es = dm.es;   // element stride of x, B, C, dx, dB, dC
-    const T *hg = h + (cvalid ? (c / dg) : 0) * hl;
+    typedef typename Filt<T>::type FT;           // element type of the filter
+    const FT *hg = (const FT *)h + (cvalid ? (c / dg) : 0) * hl;
     const int64_t g0 = c0 / dg;                                            // first group in this tile
     const int64_t clast = (c0 + CT < d ? c0 + CT : d) - 1;
     const int ngl = (int)(clast / dg - g0) + 1;                            // groups in this tile
@@ -254,7 +256,8 @@ __global__ __launch_bounds__(256) void direct_dh_reduce_kernel(const float *__re
             const int64_t gl = grp - ct * CT / dm.dg;
             s += ws[((size_t)(p * nct + ct) * gpt + gl) * dm.hl + k];
         }
-    Elem<T>::store(dh + i, s);
+    typedef typename Filt<T>::type FT;
+    Elem<FT>::store((FT *)dh + i, s);
 }
 
 struct BwdPlan { int nct, ntt, nseg, tps, gpt; int64_t nwg; };
@@ -313,6 +316,8 @@ int direct_fwd_launch(int dtype, const void *x, const void *B, const void *C, co
     case GCG_F32:  return fwd_t<float>(x, B, C, h, y, y2, bx, dm, st);
     case GCG_BF16: return fwd_t<bf16_t>(x, B, C, h, y, y2, bx, dm, st);
     case GCG_F16:  return fwd_t<f16_t>(x, B, C, h, y, y2, bx, dm, st);
+    case GCG_BF16_F32: return fwd_t<bf16w_t>(x, B, C, h, y, y2, bx, dm, st);
+    case GCG_F16_F32:  return fwd_t<f16w_t>(x, B, C, h, y, y2, bx, dm, st);
     }
     return (int)hipErrorInvalidValue;
 }
@@ -330,6 +335,8 @@ int direct_bwd_launch(int dtype, const void *dy, const void *x, const void *B, c
     case GCG_F32:  return bwd_t<float>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     case GCG_BF16: return bwd_t<bf16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     case GCG_F16:  return bwd_t<f16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    case GCG_BF16_F32: return bwd_t<bf16w_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    case GCG_F16_F32:  return bwd_t<f16w_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     }
     return (int)hipErrorInvalidValue;
 }

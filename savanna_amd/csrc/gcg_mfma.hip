@@ -127,7 +127,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 #pragma unroll
     for (int k = 0; k < HTAB / 64; ++k) htab[w][l + 64 * k] = hv[k];
     __syncthreads();
-    op_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
+    typename M::wop_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
         W0[i] = M::toeplitz(htab[w], 32 * i, j, q);
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
             unpack8<T>(lB[i - 1], Bf);
 #pragma unroll
             for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
-            store_operand_row<T>(u_wr + (i - 1) * STEP * UROW, UROW, pack8<T>(uf));
+            store_operand<T>(u_wr + (i - 1) * STEP * UROW, UROW, uf);
         }
         __syncthreads();
 #pragma unroll
@@ -165,10 +165,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                 unpack8<T>(Br, Bf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
-                const Row<T> up = pack8<T>(uf);
-                store_operand_row<T>(u_wr, UROW, up);
+                store_operand<T>(u_wr, UROW, uf);
                 const uint32_t o = lane_off + step_off(s);
-                if constexpr (EXTRA) stw_row<T>(wbx, o, up);
+                if constexpr (EXTRA) stw_row<T>(wbx, o, pack8<T>(uf));
                 __syncthreads();
                 A[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
                 {
@@ -341,7 +340,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
 #pragma unroll
     for (int k = 0; k < HTAB / 64; ++k) htab[w * HTAB + l + 64 * k] = hv[k];
     __syncthreads();
-    op_t W0[NK], W1[NK];
+    typename M::wop_t W0[NK], W1[NK];
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
         W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
@@ -357,13 +356,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
             unpack8<T>(wB_[i - 1], f1);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
-            store_operand_row<T>(u_rm + rm_off, UROW, pack8<T>(pf));
+            store_operand<T>(u_rm + rm_off, UROW, pf);
             unpack8<T>(wdy_[i - 1], f0);
             unpack8<T>(wC_[i - 1], f1);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
             unsigned char *g_slot = g_rm + (NK - 1 - i) * STEP * UROW;
-            store_operand_row<T>(g_slot + rm_off, UROW, pack8<T>(pf));
+            store_operand<T>(g_slot + rm_off, UROW, pf);
             dyq[NK - 1 - i] = wdy_[i - 1];
             __syncthreads();
             Au[NK - i] = M::load_operand(u_rm, UROW, w, j, q, false);
@@ -387,13 +386,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                 unpack8<T>(Br, Bf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[e] = xf[e] * Bf[e];
-                store_operand_row<T>(u_rm + rm_off, UROW, pack8<T>(pf));
+                store_operand<T>(u_rm + rm_off, UROW, pf);
                 unpack8<T>(dyr, tf);
                 unpack8<T>(Cr, cf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) pf[e] = tf[e] * cf[e];
                 unsigned char *g_slot = g_rm + slot_new * STEP * UROW;
-                store_operand_row<T>(g_slot + rm_off, UROW, pack8<T>(pf));
+                store_operand<T>(g_slot + rm_off, UROW, pf);
                 dyq[slot_new] = dyr;
                 __syncthreads();
                 Au[ph] = M::load_operand(u_rm, UROW, w, j, q, false);
@@ -421,7 +420,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         row0 = (row0 >= RING_ROWS) ? row0 - RING_ROWS : row0;
                         row1 = (row1 >= RING_ROWS) ? row1 - RING_ROWS : row1;
                         const op_t gn = M::load_natural(g_rm + row0 * UROW, g_rm + row1 * UROW, UROW, w, q);
-                        P[dl] = M::mfma(gn, un, P[dl]);
+                        P[dl] = M::mfma_aa(gn, un, P[dl]);
                     }
                 }
                 __syncthreads();
@@ -465,7 +464,7 @@ int fwd_launch(const void *x, const void *B, const void *C, const void *h, void 
 {
     int e = 0;
     // 16-bit: ~112 registers, 4 waves per SIMD; fp32: ~200 registers, 2 waves per SIMD
-    MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
+    MfmaPlan p = plan(dm, NW, 16, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     // Workgroup order.  With 32 or more channel blocks per row the XCD-contiguous order gives an XCD whole rows;
     // with fewer, dealing the blocks round-robin measured 3-5 % faster in the forward (d = 2048, 4096) and the same
@@ -485,8 +484,8 @@ template <typename T, int NK>
 int fwd_nk(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
            const Dims &dm, hipStream_t st)
 {
-    const int nw = choose_nw(dm, sizeof(T) == 4);
-    if constexpr (sizeof(T) == 2) {
+    const int nw = choose_nw(dm, MT<T>::SPLIT);
+    if constexpr (!MT<T>::SPLIT) {
         if (nw == 16) return fwd_launch<T, NK, 16>(x, B, C, h, y, y2, bx, dm, st);
     }
     if (nw == 8) return fwd_launch<T, NK, 8>(x, B, C, h, y, y2, bx, dm, st);
@@ -521,6 +520,8 @@ int mfma_fwd_launch(int dtype, const void *x, const void *B, const void *C, cons
     if (dtype == GCG_BF16) return fwd_t<bf16_t>(x, B, C, h, y, y2, bx, dm, st);
     if (dtype == GCG_F16) return fwd_t<f16_t>(x, B, C, h, y, y2, bx, dm, st);
     if (dtype == GCG_F32) return fwd_t<float>(x, B, C, h, y, y2, bx, dm, st);
+    if (dtype == GCG_BF16_F32) return fwd_t<bf16w_t>(x, B, C, h, y, y2, bx, dm, st);
+    if (dtype == GCG_F16_F32) return fwd_t<f16w_t>(x, B, C, h, y, y2, bx, dm, st);
     return (int)hipErrorInvalidValue;
 }
 
@@ -534,7 +535,7 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
                void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
     int e = 0;
-    MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
+    MfmaPlan p = plan_bwd(dm, MT<T>::SPLIT, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (p.fuse_dh) p.slot = next_dh_slot();
     e = launch_main((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
@@ -551,7 +552,7 @@ template <typename T, int NK>
 int bwd_nk(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
            void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    if constexpr (sizeof(T) == 2) {
+    if constexpr (!MT<T>::SPLIT) {
         if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     }
     return bwd_launch<T, NK, 4>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
@@ -574,7 +575,7 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
 
 size_t mfma_bwd_workspace(int dtype, const Dims &dm)
 {
-    const MfmaPlan p = plan_bwd(dm, dtype == GCG_F32);
+    const MfmaPlan p = plan_bwd(dm, dtype != GCG_BF16 && dtype != GCG_F16, dtype == GCG_F32 ? 4 : 2);
     return (size_t)p.nwg * p.nw * 128 * sizeof(float);
 }
 
@@ -584,6 +585,8 @@ int mfma_bwd_launch(int dtype, const void *dy, const void *x, const void *B, con
     if (dtype == GCG_BF16) return bwd_t<bf16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     if (dtype == GCG_F16) return bwd_t<f16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     if (dtype == GCG_F32) return bwd_t<float>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    if (dtype == GCG_BF16_F32) return bwd_t<bf16w_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    if (dtype == GCG_F16_F32) return bwd_t<f16w_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     return (int)hipErrorInvalidValue;
 }
 

@@ -68,13 +68,19 @@ template <typename T> __device__ __forceinline__ uint32_t pack_unit(const float 
 // one lane's unit of a row (CH channels) into a matrix-operand tile, in the tile's own element format
 template <typename T> __device__ __forceinline__ void store_operand_unit(unsigned char *p, int urow, const float *f)
 {
-    if constexpr (MT<T>::ES == 4) {
-        uint16_t v[3];
-        MT<T>::split(f[0], v[0], v[1], v[2]);
+    typedef MT<T> M;
+    if constexpr (M::SPLIT) {
+        constexpr int CH = 4 / M::ES;
+        uint16_t v[CH][M::NPA];
 #pragma unroll
-        for (int m = 0; m < 3; ++m) *(uint16_t *)(p + m * MT<T>::plane(urow)) = v[m];
+        for (int c = 0; c < CH; ++c) M::template split<M::NPA>(f[c], v[c]);
+#pragma unroll
+        for (int m = 0; m < M::NPA; ++m) {
+            if constexpr (CH == 1) *(uint16_t *)(p + m * M::plane(urow)) = v[0][m];
+            else *(uint32_t *)(p + m * M::plane(urow)) = (uint32_t)v[0][m] | ((uint32_t)v[1][m] << 16);
+        }
     } else {
-        *(uint32_t *)p = MT<T>::pack2(f[0], f[1]);
+        *(uint32_t *)p = M::pack2(f[0], f[1]);
     }
 }
 // NR units in a row vector: unpack8 then yields them in element order e = k * CH + c
@@ -171,7 +177,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
         }
     }
     __syncthreads();
-    op_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
+    typename M::wop_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
         W0[i] = M::toeplitz(htab[w], 32 * i, j, q);
@@ -379,7 +385,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
         }
     }
     __syncthreads();
-    op_t W0[NK], W1[NK];
+    typename M::wop_t W0[NK], W1[NK];
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
         W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
@@ -478,7 +484,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
                         row0 = (row0 >= RING_ROWS) ? row0 - RING_ROWS : row0;
                         row1 = (row1 >= RING_ROWS) ? row1 - RING_ROWS : row1;
                         const op_t gn = M::load_natural(g_rm + row0 * UROW, g_rm + row1 * UROW, UROW, w, q);
-                        P[dl] = M::mfma(gn, un, P[dl]);
+                        P[dl] = M::mfma_aa(gn, un, P[dl]);
                     }
                 }
                 __syncthreads();
@@ -518,7 +524,7 @@ template <typename T, int NK, int NW>
 int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
 {
     int e = 0;
-    MfmaPlan p = plan(dm, NW, 16, sizeof(T) == 4 ? 8 : 16, sizeof(T));
+    MfmaPlan p = plan(dm, NW, 16, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     // Workgroup order: dealing the channel blocks to the XCDs round-robin measured 3-4 % faster than XCD-contiguous
     // runs on interleaved operands at every width (d = 4096: 102.5 against 105.4 us, d = 8192: 376 against 389 us,
@@ -532,8 +538,8 @@ int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStre
 
 template <typename T, int NK> int fwd_nk(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
 {
-    const int nw = choose_nw(dm, sizeof(T) == 4);
-    if constexpr (sizeof(T) == 2) {
+    const int nw = choose_nw(dm, MT<T>::SPLIT);
+    if constexpr (!MT<T>::SPLIT) {
         if (nw == 16) return fwd_launch<T, NK, 16>(feat, h, y, dm, st);
     }
     if (nw == 8) return fwd_launch<T, NK, 8>(feat, h, y, dm, st);
@@ -557,7 +563,7 @@ int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, voi
                hipStream_t st)
 {
     int e = 0;
-    MfmaPlan p = plan_bwd(dm, sizeof(T) == 4);
+    MfmaPlan p = plan_bwd(dm, MT<T>::SPLIT, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (p.fuse_dh) p.slot = next_dh_slot();
     if (dm.keep_out)
@@ -577,7 +583,7 @@ template <typename T, int NK>
 int bwd_nk(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *ws, const Dims &dm,
            hipStream_t st)
 {
-    if constexpr (sizeof(T) == 2) {
+    if constexpr (!MT<T>::SPLIT) {
         if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, feat, h, dfeat, dh, ws, dm, st);
     }
     return bwd_launch<T, NK, 4>(dy, feat, h, dfeat, dh, ws, dm, st);
@@ -603,6 +609,8 @@ int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, cons
     if (dtype == GCG_BF16) return fwd_t<bf16_t>(feat, h, y, dm, st);
     if (dtype == GCG_F16) return fwd_t<f16_t>(feat, h, y, dm, st);
     if (dtype == GCG_F32) return fwd_t<float>(feat, h, y, dm, st);
+    if (dtype == GCG_BF16_F32) return fwd_t<bf16w_t>(feat, h, y, dm, st);
+    if (dtype == GCG_F16_F32) return fwd_t<f16w_t>(feat, h, y, dm, st);
     return (int)hipErrorInvalidValue;
 }
 
@@ -612,6 +620,8 @@ int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *
     if (dtype == GCG_BF16) return bwd_t<bf16_t>(dy, feat, h, dfeat, dh, ws, dm, st);
     if (dtype == GCG_F16) return bwd_t<f16_t>(dy, feat, h, dfeat, dh, ws, dm, st);
     if (dtype == GCG_F32) return bwd_t<float>(dy, feat, h, dfeat, dh, ws, dm, st);
+    if (dtype == GCG_BF16_F32) return bwd_t<bf16w_t>(dy, feat, h, dfeat, dh, ws, dm, st);
+    if (dtype == GCG_F16_F32) return bwd_t<f16w_t>(dy, feat, h, dfeat, dh, ws, dm, st);
     return (int)hipErrorInvalidValue;
 }
 

@@ -51,9 +51,11 @@ template <typename OP> struct MT16 {
     static constexpr int ES = 2;                 // bytes per element in memory
     static constexpr int RW = 1;                 // 16-byte words per 8-channel row vector
     static constexpr int LES = 2;                // bytes per element of the operand tiles in LDS
+    static constexpr bool SPLIT = false;         // operands are the tensors' own 16-bit values
     // bytes per LDS row of an operand tile of cb channels; the padding makes consecutive rows start 8 banks apart
     static constexpr int urow(int cb) { return cb * 2 + 32; }
-    typedef OP op_t;
+    typedef OP op_t;                             // operand made of activations
+    typedef OP wop_t;                            // operand made of filter taps
     typedef uint16_t hraw_t;
     static __device__ __forceinline__ int kmap(int q, int e) { return 8 * q + e; }
     static __device__ __forceinline__ op_t zero_op()
@@ -84,12 +86,6 @@ template <typename OP> struct MT16 {
         __builtin_memcpy(&r, &t4, 16);
         return r;
     }
-    // a lane's 8 channels of one row (already packed to 16 bits) into an operand tile
-    static __device__ __forceinline__ void store_u8(unsigned char *p, int urow, const uint4 &packed)
-    {
-        (void)urow;
-        *(uint4 *)p = packed;
-    }
     static __device__ __forceinline__ op_t toeplitz(const hraw_t *htab, int doff, int j, int q)
     {
         uint16_t v[8];
@@ -102,10 +98,12 @@ template <typename OP> struct MT16 {
 };
 
 template <> struct MT<bf16_t> : MT16<bf16x8> {
+    typedef bf16_t filt_t;                       // element type of h and dh
     static __device__ __forceinline__ f32x4 mfma(op_t a, op_t b, f32x4 c)
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x4 mfma_aa(op_t a, op_t b, f32x4 c) { return mfma(a, b, c); }
     static __device__ __forceinline__ void unpack2(uint32_t p, float &lo, float &hi)
     {
         lo = __uint_as_float(p << 16);
@@ -114,10 +112,12 @@ template <> struct MT<bf16_t> : MT16<bf16x8> {
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 };
 template <> struct MT<f16_t> : MT16<f16x8> {
+    typedef f16_t filt_t;
     static __device__ __forceinline__ f32x4 mfma(op_t a, op_t b, f32x4 c)
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
     }
+    static __device__ __forceinline__ f32x4 mfma_aa(op_t a, op_t b, f32x4 c) { return mfma(a, b, c); }
     static __device__ __forceinline__ void unpack2(uint32_t p, float &lo, float &hi)
     {
         typedef _Float16 h2 __attribute__((ext_vector_type(2)));
@@ -129,39 +129,44 @@ template <> struct MT<f16_t> : MT16<f16x8> {
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
 };
 
-// fp32 on the bf16 matrix cores.  An fp32 value is the exact sum of three bf16 values (8 significant bits each:
-// v1 = bf16(v), v2 = bf16(v - v1), v3 = bf16(v - v1 - v2)), and the product of two bf16 values is exact in the
-// fp32 accumulator, so  a * b  =  sum of a_m * b_n  over the planes; the six terms with m + n <= 4 carry it to
-// 2^-24 relative to |a b| (the three left out are below that), i.e. to fp32 accuracy, at 6 matrix instructions of 16
-// cycles instead of the 8 fp32 ones of 32 cycles that the same 32-deep product costs on the fp32 matrix path.
-// Operand tiles in LDS hold the three planes of a row side by side (plane m at byte offset m * plane(urow)), each
-// laid out like a 16-bit tile, so operands come from the same transposing reads.
-struct Split3 { bf16x8 p[3]; };
-template <> struct MT<float> {
-    static constexpr int ES = 4;
-    static constexpr int RW = 2;
+// fp32 arithmetic on the bf16 matrix cores.  An fp32 value is the exact sum of three bf16 values (8 significant
+// bits each: v1 = bf16(v), v2 = bf16(v - v1), v3 = bf16(v - v1 - v2)), and the product of two bf16 values is
+// exact in the fp32 accumulator, so  a * b  =  sum of a_m * b_n  over the planes; the terms with m + n <= 4 carry
+// it to 2^-24 relative to |a b| (the ones left out are below that), i.e. to fp32 accuracy, at 6 matrix
+// instructions of 16 cycles instead of the 8 fp32 ones of 32 cycles that the same 32-deep product costs on the
+// fp32 matrix path.  Operand tiles in LDS hold the planes of a row side by side (plane m at byte offset
+// m * plane(urow)), each laid out like a 16-bit tile, so operands come from the same transposing reads.
+//
+// NPA = planes of an activation operand.  fp32 tensors: 3.  bf16 tensors computed in fp32 (the pre-gate product
+// of two bf16 values has 16 significant bits): 2 exactly, which leaves 5 terms against the filter's three planes
+// and 4, all exact, in the filter-gradient product of two activation operands.
+template <int NPA> struct SplitOp { bf16x8 p[NPA]; };
+template <int NPA_> struct MTSplit {
     static constexpr int LES = 2;
-    static constexpr int NP = 3;
+    static constexpr bool SPLIT = true;
+    static constexpr int NPA = NPA_, NPW = 3;
     static constexpr int RPAD = 32;              // with it consecutive rows start an odd multiple of 8 banks apart
-    static constexpr int urow(int cb) { return NP * cb * 2 + RPAD; }
-    static __device__ __forceinline__ int plane(int urow) { return (urow - RPAD) / NP; }   // bytes between planes
-    typedef Split3 op_t;
+    static constexpr int urow(int cb) { return NPA * cb * 2 + RPAD; }
+    static __device__ __forceinline__ int plane(int urow) { return (urow - RPAD) / NPA; }   // bytes between planes
+    typedef SplitOp<NPA> op_t;
+    typedef SplitOp<NPW> wop_t;
     typedef float hraw_t;
+    typedef float filt_t;
     static __device__ __forceinline__ int kmap(int q, int e) { return 8 * q + e; }
-    static __device__ __forceinline__ void split(float v, uint16_t &v1, uint16_t &v2, uint16_t &v3)
+    template <int N> static __device__ __forceinline__ void split(float v, uint16_t (&o)[N])
     {
-        v1 = (uint16_t)float_to_bf16_bits(v);
-        const float r1 = v - bf16_bits_to_float(v1);
-        v2 = (uint16_t)float_to_bf16_bits(r1);
-        const float r2 = r1 - bf16_bits_to_float(v2);
-        v3 = (uint16_t)float_to_bf16_bits(r2);
+#pragma unroll
+        for (int m = 0; m < N; ++m) {
+            o[m] = (uint16_t)float_to_bf16_bits(v);
+            if (m + 1 < N) v -= bf16_bits_to_float(o[m]);
+        }
     }
     static __device__ __forceinline__ op_t zero_op()
     {
         op_t r;
         const uint4 z = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
-        for (int m = 0; m < NP; ++m) __builtin_memcpy(&r.p[m], &z, 16);
+        for (int m = 0; m < NPA; ++m) __builtin_memcpy(&r.p[m], &z, 16);
         return r;
     }
     static __device__ __forceinline__ op_t load_operand(const unsigned char *tile, int urow, int w, int j, int q,
@@ -169,7 +174,7 @@ template <> struct MT<float> {
     {
         op_t r;
 #pragma unroll
-        for (int m = 0; m < NP; ++m) {
+        for (int m = 0; m < NPA; ++m) {
             const uint4 t4 = tr_operand16(tile + m * plane(urow), urow, w, j, q, reversed);
             __builtin_memcpy(&r.p[m], &t4, 16);
         }
@@ -181,48 +186,83 @@ template <> struct MT<float> {
         const unsigned char *p = ((q >> 1) ? row_half1 : row_half0) + (16 * w + 8 * (q & 1)) * 2;
         op_t r;
 #pragma unroll
-        for (int m = 0; m < NP; ++m) {
+        for (int m = 0; m < NPA; ++m) {
             const uint4 t4 = *(const uint4 *)(p + m * plane(urow));
             __builtin_memcpy(&r.p[m], &t4, 16);
         }
         return r;
     }
-    static __device__ __forceinline__ op_t toeplitz(const hraw_t *htab, int doff, int j, int q)
+    static __device__ __forceinline__ wop_t toeplitz(const hraw_t *htab, int doff, int j, int q)
     {
-        uint16_t v[NP][8];
+        uint16_t v[NPW][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) split(htab[doff + j - kmap(q, e) + HPAD], v[0][e], v[1][e], v[2][e]);
-        op_t r;
+        for (int e = 0; e < 8; ++e) {
+            uint16_t o[NPW];
+            split<NPW>(htab[doff + j - kmap(q, e) + HPAD], o);
 #pragma unroll
-        for (int m = 0; m < NP; ++m) __builtin_memcpy(&r.p[m], v[m], 16);
+            for (int m = 0; m < NPW; ++m) v[m][e] = o[m];
+        }
+        wop_t r;
+#pragma unroll
+        for (int m = 0; m < NPW; ++m) __builtin_memcpy(&r.p[m], v[m], 16);
         return r;
     }
     // smallest terms first
-    static __device__ __forceinline__ f32x4 mfma(const op_t &a, const op_t &b, f32x4 c)
+    template <int NA, int NB>
+    static __device__ __forceinline__ f32x4 mfma_terms(const SplitOp<NA> &a, const SplitOp<NB> &b, f32x4 c)
     {
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[2], b.p[0], c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[1], b.p[1], c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[0], b.p[2], c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[1], b.p[0], c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[0], b.p[1], c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[0], b.p[0], c, 0, 0, 0);
+#pragma unroll
+        for (int sum = 2; sum >= 0; --sum)
+#pragma unroll
+            for (int m = 0; m <= sum; ++m)
+                if (m < NA && sum - m < NB)
+                    c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.p[m], b.p[sum - m], c, 0, 0, 0);
         return c;
     }
-    // a lane's 8 fp32 channels of one row (two 16-byte words) into the three planes of an operand tile
-    static __device__ __forceinline__ void store_u8(unsigned char *p, int urow, const uint4 &w0, const uint4 &w1)
+    static __device__ __forceinline__ f32x4 mfma(const op_t &a, const wop_t &b, f32x4 c)
     {
-        const float f[8] = {__uint_as_float(w0.x), __uint_as_float(w0.y), __uint_as_float(w0.z), __uint_as_float(w0.w),
-                            __uint_as_float(w1.x), __uint_as_float(w1.y), __uint_as_float(w1.z), __uint_as_float(w1.w)};
-        uint16_t v[NP][8];
+        return mfma_terms<NPA, NPW>(a, b, c);
+    }
+    static __device__ __forceinline__ f32x4 mfma_aa(const op_t &a, const op_t &b, f32x4 c)
+    {
+        return mfma_terms<NPA, NPA>(a, b, c);
+    }
+    // a lane's 8 channels of one row into the planes of an operand tile
+    static __device__ __forceinline__ void store_f8(unsigned char *p, int urow, const float (&f)[8])
+    {
+        uint16_t v[NPA][8];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) split(f[e], v[0][e], v[1][e], v[2][e]);
+        for (int e = 0; e < 8; ++e) {
+            uint16_t o[NPA];
+            split<NPA>(f[e], o);
 #pragma unroll
-        for (int m = 0; m < NP; ++m) {
+            for (int m = 0; m < NPA; ++m) v[m][e] = o[m];
+        }
+#pragma unroll
+        for (int m = 0; m < NPA; ++m) {
             uint4 t4;
             __builtin_memcpy(&t4, v[m], 16);
             *(uint4 *)(p + m * plane(urow)) = t4;
         }
     }
+};
+template <> struct MT<float> : MTSplit<3> {
+    static constexpr int ES = 4;                 // bytes per element in memory
+    static constexpr int RW = 2;                 // 16-byte words per 8-channel row vector
+};
+// bf16 / f16 tensors, fp32 filter, fp32 arithmetic: what a 16-bit model gets from the operator run "in fp32"
+// (every tensor cast up before it and the result cast down after), without the casts.
+template <> struct MT<bf16w_t> : MTSplit<2> {
+    static constexpr int ES = 2;
+    static constexpr int RW = 1;
+    static __device__ __forceinline__ void unpack2(uint32_t p, float &lo, float &hi) { MT<bf16_t>::unpack2(p, lo, hi); }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
+};
+template <> struct MT<f16w_t> : MTSplit<3> {
+    static constexpr int ES = 2;
+    static constexpr int RW = 1;
+    static __device__ __forceinline__ void unpack2(uint32_t p, float &lo, float &hi) { MT<f16_t>::unpack2(p, lo, hi); }
+    static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
 };
 
 // A workgroup of NW waves owns CB = 16*NW adjacent channels; LDS rows are padded (see MT<T>::urow;
@@ -278,10 +318,10 @@ template <typename T> __device__ __forceinline__ void lds_store_row(unsigned cha
 }
 
 // a lane's 8 channels of one row into a matrix-operand tile (in the tile's own element format)
-template <typename T> __device__ __forceinline__ void store_operand_row(unsigned char *p, int urow, const Row<T> &r)
+template <typename T> __device__ __forceinline__ void store_operand(unsigned char *p, int urow, const float (&f)[8])
 {
-    if constexpr (MT<T>::ES == 4) MT<T>::store_u8(p, urow, r.w[0], r.w[1]);
-    else MT<T>::store_u8(p, urow, r.w[0]);
+    if constexpr (MT<T>::SPLIT) MT<T>::store_f8(p, urow, f);
+    else *(uint4 *)p = pack8<T>(f).w[0];
 }
 
 template <typename T> __device__ __forceinline__ Row<T> lds_load_row(const unsigned char *p)
@@ -340,7 +380,8 @@ __global__ __launch_bounds__(256) void mfma_dh_reduce_kernel(const float *__rest
     for (int64_t p = 0; p < dm.bs * pl.nseg; ++p)
         for (int k = 0; k < bpg; ++k)
             sum += ws[(p * slots + grp * bpg + k) * 128 + lag];
-    Elem<T>::store(dh + i, sum);
+    typedef typename MT<T>::filt_t F;
+    Elem<F>::store((F *)dh + i, sum);
 }
 
 // ---- filter-gradient reduction at the end of the backward kernel itself ----------------------
@@ -422,7 +463,8 @@ __device__ __forceinline__ void dh_finish(const f32x4 (&P)[ND], unsigned char *s
             for (int kk = 0; kk < bpg; ++kk)
                 sum += __hip_atomic_load(ws + ((p * pl.ncb + cb) * NW + gl * bpg + kk) * 128 + lag, __ATOMIC_RELAXED,
                                          __HIP_MEMORY_SCOPE_AGENT);
-        Elem<T>::store(dh + grp * dm.hl + k, sum);
+        typedef typename MT<T>::filt_t F;
+        Elem<F>::store((F *)dh + grp * dm.hl + k, sum);
     }
 }
 
@@ -521,10 +563,10 @@ int choose_nw_bwd(const Dims &dm, bool fp32)
 }
 
 // one workgroup per CU in either geometry (fp32: one wave per SIMD by its registers alone)
-MfmaPlan plan_bwd(const Dims &dm, bool fp32)
+MfmaPlan plan_bwd(const Dims &dm, bool split, int elem_bytes)
 {
-    const int nw = choose_nw_bwd(dm, fp32);
-    MfmaPlan p = plan(dm, nw, 16, nw, fp32 ? 4 : 2);
+    const int nw = choose_nw_bwd(dm, split);
+    MfmaPlan p = plan(dm, nw, 16, nw, elem_bytes);
     // the kernel adds the partials itself when a filter group lies within one channel block
     static const int fuse = env_int("GCG_MFMA_FUSE_DH", 1);    // tuning override: 0 = always a second launch
     p.fuse_dh = fuse && (16 * nw) % dm.dg == 0 && p.ncb <= DH_UNITS;

@@ -19,6 +19,9 @@ template <> struct Vec<f16_t, 8> { typedef u32x4 raw; static constexpr int W = 4
 template <> struct Vec<float, 1> { typedef u32x1 raw; static constexpr int W = 1; };
 template <> struct Vec<bf16_t, 2> { typedef u32x1 raw; static constexpr int W = 1; };
 template <> struct Vec<f16_t, 2> { typedef u32x1 raw; static constexpr int W = 1; };
+// 16-bit tensors with an fp32 filter: the row vectors of the plain 16-bit types
+template <int VV> struct Vec<bf16w_t, VV> : Vec<bf16_t, VV> {};
+template <int VV> struct Vec<f16w_t, VV> : Vec<f16_t, VV> {};
 // the three words of an interleaved row piece in one 12-byte access
 __device__ __forceinline__ void load_piece(win_t w, uint32_t off, u32x1 (&p)[3])
 {
@@ -71,6 +74,9 @@ template <> struct Word<f16_t> {
     }
     static __device__ __forceinline__ uint32_t pack(const float *f) { return pack_f16x2(f[0], f[1]); }
 };
+
+template <> struct Word<bf16w_t> : Word<bf16_t> {};
+template <> struct Word<f16w_t> : Word<f16_t> {};
 
 template <typename T, int VV>
 __device__ __forceinline__ void unpackv(const typename Vec<T, VV>::raw &r, float (&f)[VV])

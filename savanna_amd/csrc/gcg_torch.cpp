@@ -32,6 +32,17 @@ int dtype_code(at::ScalarType t)
     }
 }
 
+// dtype code of the gated operator: the tensors' dtype, or 16-bit tensors with an fp32 filter
+int gated_code(const Tensor &x, const Tensor &h)
+{
+    const at::ScalarType t = x.scalar_type(), f = h.scalar_type();
+    if (f == t) return dtype_code(t);
+    TORCH_CHECK(f == at::kFloat && (t == at::kBFloat16 || t == at::kHalf),
+                "gcg: the filter must have the tensors' dtype, or be float32 with bfloat16 / float16 tensors; got ", t,
+                " tensors and a ", f, " filter");
+    return t == at::kBFloat16 ? GCG_BF16_F32 : GCG_F16_F32;
+}
+
 void *stream_of(const Tensor &t)
 {
     return (void *)at::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
@@ -54,9 +65,9 @@ void check_gated(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor
     TORCH_CHECK(x.dim() == 4, "gcg: x must be (bs, L, g, dg)");
     TORCH_CHECK(B.sizes() == x.sizes() && C.sizes() == x.sizes(), "gcg: x, B and C must have one shape");
     TORCH_CHECK(h.dim() == 3 && h.size(0) == x.size(2) && h.size(1) == 1, "gcg: h must be (g, 1, hl)");
-    TORCH_CHECK(B.scalar_type() == x.scalar_type() && C.scalar_type() == x.scalar_type() &&
-                    h.scalar_type() == x.scalar_type(),
-                "gcg: x, B, C and h must share one dtype");
+    TORCH_CHECK(B.scalar_type() == x.scalar_type() && C.scalar_type() == x.scalar_type(),
+                "gcg: x, B and C must share one dtype");
+    (void)gated_code(x, h);
     TORCH_CHECK(B.device() == x.device() && C.device() == x.device() && h.device() == x.device(),
                 "gcg: x, B, C and h must be on one device");
     TORCH_CHECK(x.is_contiguous() && B.is_contiguous() && C.is_contiguous() && h.is_contiguous(),
@@ -76,8 +87,8 @@ void check_feat(const Tensor &feat, const Tensor &h)
                 "gcg: feat must be a contiguous (bs, L, g, dg, 3) tensor");
     TORCH_CHECK(h.dim() == 3 && h.size(0) == feat.size(2) && h.size(1) == 1 && h.is_contiguous(),
                 "gcg: h must be a contiguous (g, 1, hl) tensor");
-    TORCH_CHECK(h.scalar_type() == feat.scalar_type() && h.device() == feat.device(),
-                "gcg: feat and h must share dtype and device");
+    TORCH_CHECK(h.device() == feat.device(), "gcg: feat and h must be on one device");
+    (void)gated_code(feat, h);
 }
 
 Tensor workspace(size_t bytes, const Tensor &like, const char *what)
@@ -101,7 +112,7 @@ std::tuple<Tensor, Tensor, Tensor> fwd_full(const Tensor &x, const Tensor &B, co
     if (x.numel() == 0) return {bx, y2, y};
     check_rc(gcg_fwd(x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), y.data_ptr(),
                      return_y2 ? y2.data_ptr() : nullptr, return_bx ? bx.data_ptr() : nullptr, x.size(0), x.size(1),
-                     (int32_t)x.size(2), (int32_t)x.size(3), (int32_t)h.size(2), dtype_code(x.scalar_type()),
+                     (int32_t)x.size(2), (int32_t)x.size(3), (int32_t)h.size(2), gated_code(x, h),
                      (int32_t)algo, stream_of(x)),
              "gcg_fwd");
     return {bx, y2, y};
@@ -122,7 +133,7 @@ void fwd_out(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &h,
     DeviceGuard guard(x.device());
     check_rc(gcg_fwd(x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), y.data_ptr(), nullptr, nullptr, x.size(0),
                      x.size(1), (int32_t)x.size(2), (int32_t)x.size(3), (int32_t)h.size(2),
-                     dtype_code(x.scalar_type()), (int32_t)algo, stream_of(x)),
+                     gated_code(x, h), (int32_t)algo, stream_of(x)),
              "gcg_fwd");
 }
 
@@ -137,7 +148,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> bwd(const Tensor &dy, const Tensor &x
     if (x.numel() == 0) return {dx, dB, dC, dh.zero_()};
     const int64_t bs = x.size(0), L = x.size(1);
     const int32_t g = (int32_t)x.size(2), dg = (int32_t)x.size(3), hl = (int32_t)h.size(2);
-    const int code = dtype_code(x.scalar_type());
+    const int code = gated_code(x, h);
     const size_t nbytes = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, (int32_t)algo);
     Tensor ws = workspace(nbytes, x, "gcg_bwd_workspace_bytes");
     check_rc(gcg_bwd(dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), dx.data_ptr(),
@@ -158,7 +169,7 @@ Tensor fwd_interleaved(const Tensor &feat, const Tensor &h, int64_t algo)
     if (y.numel() == 0) return y;
     check_rc(gcg_fwd_interleaved(feat.data_ptr(), h.data_ptr(), y.data_ptr(), feat.size(0), feat.size(1),
                                  (int32_t)feat.size(2), (int32_t)feat.size(3), (int32_t)h.size(2),
-                                 dtype_code(feat.scalar_type()), (int32_t)algo, stream_of(feat)),
+                                 gated_code(feat, h), (int32_t)algo, stream_of(feat)),
              "gcg_fwd_interleaved");
     return y;
 }
@@ -176,7 +187,7 @@ std::tuple<Tensor, Tensor> bwd_interleaved(const Tensor &dy, const Tensor &feat,
     if (dy.numel() == 0) return {dfeat, dh.zero_()};
     const int64_t bs = feat.size(0), L = feat.size(1);
     const int32_t g = (int32_t)feat.size(2), dg = (int32_t)feat.size(3), hl = (int32_t)h.size(2);
-    const int code = dtype_code(feat.scalar_type());
+    const int code = gated_code(feat, h);
     const size_t nbytes = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, (int32_t)algo);
     Tensor ws = workspace(nbytes, feat, "gcg_bwd_workspace_bytes");
     check_rc(gcg_bwd_interleaved(dy.data_ptr(), feat.data_ptr(), h.data_ptr(), dfeat.data_ptr(), dh.data_ptr(),

@@ -93,11 +93,12 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
     const int64_t L = dm.L, d = dm.d;
     const int64_t c = (int64_t)cv * V;
     const int hl = dm.hl;
-    const T *hg = h + (c / dm.dg) * hl;
+    typedef typename Filt<T>::type FT;           // element type of the filter
+    const FT *hg = (const FT *)h + (c / dm.dg) * hl;
 
     float hr[HL];  // hr[j] multiplies the sample j rows in the past
 #pragma unroll
-    for (int j = 0; j < HL; ++j) hr[j] = (j < hl) ? Elem<T>::load(hg + hl - 1 - j) : 0.f;
+    for (int j = 0; j < HL; ++j) hr[j] = (j < hl) ? Elem<FT>::load(hg + hl - 1 - j) : 0.f;
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
@@ -217,11 +218,12 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
     const int64_t L = dm.L, d = dm.d;
     const int64_t c = (int64_t)cv * V;
     const int hl = dm.hl;
-    const T *hg = h + (c / dm.dg) * hl;
+    typedef typename Filt<T>::type FT;           // element type of the filter
+    const FT *hg = (const FT *)h + (c / dm.dg) * hl;
 
     float hr[HL];
 #pragma unroll
-    for (int j = 0; j < HL; ++j) hr[j] = (j < hl) ? Elem<T>::load(hg + hl - 1 - j) : 0.f;
+    for (int j = 0; j < HL; ++j) hr[j] = (j < hl) ? Elem<FT>::load(hg + hl - 1 - j) : 0.f;
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
@@ -451,7 +453,8 @@ int bwd_t(const void *dy, const void *x, const void *B, const void *C, const voi
                            (T *)dC, (float *)ws, dm, p);
     if (e) return e;
     // partials are ws[tap][(batch, run)][lane]; a filter owns dg / v adjacent lanes
-    return launch_colsum_reduce<T>((const float *)ws, (T *)dh, dm.bs * p.nseg, p.nvec, dm.dg / p.v, dm.g, dm.hl, st);
+    typedef typename Filt<T>::type FT;
+    return launch_colsum_reduce<FT>((const float *)ws, (FT *)dh, dm.bs * p.nseg, p.nvec, dm.dg / p.v, dm.g, dm.hl, st);
 }
 
 // Four channels per lane in both directions.  Eight (16-byte vectors for the 16-bit types) was
@@ -496,6 +499,8 @@ int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, co
     case GCG_F32:  return fwd_hl<float>(x, B, C, h, y, y2, bx, dm, st);
     case GCG_BF16: return fwd_hl<bf16_t>(x, B, C, h, y, y2, bx, dm, st);
     case GCG_F16:  return fwd_hl<f16_t>(x, B, C, h, y, y2, bx, dm, st);
+    case GCG_BF16_F32: return fwd_hl<bf16w_t>(x, B, C, h, y, y2, bx, dm, st);
+    case GCG_F16_F32:  return fwd_hl<f16w_t>(x, B, C, h, y, y2, bx, dm, st);
     }
     return (int)hipErrorInvalidValue;
 }
@@ -520,6 +525,8 @@ int window_bwd_launch(int dtype, const void *dy, const void *x, const void *B, c
     case GCG_F32:  return bwd_hl<float>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     case GCG_BF16: return bwd_hl<bf16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     case GCG_F16:  return bwd_hl<f16_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    case GCG_BF16_F32: return bwd_hl<bf16w_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    case GCG_F16_F32:  return bwd_hl<f16w_t>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     }
     return (int)hipErrorInvalidValue;
 }

@@ -40,5 +40,6 @@ def two_pass_bwd_refactor(
         assert dy.shape == (bs, seqlen, g, dg)
     assert h.dim() == 3 and h.shape[0] == x.shape[2] and h.shape[1] == 1
     assert all(t.is_contiguous() for t in (dy, x, B, C, h))
-    assert dy.dtype == x.dtype == B.dtype == C.dtype == h.dtype
+    assert dy.dtype == x.dtype == B.dtype == C.dtype
+    _lib.gated_code(x, h)       # h: the same dtype, or float32 with 16-bit tensors
     return _lib.bwd(dy, x, B, C, h, algo=algo)

@@ -31,7 +31,8 @@ def two_pass_fwd_grouped(
     assert x.shape == B.shape == C.shape, "x, B, C must share one shape"
     assert h.dim() == 3 and h.shape[0] == g and h.shape[1] == 1, "h must be (g, 1, hl)"
     assert x.is_contiguous() and B.is_contiguous() and C.is_contiguous() and h.is_contiguous()
-    assert x.dtype == B.dtype == C.dtype == h.dtype, "x, B, C, h must share one dtype"
+    assert x.dtype == B.dtype == C.dtype, "x, B, C must share one dtype"
+    _lib.gated_code(x, h)       # h: the same dtype, or float32 with 16-bit tensors (fp32 arithmetic, no casts)
     if schedule == "persistent":
         raise NotImplementedError("Skip persistent for now")
     if schedule != "default":

@@ -145,10 +145,15 @@ class _CgcgOperatorBase(nn.Module):
         """x1 (post-gate), x2, v (pre-gate pair): (b, l, g, dg) -> z: (b, l, g*dg)."""
         dtype = x1.dtype
         h = self._filter(x1.shape[1])
-        if self.cgcg_dtype != dtype:
+        x, B, C = v, x2, x1
+        cast = self.cgcg_dtype != dtype
+        if cast and self._fp32_inside(dtype, x1):
+            # hyena.py:499-503, :533-534 cast the three tensors up and the result down around the call; here the
+            # kernels read the 16-bit tensors, keep the filter and all arithmetic in fp32, and round the result once
+            h, cast = h.to(torch.float32), False
+        elif cast:
             x, B, C, h = (t.to(self.cgcg_dtype) for t in (v, x2, x1, h))
         else:
-            x, B, C = v, x2, x1
             h = h.to(dtype)             # parameters kept in another precision than the activations
         bs, seqlen, g, dg = x.shape
         z = self.cgcg_fn(
@@ -160,7 +165,11 @@ class _CgcgOperatorBase(nn.Module):
             bwd_kernel_cfg=None if self.cfg.cgcg_bwd_autotune else self.cgcg_bwd_config,
         )
         z = z.reshape(bs, seqlen, g * dg)
-        return z.to(dtype) if self.cgcg_dtype != dtype else z
+        return z.to(dtype) if cast else z
+
+    def _fp32_inside(self, dtype: torch.dtype, t: torch.Tensor) -> bool:
+        """16-bit activations with ``cgcg_dtype`` float32 on the GPU: one kernel instead of casts around it."""
+        return self.cgcg_dtype == torch.float32 and dtype in (torch.bfloat16, torch.float16) and t.is_cuda
 
     def forward_features(self, features: torch.Tensor, from_featurizer: bool = False) -> torch.Tensor:
         """The same on the projected features before their split: (b, l, 3*g*dg) laid out
@@ -172,12 +181,13 @@ class _CgcgOperatorBase(nn.Module):
         g, dg = self.num_groups, self.group_dim
         assert d3 == 3 * g * dg
         h = self._filter(seqlen)
-        if self.cgcg_dtype != dtype:
+        cast = self.cgcg_dtype != dtype and not self._fp32_inside(dtype, features)
+        if cast:
             features = features.to(self.cgcg_dtype)
         z = two_pass_chunked_gate_conv_gate_interleaved(features, h.to(self.cgcg_dtype), bs, seqlen, g, dg,
                                                         keep_dfeatures=from_featurizer)
         z = z.reshape(bs, seqlen, g * dg)
-        return z.to(dtype) if self.cgcg_dtype != dtype else z
+        return z.to(dtype) if cast else z
 
 
 class HyenaMROperator(_CgcgOperatorBase):

@@ -54,7 +54,13 @@ def test_meta_implementations_check_arguments(gcg_lib):
     with pytest.raises(RuntimeError, match=r"\(g, 1, hl\)"):
         torch.ops.gcg.fwd(x, x, x, h[:2])
     with pytest.raises(RuntimeError, match="one dtype"):
+        torch.ops.gcg.fwd(x, x.to(torch.bfloat16), x, h)
+    with pytest.raises(RuntimeError, match="filter must have the tensors' dtype"):
         torch.ops.gcg.fwd(x, x, x, h.to(torch.bfloat16))
+    # 16-bit tensors with a float32 filter: fp32 arithmetic inside, 16-bit result, float32 filter gradient
+    xb = x.to(torch.bfloat16)
+    assert torch.ops.gcg.fwd(xb, xb, xb, h).dtype == torch.bfloat16
+    assert [t.dtype for t in torch.ops.gcg.bwd(xb, xb, xb, xb, h)] == [torch.bfloat16] * 3 + [torch.float32]
     with pytest.raises(RuntimeError, match="contiguous"):
         torch.ops.gcg.fwd(x, x, x, torch.empty(4, 1, 14, device="meta")[:, :, ::2])
 
