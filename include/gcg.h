@@ -302,6 +302,40 @@ GCG_API int gcg_filter_decay_fwd(const float *w, const float *decay, void *h,
 GCG_API int gcg_filter_decay_bwd(const void *dh, const float *decay, float *dw,
             int32_t g, int32_t l_cache, int32_t hl, int32_t dtype, void *stream);
 
+/*
+ * The gated convolution of Hyena-MR with its explicit decayed filter built inside the kernels: the filter
+ * table a workgroup keeps on chip is filled with F(w[g, k] * decay[g, k]) (F = element type of the filter for
+ * `dtype`: the tensors' type, or fp32 for GCG_F32 / GCG_BF16_F32 / GCG_F16_F32) instead of being read from h,
+ * and the backward's filter-gradient reduction writes the gradient of the parameter itself,
+ *   dw[g, k] = float(F(dh[g, 0, k])) * decay[g, k]  for k < hl,  0 for hl <= k < l_cache,
+ * so neither h nor dh exists in memory and the layer needs no launch besides the convolution's.
+ * Replaces, around two_pass_fwd_grouped / two_pass_bwd_refactor, ExplicitSingleDecayFilter.filter
+ * (savanna/model/operators/hyena/parametrization/explicit.py:68-75), the [:, None] and cast of
+ * savanna/model/operators/hyena/hyena.py:440-441 and :499-503, and what autograd derives for them.
+ * The values are those of gcg_filter_decay_fwd -> gcg_fwd (gcg_bwd -> gcg_filter_decay_bwd), bit for bit.
+ *
+ * Matrix-core kernels only: hl <= 128, dg % 16 == 0, 16-byte aligned tensors, else GCG_ERR_UNSUPPORTED
+ * (make the filter with gcg_filter_decay_fwd then).  w, decay: (g, l_cache) fp32; dw: out, (g, l_cache)
+ * fp32, overwritten; workspace as for gcg_bwd (gcg_bwd_workspace_bytes with GCG_ALGO_MFMA).
+ */
+GCG_API int gcg_fwd_decay(const void *x, const void *B, const void *C,
+            const float *w, const float *decay, int32_t l_cache, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, void *stream);
+GCG_API int gcg_bwd_decay(const void *dy, const void *x, const void *B, const void *C,
+            const float *w, const float *decay, int32_t l_cache,
+            void *dx, void *dB, void *dC, float *dw,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, void *stream);
+/* The same on the interleaved features tensor (gcg_fwd_interleaved / gcg_bwd_interleaved). */
+GCG_API int gcg_fwd_interleaved_decay(const void *feat,
+            const float *w, const float *decay, int32_t l_cache, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, void *stream);
+GCG_API int gcg_bwd_interleaved_decay(const void *dy, const void *feat,
+            const float *w, const float *decay, int32_t l_cache,
+            void *dfeat, float *dw,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t flags, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,6 +35,7 @@ EXPORTS = (
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
+    "gcg_fwd_decay", "gcg_bwd_decay", "gcg_fwd_interleaved_decay", "gcg_bwd_interleaved_decay",
 )
 
 _lock = threading.Lock()
@@ -98,6 +99,14 @@ def load() -> ctypes.CDLL:
         lib.gcg_filter_decay_fwd.restype = ctypes.c_int
         lib.gcg_filter_decay_bwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
         lib.gcg_filter_decay_bwd.restype = ctypes.c_int
+        lib.gcg_fwd_decay.argtypes = [vp] * 5 + [i32, vp, i64, i64, i32, i32, i32, i32, vp]
+        lib.gcg_fwd_decay.restype = ctypes.c_int
+        lib.gcg_bwd_decay.argtypes = [vp] * 6 + [i32] + [vp] * 5 + [sz, i64, i64, i32, i32, i32, i32, vp]
+        lib.gcg_bwd_decay.restype = ctypes.c_int
+        lib.gcg_fwd_interleaved_decay.argtypes = [vp] * 3 + [i32, vp, i64, i64, i32, i32, i32, i32, vp]
+        lib.gcg_fwd_interleaved_decay.restype = ctypes.c_int
+        lib.gcg_bwd_interleaved_decay.argtypes = [vp] * 4 + [i32] + [vp] * 3 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_bwd_interleaved_decay.restype = ctypes.c_int
         _lib = lib
         return lib
 
@@ -478,6 +487,109 @@ def filter_decay_bwd(dh, decay):
                                       dtype_code(dh.dtype), st)
     check(rc, "gcg_filter_decay_bwd")
     return dw
+
+
+
+# ---- the gated convolution with the decayed explicit filter built inside the kernels -------------
+
+def decay_supported(g: int, dg: int, hl: int, *tensors) -> bool:
+    """Whether the *_decay entry points take these sizes: matrix-core kernels only
+    (hl <= 128, dg a multiple of 16, 16-byte aligned tensors; a tensor that is not contiguous is
+    copied or read through its interleaved source before it reaches them)."""
+    return hl <= 128 and dg % 16 == 0 and all(t.data_ptr() % 16 == 0 for t in tensors if t.is_contiguous())
+
+
+def _decay_code(t: torch.Tensor, filt: torch.dtype) -> int:
+    if filt == t.dtype:
+        return dtype_code(t.dtype)
+    if filt == torch.float32 and t.dtype in (torch.bfloat16, torch.float16):
+        return GCG_BF16_F32 if t.dtype == torch.bfloat16 else GCG_F16_F32
+    raise TypeError(f"filter type {filt} with {t.dtype} tensors")
+
+
+def fwd_decay(x, B, C, w, decay, hl: int, filt: torch.dtype):
+    """gcg_fwd with h = filt(w[:, :hl] * decay[:, :hl]) formed inside the kernel; w, decay: (g, L_cache) fp32."""
+    _require_gpu(x)
+    if TORCH_OPS:
+        return torch.ops.gcg.fwd_decay(x, B, C, w, decay, hl, filt)
+    lib = load()
+    _check_filter_params(w, decay)
+    bs, L, g, dg = x.shape
+    y = torch.empty_like(x)
+    if x.numel() == 0:
+        return y
+    with _on_device(x.device):
+        rc = lib.gcg_fwd_decay(x.data_ptr(), B.data_ptr(), C.data_ptr(), w.data_ptr(), decay.data_ptr(), w.shape[1],
+                               y.data_ptr(), bs, L, g, dg, hl, _decay_code(x, filt),
+                               torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_fwd_decay")
+    return y
+
+
+def bwd_decay(dy, x, B, C, w, decay, hl: int, filt: torch.dtype):
+    """(dx, dB, dC, dw): gcg_bwd whose filter-gradient reduction writes the (g, L_cache) fp32 gradient of w."""
+    _require_gpu(x)
+    if TORCH_OPS:
+        return torch.ops.gcg.bwd_decay(dy, x, B, C, w, decay, hl, filt)
+    lib = load()
+    _check_filter_params(w, decay)
+    bs, L, g, dg = x.shape
+    dx, dB, dC, dw = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x), torch.empty_like(w)
+    if x.numel() == 0:
+        return dx, dB, dC, dw.zero_()
+    code = _decay_code(x, filt)
+    nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, ALGO_NAMES["mfma"])
+    if nbytes == 0:
+        raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")
+    with _on_device(x.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        rc = lib.gcg_bwd_decay(dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), w.data_ptr(), decay.data_ptr(),
+                               w.shape[1], dx.data_ptr(), dB.data_ptr(), dC.data_ptr(), dw.data_ptr(), ws.data_ptr(),
+                               nbytes, bs, L, g, dg, hl, code, torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_bwd_decay")
+    return dx, dB, dC, dw
+
+
+def fwd_interleaved_decay(feat, w, decay, hl: int, filt: torch.dtype):
+    _require_gpu(feat)
+    if TORCH_OPS:
+        return torch.ops.gcg.fwd_interleaved_decay(feat, w, decay, hl, filt)
+    lib = load()
+    _check_filter_params(w, decay)
+    bs, L, g, dg, _ = feat.shape
+    y = torch.empty(bs, L, g, dg, dtype=feat.dtype, device=feat.device)
+    if y.numel() == 0:
+        return y
+    with _on_device(feat.device):
+        rc = lib.gcg_fwd_interleaved_decay(feat.data_ptr(), w.data_ptr(), decay.data_ptr(), w.shape[1], y.data_ptr(),
+                                           bs, L, g, dg, hl, _decay_code(feat, filt),
+                                           torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_fwd_interleaved_decay")
+    return y
+
+
+def bwd_interleaved_decay(dy, feat, w, decay, hl: int, filt: torch.dtype, keep_output=False):
+    _require_gpu(feat)
+    if TORCH_OPS:
+        return torch.ops.gcg.bwd_interleaved_decay(dy, feat, w, decay, hl, filt, keep_output)
+    lib = load()
+    _check_filter_params(w, decay)
+    bs, L, g, dg, _ = feat.shape
+    dfeat, dw = torch.empty_like(feat), torch.empty_like(w)
+    if dy.numel() == 0:
+        return dfeat, dw.zero_()
+    code = _decay_code(feat, filt)
+    nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, ALGO_NAMES["mfma"])
+    if nbytes == 0:
+        raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")
+    with _on_device(feat.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=feat.device)
+        rc = lib.gcg_bwd_interleaved_decay(dy.data_ptr(), feat.data_ptr(), w.data_ptr(), decay.data_ptr(), w.shape[1],
+                                           dfeat.data_ptr(), dw.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl,
+                                           code, KEEP_OUTPUT if keep_output else 0,
+                                           torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_bwd_interleaved_decay")
+    return dfeat, dw
 
 
 def select_algo(bs, L, g, dg, hl, dtype: torch.dtype, backward=False) -> str:

@@ -40,6 +40,7 @@ int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t 
     const bool mixed = dtype == GCG_BF16_F32 || dtype == GCG_F16_F32;
     if (!plain && !(mixed && mixed_ok)) return GCG_ERR_BAD_ARG;
     dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg; dm->es = 1; dm->keep_out = 0;
+    dm->fw = dm->fdecay = nullptr; dm->lc = 0;
     return GCG_OK;
 }
 
@@ -309,6 +310,95 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
         return finish(gcg::mfma_il_bwd_launch(dtype, dy, feat, h, dfeat, dh, workspace, dm, st));
     }
     return GCG_ERR_BAD_ARG;
+}
+
+// ---- the gated convolution with the decayed explicit filter built inside the kernels ---------------
+// Matrix-core kernels only (hl <= 128, dg % 16 == 0, 16-byte aligned tensors); other shapes are refused and
+// the caller makes the filter with gcg_filter_decay_fwd.
+
+namespace {
+int decay_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, const float *w,
+               const float *decay, int32_t l_cache, gcg::Dims *dm)
+{
+    if (!w || !decay || l_cache < hl) return GCG_ERR_BAD_ARG;
+    const int rc = make_dims(bs, L, g, dg, hl, dtype, dm, true);
+    if (rc) return rc;
+    dm->fw = w; dm->fdecay = decay; dm->lc = l_cache;
+    return GCG_OK;
+}
+} // namespace
+
+GCG_API int gcg_fwd_decay(const void *x, const void *B, const void *C, const float *w, const float *decay,
+                          int32_t l_cache, void *y, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                          int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!x || !B || !C || !y) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = decay_dims(bs, L, g, dg, hl, dtype, w, decay, l_cache, &dm);
+    if (rc) return rc;
+    const int a = resolve_algo(GCG_ALGO_MFMA, dtype, dm, false, all_aligned16({x, B, C, y}));
+    if (a < 0) return a;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::mfma_fwd_launch(dtype, x, B, C, nullptr, y, nullptr, nullptr, dm, (hipStream_t)stream));
+}
+
+GCG_API int gcg_bwd_decay(const void *dy, const void *x, const void *B, const void *C, const float *w,
+                          const float *decay, int32_t l_cache, void *dx, void *dB, void *dC, float *dw,
+                          void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg,
+                          int32_t hl, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !x || !B || !C || !dx || !dB || !dC || !dw) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = decay_dims(bs, L, g, dg, hl, dtype, w, decay, l_cache, &dm);
+    if (rc) return rc;
+    const int a = resolve_algo(GCG_ALGO_MFMA, dtype, dm, true, all_aligned16({dy, x, B, C, dx, dB, dC}));
+    if (a < 0) return a;
+    const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::mfma_bwd_launch(dtype, dy, x, B, C, nullptr, dx, dB, dC, dw, workspace, dm, (hipStream_t)stream));
+}
+
+GCG_API int gcg_fwd_interleaved_decay(const void *feat, const float *w, const float *decay, int32_t l_cache, void *y,
+                                      int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype,
+                                      void *stream)
+{
+    TimerScope timer_scope;
+    if (!feat || !y) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = decay_dims(bs, L, g, dg, hl, dtype, w, decay, l_cache, &dm);
+    if (rc) return rc;
+    dm.es = 3;
+    const int a = resolve_algo(GCG_ALGO_MFMA, dtype, dm, false, all_aligned16({feat, y}));
+    if (a < 0) return a;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::mfma_il_fwd_launch(dtype, feat, nullptr, y, dm, (hipStream_t)stream));
+}
+
+GCG_API int gcg_bwd_interleaved_decay(const void *dy, const void *feat, const float *w, const float *decay,
+                                      int32_t l_cache, void *dfeat, float *dw, void *workspace, size_t workspace_bytes,
+                                      int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype,
+                                      int32_t flags, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !feat || !dfeat || !dw || (flags & ~GCG_KEEP_OUTPUT)) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = decay_dims(bs, L, g, dg, hl, dtype, w, decay, l_cache, &dm);
+    if (rc) return rc;
+    dm.es = 3;
+    dm.keep_out = flags & GCG_KEEP_OUTPUT;
+    const int a = resolve_algo(GCG_ALGO_MFMA, dtype, dm, true, all_aligned16({dy, feat, dfeat}));
+    if (a < 0) return a;
+    const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::mfma_il_bwd_launch(dtype, dy, feat, nullptr, dfeat, dw, workspace, dm, (hipStream_t)stream));
 }
 
 // ---- ungated short causal depthwise convolution (featurizer)

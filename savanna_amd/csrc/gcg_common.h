@@ -121,6 +121,15 @@ template <> __device__ __forceinline__ uint32_t win_load<uint32_t>(win_t w, uint
 {
     return __builtin_amdgcn_raw_buffer_load_b32(w, (int)off, 0, WIN_NT);
 }
+// a 16-bit element (zero-extended)
+__device__ __forceinline__ uint32_t win_load_u16(win_t w, uint32_t off)
+{
+    return (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(w, (int)off, 0, 0);
+}
+__device__ __forceinline__ float win_load_f32_cached(win_t w, uint32_t off)
+{
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(w, (int)off, 0, 0));
+}
 template <> __device__ __forceinline__ u32x1 win_load<u32x1>(win_t w, uint32_t off)
 {
     u32x1 r;
@@ -201,6 +210,11 @@ struct Dims {
     // (and dC, dB, dx likewise).  y, y2, bx and dy are always plain.
     int32_t es;
     int32_t keep_out;   // GCG_KEEP_OUTPUT: store the main output through the cache (kernels that have the variant)
+    // Decayed explicit filter built inside the matrix-core kernels (the *_decay entry points): when fw is set
+    // the filter is h[g, k] = F(fw[g * lc + k] * fdecay[g * lc + k]) for k < hl (F = element type of the filter),
+    // the kernels' h argument is unused, and their dh argument is the (g, lc) fp32 gradient of fw.
+    const float *fw, *fdecay;
+    int32_t lc;
 };
 
 constexpr int kWave = 64;

@@ -88,18 +88,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     // order of issue, so taps requested after the rows would arrive after all of them).
     // htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0.
     hraw_t hv[HTAB / 64];
-    {
-        const int64_t cw = c0 + 16 * w;
-        const int64_t grp = (cw < d) ? cw / dm.dg : 0;
-        const hraw_t *hg = (const hraw_t *)h + grp * hl;
-#pragma unroll
-        for (int k = 0; k < HTAB / 64; ++k) {
-            const int lag = l + 64 * k - HPAD;
-            const bool in = lag >= 0 && lag < hl;
-            const hraw_t v = hg[in ? hl - 1 - lag : 0];          // no branch around the load
-            hv[k] = in ? v : (hraw_t)0;
-        }
-    }
+    load_taps<T>(dm, h, (c0 + 16 * w < d) ? (c0 + 16 * w) / dm.dg : 0, l, hv);
 
     // The operands of the NK-1 steps before the segment are rebuilt first (zero before the
     // start of the sequence).  Their rows are requested together, so the replay costs one
@@ -124,8 +113,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     };
     fetch(s_lo, xr, Br, Cr);
 
-#pragma unroll
-    for (int k = 0; k < HTAB / 64; ++k) htab[w][l + 64 * k] = hv[k];
+    store_taps(htab[w], l, hv);
     __syncthreads();
     typename M::wop_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
 #pragma unroll
@@ -303,17 +291,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     // The filter taps of this wave's group are requested before any row, so that the filter table
     // and the Toeplitz tiles are built while the rows are in flight (loads complete in order of issue).
     hraw_t hv[HTAB / 64];
-    {
-        const int64_t grp = wave_valid ? (c0 + 16 * w) / dm.dg : 0;
-        const hraw_t *hg = (const hraw_t *)h + grp * hl;
-#pragma unroll
-        for (int k = 0; k < HTAB / 64; ++k) {
-            const int lag = l + 64 * k - HPAD;
-            const bool in = lag >= 0 && lag < hl;
-            const hraw_t v = hg[in ? hl - 1 - lag : 0];          // no branch around the load
-            hv[k] = in ? v : (hraw_t)0;
-        }
-    }
+    load_taps<T>(dm, h, wave_valid ? (c0 + 16 * w) / dm.dg : 0, l, hv);
 
     // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the windows)
     auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
@@ -337,8 +315,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     Row<T> xr, Br, dyr, Cr;
     fetch(s_lo, xr, Br, dyr, Cr);
 
-#pragma unroll
-    for (int k = 0; k < HTAB / 64; ++k) htab[w * HTAB + l + 64 * k] = hv[k];
+    store_taps(htab + w * HTAB, l, hv);
     __syncthreads();
     typename M::wop_t W0[NK], W1[NK];
 #pragma unroll
@@ -542,7 +519,7 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
                        (T *)dh, (float *)ws, dm, p);
     if (e || p.fuse_dh) return e;
-    const int64_t n = (int64_t)dm.g * dm.hl;
+    const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
                        (const float *)ws, (T *)dh, dm, p);
     return e;

@@ -153,29 +153,25 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 #pragma unroll
         for (int k = 0; k < NR; ++k) store_operand_unit<T>(u_wr + RP * k * UROW, UROW, &uf[CH * k]);
     };
-    u32x3 in[NR];
-    fetch(s_lo, in);
+    // The filter taps of this wave's group are requested before any row, so that the filter table and the
+    // Toeplitz tiles are built while the rows are in flight (loads complete in order of issue).
+    hraw_t hv[HTAB / 64];
+    load_taps<T>(dm, h, (c0 + 16 * w < d) ? (c0 + 16 * w) / dm.dg : 0, l, hv);
 
     // A segment that starts inside the sequence first rebuilds the operands of the NK-1 steps
     // before it; their rows are requested together (one memory latency instead of NK-1) and
-    // step s_lo-i lands in ring slot NK-i, where phase 0 expects it.
+    // step s_lo-i lands in ring slot NK-i, where phase 0 expects it.  The rows of the first step
+    // follow them: they are needed last.
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
     u32x3 lead[NLEAD][NR];
     if constexpr (NK > 1) {
 #pragma unroll
         for (int i = 1; i < NK; ++i) fetch(s_lo - i, lead[i - 1]);
     }
+    u32x3 in[NR];
+    fetch(s_lo, in);
 
-    // filter table of this wave's group, htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0
-    {
-        const int64_t cw = c0 + 16 * w;
-        const int64_t grp = (cw < d) ? cw / dm.dg : 0;
-        const hraw_t *hg = (const hraw_t *)h + grp * hl;
-        for (int i = l; i < HTAB; i += 64) {
-            const int lag = i - HPAD;
-            htab[w][i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
-        }
-    }
+    store_taps(htab[w], l, hv);
     __syncthreads();
     typename M::wop_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
 #pragma unroll
@@ -357,12 +353,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     // iteration sigma brings the interleaved rows and dy of step sigma+NK-1
     u32x3 in[NR];
     Row<T> dyr;
-    fetch_feat(s_lo + NK - 1, in);
-    fetch_dy(s_lo + NK - 1, dyr);
+    // The filter taps of this wave's group are requested before any row (loads complete in order of issue).
+    hraw_t hv[HTAB / 64];
+    load_taps<T>(dm, h, wave_valid ? (c0 + 16 * w) / dm.dg : 0, l, hv);
 
     // Lead-in: the rows of the NK-1 steps before the segment (for u) and of its first NK-1 steps
     // (for g2, and x, B to wait in the ring), i.e. what iterations s_lo-NK+1 .. s_lo-1 would have
-    // brought.  Requested together, so the lead-in costs one memory latency instead of NK-1.
+    // brought.  Requested together, so the lead-in costs one memory latency instead of NK-1; the rows
+    // of the first iteration follow them (needed last).
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
     u32x3 past[NLEAD][NR], lead[NLEAD][NR];
     Row<T> wdy[NLEAD];
@@ -374,16 +372,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
             fetch_dy(s_lo + NK - 1 - i, wdy[i - 1]);
         }
     }
+    fetch_feat(s_lo + NK - 1, in);
+    fetch_dy(s_lo + NK - 1, dyr);
 
-    // While those rows are in flight: the filter table of this wave's group and the Toeplitz tiles.
-    {
-        const int64_t grp = wave_valid ? (c0 + 16 * w) / dm.dg : 0;
-        const hraw_t *hg = (const hraw_t *)h + grp * hl;
-        for (int i = l; i < HTAB; i += 64) {
-            const int lag = i - HPAD;
-            htab[w * HTAB + i] = (lag >= 0 && lag < hl) ? hg[hl - 1 - lag] : (hraw_t)0;
-        }
-    }
+    store_taps(htab + w * HTAB, l, hv);
     __syncthreads();
     typename M::wop_t W0[NK], W1[NK];
 #pragma unroll
@@ -573,7 +565,7 @@ int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, voi
         e = launch_main((mfma_il_bwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (T *)dh, (float *)ws, dm, p);
     if (e || p.fuse_dh) return e;
-    const int64_t n = (int64_t)dm.g * dm.hl;
+    const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
                        (const float *)ws, (T *)dh, dm, p);
     return e;

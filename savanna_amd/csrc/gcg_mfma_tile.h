@@ -99,6 +99,8 @@ template <typename OP> struct MT16 {
 
 template <> struct MT<bf16_t> : MT16<bf16x8> {
     typedef bf16_t filt_t;                       // element type of h and dh
+    static __device__ __forceinline__ hraw_t to_hraw(float v) { return (hraw_t)float_to_bf16_bits(v); }
+    static __device__ __forceinline__ float from_hraw(hraw_t v) { return bf16_bits_to_float(v); }
     static __device__ __forceinline__ f32x4 mfma(op_t a, op_t b, f32x4 c)
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
@@ -113,6 +115,19 @@ template <> struct MT<bf16_t> : MT16<bf16x8> {
 };
 template <> struct MT<f16_t> : MT16<f16x8> {
     typedef f16_t filt_t;
+    static __device__ __forceinline__ hraw_t to_hraw(float v)
+    {
+        const _Float16 hv = (_Float16)v;
+        hraw_t r;
+        __builtin_memcpy(&r, &hv, 2);
+        return r;
+    }
+    static __device__ __forceinline__ float from_hraw(hraw_t v)
+    {
+        _Float16 hv;
+        __builtin_memcpy(&hv, &v, 2);
+        return (float)hv;
+    }
     static __device__ __forceinline__ f32x4 mfma(op_t a, op_t b, f32x4 c)
     {
         return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
@@ -152,6 +167,8 @@ template <int NPA_> struct MTSplit {
     typedef SplitOp<NPW> wop_t;
     typedef float hraw_t;
     typedef float filt_t;
+    static __device__ __forceinline__ hraw_t to_hraw(float v) { return v; }
+    static __device__ __forceinline__ float from_hraw(hraw_t v) { return v; }
     static __device__ __forceinline__ int kmap(int q, int e) { return 8 * q + e; }
     template <int N> static __device__ __forceinline__ void split(float v, uint16_t (&o)[N])
     {
@@ -359,6 +376,52 @@ template <typename T> __device__ __forceinline__ void stw_row(win_t w, uint32_t 
     for (int i = 0; i < MT<T>::RW; ++i) stw16(w, off + 16 * i, r.w[i]);
 }
 
+// The filter table of a wave's group: tab[lag + HPAD] = h[hl-1-lag] for 0 <= lag < hl, else 0; lane l
+// holds entries l, l + 64, l + 128 between load_taps and store_taps.  The taps come from h, or -- decayed
+// explicit filter -- are formed here as F(fw * fdecay).  Both sources are read through windows, the one not
+// in use empty (its loads return zero and touch no memory), so there is no branch around a load: the taps
+// are requested before the first tensor rows, and a branch would make their use wait for those rows too.
+template <typename T>
+__device__ __forceinline__ void load_taps(const Dims &dm, const void *h, int64_t grp, int l,
+                                          typename MT<T>::hraw_t (&hv)[HTAB / 64])
+{
+    typedef MT<T> M;
+    typedef typename M::hraw_t hraw_t;
+    const bool dec = dm.fw != nullptr;
+    const int hl = dm.hl;
+    const win_t wh = make_window(h, dec ? 0 : (int64_t)dm.g * hl * (int64_t)sizeof(hraw_t));
+    const win_t ww = make_window(dm.fw, dec ? (int64_t)dm.g * dm.lc * 4 : 0);
+    const win_t wd = make_window(dm.fdecay, dec ? (int64_t)dm.g * dm.lc * 4 : 0);
+#pragma unroll
+    for (int k = 0; k < HTAB / 64; ++k) {
+        const int lag = l + 64 * k - HPAD;
+        const bool in = lag >= 0 && lag < hl;
+        const int tap = in ? hl - 1 - lag : 0;
+        const uint32_t oh = (uint32_t)((grp * hl + tap) * (int64_t)sizeof(hraw_t));
+        const uint32_t od = (uint32_t)((grp * dm.lc + tap) * 4);
+        hraw_t plain;
+        if constexpr (sizeof(hraw_t) == 2) plain = (hraw_t)win_load_u16(wh, oh);
+        else plain = win_load_f32_cached(wh, oh);
+        const hraw_t made = M::to_hraw(win_load_f32_cached(ww, od) * win_load_f32_cached(wd, od));
+        const hraw_t v = dec ? made : plain;
+        hv[k] = in ? v : (hraw_t)0;
+    }
+}
+template <typename H> __device__ __forceinline__ void store_taps(H *tab, int l, const H (&hv)[HTAB / 64])
+{
+#pragma unroll
+    for (int k = 0; k < HTAB / 64; ++k) tab[l + 64 * k] = hv[k];
+}
+// one value of the filter gradient: dh[grp, k] in the filter's element type, or -- decayed filter -- the
+// gradient of fw, dw[grp, k] = float(F(dh[grp, k])) * fdecay[grp, k]
+template <typename T> __device__ __forceinline__ void store_dh(void *dh, const Dims &dm, int64_t grp, int k, float sum)
+{
+    typedef MT<T> M;
+    typedef typename M::filt_t F;
+    if (dm.fw) ((float *)dh)[grp * dm.lc + k] = M::from_hraw(M::to_hraw(sum)) * dm.fdecay[grp * dm.lc + k];
+    else Elem<F>::store((F *)dh + grp * dm.hl + k, sum);
+}
+
 struct MfmaPlan { int ncb, nseg, steps_per_seg, nw, xcd; int64_t nsteps, nwg; int fuse_dh, slot; };
 
 // Operand tile of the banded Toeplitz matrix at row offset doff = (out time) - (in time) of the
@@ -371,17 +434,22 @@ __global__ __launch_bounds__(256) void mfma_dh_reduce_kernel(const float *__rest
                                                              Dims dm, MfmaPlan pl)
 {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= (int64_t)dm.g * dm.hl) return;
-    const int64_t grp = i / dm.hl;
-    const int lag = dm.hl - 1 - (int)(i % dm.hl);
+    const int row = dm.fw ? dm.lc : dm.hl;                // taps per group in the output
+    if (i >= (int64_t)dm.g * row) return;
+    const int64_t grp = i / row;
+    const int k = (int)(i % row);
+    if (k >= dm.hl) {                                    // the parameter's taps beyond the filter in use
+        ((float *)dh)[i] = 0.f;
+        return;
+    }
+    const int lag = dm.hl - 1 - k;
     const int bpg = dm.dg / 16;                          // 16-channel blocks per group
     const int64_t slots = (int64_t)pl.ncb * pl.nw;       // block slots per (batch, segment)
     float sum = 0.f;
     for (int64_t p = 0; p < dm.bs * pl.nseg; ++p)
-        for (int k = 0; k < bpg; ++k)
-            sum += ws[(p * slots + grp * bpg + k) * 128 + lag];
-    typedef typename MT<T>::filt_t F;
-    Elem<F>::store((F *)dh + i, sum);
+        for (int kk = 0; kk < bpg; ++kk)
+            sum += ws[(p * slots + grp * bpg + kk) * 128 + lag];
+    store_dh<T>(dh, dm, grp, k, sum);
 }
 
 // ---- filter-gradient reduction at the end of the backward kernel itself ----------------------
@@ -453,18 +521,22 @@ __device__ __forceinline__ void dh_finish(const f32x4 (&P)[ND], unsigned char *s
     constexpr int CB = 16 * NW;
     const int gpc = CB / dm.dg, bpg = dm.dg / 16;      // filter groups per channel block, 16-channel blocks per group
     const int64_t np = dm.bs * pl.nseg;
-    for (int idx = tid; idx < gpc * dm.hl; idx += 64 * NW) {
-        const int gl = idx / dm.hl, k = idx % dm.hl;
+    const int row = dm.fw ? dm.lc : dm.hl;              // taps per group in the output
+    for (int idx = tid; idx < gpc * row; idx += 64 * NW) {
+        const int gl = idx / row, k = idx % row;
         const int64_t grp = (int64_t)cb * gpc + gl;
         if (grp >= dm.g) continue;
+        if (k >= dm.hl) {                                // the parameter's taps beyond the filter in use
+            ((float *)dh)[grp * row + k] = 0.f;
+            continue;
+        }
         const int lag = dm.hl - 1 - k;
         float sum = 0.f;
         for (int64_t p = 0; p < np; ++p)
             for (int kk = 0; kk < bpg; ++kk)
                 sum += __hip_atomic_load(ws + ((p * pl.ncb + cb) * NW + gl * bpg + kk) * 128 + lag, __ATOMIC_RELAXED,
                                          __HIP_MEMORY_SCOPE_AGENT);
-        typedef typename MT<T>::filt_t F;
-        Elem<F>::store((F *)dh + grp * dm.hl + k, sum);
+        store_dh<T>(dh, dm, grp, k, sum);
     }
 }
 

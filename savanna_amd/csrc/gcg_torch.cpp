@@ -334,6 +334,122 @@ Tensor filter_decay_bwd(const Tensor &dh, const Tensor &decay)
     return dw;
 }
 
+// ---- gated convolution with the decayed explicit filter built inside the kernels ---------------
+
+// dtype code for tensors of type t with a filter of element type filt
+int gated_code_for(at::ScalarType t, at::ScalarType filt)
+{
+    if (filt == t) return dtype_code(t);
+    TORCH_CHECK(filt == at::kFloat && (t == at::kBFloat16 || t == at::kHalf),
+                "gcg: the filter must have the tensors' dtype, or be float32 with bfloat16 / float16 tensors; got ", t,
+                " tensors and a ", filt, " filter");
+    return t == at::kBFloat16 ? GCG_BF16_F32 : GCG_F16_F32;
+}
+
+void check_decay(const Tensor &w, const Tensor &decay, int64_t hl, int64_t g, const Tensor &on)
+{
+    check_filter_params(w, decay);
+    TORCH_CHECK(w.size(0) == g && hl > 0 && hl <= w.size(1) && w.device() == on.device(),
+                "gcg: w and decay must be (g, L_cache) on the tensors' device with 0 < hl <= L_cache");
+}
+
+void check_xbc(const Tensor &x, const Tensor &B, const Tensor &C)
+{
+    TORCH_CHECK(x.dim() == 4 && B.sizes() == x.sizes() && C.sizes() == x.sizes(), "gcg: x, B and C must be (bs, L, g, dg) of one shape");
+    TORCH_CHECK(B.scalar_type() == x.scalar_type() && C.scalar_type() == x.scalar_type() && B.device() == x.device() &&
+                    C.device() == x.device() && x.is_contiguous() && B.is_contiguous() && C.is_contiguous(),
+                "gcg: x, B and C must be contiguous and share one dtype and device");
+}
+
+Tensor fwd_decay(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &w, const Tensor &decay, int64_t hl,
+                 at::ScalarType filt)
+{
+    require_gpu(x, "x");
+    check_xbc(x, B, C);
+    check_decay(w, decay, hl, x.size(2), x);
+    const int code = gated_code_for(x.scalar_type(), filt);
+    DeviceGuard guard(x.device());
+    Tensor y = at::empty_like(x);
+    if (x.numel() == 0) return y;
+    check_rc(gcg_fwd_decay(x.data_ptr(), B.data_ptr(), C.data_ptr(), (const float *)w.data_ptr(),
+                           (const float *)decay.data_ptr(), (int32_t)w.size(1), y.data_ptr(), x.size(0), x.size(1),
+                           (int32_t)x.size(2), (int32_t)x.size(3), (int32_t)hl, code, stream_of(x)),
+             "gcg_fwd_decay");
+    return y;
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> bwd_decay(const Tensor &dy, const Tensor &x, const Tensor &B, const Tensor &C,
+                                                     const Tensor &w, const Tensor &decay, int64_t hl,
+                                                     at::ScalarType filt)
+{
+    require_gpu(x, "x");
+    check_xbc(x, B, C);
+    check_like(dy, x, "dy");
+    check_decay(w, decay, hl, x.size(2), x);
+    const int code = gated_code_for(x.scalar_type(), filt);
+    DeviceGuard guard(x.device());
+    Tensor dx = at::empty_like(x), dB = at::empty_like(x), dC = at::empty_like(x), dw = at::empty_like(w);
+    if (x.numel() == 0) return {dx, dB, dC, dw.zero_()};
+    const int64_t bs = x.size(0), L = x.size(1);
+    const int32_t g = (int32_t)x.size(2), dg = (int32_t)x.size(3);
+    const size_t nbytes = gcg_bwd_workspace_bytes(bs, L, g, dg, (int32_t)hl, code, GCG_ALGO_MFMA);
+    Tensor ws = workspace(nbytes, x, "gcg_bwd_workspace_bytes");
+    check_rc(gcg_bwd_decay(dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), (const float *)w.data_ptr(),
+                           (const float *)decay.data_ptr(), (int32_t)w.size(1), dx.data_ptr(), dB.data_ptr(),
+                           dC.data_ptr(), (float *)dw.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, (int32_t)hl,
+                           code, stream_of(x)),
+             "gcg_bwd_decay");
+    return {dx, dB, dC, dw};
+}
+
+void check_feat_only(const Tensor &feat)
+{
+    TORCH_CHECK(feat.dim() == 5 && feat.size(4) == 3 && feat.is_contiguous(),
+                "gcg: feat must be a contiguous (bs, L, g, dg, 3) tensor");
+}
+
+Tensor fwd_interleaved_decay(const Tensor &feat, const Tensor &w, const Tensor &decay, int64_t hl, at::ScalarType filt)
+{
+    require_gpu(feat, "feat");
+    check_feat_only(feat);
+    check_decay(w, decay, hl, feat.size(2), feat);
+    const int code = gated_code_for(feat.scalar_type(), filt);
+    DeviceGuard guard(feat.device());
+    Tensor y = at::empty({feat.size(0), feat.size(1), feat.size(2), feat.size(3)}, feat.options());
+    if (y.numel() == 0) return y;
+    check_rc(gcg_fwd_interleaved_decay(feat.data_ptr(), (const float *)w.data_ptr(), (const float *)decay.data_ptr(),
+                                       (int32_t)w.size(1), y.data_ptr(), feat.size(0), feat.size(1),
+                                       (int32_t)feat.size(2), (int32_t)feat.size(3), (int32_t)hl, code,
+                                       stream_of(feat)),
+             "gcg_fwd_interleaved_decay");
+    return y;
+}
+
+std::tuple<Tensor, Tensor> bwd_interleaved_decay(const Tensor &dy, const Tensor &feat, const Tensor &w,
+                                                 const Tensor &decay, int64_t hl, at::ScalarType filt, bool keep_output)
+{
+    require_gpu(feat, "feat");
+    check_feat_only(feat);
+    check_decay(w, decay, hl, feat.size(2), feat);
+    TORCH_CHECK(dy.dim() == 4 && dy.sizes() == feat.sizes().slice(0, 4) && dy.scalar_type() == feat.scalar_type() &&
+                    dy.device() == feat.device() && dy.is_contiguous(),
+                "gcg: dy must be a contiguous (bs, L, g, dg) tensor of feat's dtype and device");
+    const int code = gated_code_for(feat.scalar_type(), filt);
+    DeviceGuard guard(feat.device());
+    Tensor dfeat = at::empty_like(feat), dw = at::empty_like(w);
+    if (dy.numel() == 0) return {dfeat, dw.zero_()};
+    const int64_t bs = feat.size(0), L = feat.size(1);
+    const int32_t g = (int32_t)feat.size(2), dg = (int32_t)feat.size(3);
+    const size_t nbytes = gcg_bwd_workspace_bytes(bs, L, g, dg, (int32_t)hl, code, GCG_ALGO_MFMA);
+    Tensor ws = workspace(nbytes, feat, "gcg_bwd_workspace_bytes");
+    check_rc(gcg_bwd_interleaved_decay(dy.data_ptr(), feat.data_ptr(), (const float *)w.data_ptr(),
+                                       (const float *)decay.data_ptr(), (int32_t)w.size(1), dfeat.data_ptr(),
+                                       (float *)dw.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, (int32_t)hl, code,
+                                       keep_output ? GCG_KEEP_OUTPUT : 0, stream_of(feat)),
+             "gcg_bwd_interleaved_decay");
+    return {dfeat, dw};
+}
+
 // ---- meta implementations: shapes and dtypes only (fake tensors, torch.compile) ----------------
 
 std::tuple<Tensor, Tensor, Tensor> fwd_full_meta(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &h,
@@ -407,6 +523,42 @@ Tensor filter_decay_bwd_meta(const Tensor &dh, const Tensor &decay)
     return at::empty_like(decay);
 }
 
+Tensor fwd_decay_meta(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &w, const Tensor &decay,
+                      int64_t hl, at::ScalarType filt)
+{
+    check_xbc(x, B, C);
+    check_decay(w, decay, hl, x.size(2), x);
+    (void)gated_code_for(x.scalar_type(), filt);
+    return at::empty_like(x);
+}
+std::tuple<Tensor, Tensor, Tensor, Tensor> bwd_decay_meta(const Tensor &dy, const Tensor &x, const Tensor &B,
+                                                          const Tensor &C, const Tensor &w, const Tensor &decay,
+                                                          int64_t hl, at::ScalarType filt)
+{
+    check_xbc(x, B, C);
+    check_like(dy, x, "dy");
+    check_decay(w, decay, hl, x.size(2), x);
+    (void)gated_code_for(x.scalar_type(), filt);
+    return {at::empty_like(x), at::empty_like(x), at::empty_like(x), at::empty_like(w)};
+}
+Tensor fwd_interleaved_decay_meta(const Tensor &feat, const Tensor &w, const Tensor &decay, int64_t hl,
+                                  at::ScalarType filt)
+{
+    check_feat_only(feat);
+    check_decay(w, decay, hl, feat.size(2), feat);
+    (void)gated_code_for(feat.scalar_type(), filt);
+    return at::empty({feat.size(0), feat.size(1), feat.size(2), feat.size(3)}, feat.options());
+}
+std::tuple<Tensor, Tensor> bwd_interleaved_decay_meta(const Tensor &dy, const Tensor &feat, const Tensor &w,
+                                                      const Tensor &decay, int64_t hl, at::ScalarType filt, bool)
+{
+    check_feat_only(feat);
+    check_decay(w, decay, hl, feat.size(2), feat);
+    (void)dy;
+    (void)gated_code_for(feat.scalar_type(), filt);
+    return {at::empty_like(feat), at::empty_like(w)};
+}
+
 } // namespace
 
 TORCH_LIBRARY(gcg, m)
@@ -424,6 +576,12 @@ TORCH_LIBRARY(gcg, m)
     m.def("mixer_se_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h) -> (Tensor, Tensor, Tensor)");
     m.def("filter_decay_fwd(Tensor w, Tensor decay, int hl, ScalarType dtype) -> Tensor");
     m.def("filter_decay_bwd(Tensor dh, Tensor decay) -> Tensor");
+    m.def("fwd_decay(Tensor x, Tensor B, Tensor C, Tensor w, Tensor decay, int hl, ScalarType filt) -> Tensor");
+    m.def("bwd_decay(Tensor dy, Tensor x, Tensor B, Tensor C, Tensor w, Tensor decay, int hl, ScalarType filt)"
+          " -> (Tensor, Tensor, Tensor, Tensor)");
+    m.def("fwd_interleaved_decay(Tensor feat, Tensor w, Tensor decay, int hl, ScalarType filt) -> Tensor");
+    m.def("bwd_interleaved_decay(Tensor dy, Tensor feat, Tensor w, Tensor decay, int hl, ScalarType filt,"
+          " bool keep_output=False) -> (Tensor, Tensor)");
 }
 
 TORCH_LIBRARY_IMPL(gcg, CUDA, m)
@@ -440,6 +598,10 @@ TORCH_LIBRARY_IMPL(gcg, CUDA, m)
     m.impl("mixer_se_bwd", &mixer_se_bwd);
     m.impl("filter_decay_fwd", &filter_decay_fwd);
     m.impl("filter_decay_bwd", &filter_decay_bwd);
+    m.impl("fwd_decay", &fwd_decay);
+    m.impl("bwd_decay", &bwd_decay);
+    m.impl("fwd_interleaved_decay", &fwd_interleaved_decay);
+    m.impl("bwd_interleaved_decay", &bwd_interleaved_decay);
 }
 
 TORCH_LIBRARY_IMPL(gcg, Meta, m)
@@ -456,4 +618,8 @@ TORCH_LIBRARY_IMPL(gcg, Meta, m)
     m.impl("mixer_se_bwd", &mixer_se_bwd_meta);
     m.impl("filter_decay_fwd", &filter_decay_fwd_meta);
     m.impl("filter_decay_bwd", &filter_decay_bwd_meta);
+    m.impl("fwd_decay", &fwd_decay_meta);
+    m.impl("bwd_decay", &bwd_decay_meta);
+    m.impl("fwd_interleaved_decay", &fwd_interleaved_decay_meta);
+    m.impl("bwd_interleaved_decay", &bwd_interleaved_decay_meta);
 }

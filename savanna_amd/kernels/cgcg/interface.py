@@ -150,3 +150,54 @@ def two_pass_chunked_gate_conv_gate_interleaved(features: torch.Tensor, h: torch
     assert features.numel() == bs * seqlen * g * dg * 3, "features must hold 3*g*dg values per position"
     assert h.dim() == 3 and h.shape[0] == g and h.shape[1] == 1, "h must be (g, 1, hl)"
     return InterleavedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3), h, keep_dfeatures)
+
+
+class DecayedGateConvGate(torch.autograd.Function):
+    """y = C * conv(B * x, h) with the Hyena-MR filter h = filt(w[:, :hl] * decay[:, :hl]) formed inside the
+    convolution kernels, and the gradient of w written by the backward kernel's own filter-gradient
+    reduction: neither h nor dh exists in memory and the layer launches nothing besides the convolution.
+    Counterpart of ExplicitSingleDecayFilter.filter (savanna/model/operators/hyena/parametrization/
+    explicit.py:68-75), the slice and cast of savanna/model/operators/hyena/hyena.py:440-441, :499-503 and
+    TwoPassChunkedGateConvGate (cgcg/interface.py:27-127) taken together.  Matrix-core shapes only
+    (``_lib.decay_supported``).  Three views of one interleaved features tensor are read in place."""
+
+    @staticmethod
+    def forward(ctx, x, B, C, w, decay, hl, filt):
+        w, decay = _contig(w), _contig(decay)
+        feat = interleaved_source(x, B, C) if x.numel() > 0 and not torch.compiler.is_compiling() else None
+        ctx.interleaved = feat is not None
+        ctx.hl, ctx.filt = hl, filt
+        if feat is not None:
+            ctx.save_for_backward(feat, w, decay)
+            return _lib.fwd_interleaved_decay(feat, w, decay, hl, filt)
+        x, B, C = _contig(x), _contig(B), _contig(C)
+        ctx.save_for_backward(x, B, C, w, decay)
+        return _lib.fwd_decay(x, B, C, w, decay, hl, filt)
+
+    @staticmethod
+    def backward(ctx, dy):
+        if ctx.interleaved:
+            feat, w, decay = ctx.saved_tensors
+            dfeat, dw = _lib.bwd_interleaved_decay(_contig(dy), feat, w, decay, ctx.hl, ctx.filt)
+            return dfeat[..., 2], dfeat[..., 1], dfeat[..., 0], dw, None, None, None
+        x, B, C, w, decay = ctx.saved_tensors
+        dx, dB, dC, dw = _lib.bwd_decay(_contig(dy), x, B, C, w, decay, ctx.hl, ctx.filt)
+        return dx, dB, dC, dw, None, None, None
+
+
+class InterleavedDecayedGateConvGate(torch.autograd.Function):
+    """The same on the interleaved features tensor itself (gradient in the features' layout)."""
+
+    @staticmethod
+    def forward(ctx, feat, w, decay, hl, filt, keep_dfeatures=False):
+        feat, w, decay = _contig(feat), _contig(w), _contig(decay)
+        ctx.save_for_backward(feat, w, decay)
+        ctx.hl, ctx.filt, ctx.keep_dfeatures = hl, filt, keep_dfeatures
+        return _lib.fwd_interleaved_decay(feat, w, decay, hl, filt)
+
+    @staticmethod
+    def backward(ctx, dy):
+        feat, w, decay = ctx.saved_tensors
+        dfeat, dw = _lib.bwd_interleaved_decay(_contig(dy), feat, w, decay, ctx.hl, ctx.filt,
+                                               keep_output=ctx.keep_dfeatures)
+        return dfeat, dw, None, None, None, None

@@ -26,7 +26,8 @@ import torch
 import torch.nn as nn
 
 from .. import _lib
-from ..kernels.cgcg.interface import two_pass_chunked_gate_conv_gate, two_pass_chunked_gate_conv_gate_interleaved
+from ..kernels.cgcg.interface import (DecayedGateConvGate, InterleavedDecayedGateConvGate,
+                                       two_pass_chunked_gate_conv_gate, two_pass_chunked_gate_conv_gate_interleaved)
 from ..kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
 
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
@@ -144,6 +145,11 @@ class _CgcgOperatorBase(nn.Module):
     def forward(self, x1: torch.Tensor, x2: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
         """x1 (post-gate), x2, v (pre-gate pair): (b, l, g, dg) -> z: (b, l, g*dg)."""
         dtype = x1.dtype
+        fused = self._filter_in_kernel(x1.shape[1], x1.shape[2], x1.shape[3], dtype, x1, x2, v)
+        if fused is not None:
+            hl, filt = fused
+            z = DecayedGateConvGate.apply(v, x2, x1, self.filter.h, self.filter.decay, hl, filt)
+            return z.reshape(z.shape[0], z.shape[1], -1)
         h = self._filter(x1.shape[1])
         x, B, C = v, x2, x1
         cast = self.cgcg_dtype != dtype
@@ -167,6 +173,10 @@ class _CgcgOperatorBase(nn.Module):
         z = z.reshape(bs, seqlen, g * dg)
         return z.to(dtype) if cast else z
 
+    def _filter_in_kernel(self, L, g, dg, dtype, *tensors):
+        """(hl, filter dtype) when the convolution kernels can form the decayed filter themselves, else None."""
+        return None
+
     def _fp32_inside(self, dtype: torch.dtype, t: torch.Tensor) -> bool:
         """16-bit activations with ``cgcg_dtype`` float32 on the GPU: one kernel instead of casts around it."""
         return self.cgcg_dtype == torch.float32 and dtype in (torch.bfloat16, torch.float16) and t.is_cuda
@@ -180,6 +190,12 @@ class _CgcgOperatorBase(nn.Module):
         bs, seqlen, d3 = features.shape
         g, dg = self.num_groups, self.group_dim
         assert d3 == 3 * g * dg
+        fused = self._filter_in_kernel(seqlen, g, dg, dtype, features)
+        if fused is not None:
+            hl, filt = fused
+            z = InterleavedDecayedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3), self.filter.h,
+                                                     self.filter.decay, hl, filt, from_featurizer)
+            return z.reshape(bs, seqlen, g * dg)
         h = self._filter(seqlen)
         cast = self.cgcg_dtype != dtype and not self._fp32_inside(dtype, features)
         if cast:
@@ -194,11 +210,23 @@ class HyenaMROperator(_CgcgOperatorBase):
     """Hyena-MR: explicit decayed filter of length ``hyena_mr_len`` (128 in the 7B configs)."""
 
     def __init__(self, hidden_size: int, num_groups: int, hyena_mr_len: int = 128, cfg: Optional[CgcgConfig] = None,
-                 decay_preset: str = "strong", small_init: bool = True, device=None):
+                 decay_preset: str = "strong", small_init: bool = True, device=None, fuse_filter: bool = True):
         super().__init__(hidden_size, num_groups, cfg)
         self.hyena_mr_len = hyena_mr_len
+        self.fuse_filter = fuse_filter       # form the filter inside the convolution kernels where they can
         self.filter = ExplicitSingleDecayFilter(self.num_groups, hyena_mr_len, decay_preset=decay_preset,
                                                 small_init=small_init, device=device)
+
+    def _filter_in_kernel(self, L, g, dg, dtype, *tensors):
+        w = self.filter.h
+        if not (self.fuse_filter and w.is_cuda and w.dtype == torch.float32 and all(t.is_cuda for t in tensors)):
+            return None
+        if self.cgcg_dtype != dtype and not self._fp32_inside(dtype, tensors[0]):
+            return None                                             # a cast the kernels do not fold
+        hl = min(self.hyena_mr_len, L)
+        if not _lib.decay_supported(g, dg, hl, *tensors):
+            return None
+        return hl, self.cgcg_dtype
 
     def _filter(self, L: int) -> torch.Tensor:
         hl = min(self.hyena_mr_len, L)                              # hyena.py:440-441, :503
