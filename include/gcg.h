@@ -336,6 +336,25 @@ GCG_API int gcg_bwd_interleaved_decay(const void *dy, const void *feat,
             void *workspace, size_t workspace_bytes,
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t flags, void *stream);
 
+/*
+ * The short-filter operator on time-major operands: x, B, C (and dx, dB, dC) are (L, bs, g, dg) contiguous,
+ * y and dy are (bs, L, g, dg).  This is the input layout of the reference's other short-filter kernel family,
+ * run_short_hyena / ShortHyenaOperator (savanna/kernels/triton_src/short_hyena/interface.py:8-119: q, k, v of
+ * shape (seqlen, bs, g, dg), which its pre-convolution kernel permutes, short_hyena/fwd.py:245-247); with
+ * C = q, B = k, x = v the operator is the same gated convolution, read here where it lies instead of from
+ * three permuted copies, and the gradients are written in the operands' own layout.
+ * Register-window kernels only: hl <= 8, dg % 4 == 0, 16-byte aligned tensors, else GCG_ERR_UNSUPPORTED.
+ * dtype: any, GCG_BF16_F32 / GCG_F16_F32 included.  workspace: gcg_bwd_time_major_workspace_bytes, 256-byte aligned.
+ */
+GCG_API int gcg_fwd_time_major(const void *x, const void *B, const void *C, const void *h, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, void *stream);
+GCG_API size_t gcg_bwd_time_major_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype);
+GCG_API int gcg_bwd_time_major(const void *dy, const void *x, const void *B, const void *C, const void *h,
+            void *dx, void *dB, void *dC, void *dh,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -35,6 +35,7 @@ EXPORTS = (
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
+    "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
     "gcg_fwd_decay", "gcg_bwd_decay", "gcg_fwd_interleaved_decay", "gcg_bwd_interleaved_decay",
 )
 
@@ -99,6 +100,12 @@ def load() -> ctypes.CDLL:
         lib.gcg_filter_decay_fwd.restype = ctypes.c_int
         lib.gcg_filter_decay_bwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
         lib.gcg_filter_decay_bwd.restype = ctypes.c_int
+        lib.gcg_fwd_time_major.argtypes = [vp] * 5 + [i64, i64, i32, i32, i32, i32, vp]
+        lib.gcg_fwd_time_major.restype = ctypes.c_int
+        lib.gcg_bwd_time_major_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32]
+        lib.gcg_bwd_time_major_workspace_bytes.restype = sz
+        lib.gcg_bwd_time_major.argtypes = [vp] * 10 + [sz, i64, i64, i32, i32, i32, i32, vp]
+        lib.gcg_bwd_time_major.restype = ctypes.c_int
         lib.gcg_fwd_decay.argtypes = [vp] * 5 + [i32, vp, i64, i64, i32, i32, i32, i32, vp]
         lib.gcg_fwd_decay.restype = ctypes.c_int
         lib.gcg_bwd_decay.argtypes = [vp] * 6 + [i32] + [vp] * 5 + [sz, i64, i64, i32, i32, i32, i32, vp]
@@ -488,6 +495,54 @@ def filter_decay_bwd(dh, decay):
     check(rc, "gcg_filter_decay_bwd")
     return dw
 
+
+
+# ---- the short-filter operator on time-major operands (seqlen, bs, g, dg) ------------------------
+
+def time_major_supported(dg: int, hl: int, *tensors) -> bool:
+    """Whether gcg_fwd_time_major / gcg_bwd_time_major take these sizes (register-window kernels)."""
+    return hl <= 8 and dg % 4 == 0 and all(t.is_contiguous() and t.data_ptr() % 16 == 0 for t in tensors)
+
+
+def fwd_time_major(x, B, C, h):
+    """y (bs, seqlen, g, dg) for x, B, C of shape (seqlen, bs, g, dg), read where they lie."""
+    _require_gpu(x)
+    if TORCH_OPS:
+        return torch.ops.gcg.fwd_time_major(x, B, C, h)
+    lib = load()
+    L, bs, g, dg = x.shape
+    y = torch.empty(bs, L, g, dg, dtype=x.dtype, device=x.device)
+    if x.numel() == 0:
+        return y
+    with _on_device(x.device):
+        rc = lib.gcg_fwd_time_major(x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg,
+                                    h.shape[-1], gated_code(x, h), torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_fwd_time_major")
+    return y
+
+
+def bwd_time_major(dy, x, B, C, h):
+    """(dx, dB, dC, dh) with dx, dB, dC in the operands' (seqlen, bs, g, dg) layout; dy is (bs, seqlen, g, dg)."""
+    _require_gpu(x)
+    if TORCH_OPS:
+        return torch.ops.gcg.bwd_time_major(dy, x, B, C, h)
+    lib = load()
+    L, bs, g, dg = x.shape
+    hl = h.shape[-1]
+    dx, dB, dC, dh = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x), torch.empty_like(h)
+    if x.numel() == 0:
+        return dx, dB, dC, dh.zero_()
+    code = gated_code(x, h)
+    nbytes = lib.gcg_bwd_time_major_workspace_bytes(bs, L, g, dg, hl, code)
+    if nbytes == 0:
+        raise GcgError("gcg_bwd_time_major_workspace_bytes: arguments rejected")
+    with _on_device(x.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        rc = lib.gcg_bwd_time_major(dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), dx.data_ptr(),
+                                    dB.data_ptr(), dC.data_ptr(), dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg,
+                                    hl, code, torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_bwd_time_major")
+    return dx, dB, dC, dh
 
 
 # ---- the gated convolution with the decayed explicit filter built inside the kernels -------------

@@ -40,7 +40,7 @@ int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t 
     const bool mixed = dtype == GCG_BF16_F32 || dtype == GCG_F16_F32;
     if (!plain && !(mixed && mixed_ok)) return GCG_ERR_BAD_ARG;
     dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg; dm->es = 1; dm->keep_out = 0;
-    dm->fw = dm->fdecay = nullptr; dm->lc = 0;
+    dm->fw = dm->fdecay = nullptr; dm->lc = 0; dm->tmajor = 0;
     return GCG_OK;
 }
 
@@ -399,6 +399,54 @@ GCG_API int gcg_bwd_interleaved_decay(const void *dy, const void *feat, const fl
     rc = check_device();
     if (rc) return rc;
     return finish(gcg::mfma_il_bwd_launch(dtype, dy, feat, nullptr, dfeat, dw, workspace, dm, (hipStream_t)stream));
+}
+
+// ---- the short-filter operator on time-major operands (the layout of run_short_hyena) ------------
+// Register-window kernels only (hl <= 8, dg % 4 == 0, 16-byte aligned tensors).
+
+GCG_API int gcg_fwd_time_major(const void *x, const void *B, const void *C, const void *h, void *y, int64_t bs,
+                               int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!x || !B || !C || !h || !y) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    if (rc) return rc;
+    dm.tmajor = 1;
+    const int a = resolve_algo(GCG_ALGO_WINDOW, dtype, dm, false, all_aligned16({x, B, C, y}));
+    if (a < 0) return a;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::window_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, (hipStream_t)stream));
+}
+
+GCG_API size_t gcg_bwd_time_major_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                                                  int32_t dtype)
+{
+    gcg::Dims dm;
+    if (make_dims(bs, L, g, dg, hl, dtype, &dm, true)) return 0;
+    dm.tmajor = 1;
+    if (!gcg::window_supported(dm)) return 0;
+    return (gcg::window_bwd_workspace(dm) + 255) & ~(size_t)255;
+}
+
+GCG_API int gcg_bwd_time_major(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx,
+                               void *dB, void *dC, void *dh, void *workspace, size_t workspace_bytes, int64_t bs,
+                               int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !x || !B || !C || !h || !dx || !dB || !dC || !dh) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    if (rc) return rc;
+    dm.tmajor = 1;
+    const int a = resolve_algo(GCG_ALGO_WINDOW, dtype, dm, true, all_aligned16({dy, x, B, C, dx, dB, dC}));
+    if (a < 0) return a;
+    const size_t need = gcg_bwd_time_major_workspace_bytes(bs, L, g, dg, hl, dtype);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::window_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, (hipStream_t)stream));
 }
 
 // ---- ungated short causal depthwise convolution (featurizer)

@@ -215,6 +215,9 @@ struct Dims {
     // the kernels' h argument is unused, and their dh argument is the (g, lc) fp32 gradient of fw.
     const float *fw, *fdecay;
     int32_t lc;
+    // Time-major operands (register-window kernels, separate tensors): x, B, C and dx, dB, dC are laid out
+    // (L, bs, g, dg) -- the rows of one batch entry lie bs * d elements apart -- while y and dy stay (bs, L, g, dg).
+    int32_t tmajor;
 };
 
 constexpr int kWave = 64;

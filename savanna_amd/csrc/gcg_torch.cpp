@@ -450,6 +450,58 @@ std::tuple<Tensor, Tensor> bwd_interleaved_decay(const Tensor &dy, const Tensor 
     return {dfeat, dw};
 }
 
+// ---- short-filter operator on time-major operands (seqlen, bs, g, dg) --------------------------
+
+void check_time_major(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &h)
+{
+    TORCH_CHECK(x.dim() == 4 && B.sizes() == x.sizes() && C.sizes() == x.sizes(),
+                "gcg: x, B and C must be (seqlen, bs, g, dg) of one shape");
+    TORCH_CHECK(h.dim() == 3 && h.size(0) == x.size(2) && h.size(1) == 1 && h.is_contiguous(), "gcg: h must be a contiguous (g, 1, hl) tensor");
+    TORCH_CHECK(B.scalar_type() == x.scalar_type() && C.scalar_type() == x.scalar_type() && B.device() == x.device() &&
+                    C.device() == x.device() && h.device() == x.device() && x.is_contiguous() && B.is_contiguous() &&
+                    C.is_contiguous(),
+                "gcg: x, B and C must be contiguous and share one dtype and device");
+}
+
+Tensor fwd_time_major(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &h)
+{
+    require_gpu(x, "x");
+    check_time_major(x, B, C, h);
+    const int code = gated_code(x, h);
+    DeviceGuard guard(x.device());
+    Tensor y = at::empty({x.size(1), x.size(0), x.size(2), x.size(3)}, x.options());
+    if (x.numel() == 0) return y;
+    check_rc(gcg_fwd_time_major(x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), y.data_ptr(), x.size(1),
+                                x.size(0), (int32_t)x.size(2), (int32_t)x.size(3), (int32_t)h.size(2), code,
+                                stream_of(x)),
+             "gcg_fwd_time_major");
+    return y;
+}
+
+std::tuple<Tensor, Tensor, Tensor, Tensor> bwd_time_major(const Tensor &dy, const Tensor &x, const Tensor &B,
+                                                          const Tensor &C, const Tensor &h)
+{
+    require_gpu(x, "x");
+    check_time_major(x, B, C, h);
+    TORCH_CHECK(dy.dim() == 4 && dy.size(0) == x.size(1) && dy.size(1) == x.size(0) && dy.size(2) == x.size(2) &&
+                    dy.size(3) == x.size(3) && dy.scalar_type() == x.scalar_type() && dy.device() == x.device() &&
+                    dy.is_contiguous(),
+                "gcg: dy must be a contiguous (bs, seqlen, g, dg) tensor of x's dtype and device");
+    const int code = gated_code(x, h);
+    DeviceGuard guard(x.device());
+    Tensor dx = at::empty_like(x), dB = at::empty_like(x), dC = at::empty_like(x), dh = at::empty_like(h);
+    if (x.numel() == 0) return {dx, dB, dC, dh.zero_()};
+    const int64_t L = x.size(0), bs = x.size(1);
+    const int32_t g = (int32_t)x.size(2), dg = (int32_t)x.size(3), hl = (int32_t)h.size(2);
+    const size_t nbytes = gcg_bwd_time_major_workspace_bytes(bs, L, g, dg, hl, code);
+    Tensor ws = workspace(nbytes, x, "gcg_bwd_time_major_workspace_bytes");
+    check_rc(gcg_bwd_time_major(dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(), dx.data_ptr(),
+                                dB.data_ptr(), dC.data_ptr(), dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl,
+                                code, stream_of(x)),
+             "gcg_bwd_time_major");
+    return {dx, dB, dC, dh};
+}
+
 // ---- meta implementations: shapes and dtypes only (fake tensors, torch.compile) ----------------
 
 std::tuple<Tensor, Tensor, Tensor> fwd_full_meta(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &h,
@@ -559,6 +611,20 @@ std::tuple<Tensor, Tensor> bwd_interleaved_decay_meta(const Tensor &dy, const Te
     return {at::empty_like(feat), at::empty_like(w)};
 }
 
+Tensor fwd_time_major_meta(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &h)
+{
+    check_time_major(x, B, C, h);
+    (void)gated_code(x, h);
+    return at::empty({x.size(1), x.size(0), x.size(2), x.size(3)}, x.options());
+}
+std::tuple<Tensor, Tensor, Tensor, Tensor> bwd_time_major_meta(const Tensor &dy, const Tensor &x, const Tensor &B,
+                                                               const Tensor &C, const Tensor &h)
+{
+    check_time_major(x, B, C, h);
+    (void)dy;
+    return {at::empty_like(x), at::empty_like(x), at::empty_like(x), at::empty_like(h)};
+}
+
 } // namespace
 
 TORCH_LIBRARY(gcg, m)
@@ -576,6 +642,8 @@ TORCH_LIBRARY(gcg, m)
     m.def("mixer_se_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h) -> (Tensor, Tensor, Tensor)");
     m.def("filter_decay_fwd(Tensor w, Tensor decay, int hl, ScalarType dtype) -> Tensor");
     m.def("filter_decay_bwd(Tensor dh, Tensor decay) -> Tensor");
+    m.def("fwd_time_major(Tensor x, Tensor B, Tensor C, Tensor h) -> Tensor");
+    m.def("bwd_time_major(Tensor dy, Tensor x, Tensor B, Tensor C, Tensor h) -> (Tensor, Tensor, Tensor, Tensor)");
     m.def("fwd_decay(Tensor x, Tensor B, Tensor C, Tensor w, Tensor decay, int hl, ScalarType filt) -> Tensor");
     m.def("bwd_decay(Tensor dy, Tensor x, Tensor B, Tensor C, Tensor w, Tensor decay, int hl, ScalarType filt)"
           " -> (Tensor, Tensor, Tensor, Tensor)");
@@ -598,6 +666,8 @@ TORCH_LIBRARY_IMPL(gcg, CUDA, m)
     m.impl("mixer_se_bwd", &mixer_se_bwd);
     m.impl("filter_decay_fwd", &filter_decay_fwd);
     m.impl("filter_decay_bwd", &filter_decay_bwd);
+    m.impl("fwd_time_major", &fwd_time_major);
+    m.impl("bwd_time_major", &bwd_time_major);
     m.impl("fwd_decay", &fwd_decay);
     m.impl("bwd_decay", &bwd_decay);
     m.impl("fwd_interleaved_decay", &fwd_interleaved_decay);
@@ -618,6 +688,8 @@ TORCH_LIBRARY_IMPL(gcg, Meta, m)
     m.impl("mixer_se_bwd", &mixer_se_bwd_meta);
     m.impl("filter_decay_fwd", &filter_decay_fwd_meta);
     m.impl("filter_decay_bwd", &filter_decay_bwd_meta);
+    m.impl("fwd_time_major", &fwd_time_major_meta);
+    m.impl("bwd_time_major", &bwd_time_major_meta);
     m.impl("fwd_decay", &fwd_decay_meta);
     m.impl("bwd_decay", &bwd_decay_meta);
     m.impl("fwd_interleaved_decay", &fwd_interleaved_decay_meta);

@@ -104,9 +104,12 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
     const int64_t t0 = t_start - (HL - 1) > 0 ? t_start - (HL - 1) : 0;       // first row of the windows
     const int64_t origin = (b * L + t0) * d, rows = t_end - t0;
-    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow;               // bytes per row: outputs, inputs
-    const win_t wx = make_window((PK ? C : x) + IS * origin, rows * irow);
-    const win_t wB = make_window(B + origin, PK ? 0 : rows * irow), wC = make_window(C + origin, PK ? 0 : rows * irow);
+    // time-major inputs: the rows of this batch entry lie bs rows apart (a window then spans the other
+    // entries' rows in between, which no offset of this lane reaches)
+    const int64_t in_origin = dm.tmajor ? (t0 * dm.bs + b) * d : origin;
+    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow * (uint32_t)(dm.tmajor ? dm.bs : 1);   // bytes per row: outputs, inputs
+    const win_t wx = make_window((PK ? C : x) + IS * in_origin, rows * irow);
+    const win_t wB = make_window(B + in_origin, PK ? 0 : rows * irow), wC = make_window(C + in_origin, PK ? 0 : rows * irow);
     const win_t wy = make_window(y + origin, rows * orow);
     const win_t wy2 = make_window(EXTRA && y2 ? y2 + origin : y + origin, EXTRA && y2 ? rows * orow : 0);
     const win_t wbx = make_window(EXTRA && bx ? bx + origin : y + origin, EXTRA && bx ? rows * orow : 0);
@@ -230,12 +233,15 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
     const int64_t t_stop = t_end + (HL - 1);                     // exclusive bound of the walk
     const int64_t t0 = t_start - (HL - 1) > 0 ? t_start - (HL - 1) : 0;
     const int64_t t_far = t_stop < L ? t_stop : L;
-    const int64_t origin = (b * L + t0) * d, out_origin = (b * L + t_start) * d;
-    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow;
+    const int64_t origin = (b * L + t0) * d;
+    // time-major x, B, C, dx, dB, dC: the rows of this batch entry lie bs rows apart
+    const int64_t in_origin = dm.tmajor ? (t0 * dm.bs + b) * d : origin;
+    const int64_t out_origin = dm.tmajor ? (t_start * dm.bs + b) * d : (b * L + t_start) * d;
+    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow * (uint32_t)(dm.tmajor ? dm.bs : 1);
     // PK: wx is the interleaved tensor and reaches as far as dy (C is part of it)
-    const win_t wx = make_window((PK ? C : x) + IS * origin, ((PK ? t_far : t_end) - t0) * irow);
-    const win_t wB = make_window(B + origin, PK ? 0 : (t_end - t0) * irow);
-    const win_t wC = make_window(C + origin, PK ? 0 : (t_far - t0) * irow);
+    const win_t wx = make_window((PK ? C : x) + IS * in_origin, ((PK ? t_far : t_end) - t0) * irow);
+    const win_t wB = make_window(B + in_origin, PK ? 0 : (t_end - t0) * irow);
+    const win_t wC = make_window(C + in_origin, PK ? 0 : (t_far - t0) * irow);
     const win_t wdy = make_window(dy + origin, (t_far - t0) * orow);
     const win_t wdC = make_window(dC + IS * out_origin, (t_end - t_start) * irow);
     const win_t wdx = make_window(dx + out_origin, PK ? 0 : (t_end - t_start) * irow);
@@ -334,7 +340,7 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
 #pragma unroll
                     for (int v = 0; v < V; ++v) o[v] = dyf[v] * y2v[v];
                     if constexpr (PK) dCs[k] = packv<T, V>(o);
-                    else win_store(wdC, lane_o + (uint32_t)(t - t_start) * orow, packv<T, V>(o));
+                    else win_store(wdC, lane_o + (uint32_t)(t - t_start) * irow, packv<T, V>(o));
                 }
                 // du for row t-(HL-1): sum_j hr[j] * g2[row + j]; rows before the run fall outside
                 // the output windows
@@ -361,7 +367,7 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
                         if constexpr (KEEP) store_piece_as<true>(wdC, q, p);
                         else store_piece(wdC, q, p);
                     } else {
-                        const uint32_t q = lane_o + (uint32_t)(out_t - t_start) * orow;
+                        const uint32_t q = lane_o + (uint32_t)(out_t - t_start) * irow;
 #pragma unroll
                         for (int v = 0; v < V; ++v) o[v] = du[v] * Bo[v];
                         win_store(wdx, q, packv<T, V>(o));
@@ -393,7 +399,7 @@ WinPlan plan(const Dims &dm, int v)
     static const char *env = getenv("GCG_WINDOW_ROWS");   // tuning override: rows per lane, a multiple of 8
     if (env && atoi(env) >= 8 && atoi(env) % 8 == 0) p.ts = atoi(env);
     // the rows of a run, its halo and an interleaved fp32 row width must fit one tensor window
-    while (p.ts > 8 && (int64_t)(p.ts + 2 * RING) * 3 * dm.d * 4 > WIN_MAX_BYTES) p.ts >>= 1;
+    while (p.ts > 8 && (int64_t)(p.ts + 2 * RING) * 3 * dm.d * 4 * (dm.tmajor ? dm.bs : 1) > WIN_MAX_BYTES) p.ts >>= 1;
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);
     p.nthreads = dm.bs * p.nseg * p.nvec;       // workspace slots (one per lane with work)
     p.threads = p.nvec >= 256 ? 256 : ((p.nvec + 63) / 64) * 64;   // narrow tensors: fewer idle lanes
@@ -489,7 +495,7 @@ int bwd_hl(const void *dy, const void *x, const void *B, const void *C, const vo
 bool window_supported(const Dims &dm)
 {
     return dm.hl <= RING && dm.dg % 4 == 0 && (int64_t)dm.g * dm.hl <= 0x7fffffffLL &&
-           (int64_t)(3 * RING) * 3 * dm.d * 4 <= WIN_MAX_BYTES;
+           (int64_t)(3 * RING) * 3 * dm.d * 4 * (dm.tmajor ? dm.bs : 1) <= WIN_MAX_BYTES && !(dm.tmajor && dm.es == 3);
 }
 
 int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h, void *y,

@@ -4,17 +4,37 @@
 That family computes the same operator, ``out = q * conv(k * v, w)`` with a causal
 cross-correlation (short_hyena/utils.py:14-28, ref_hyena_mlp :36-66), on another layout: inputs
 ``(seqlen, bs, g, dg)``, output ``(bs, g, seqlen, dg)`` (short_hyena/fwd.py:245-247).  Here it maps
-onto the gated convolution kernels (C = q, B = k, x = v); the two layout changes are views on the
-way in (made contiguous by the autograd boundary) and a permuted view of the result on the way out.
+onto the gated convolution kernels (C = q, B = k, x = v).  With one filter per group of at most 8 taps
+the register-window kernels read q, k, v where they lie -- rows of one batch entry ``bs * g * dg``
+elements apart -- and write dq, dk, dv in that layout, so nothing is permuted on the way in
+(gcg_fwd_time_major / gcg_bwd_time_major); the result is computed as (bs, seqlen, g, dg) and returned as the
+permuted view the reference's shape asks for.  Other shapes take two layout changes around the general kernels.
 """
 from __future__ import annotations
 
 import torch
 
+from ... import _lib
 from ..cgcg.interface import two_pass_chunked_gate_conv_gate
 from ..cgcg.src.kernel_utils import FwdKernelConfigRefactor
 
 _FWD_CFG = FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row")
+
+
+class _TimeMajorShortHyena(torch.autograd.Function):
+    """q * conv(k * v, w) on (seqlen, bs, g, dg) operands in place -> (bs, seqlen, g, dg); saves the inputs only
+    (ShortHyenaOperator also saves three permuted intermediates, interface.py:47)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, w):
+        ctx.save_for_backward(q, k, v, w)
+        return _lib.fwd_time_major(v, k, q, w)
+
+    @staticmethod
+    def backward(ctx, dy):
+        q, k, v, w = ctx.saved_tensors
+        dv, dk, dq, dw = _lib.bwd_time_major(dy if dy.is_contiguous() else dy.contiguous(), v, k, q, w)
+        return dq, dk, dv, dw
 
 
 def run_short_hyena(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.Tensor,
@@ -40,6 +60,10 @@ def run_short_hyena(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.
     else:
         assert w.shape[0] == g * dg
         groups, width = g * dg, 1
+    if repeat_interleave and q.is_cuda and _lib.time_major_supported(dg, hl, q, k, v):
+        w3 = w.reshape(g, 1, hl)
+        y = _TimeMajorShortHyena.apply(q, k, v, w3 if w3.is_contiguous() else w3.contiguous())
+        return y.permute(0, 2, 1, 3)
     to_blgd = lambda t: t.permute(1, 0, 2, 3).reshape(bs, seqlen, groups, width)
     y = two_pass_chunked_gate_conv_gate(to_blgd(v), to_blgd(k), to_blgd(q), w.reshape(groups, 1, hl),
                                         bs, seqlen, groups, width, fwd_kernel_cfg=_FWD_CFG, bwd_autotune=True)

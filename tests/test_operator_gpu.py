@@ -6,7 +6,7 @@ import torch
 
 import oracle
 from helpers import TOL, TOL_DH, assert_close
-from savanna_amd import two_pass_chunked_gate_conv_gate
+from savanna_amd import _lib, two_pass_chunked_gate_conv_gate
 from savanna_amd.kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
 from savanna_amd.operators import hyena
 
@@ -219,6 +219,55 @@ def test_run_short_hyena_layout(gcg_lib, repeat_interleave):
         assert_close(a.grad, r.grad, TOL_DH[torch.float32] if n == "dw" else TOL[torch.float32], n)
     with pytest.raises(AssertionError, match="Must specify"):
         run_short_hyena(*dev)
+
+
+@pytest.mark.parametrize("seqlen,bs,g,dg,hl,dtype", [
+    (8192, 16, 48, 16, 7, torch.bfloat16),     # the reference's own case: d_model 768, group size 16, kernel 7
+    (1000, 3, 5, 20, 4, torch.float32),        # ragged length, odd batch, dg not a power of two
+    (513, 2, 6, 16, 8, torch.float16),
+    (300, 4, 3, 32, 5, "bf16-fp32"),           # bf16 tensors with an fp32 filter
+], ids=["ref-shape-bf16", "ragged-f32", "f16", "bf16-fp32-filter"])
+def test_run_short_hyena_in_place(gcg_lib, seqlen, bs, g, dg, hl, dtype):
+    """run_short_hyena reads (seqlen, bs, g, dg) operands where they lie: the reference's test shape
+    (tests/model/test_kernels.py:133-137, seqlen 8192, bs 16, d_model 768 in groups of 16, 7 taps, bf16), against
+    the oracle on whole filter groups, and a kernel trace without any copy or permute kernel."""
+    from savanna_amd.kernels.short_hyena import run_short_hyena
+
+    mixed = dtype == "bf16-fp32"
+    tdt = torch.bfloat16 if mixed else dtype
+    gen = torch.Generator().manual_seed(5)
+    q, k, v = (torch.randn(seqlen, bs, g, dg, generator=gen).to(tdt) for _ in range(3))
+    w = (torch.randn(g, 1, hl, generator=gen) / hl ** 0.5).to(torch.float32 if mixed else tdt)
+    dy = (0.1 * torch.randn(bs, seqlen, g, dg, generator=gen)).to(tdt)
+    dev = [t.to(DEV).requires_grad_(True) for t in (q, k, v, w)]
+    dyd = dy.to(DEV)
+    from torch.profiler import ProfilerActivity, profile
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        out = run_short_hyena(*dev, autotune=True)
+        out.backward(dyd.permute(0, 2, 1, 3))          # a gradient laid out like the kernel's own result
+        torch.cuda.synchronize()
+    assert out.shape == (bs, g, seqlen, dg)
+    names = [e.key for e in prof.key_averages() if e.device_time_total > 0 and "Memcpy" not in e.key and "Memset" not in e.key]
+    assert all("gcg::" in n for n in names) and len(names) == 3, names     # forward, backward, filter-gradient reduction
+    # oracle on a few whole filter groups of every batch entry (the operator is independent across groups)
+    gs = sorted({0, g // 2, g - 1})
+    to_blgd = lambda t: t[:, :, gs].permute(1, 0, 2, 3).float()
+    ref_y = oracle.gcg_fwd_oracle(to_blgd(v), to_blgd(k), to_blgd(q), w[gs].float())
+    ref = oracle.gcg_bwd_oracle(dy[:, :, gs].float(), to_blgd(v), to_blgd(k), to_blgd(q), w[gs].float())
+    tol = 1.1 * 2.0 ** -8 if mixed else TOL[tdt]
+    assert_close(out.permute(0, 2, 1, 3)[:, :, gs], ref_y, tol, "out")
+    for a, r, n in zip((dev[2], dev[1], dev[0]), ref[:3], ("dv", "dk", "dq")):
+        assert a.grad.shape == (seqlen, bs, g, dg) and a.grad.is_contiguous()
+        assert_close(a.grad[:, :, gs].permute(1, 0, 2, 3), r, tol, n)
+    assert dev[3].grad.dtype == w.dtype
+    assert_close(dev[3].grad[gs], ref[3], TOL_DH[w.dtype], "dw")
+    # and bit for bit what the batch-major kernels give on permuted copies
+    x_, B_, C_ = (t.detach().permute(1, 0, 2, 3).contiguous() for t in (dev[2], dev[1], dev[0]))
+    _, _, y2 = _lib.fwd(x_, B_, C_, dev[3].detach(), algo="window")
+    assert torch.equal(out.permute(0, 2, 1, 3), y2)
+    dx2, dB2, dC2, dh2 = _lib.bwd(dyd, x_, B_, C_, dev[3].detach(), algo="window")
+    assert torch.equal(dev[2].grad.permute(1, 0, 2, 3), dx2) and torch.equal(dev[0].grad.permute(1, 0, 2, 3), dC2)
+    assert torch.equal(dev[3].grad, dh2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
