@@ -138,7 +138,8 @@ class Op:
         from savanna_amd.kernels.cgcg.interface import (two_pass_chunked_gate_conv_gate,
                                                         two_pass_chunked_gate_conv_gate_interleaved)
         from savanna_amd.kernels.cgcg.src.kernel_utils import FwdKernelConfigRefactor
-        from savanna_amd.operators.hyena import _CausalDepthwiseConv, _FeaturizedShortGateConvGate
+        from savanna_amd.operators.hyena import (_CausalDepthwiseConv, _FeaturizedGateConvGate,
+                                                 _FeaturizedShortGateConvGate)
 
         wl = self.wl
         raw, wf, h = t["raw"], t["wf"], t["h"]
@@ -146,7 +147,8 @@ class Op:
         if ev is not None:
             ev[0].record()
         if self.layout == "mixer_fused":
-            y = _FeaturizedShortGateConvGate.apply(raw.reshape(wl.bs, wl.L, wl.g, wl.dg, 3), wf, h)
+            fused = _FeaturizedShortGateConvGate if self.hl <= 8 else _FeaturizedGateConvGate
+            y = fused.apply(raw.reshape(wl.bs, wl.L, wl.g, wl.dg, 3), wf, h)
         elif self.layout == "mixer":
             f = _CausalDepthwiseConv.apply(raw.reshape(wl.bs, wl.L, 3 * wl.d, 1), wf, KEEP_INTERMEDIATES)
             y = two_pass_chunked_gate_conv_gate_interleaved(f, h, wl.bs, wl.L, wl.g, wl.dg,
@@ -466,7 +468,8 @@ def main():
         # featurizer conv, and the two chained through autograd
         extra = {}
         for name in ("mr_fwdbwd_7b_interleaved", "se_fwdbwd_40b_interleaved", "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b",
-                     "mixer_se_fwdbwd_40b", "mixer_se_fwdbwd_40b_fused"):
+                     "mixer_fwdbwd_7b_fused", "mixer_fwd_7b", "mixer_fwd_7b_fused", "mixer_se_fwdbwd_40b",
+                     "mixer_se_fwdbwd_40b_fused"):
             r = time_workload(WORKLOADS[name], device, max(10, args.steps // 2), 4)
             extra[name] = {k: r[k] for k in ("ms_per_step", "tokens_per_s", "step_gbs", "step_hbm_frac")}
         line["next_rows"] = extra

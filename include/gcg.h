@@ -283,6 +283,36 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
             int32_t dtype, void *stream);
 
 /*
+ * Featurizer and Hyena-MR operator without the featurized tensor: gcg_dwconv_fwd followed by
+ * gcg_fwd_interleaved as one kernel that makes every row of (C, B, x) on the way
+ * (savanna/model/block.py:867-890 -> hyena.py:517-531), and a backward that needs the projection output only.
+ * Every row of the features is the featurizer's result rounded to the tensors' type, exactly what the two-call
+ * chain stores and reads back, so y, dh and the gradients are the chain's (bit for bit at bf16 and fp32; at
+ * f16 the compiler sums the featurizer's taps in another grouping in the two kernels, which moves a few results
+ * in 10^5 by one unit in the last place).
+ *   raw  (bs, L, g, dg, 3)   wf  (3 * g * dg, 1, kf), tensors' type   h  (g, 1, hl)   y  out, (bs, L, g, dg)
+ * Forward: reads raw, writes y -- 4 N s of memory traffic instead of 10 N s.
+ * Backward: one kernel recomputes the features from raw and writes their gradient into dfeat_scratch
+ * ((bs, L, g, dg, 3), caller's memory, contents on return unspecified), then the featurizer's own backward
+ * turns it into draw and dwf: the traffic of the two-call chain (16 N s), but nothing of size 3 N is kept
+ * between forward and backward.
+ *   draw  out, (bs, L, g, dg, 3)   dwf  out, (3 * g * dg, 1, kf)   dh  out, (g, 1, hl), filter's type
+ *   workspace  gcg_mixer_mr_bwd_workspace_bytes(...) bytes, 256-byte aligned
+ * Matrix-core kernels with full-length filters only: 98 <= hl <= 128, dg % 16 == 0, kf <= 3, 16-byte aligned
+ * tensors; otherwise GCG_ERR_UNSUPPORTED (use the two calls).  dtype: any, GCG_BF16_F32 / GCG_F16_F32 included.
+ */
+GCG_API int gcg_mixer_mr_fwd(const void *raw, const void *wf, const void *h, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+GCG_API size_t gcg_mixer_mr_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t kf, int32_t dtype);
+GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, const void *h,
+            void *draw, void *dwf, void *dh, void *dfeat_scratch,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+
+/*
  * Explicit decayed filter of Hyena-MR, ready for gcg_fwd, in one launch.
  * Replaces ExplicitSingleDecayFilter.filter (savanna/model/operators/hyena/parametrization/
  * explicit.py:68-75: h = self.h[:, :L] * self.decay[:, :L]) with L = min(hyena_mr_len, seq_len),

@@ -35,7 +35,7 @@ EXPORTS = (
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
-    "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
+    "gcg_mixer_mr_fwd", "gcg_mixer_mr_bwd_workspace_bytes", "gcg_mixer_mr_bwd", "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
     "gcg_fwd_decay", "gcg_bwd_decay", "gcg_fwd_interleaved_decay", "gcg_bwd_interleaved_decay",
 )
 
@@ -100,6 +100,12 @@ def load() -> ctypes.CDLL:
         lib.gcg_filter_decay_fwd.restype = ctypes.c_int
         lib.gcg_filter_decay_bwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
         lib.gcg_filter_decay_bwd.restype = ctypes.c_int
+        lib.gcg_mixer_mr_fwd.argtypes = [vp] * 4 + [i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_mixer_mr_fwd.restype = ctypes.c_int
+        lib.gcg_mixer_mr_bwd_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32, i32]
+        lib.gcg_mixer_mr_bwd_workspace_bytes.restype = sz
+        lib.gcg_mixer_mr_bwd.argtypes = [vp] * 9 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_mixer_mr_bwd.restype = ctypes.c_int
         lib.gcg_fwd_time_major.argtypes = [vp] * 5 + [i64, i64, i32, i32, i32, i32, vp]
         lib.gcg_fwd_time_major.restype = ctypes.c_int
         lib.gcg_bwd_time_major_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32]
@@ -495,6 +501,69 @@ def filter_decay_bwd(dh, decay):
     check(rc, "gcg_filter_decay_bwd")
     return dw
 
+
+
+def _check_mixer_mr(raw, wf, h):
+    if raw.dim() != 5 or raw.shape[-1] != 3 or not raw.is_contiguous():
+        raise ValueError("raw must be a contiguous (bs, L, g, dg, 3) tensor")
+    bs, L, g, dg, _ = raw.shape
+    if wf.dim() != 3 or wf.shape[0] != 3 * g * dg or wf.shape[1] != 1 or not wf.is_contiguous() or wf.dtype != raw.dtype:
+        raise ValueError("wf must be a contiguous (3 * g * dg, 1, kf) tensor of raw's dtype")
+    if h.dim() != 3 or h.shape[0] != g or h.shape[1] != 1 or not h.is_contiguous():
+        raise ValueError("h must be a contiguous (g, 1, hl) tensor")
+    if wf.device != raw.device or h.device != raw.device:
+        raise ValueError("raw, wf and h must be on one device")
+
+
+def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors) -> bool:
+    """Whether gcg_mixer_mr_fwd / _bwd take these sizes (matrix-core kernels, full-length filter, short featurizer)."""
+    return 98 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and all(t.data_ptr() % 16 == 0 for t in tensors)
+
+
+def mixer_mr_fwd(raw, wf, h):
+    """Featurizer conv and Hyena-MR operator in one pass: y (bs, L, g, dg) from the projection output
+    raw (bs, L, g, dg, 3), without the featurized tensor; the same values as dwconv_fwd followed by fwd_interleaved."""
+    _require_gpu(raw)
+    if TORCH_OPS:
+        return torch.ops.gcg.mixer_mr_fwd(raw, wf, h)
+    lib = load()
+    _check_mixer_mr(raw, wf, h)
+    bs, L, g, dg, _ = raw.shape
+    y = torch.empty(bs, L, g, dg, dtype=raw.dtype, device=raw.device)
+    if y.numel() == 0:
+        return y
+    with _on_device(raw.device):
+        rc = lib.gcg_mixer_mr_fwd(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg,
+                                  h.shape[-1], wf.shape[-1], gated_code(raw, h), torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_mixer_mr_fwd")
+    return y
+
+
+def mixer_mr_bwd(dy, raw, wf, h):
+    """(draw, dwf, dh) of mixer_mr_fwd from the projection output alone: the features are recomputed, their
+    gradient lives in a scratch tensor for the duration of the call."""
+    _require_gpu(raw)
+    if TORCH_OPS:
+        return torch.ops.gcg.mixer_mr_bwd(dy, raw, wf, h)
+    lib = load()
+    _check_mixer_mr(raw, wf, h)
+    bs, L, g, dg, _ = raw.shape
+    hl, kf = h.shape[-1], wf.shape[-1]
+    draw, dwf, dh = torch.empty_like(raw), torch.empty_like(wf), torch.empty_like(h)
+    if dy.numel() == 0:
+        return draw, dwf.zero_(), dh.zero_()
+    code = gated_code(raw, h)
+    nbytes = lib.gcg_mixer_mr_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code)
+    if nbytes == 0:
+        check(-2, "gcg_mixer_mr_bwd_workspace_bytes")
+    with _on_device(raw.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
+        scratch = torch.empty_like(raw)
+        rc = lib.gcg_mixer_mr_bwd(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
+                                  dwf.data_ptr(), dh.data_ptr(), scratch.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg,
+                                  hl, kf, code, torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_mixer_mr_bwd")
+    return draw, dwf, dh
 
 
 # ---- the short-filter operator on time-major operands (seqlen, bs, g, dg) ------------------------

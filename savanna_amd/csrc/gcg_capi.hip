@@ -533,6 +533,64 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
     return finish(gcg::mixer_se_bwd_launch(dtype, dy, raw, wf, h, draw, dwf, dh, workspace, dm, kf, (hipStream_t)stream));
 }
 
+// ---- featurizer and Hyena-MR operator: the forward in one pass
+
+GCG_API int gcg_mixer_mr_fwd(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L, int32_t g,
+                             int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!raw || !wf || !h || !y || kf <= 0) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    if (rc) return rc;
+    dm.es = 3;
+    if (!all_aligned16({raw, y}) || !gcg::mfma_feat_supported(dtype, dm, kf)) return GCG_ERR_UNSUPPORTED;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::mfma_il_fwd_feat_launch(dtype, raw, wf, kf, h, y, dm, (hipStream_t)stream));
+}
+
+namespace {
+int plain_tensor_code(int dtype) { return dtype == GCG_BF16_F32 ? GCG_BF16 : dtype == GCG_F16_F32 ? GCG_F16 : dtype; }
+size_t up256(size_t n) { return (n + 255) & ~(size_t)255; }
+} // namespace
+
+GCG_API size_t gcg_mixer_mr_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+                                                int32_t dtype)
+{
+    gcg::Dims dm, df;
+    if (kf <= 0 || make_dims(bs, L, g, dg, hl, dtype, &dm, true)) return 0;
+    if (!gcg::mfma_feat_supported(dtype, dm, kf)) return 0;
+    if (make_dims(bs, L, 3 * g * dg, 1, kf, plain_tensor_code(dtype), &df) || !gcg::dwconv_supported(df)) return 0;
+    return up256(gcg::mfma_feat_bwd_workspace(dtype, dm)) + up256(gcg::dwconv_bwd_workspace(df));
+}
+
+GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf,
+                             void *dh, void *dfeat_scratch, void *workspace, size_t workspace_bytes, int64_t bs,
+                             int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !raw || !wf || !h || !draw || !dwf || !dh || !dfeat_scratch || kf <= 0) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm, df;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    if (rc) return rc;
+    dm.es = 3;
+    dm.keep_out = 1;
+    if (!all_aligned16({dy, raw, draw, dfeat_scratch}) || !gcg::mfma_feat_supported(dtype, dm, kf)) return GCG_ERR_UNSUPPORTED;
+    rc = make_dims(bs, L, 3 * g * dg, 1, kf, plain_tensor_code(dtype), &df);
+    if (rc) return rc;
+    if (!gcg::dwconv_supported(df)) return GCG_ERR_UNSUPPORTED;
+    const size_t need = gcg_mixer_mr_bwd_workspace_bytes(bs, L, g, dg, hl, kf, dtype);
+    if (!need || !workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    void *ws2 = (char *)workspace + up256(gcg::mfma_feat_bwd_workspace(dtype, dm));
+    int e = gcg::mfma_il_bwd_feat_launch(dtype, dy, raw, wf, kf, h, dfeat_scratch, dh, workspace, dm, st);
+    if (e) return finish(e);
+    return finish(gcg::dwconv_bwd_launch(plain_tensor_code(dtype), dfeat_scratch, raw, wf, draw, dwf, ws2, df, st));
+}
+
 // ---- explicit decayed filter (Hyena-MR parametrization)
 
 GCG_API int gcg_filter_decay_fwd(const float *w, const float *decay, void *h, int32_t g, int32_t l_cache, int32_t hl,

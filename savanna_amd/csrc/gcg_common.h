@@ -294,6 +294,14 @@ int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, cons
 int mfma_il_bwd_launch(int dtype, const void *dy, const void *feat, const void *h, void *dfeat, void *dh,
                        void *ws, const Dims &dm, hipStream_t st);
 
+// the same forward with the featurizer in front: raw is the projection output, wfeat (3 * d, 1, kf)
+bool mfma_feat_supported(int dtype, const Dims &dm, int kf);
+size_t mfma_feat_bwd_workspace(int dtype, const Dims &dm);
+int mfma_il_fwd_feat_launch(int dtype, const void *raw, const void *wfeat, int kf, const void *h, void *y,
+                            const Dims &dm, hipStream_t st);
+int mfma_il_bwd_feat_launch(int dtype, const void *dy, const void *raw, const void *wfeat, int kf, const void *h,
+                            void *dfeat, void *dh, void *ws, const Dims &dm, hipStream_t st);
+
 // ungated short causal depthwise convolution (the featurizer), (bs, L, g, dg) channel-fastest
 bool dwconv_supported(const Dims &dm);
 int dwconv_fwd_launch(int dtype, const void *x, const void *w, void *y, const Dims &dm, hipStream_t st);

@@ -92,10 +92,70 @@ template <typename T, int NR> __device__ __forceinline__ Row<T> units_row(const 
     return r;
 }
 
+// ---- featurizer in front of the operator ------------------------------------------------------
+// The features need not be given: a kernel with KF > 0 takes the projection output instead and makes every
+// row of (C, B, x) on the way -- a short causal depthwise convolution with one filter per feature channel
+// (wfeat: (3 * d, 1, kf), kf <= KF), rounded to T as if the featurizer had stored it and the kernel had read
+// it back.  A lane then owns NR consecutive rows of a step instead of rows RP apart, and also fetches the
+// KF-1 rows before them: rows its neighbours own and request at the same time, so they cost cache hits, not
+// memory traffic.
+// tap[m][v]: what feature channel f0 + v multiplies the row KF-1-m rows in the past with (zero where kf < KF)
+template <typename T, int KF, int NV>
+__device__ __forceinline__ void load_feat_taps(const T *wfeat, int64_t f0, int kf, float (&tap)[KF][NV])
+{
+#pragma unroll
+    for (int v = 0; v < NV; ++v)
+#pragma unroll
+        for (int m = 0; m < KF; ++m) {
+            const int kk = m - (KF - kf);                // index into the kf taps of the filter
+            const float t = Elem<T>::load(wfeat + (f0 + v) * kf + (kk >= 0 ? kk : 0));
+            tap[m][v] = kk >= 0 ? t : 0.f;
+        }
+}
+// (C, B, x) of a lane's NR rows from the KF-1 + NR fetched pieces of the projection output, oldest row first;
+// sums in the featurizer kernel's order (oldest sample first, fp32) and rounded to T like its output
+template <typename T, int NR, int KF>
+__device__ __forceinline__ void featurized_rows(const u32x3 (&p)[KF - 1 + NR], const float (&tap)[KF][3 * (4 / MT<T>::ES)],
+                                                float (&xf)[8], float (&Bf)[8], float (&Cf)[8])
+{
+    typedef MT<T> M;
+    constexpr int NV = 3 * (4 / M::ES);
+    float rv[KF - 1 + NR][NV];
+#pragma unroll
+    for (int k = 0; k < KF - 1 + NR; ++k) {
+        if constexpr (M::ES == 4) {
+            rv[k][0] = __uint_as_float(p[k][0]); rv[k][1] = __uint_as_float(p[k][1]); rv[k][2] = __uint_as_float(p[k][2]);
+        } else {
+            M::unpack2(p[k][0], rv[k][0], rv[k][1]);
+            M::unpack2(p[k][1], rv[k][2], rv[k][3]);
+            M::unpack2(p[k][2], rv[k][4], rv[k][5]);
+        }
+    }
+    u32x3 fp[NR];
+#pragma unroll
+    for (int k = 0; k < NR; ++k) {
+        float acc[NV];
+#pragma unroll
+        for (int v = 0; v < NV; ++v) acc[v] = 0.f;
+#pragma unroll
+        for (int m = 0; m < KF; ++m)
+#pragma unroll
+            for (int v = 0; v < NV; ++v) acc[v] = fmaf(tap[m][v], rv[k + m][v], acc[v]);
+        if constexpr (M::ES == 4) {
+            fp[k][0] = __float_as_uint(acc[0]); fp[k][1] = __float_as_uint(acc[1]); fp[k][2] = __float_as_uint(acc[2]);
+        } else {
+            fp[k][0] = M::pack2(acc[0], acc[1]); fp[k][1] = M::pack2(acc[2], acc[3]); fp[k][2] = M::pack2(acc[4], acc[5]);
+        }
+    }
+    il_split<T, NR>(fp, xf, Bf, Cf);
+}
+
 // ---------------------------------------------------------------------------- forward
-template <typename T, int NK, int NW>
+// KF > 0: `feat` is the projection output and wfeat the featurizer's filters (see above).
+template <typename T, int NK, int NW, int KF>
 __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restrict__ feat, const T *__restrict__ h,
-                                                          T *__restrict__ y, Dims dm, MfmaPlan pl)
+                                                          const T *__restrict__ wfeat, T *__restrict__ y, Dims dm,
+                                                          MfmaPlan pl, int kf)
 {
     typedef MT<T> M;
     typedef typename M::op_t op_t;
@@ -104,6 +164,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     typedef GeoIL<T, NW> I;
     constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW;
     constexpr int CH = I::CH, LPR = I::LPR, RP = I::RP, NR = I::NR;
+    constexpr bool FEAT = KF > 0;
+    constexpr int NH = FEAT ? KF - 1 : 0;           // rows fetched before the lane's own
+    constexpr int KS = FEAT ? 1 : RP;               // rows between a lane's consecutive rows
+    constexpr int NV = 3 * CH;                      // feature values of a lane's row piece
     __shared__ __attribute__((aligned(16))) unsigned char u_rm[STEP * UROW];
     __shared__ __attribute__((aligned(16))) unsigned char y_st[STEP * YROW];
     __shared__ hraw_t htab[NW][HTAB];
@@ -114,44 +178,55 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     const int64_t b = wg / pl.nseg;
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
-    const int rr = tid / LPR, a = tid % LPR;        // memory layout: rows rr + RP*k, channels CH*a ..
+    const int rr = tid / LPR, a = tid % LPR;        // memory layout: rows row0 + KS*k, channels CH*a ..
+    const int row0 = FEAT ? NR * rr : rr;
     const int j = l & 15, q = l >> 4;               // matrix layout
     const int64_t d = dm.d, L = dm.L;
     const int64_t c0 = (int64_t)cb * CB;
-    const int hl = dm.hl;
 
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
     const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
 
     // Windows over rows [t0, t1) of this batch row (12-byte pieces are only 4-byte aligned, which
     // buffer accesses take).  A lane's offset into y is lane_off + k * pass_off + step_off(s); into
-    // the features three times that.
+    // the features three times that.  (With the featurizer the features' window starts NH rows earlier.)
     const int64_t t0 = (s_lo - (NK - 1)) * STEP > 0 ? (s_lo - (NK - 1)) * STEP : 0;
     const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
+    const int64_t tf = t0 - NH > 0 ? t0 - NH : 0;
     const int64_t row_bytes = d * M::ES, win_bytes = (t1 - t0) * row_bytes;
     const int64_t origin = (b * L + t0) * d;
-    const win_t wf = make_window(feat + 3 * origin, 3 * win_bytes), wy = make_window(y + origin, win_bytes);
+    const win_t wf = make_window(feat + 3 * (b * L + tf) * d, 3 * (t1 - tf) * row_bytes);
+    const win_t wy = make_window(y + origin, win_bytes);
     const bool cvalid = c0 + CH * a < d;
-    const uint32_t lane_off = (uint32_t)(rr * row_bytes + (c0 + CH * a) * M::ES);
-    const uint32_t pass_off = (uint32_t)(RP * row_bytes), bad = cvalid ? 0u : WIN_OFF;
+    const uint32_t lane_off = (uint32_t)(row0 * row_bytes + (c0 + CH * a) * M::ES);
+    const uint32_t feat_off = lane_off + (uint32_t)((t0 - tf) * row_bytes);
+    const uint32_t pass_off = (uint32_t)(KS * row_bytes), bad = cvalid ? 0u : WIN_OFF;
     auto step_off = [&](int64_t s) { return (uint32_t)((s * STEP - t0) * row_bytes); };
 
     op_t A[NK];            // A[(ph - i + NK) % NK]: operand of step s-i while step s runs in phase ph
 #pragma unroll
     for (int i = 0; i < NK; ++i) A[i] = M::zero_op();
 
-    unsigned char *u_wr = u_rm + rr * UROW + M::LES * CH * a;
+    unsigned char *u_wr = u_rm + row0 * UROW + M::LES * CH * a;
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
-    const unsigned char *y_rd = y_st + rr * YROW + 4 * CH * a;
+    const unsigned char *y_rd = y_st + row0 * YROW + 4 * CH * a;
 
-    auto fetch = [&](int64_t s, u32x3 (&p)[NR]) {
-        const uint32_t o = lane_off + step_off(s);
+    // rows of step s: the NH rows before the lane's own first, then its NR rows
+    auto fetch = [&](int64_t s, u32x3 (&p)[NH + NR]) {
+        const uint32_t o = feat_off + step_off(s);
 #pragma unroll
-        for (int k = 0; k < NR; ++k) p[k] = ldw12(wf, 3 * (o + k * pass_off) + bad);
+        for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, 3 * (o + (k - NH) * pass_off) + bad);
     };
     auto store_u = [&](const float (&uf)[8]) {
 #pragma unroll
-        for (int k = 0; k < NR; ++k) store_operand_unit<T>(u_wr + RP * k * UROW, UROW, &uf[CH * k]);
+        for (int k = 0; k < NR; ++k) store_operand_unit<T>(u_wr + KS * k * UROW, UROW, &uf[CH * k]);
+    };
+    float tap[FEAT ? KF : 1][NV];
+    if constexpr (FEAT) load_feat_taps<T, KF, NV>(wfeat, cvalid ? 3 * (c0 + CH * a) : 0, kf, tap);
+    // (C, B, x) of the lane's rows from the fetched pieces
+    auto rows_of = [&](const u32x3 (&p)[NH + NR], float (&xf)[8], float (&Bf)[8], float (&Cf)[8]) {
+        if constexpr (FEAT) featurized_rows<T, NR, KF>(p, tap, xf, Bf, Cf);
+        else il_split<T, NR>(p, xf, Bf, Cf);
     };
     // The filter taps of this wave's group are requested before any row, so that the filter table and the
     // Toeplitz tiles are built while the rows are in flight (loads complete in order of issue).
@@ -163,12 +238,12 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     // step s_lo-i lands in ring slot NK-i, where phase 0 expects it.  The rows of the first step
     // follow them: they are needed last.
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
-    u32x3 lead[NLEAD][NR];
+    u32x3 lead[NLEAD][NH + NR];
     if constexpr (NK > 1) {
 #pragma unroll
         for (int i = 1; i < NK; ++i) fetch(s_lo - i, lead[i - 1]);
     }
-    u32x3 in[NR];
+    u32x3 in[NH + NR];
     fetch(s_lo, in);
 
     store_taps(htab[w], l, hv);
@@ -184,7 +259,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
             float xf[8], Bf[8], Cf[8], uf[8];
-            il_split<T, NR>(lead[i - 1], xf, Bf, Cf);
+            rows_of(lead[i - 1], xf, Bf, Cf);
 #pragma unroll
             for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
             store_u(uf);
@@ -199,11 +274,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
-                u32x3 nx[NR];        // rows of the next step; past the segment they fall outside the window
+                u32x3 nx[NH + NR];   // rows of the next step; past the segment they fall outside the window
                 fetch(s + 1, nx);
 
                 float xf[8], Bf[8], Cf[8], uf[8];
-                il_split<T, NR>(in, xf, Bf, Cf);
+                rows_of(in, xf, Bf, Cf);
 #pragma unroll
                 for (int e = 0; e < 8; ++e) uf[e] = xf[e] * Bf[e];
                 store_u(uf);
@@ -226,11 +301,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
                     float yf[CH];
 #pragma unroll
                     for (int c = 0; c < CH; ++c)
-                        yf[c] = Cf[CH * k + c] * *(const float *)(y_rd + RP * k * YROW + 4 * c);
+                        yf[c] = Cf[CH * k + c] * *(const float *)(y_rd + KS * k * YROW + 4 * c);
                     stw4(wy, o + k * pass_off, pack_unit<T>(yf));
                 }
 #pragma unroll
-                for (int k = 0; k < NR; ++k) in[k] = nx[k];
+                for (int k = 0; k < NH + NR; ++k) in[k] = nx[k];
                 ++s;
             }
         }
@@ -244,9 +319,12 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 // iterations before those are used, and the outputs of a row leave as one interleaved row.
 // The early x, B values wait in LDS: each lane parks its own two row vectors in a ring of NK-1
 // slots and reads them back itself, so the ring needs no barrier.
-template <typename T, int NK, int NW, bool KEEP>
+// KF > 0: `feat` is the projection output and wfeat the featurizer's filters (see above); dfeat is still the
+// gradient of the featurized features, which the featurizer's own backward then takes.
+template <typename T, int NK, int NW, bool KEEP, int KF>
 __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ feat,
-                                                          const T *__restrict__ h, T *__restrict__ dfeat,
+                                                          const T *__restrict__ h, const T *__restrict__ wfeat,
+                                                          int kf, T *__restrict__ dfeat,
                                                           T *__restrict__ dh, float *__restrict__ ws, Dims dm,
                                                           MfmaPlan pl)
 {
@@ -257,6 +335,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     typedef GeoIL<T, NW> I;
     constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW;
     constexpr int CH = I::CH, LPR = I::LPR, RP = I::RP, NR = I::NR;
+    constexpr bool FEAT = KF > 0;
+    constexpr int NH = FEAT ? KF - 1 : 0;           // rows fetched before the lane's own
+    constexpr int KS = FEAT ? 1 : RP;               // rows between a lane's consecutive rows
+    constexpr int NV = 3 * CH;                      // feature values of a lane's row piece
     constexpr int ND = 2 * NK - 1;
     constexpr int RING_ROWS = STEP * NK;
     constexpr int OFF_U = 0;                                // u of the current step, row-major
@@ -286,7 +368,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     const int64_t b = wg / pl.nseg;
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
-    const int rr = tid / LPR, a = tid % LPR;        // memory layout: rows rr + RP*k, channels CH*a ..
+    const int rr = tid / LPR, a = tid % LPR;        // memory layout: rows row0 + KS*k, channels CH*a ..
+    const int row0 = FEAT ? NR * rr : rr;
     const int j = l & 15, q = l >> 4;               // matrix layout
     const int64_t d = dm.d, L = dm.L;
     const int64_t c0 = (int64_t)cb * CB;
@@ -301,13 +384,15 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     const int64_t t0 = (s_lo - (NK - 1)) * STEP > 0 ? (s_lo - (NK - 1)) * STEP : 0;
     const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
     const int64_t t2 = (s_hi + NK - 1) * STEP < L ? (s_hi + NK - 1) * STEP : L;
+    const int64_t tf = t0 - NH > 0 ? t0 - NH : 0;        // the featurizer looks NH rows further back
     const int64_t row_bytes = d * M::ES, origin = (b * L + t0) * d;
-    const win_t wf = make_window(feat + 3 * origin, 3 * (t2 - t0) * row_bytes);
+    const win_t wf = make_window(feat + 3 * (b * L + tf) * d, 3 * (t2 - tf) * row_bytes);
     const win_t wdyw = make_window(dy + origin, (t2 - t0) * row_bytes);
     const win_t wdf = make_window(dfeat + 3 * origin, 3 * (t1 - t0) * row_bytes);
     const bool cvalid = c0 + CH * a < d;
-    const uint32_t lane_off = (uint32_t)(rr * row_bytes + (c0 + CH * a) * M::ES);
-    const uint32_t pass_off = (uint32_t)(RP * row_bytes), bad = cvalid ? 0u : WIN_OFF;
+    const uint32_t lane_off = (uint32_t)(row0 * row_bytes + (c0 + CH * a) * M::ES);
+    const uint32_t feat_off = lane_off + (uint32_t)((t0 - tf) * row_bytes);
+    const uint32_t pass_off = (uint32_t)(KS * row_bytes), bad = cvalid ? 0u : WIN_OFF;
     auto step_off = [&](int64_t sg) { return (uint32_t)((sg * STEP - t0) * row_bytes); };
 
     // While step s runs in phase ph:  Au[(ph - i + NK) % NK] is the u operand of step s-i,
@@ -325,18 +410,26 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // LDS addresses of this lane
-    const int rm_off = rr * UROW + M::LES * CH * a;                                    // memory layout, row rr
+    const int rm_off = row0 * UROW + M::LES * CH * a;                                  // memory layout, row row0
     unsigned char *y_wr = y_st + j * YROW + (16 * w + 4 * q) * 4;
     unsigned char *d_wr = d_st + (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
-    const unsigned char *y_rd = y_st + rr * YROW + 4 * CH * a;
-    const unsigned char *d_rd = d_st + rr * YROW + 4 * CH * a;
+    const unsigned char *y_rd = y_st + row0 * YROW + 4 * CH * a;
+    const unsigned char *d_rd = d_st + row0 * YROW + 4 * CH * a;
     unsigned char *xb_own = smem + OFF_XB + tid * 16 * M::RW;                 // slot k at + k * 2 * XB_VEC
 
     // interleaved rows and dy of one step (zero outside the sequence)
-    auto fetch_feat = [&](int64_t step, u32x3 (&p)[NR]) {
-        const uint32_t o = lane_off + step_off(step);
+    // (with the featurizer: the NH rows before the lane's own first, then its NR rows)
+    auto fetch_feat = [&](int64_t step, u32x3 (&p)[NH + NR]) {
+        const uint32_t o = feat_off + step_off(step);
 #pragma unroll
-        for (int k = 0; k < NR; ++k) p[k] = ldw12(wf, 3 * (o + k * pass_off) + bad);
+        for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, 3 * (o + (k - NH) * pass_off) + bad);
+    };
+    float tap[FEAT ? KF : 1][NV];
+    if constexpr (FEAT) load_feat_taps<T, KF, NV>(wfeat, cvalid ? 3 * (c0 + CH * a) : 0, kf, tap);
+    // x, B, C of the lane's rows from the fetched pieces
+    auto rows_of = [&](const u32x3 (&p)[NH + NR], float (&xo)[8], float (&Bo)[8], float (&Co)[8]) {
+        if constexpr (FEAT) featurized_rows<T, NR, KF>(p, tap, xo, Bo, Co);
+        else il_split<T, NR>(p, xo, Bo, Co);
     };
     auto fetch_dy = [&](int64_t step, Row<T> &out) {
         const uint32_t o = lane_off + step_off(step) + bad;
@@ -347,11 +440,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     };
     auto store_rows = [&](unsigned char *tile, const float (&f)[8]) {
 #pragma unroll
-        for (int k = 0; k < NR; ++k) store_operand_unit<T>(tile + rm_off + RP * k * UROW, UROW, &f[CH * k]);
+        for (int k = 0; k < NR; ++k) store_operand_unit<T>(tile + rm_off + KS * k * UROW, UROW, &f[CH * k]);
     };
 
     // iteration sigma brings the interleaved rows and dy of step sigma+NK-1
-    u32x3 in[NR];
+    u32x3 in[NH + NR];
     Row<T> dyr;
     // The filter taps of this wave's group are requested before any row (loads complete in order of issue).
     hraw_t hv[HTAB / 64];
@@ -362,7 +455,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     // brought.  Requested together, so the lead-in costs one memory latency instead of NK-1; the rows
     // of the first iteration follow them (needed last).
     constexpr int NLEAD = NK > 1 ? NK - 1 : 1;
-    u32x3 past[NLEAD][NR], lead[NLEAD][NR];
+    u32x3 past[NLEAD][NH + NR], lead[NLEAD][NH + NR];
     Row<T> wdy[NLEAD];
     if constexpr (NK > 1) {
 #pragma unroll
@@ -390,12 +483,12 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
         for (int i = 1; i < NK; ++i) {
             // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
             float f0[8], f1[8], f2[8], tf[8], pf[8];
-            il_split<T, NR>(past[i - 1], f0, f1, f2);
+            rows_of(past[i - 1], f0, f1, f2);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
             store_rows(u_rm, pf);
             // x, B of step s_lo+NK-1-i wait in ring slot (NK-1-i) % (NK-1) for iteration s_lo+NK-1-i
-            il_split<T, NR>(lead[i - 1], f0, f1, f2);
+            rows_of(lead[i - 1], f0, f1, f2);
             unsigned char *slot = xb_own + ((NK - 1 - i) % (NK - 1)) * 2 * XB_VEC;
             lds_store_row<T>(slot, pack8<T>(f0));
             lds_store_row<T>(slot + XB_VEC, pack8<T>(f1));
@@ -419,7 +512,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
                 const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
-                u32x3 nx[NR];        // rows of the next iteration; past the segment's reach they are
+                u32x3 nx[NH + NR];   // rows of the next iteration; past the segment's reach they are
                 Row<T> dyn;          // outside the windows
                 fetch_feat(s + NK, nx);
                 fetch_dy(s + NK, dyn);
@@ -427,7 +520,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
                 float xf[8], Bf[8], tf[8], cf[8], pf[8];
                 {
                     float xa[8], Ba[8];
-                    il_split<T, NR>(in, xa, Ba, cf);          // x, B, C of step s+NK-1
+                    rows_of(in, xa, Ba, cf);                  // x, B, C of step s+NK-1
                     if constexpr (NK > 1) {
                         unsigned char *slot = xb_own + xb_slot * 2 * XB_VEC;
                         const Row<T> xw = lds_load_row<T>(slot), Bw = lds_load_row<T>(slot + XB_VEC);
@@ -488,8 +581,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
 #pragma unroll
                         for (int c = 0; c < CH; ++c) {
                             const int e = CH * k + c;
-                            const float y2v = *(const float *)(y_rd + RP * k * YROW + 4 * c);
-                            const float duv = *(const float *)(d_rd + RP * k * YROW + 4 * c);
+                            const float y2v = *(const float *)(y_rd + KS * k * YROW + 4 * c);
+                            const float duv = *(const float *)(d_rd + KS * k * YROW + 4 * c);
                             oC[e] = dyf[e] * y2v;
                             ox[e] = duv * Bf[e];
                             oB[e] = duv * xf[e];
@@ -501,7 +594,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
                     for (int k = 0; k < NR; ++k) win_store_as<KEEP>(wdf, 3 * (o + k * pass_off) + bad, po[k]);
                 }
 #pragma unroll
-                for (int k = 0; k < NR; ++k) in[k] = nx[k];
+                for (int k = 0; k < NH + NR; ++k) in[k] = nx[k];
                 dyr = dyn;
                 ++s;
             }
@@ -523,9 +616,36 @@ int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStre
     // d = 16384: 361 against 375 us).
     static const int order = env_int("GCG_MFMA_FWD_ORDER", -1);   // tuning override: 0 round-robin, 1 XCD-contiguous
     p.xcd = order >= 0 ? (order != 0) : 0;
-    e = launch_main((mfma_il_fwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)feat,
-                       (const T *)h, (T *)y, dm, p);
+    e = launch_main((mfma_il_fwd_kernel<T, NK, NW, 0>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)feat,
+                       (const T *)h, (const T *)nullptr, (T *)y, dm, p, 0);
     return e;
+}
+
+// the forward with the featurizer in front: full-length filters only (the five-slice walk), up to FEAT_KF taps
+constexpr int FEAT_KF = 3;
+template <typename T, int NW>
+int fwd_feat_launch(const void *raw, const void *wfeat, int kf, const void *h, void *y, const Dims &dm, hipStream_t st)
+{
+    MfmaPlan p = plan(dm, NW, 16, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
+    if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    static const int order = env_int("GCG_MFMA_FWD_ORDER", -1);
+    p.xcd = order >= 0 ? (order != 0) : 0;
+    return launch_main((mfma_il_fwd_kernel<T, 5, NW, FEAT_KF>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+                       (const T *)raw, (const T *)h, (const T *)wfeat, (T *)y, dm, p, kf);
+}
+template <typename T>
+int fwd_feat_t(const void *raw, const void *wfeat, int kf, const void *h, void *y, const Dims &dm, hipStream_t st)
+{
+    static const int forced = env_int("GCG_MFMA_FEAT_NW", 0);   // tuning override: 4, 8 or 16
+    // the featurizer's registers leave room for three waves per SIMD: 8-wave workgroups at most (16 spill)
+    int nw = choose_nw(dm, MT<T>::SPLIT);
+    if (nw > 8) nw = 8;
+    if (forced == 4 || forced == 8 || (forced == 16 && !MT<T>::SPLIT)) nw = forced;
+    if constexpr (!MT<T>::SPLIT) {
+        if (nw == 16) return fwd_feat_launch<T, 16>(raw, wfeat, kf, h, y, dm, st);
+    }
+    if (nw == 8) return fwd_feat_launch<T, 8>(raw, wfeat, kf, h, y, dm, st);
+    return fwd_feat_launch<T, 4>(raw, wfeat, kf, h, y, dm, st);
 }
 
 template <typename T, int NK> int fwd_nk(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
@@ -559,16 +679,45 @@ int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, voi
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (p.fuse_dh) p.slot = next_dh_slot();
     if (dm.keep_out)
-        e = launch_main((mfma_il_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
-                           (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (T *)dh, (float *)ws, dm, p);
+        e = launch_main((mfma_il_bwd_kernel<T, NK, NW, true, 0>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+                           (const T *)dy, (const T *)feat, (const T *)h, (const T *)nullptr, 0, (T *)dfeat, (T *)dh,
+                           (float *)ws, dm, p);
     else
-        e = launch_main((mfma_il_bwd_kernel<T, NK, NW, false>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
-                           (const T *)dy, (const T *)feat, (const T *)h, (T *)dfeat, (T *)dh, (float *)ws, dm, p);
+        e = launch_main((mfma_il_bwd_kernel<T, NK, NW, false, 0>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+                           (const T *)dy, (const T *)feat, (const T *)h, (const T *)nullptr, 0, (T *)dfeat, (T *)dh,
+                           (float *)ws, dm, p);
     if (e || p.fuse_dh) return e;
     const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
                        (const float *)ws, (T *)dh, dm, p);
     return e;
+}
+
+// the backward from the projection output (full-length filters; 4-wave workgroups; dfeat goes to the featurizer's
+// backward next, so it is stored through the cache)
+template <typename T, int NW>
+int bwd_feat_launch(const void *dy, const void *raw, const void *wfeat, int kf, const void *h, void *dfeat, void *dh,
+                    void *ws, const Dims &dm, MfmaPlan p, hipStream_t st)
+{
+    int e = launch_main((mfma_il_bwd_kernel<T, 5, NW, true, FEAT_KF>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+                        (const T *)dy, (const T *)raw, (const T *)h, (const T *)wfeat, kf, (T *)dfeat, (T *)dh,
+                        (float *)ws, dm, p);
+    if (e || p.fuse_dh) return e;
+    const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
+    return launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
+                        (const float *)ws, (T *)dh, dm, p);
+}
+template <typename T>
+int bwd_feat_t(const void *dy, const void *raw, const void *wfeat, int kf, const void *h, void *dfeat, void *dh,
+               void *ws, const Dims &dm, hipStream_t st)
+{
+    MfmaPlan p = plan_bwd_nw(dm, choose_nw_bwd_feat(MT<T>::SPLIT), MT<T>::ES);
+    if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    if (p.fuse_dh) p.slot = next_dh_slot();
+    if constexpr (!MT<T>::SPLIT) {
+        if (p.nw == 8) return bwd_feat_launch<T, 8>(dy, raw, wfeat, kf, h, dfeat, dh, ws, dm, p, st);
+    }
+    return bwd_feat_launch<T, 4>(dy, raw, wfeat, kf, h, dfeat, dh, ws, dm, p, st);
 }
 
 template <typename T, int NK>
@@ -603,6 +752,40 @@ int mfma_il_fwd_launch(int dtype, const void *feat, const void *h, void *y, cons
     if (dtype == GCG_F32) return fwd_t<float>(feat, h, y, dm, st);
     if (dtype == GCG_BF16_F32) return fwd_t<bf16w_t>(feat, h, y, dm, st);
     if (dtype == GCG_F16_F32) return fwd_t<f16w_t>(feat, h, y, dm, st);
+    return (int)hipErrorInvalidValue;
+}
+
+size_t mfma_feat_bwd_workspace(int dtype, const Dims &dm)
+{
+    const bool split = dtype != GCG_BF16 && dtype != GCG_F16;
+    const MfmaPlan p = plan_bwd_nw(dm, choose_nw_bwd_feat(split), dtype == GCG_F32 ? 4 : 2);
+    return (size_t)p.nwg * p.nw * 128 * sizeof(float);
+}
+
+bool mfma_feat_supported(int dtype, const Dims &dm, int kf)
+{
+    return kf >= 1 && kf <= FEAT_KF && nk_for(dm.hl) == 5 && mfma_supported(dtype, dm);
+}
+
+int mfma_il_fwd_feat_launch(int dtype, const void *raw, const void *wfeat, int kf, const void *h, void *y,
+                            const Dims &dm, hipStream_t st)
+{
+    if (dtype == GCG_BF16) return fwd_feat_t<bf16_t>(raw, wfeat, kf, h, y, dm, st);
+    if (dtype == GCG_F16) return fwd_feat_t<f16_t>(raw, wfeat, kf, h, y, dm, st);
+    if (dtype == GCG_F32) return fwd_feat_t<float>(raw, wfeat, kf, h, y, dm, st);
+    if (dtype == GCG_BF16_F32) return fwd_feat_t<bf16w_t>(raw, wfeat, kf, h, y, dm, st);
+    if (dtype == GCG_F16_F32) return fwd_feat_t<f16w_t>(raw, wfeat, kf, h, y, dm, st);
+    return (int)hipErrorInvalidValue;
+}
+
+int mfma_il_bwd_feat_launch(int dtype, const void *dy, const void *raw, const void *wfeat, int kf, const void *h,
+                            void *dfeat, void *dh, void *ws, const Dims &dm, hipStream_t st)
+{
+    if (dtype == GCG_BF16) return bwd_feat_t<bf16_t>(dy, raw, wfeat, kf, h, dfeat, dh, ws, dm, st);
+    if (dtype == GCG_F16) return bwd_feat_t<f16_t>(dy, raw, wfeat, kf, h, dfeat, dh, ws, dm, st);
+    if (dtype == GCG_F32) return bwd_feat_t<float>(dy, raw, wfeat, kf, h, dfeat, dh, ws, dm, st);
+    if (dtype == GCG_BF16_F32) return bwd_feat_t<bf16w_t>(dy, raw, wfeat, kf, h, dfeat, dh, ws, dm, st);
+    if (dtype == GCG_F16_F32) return bwd_feat_t<f16w_t>(dy, raw, wfeat, kf, h, dfeat, dh, ws, dm, st);
     return (int)hipErrorInvalidValue;
 }
 

@@ -635,9 +635,21 @@ int choose_nw_bwd(const Dims &dm, bool fp32)
 }
 
 // one workgroup per CU in either geometry (fp32: one wave per SIMD by its registers alone)
+MfmaPlan plan_bwd_nw(const Dims &dm, int nw, int elem_bytes);
 MfmaPlan plan_bwd(const Dims &dm, bool split, int elem_bytes)
 {
-    const int nw = choose_nw_bwd(dm, split);
+    return plan_bwd_nw(dm, choose_nw_bwd(dm, split), elem_bytes);
+}
+// The backward that recomputes the featurizer spends twice the vector instructions per row: with two waves per
+// SIMD they hide behind each other (8-wave workgroups: 220 us at the 7B shape against 263 with 4 waves).
+int choose_nw_bwd_feat(bool split)
+{
+    static const int forced = env_int("GCG_MFMA_FEAT_BWD_NW", 0);   // tuning override: 4 or 8
+    if (forced == 4 || (forced == 8 && !split)) return forced;
+    return split ? 4 : 8;
+}
+MfmaPlan plan_bwd_nw(const Dims &dm, int nw, int elem_bytes)
+{
     MfmaPlan p = plan(dm, nw, 16, nw, elem_bytes);
     // the kernel adds the partials itself when a filter group lies within one channel block
     static const int fuse = env_int("GCG_MFMA_FUSE_DH", 1);    // tuning override: 0 = always a second launch

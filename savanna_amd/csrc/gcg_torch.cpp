@@ -502,6 +502,58 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> bwd_time_major(const Tensor &dy, cons
     return {dx, dB, dC, dh};
 }
 
+// ---- featurizer and Hyena-MR operator without the featurized tensor ----------------------------
+
+void check_mixer_mr(const Tensor &raw, const Tensor &wf, const Tensor &h)
+{
+    TORCH_CHECK(raw.dim() == 5 && raw.size(4) == 3 && raw.is_contiguous(),
+                "gcg: raw must be a contiguous (bs, L, g, dg, 3) tensor");
+    TORCH_CHECK(wf.dim() == 3 && wf.size(0) == 3 * raw.size(2) * raw.size(3) && wf.size(1) == 1 && wf.is_contiguous() &&
+                    wf.scalar_type() == raw.scalar_type(),
+                "gcg: wf must be a contiguous (3 * g * dg, 1, kf) tensor of raw's dtype");
+    TORCH_CHECK(h.dim() == 3 && h.size(0) == raw.size(2) && h.size(1) == 1 && h.is_contiguous(),
+                "gcg: h must be a contiguous (g, 1, hl) tensor");
+    TORCH_CHECK(wf.device() == raw.device() && h.device() == raw.device(), "gcg: raw, wf and h must be on one device");
+    (void)gated_code(raw, h);
+}
+
+Tensor mixer_mr_fwd(const Tensor &raw, const Tensor &wf, const Tensor &h)
+{
+    require_gpu(raw, "raw");
+    check_mixer_mr(raw, wf, h);
+    DeviceGuard guard(raw.device());
+    Tensor y = at::empty({raw.size(0), raw.size(1), raw.size(2), raw.size(3)}, raw.options());
+    if (y.numel() == 0) return y;
+    check_rc(gcg_mixer_mr_fwd(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), raw.size(0), raw.size(1),
+                              (int32_t)raw.size(2), (int32_t)raw.size(3), (int32_t)h.size(2), (int32_t)wf.size(2),
+                              gated_code(raw, h), stream_of(raw)),
+             "gcg_mixer_mr_fwd");
+    return y;
+}
+
+std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd(const Tensor &dy, const Tensor &raw, const Tensor &wf, const Tensor &h)
+{
+    require_gpu(raw, "raw");
+    check_mixer_mr(raw, wf, h);
+    TORCH_CHECK(dy.dim() == 4 && dy.sizes() == raw.sizes().slice(0, 4) && dy.scalar_type() == raw.scalar_type() &&
+                    dy.device() == raw.device() && dy.is_contiguous(),
+                "gcg: dy must be a contiguous (bs, L, g, dg) tensor of raw's dtype and device");
+    DeviceGuard guard(raw.device());
+    Tensor draw = at::empty_like(raw), dwf = at::empty_like(wf), dh = at::empty_like(h);
+    if (dy.numel() == 0) return {draw, dwf.zero_(), dh.zero_()};
+    const int64_t bs = raw.size(0), L = raw.size(1);
+    const int32_t g = (int32_t)raw.size(2), dg = (int32_t)raw.size(3), hl = (int32_t)h.size(2), kf = (int32_t)wf.size(2);
+    const int code = gated_code(raw, h);
+    const size_t nbytes = gcg_mixer_mr_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code);
+    Tensor ws = workspace(nbytes, raw, "gcg_mixer_mr_bwd_workspace_bytes");
+    Tensor scratch = at::empty_like(raw);      // gradient of the featurized features, for the duration of the call
+    check_rc(gcg_mixer_mr_bwd(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
+                              dwf.data_ptr(), dh.data_ptr(), scratch.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl,
+                              kf, code, stream_of(raw)),
+             "gcg_mixer_mr_bwd");
+    return {draw, dwf, dh};
+}
+
 // ---- meta implementations: shapes and dtypes only (fake tensors, torch.compile) ----------------
 
 std::tuple<Tensor, Tensor, Tensor> fwd_full_meta(const Tensor &x, const Tensor &B, const Tensor &C, const Tensor &h,
@@ -625,6 +677,19 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> bwd_time_major_meta(const Tensor &dy,
     return {at::empty_like(x), at::empty_like(x), at::empty_like(x), at::empty_like(h)};
 }
 
+Tensor mixer_mr_fwd_meta(const Tensor &raw, const Tensor &wf, const Tensor &h)
+{
+    check_mixer_mr(raw, wf, h);
+    return at::empty({raw.size(0), raw.size(1), raw.size(2), raw.size(3)}, raw.options());
+}
+std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd_meta(const Tensor &dy, const Tensor &raw, const Tensor &wf,
+                                                     const Tensor &h)
+{
+    check_mixer_mr(raw, wf, h);
+    (void)dy;
+    return {at::empty_like(raw), at::empty_like(wf), at::empty_like(h)};
+}
+
 } // namespace
 
 TORCH_LIBRARY(gcg, m)
@@ -642,6 +707,8 @@ TORCH_LIBRARY(gcg, m)
     m.def("mixer_se_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h) -> (Tensor, Tensor, Tensor)");
     m.def("filter_decay_fwd(Tensor w, Tensor decay, int hl, ScalarType dtype) -> Tensor");
     m.def("filter_decay_bwd(Tensor dh, Tensor decay) -> Tensor");
+    m.def("mixer_mr_fwd(Tensor raw, Tensor wf, Tensor h) -> Tensor");
+    m.def("mixer_mr_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h) -> (Tensor, Tensor, Tensor)");
     m.def("fwd_time_major(Tensor x, Tensor B, Tensor C, Tensor h) -> Tensor");
     m.def("bwd_time_major(Tensor dy, Tensor x, Tensor B, Tensor C, Tensor h) -> (Tensor, Tensor, Tensor, Tensor)");
     m.def("fwd_decay(Tensor x, Tensor B, Tensor C, Tensor w, Tensor decay, int hl, ScalarType filt) -> Tensor");
@@ -666,6 +733,8 @@ TORCH_LIBRARY_IMPL(gcg, CUDA, m)
     m.impl("mixer_se_bwd", &mixer_se_bwd);
     m.impl("filter_decay_fwd", &filter_decay_fwd);
     m.impl("filter_decay_bwd", &filter_decay_bwd);
+    m.impl("mixer_mr_fwd", &mixer_mr_fwd);
+    m.impl("mixer_mr_bwd", &mixer_mr_bwd);
     m.impl("fwd_time_major", &fwd_time_major);
     m.impl("bwd_time_major", &bwd_time_major);
     m.impl("fwd_decay", &fwd_decay);
@@ -688,6 +757,8 @@ TORCH_LIBRARY_IMPL(gcg, Meta, m)
     m.impl("mixer_se_bwd", &mixer_se_bwd_meta);
     m.impl("filter_decay_fwd", &filter_decay_fwd_meta);
     m.impl("filter_decay_bwd", &filter_decay_bwd_meta);
+    m.impl("mixer_mr_fwd", &mixer_mr_fwd_meta);
+    m.impl("mixer_mr_bwd", &mixer_mr_bwd_meta);
     m.impl("fwd_time_major", &fwd_time_major_meta);
     m.impl("bwd_time_major", &bwd_time_major_meta);
     m.impl("fwd_decay", &fwd_decay_meta);

@@ -317,6 +317,23 @@ class _FeaturizedShortGateConvGate(torch.autograd.Function):
         return _lib.mixer_se_bwd(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, h)
 
 
+class _FeaturizedGateConvGate(torch.autograd.Function):
+    """z = gated Hyena-MR convolution of the featurized projection, raw (b, l, g, dg, 3) -> (b, l, g, dg), without
+    the featurized tensor: the forward makes its rows on the way, the backward recomputes them from raw and hands
+    their gradient to the featurizer's backward inside the same call.  Only raw, wf and h are saved."""
+
+    @staticmethod
+    def forward(ctx, raw, wf, h):
+        raw, wf, h = (t if t.is_contiguous() else t.contiguous() for t in (raw, wf, h))
+        ctx.save_for_backward(raw, wf, h)
+        return _lib.mixer_mr_fwd(raw, wf, h)
+
+    @staticmethod
+    def backward(ctx, dz):
+        raw, wf, h = ctx.saved_tensors
+        return _lib.mixer_mr_bwd(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, h)
+
+
 class HyenaMixer(nn.Module):
     """The convolutional part of ParallelSequenceMixer.forward for the hyena operators
     (savanna/model/block.py:865-890): featurizer conv on the projected features, interleaved split,
@@ -325,13 +342,16 @@ class HyenaMixer(nn.Module):
 
     With a short operator filter (Hyena-SE: at most 8 taps, featurizer of at most 4, one filter per
     feature channel) the two convolutions run as one kernel each way (``fuse_short``); the result
-    differs from the two-kernel chain by the rounding of fp32 sums only."""
+    differs from the two-kernel chain by the rounding of fp32 sums only.  With a full-length Hyena-MR filter
+    (98 to 128 taps) and a featurizer of at most 3 taps the featurized tensor is never stored (``fuse_medium``):
+    the operator's kernels make its rows from the projection output, forward and backward, with the chain's results."""
 
     def __init__(self, operator: _CgcgOperatorBase, short_conv_L: int = 3, dtype=torch.float32, device=None,
-                 fuse_short: bool = True):
+                 fuse_short: bool = True, fuse_medium: bool = True):
         super().__init__()
         self.mixer = operator
         self.fuse_short = fuse_short
+        self.fuse_medium = fuse_medium
         self.hyena_proj_conv = CausalDepthwiseConv1d(3 * operator.hidden_size, short_conv_L, dtype=dtype, device=device)
 
     def _fusable(self, features: torch.Tensor, hl: int) -> bool:
@@ -343,6 +363,15 @@ class HyenaMixer(nn.Module):
         op = self.mixer
         bs, seqlen, d3 = features.shape
         h = op._filter(seqlen)
+        conv = self.hyena_proj_conv
+        if (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and
+                _lib.mixer_mr_supported(op.group_dim, h.shape[-1], conv.kernel_size, features) and
+                (op.cgcg_dtype == features.dtype or op._fp32_inside(features.dtype, features))):
+            g, dg = op.num_groups, op.group_dim
+            assert d3 == 3 * g * dg
+            z = _FeaturizedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3),
+                                              conv.short_conv_weight.to(features.dtype), h.to(op.cgcg_dtype))
+            return z.reshape(bs, seqlen, g * dg)
         if not self._fusable(features, h.shape[-1]):
             return op.forward_features(self.hyena_proj_conv.forward_bld(features, feeds_operator=True),
                                        from_featurizer=True)

@@ -54,7 +54,7 @@ class Workload:
     def algorithmic_bytes(self) -> int:
         if self.layout.startswith("mixer"):
             # forward: read raw features 3N, write y N; backward: read dy N and raw features 3N, write d features 3N
-            return 11 * self.bs * self.L * self.d * self.elem_bytes * len(self.filters)
+            return (11 if self.backward else 4) * self.bs * self.L * self.d * self.elem_bytes * len(self.filters)
         if self.layout == "dwconv":      # ungated: forward reads x, writes y; backward reads dy, x, writes dx
             return (5 if self.backward else 2) * self.bs * self.L * self.d * self.elem_bytes * len(self.filters)
         return self._gated_bytes()
@@ -109,6 +109,15 @@ WORKLOADS = {
     "mixer_fwdbwd_7b": Workload("mixer_fwdbwd_7b", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
                                 "featurizer conv + Hyena-MR on interleaved features, forward+backward, bf16, B=2 L=8192 "
                                 "D=4096 G=256 hl=128", layout="mixer"),
+    "mixer_fwdbwd_7b_fused": Workload("mixer_fwdbwd_7b_fused", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
+                                      "the same without the featurized tensor: the operator's kernels make its rows "
+                                      "from the projection output, forward and backward", layout="mixer_fused"),
+    "mixer_fwd_7b": Workload("mixer_fwd_7b", 2, 8192, 256, 16, (128,), torch.bfloat16, False,
+                             "featurizer conv + Hyena-MR on interleaved features, forward only (prefill), bf16, "
+                             "B=2 L=8192 D=4096 G=256 hl=128", layout="mixer"),
+    "mixer_fwd_7b_fused": Workload("mixer_fwd_7b_fused", 2, 8192, 256, 16, (128,), torch.bfloat16, False,
+                                   "the same as one kernel (the featurized tensor is never stored)",
+                                   layout="mixer_fused"),
     "mixer_fwdbwd_7b_reference_flow": Workload("mixer_fwdbwd_7b_reference_flow", 2, 8192, 256, 16, (128,),
                                                torch.bfloat16, True,
                                                "the same chain with the reference's data flow (permutes, F.conv1d on "

@@ -1,0 +1,132 @@
+"""Featurizer conv and Hyena-MR operator without the featurized tensor in memory (gcg_mixer_mr_fwd /
+gcg_mixer_mr_bwd): the chain of savanna/model/block.py:867-890 (featurizer conv on the projected features,
+interleaved split) into ParallelHyenaOperator's cgcg branch (hyena.py:517-531), with the rows of the features made
+inside the operator's kernels.  Checked against the oracle applied twice (featurizer with both gates at one and
+the intermediate rounded to the tensors' type, then the operator) and against the two-call chain of entry points."""
+import pytest
+import torch
+
+import oracle
+from helpers import TOL, TOL_DH, assert_close
+from savanna_amd import _lib
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+# (bs, L, g, dg, hl, kf)
+SHAPES = [
+    (2, 300, 3, 16, 128, 3),
+    (1, 1000, 5, 16, 100, 3),     # partial channel tile
+    (3, 2500, 10, 16, 128, 2),    # several runs per column; two taps
+    (1, 2049, 20, 16, 98, 3),
+    (2, 40, 2, 32, 128, 1),       # one tap: the featurizer scales its channels
+    (1, 700, 17, 16, 128, 3),     # d = 272
+]
+TYPES = [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.float32, torch.float32),
+         (torch.bfloat16, torch.float32)]
+
+
+def make(bs, L, g, dg, hl, kf, dtype, filt, seed=0):
+    gen = torch.Generator().manual_seed(seed)
+    raw = torch.randn(bs, L, g, dg, 3, generator=gen).to(dtype)
+    wf = (torch.randn(3 * g * dg, 1, kf, generator=gen) / kf ** 0.5).to(dtype)
+    h = (torch.randn(g, 1, hl, generator=gen) / hl ** 0.5).to(filt)
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen)).to(dtype)
+    return raw, wf, h, dy
+
+
+def chain(raw, wf, h, dy):
+    bs, L, g, dg, _ = raw.shape
+    flat = raw.reshape(bs, L, 3 * g * dg, 1)
+    f = _lib.dwconv_fwd(flat, wf)
+    y = _lib.fwd_interleaved(f.reshape(bs, L, g, dg, 3), h)
+    dfeat, dh = _lib.bwd_interleaved(dy, f.reshape(bs, L, g, dg, 3), h)
+    draw, dwf = _lib.dwconv_bwd(dfeat.reshape(bs, L, 3 * g * dg, 1), flat, wf)
+    return y, draw.reshape(raw.shape), dwf, dh
+
+
+def _cases():
+    for shape in SHAPES:
+        for dtype, filt in TYPES:
+            yield pytest.param(*shape, dtype, filt, id="x".join(map(str, shape)) + f"-{str(dtype)[6:]}-{str(filt)[6:]}")
+
+
+@pytest.mark.parametrize("bs,L,g,dg,hl,kf,dtype,filt", list(_cases()))
+def test_against_oracle_and_chain(gcg_lib, bs, L, g, dg, hl, kf, dtype, filt):
+    raw, wf, h, dy = make(bs, L, g, dg, hl, kf, dtype, filt)
+    rd, wd, hd, dyd = (t.to(DEV) for t in (raw, wf, h, dy))
+    y = _lib.mixer_mr_fwd(rd, wd, hd)
+    draw, dwf, dh = _lib.mixer_mr_bwd(dyd, rd, wd, hd)
+    torch.cuda.synchronize()
+    assert y.shape == (bs, L, g, dg) and draw.shape == raw.shape and dwf.shape == wf.shape and dh.shape == h.shape
+    assert y.dtype == dtype and draw.dtype == dtype and dwf.dtype == dtype and dh.dtype == filt
+    # oracle twice: the featurizer is the gated oracle with both gates at one and one filter per feature channel
+    flat = raw.float().reshape(bs, L, 3 * g * dg, 1)
+    one = torch.ones_like(flat)
+    f = oracle.gcg_fwd_oracle(flat, one, one, wf.float()).to(dtype).float().reshape(bs, L, g, dg, 3)
+    C, B, x = f[..., 0], f[..., 1], f[..., 2]
+    tol = TOL[dtype] if filt == dtype else 1.1 * 2.0 ** -8
+    assert_close(y, oracle.gcg_fwd_oracle(x, B, C, h.float()), tol, "y")
+    dx, dB, dC, dh_ref = oracle.gcg_bwd_oracle(dy.float(), x, B, C, h.float())
+    assert_close(dh, dh_ref, TOL_DH[filt], "dh")
+    dfeat = torch.stack([dC, dB, dx], dim=-1).to(dtype).float().reshape(bs, L, 3 * g * dg, 1)
+    draw_ref, _, _, dwf_ref = oracle.gcg_bwd_oracle(dfeat, flat, one, one, wf.float())
+    assert_close(draw.reshape(flat.shape), draw_ref, TOL[dtype], "draw")
+    assert_close(dwf, dwf_ref, TOL_DH[dtype], "dwf")
+    # the two-call chain: same arithmetic on the same values
+    exact = dtype != torch.float16       # (f16: the featurizer's taps are summed in another grouping in the two kernels)
+    for a, b, n in zip((y, draw, dwf, dh), chain(rd, wd, hd, dyd), ("y", "draw", "dwf", "dh")):
+        if exact and n != "dh":
+            assert torch.equal(a, b), n
+        elif n == "dh":
+            assert_close(a, b, 1e-6 if filt == torch.float32 else TOL_DH[filt], n)     # other run lengths, other order of partial sums
+        else:
+            assert (a == b).float().mean().item() > 0.99 and torch.allclose(a.float(), b.float(), rtol=2e-3, atol=1e-3), n
+
+
+def test_refused_shapes(gcg_lib):
+    raw, wf, h, dy = (t.to(DEV) for t in make(1, 64, 2, 16, 64, 3, torch.bfloat16, torch.bfloat16))
+    with pytest.raises(RuntimeError, match="not supported"):
+        _lib.mixer_mr_fwd(raw, wf, h)                      # short filter: fewer slices than the fused kernels walk
+    raw, wf, h, dy = (t.to(DEV) for t in make(1, 64, 2, 16, 128, 4, torch.bfloat16, torch.bfloat16))
+    with pytest.raises(RuntimeError, match="not supported"):
+        _lib.mixer_mr_bwd(dy, raw, wf, h)                  # four featurizer taps
+    assert not _lib.mixer_mr_supported(16, 64, 3) and not _lib.mixer_mr_supported(16, 128, 4) and _lib.mixer_mr_supported(16, 128, 3)
+
+
+@pytest.mark.parametrize("act,cgcg", [(torch.bfloat16, "bfloat16"), (torch.float32, "float32"), (torch.bfloat16, "float32")])
+def test_hyena_mixer_keeps_no_featurized_tensor(gcg_lib, act, cgcg):
+    """HyenaMixer with a Hyena-MR operator: same output and gradients with and without the featurized tensor,
+    and the fused path runs three kernels (forward; backward; featurizer backward) plus its small reductions."""
+    from savanna_amd.operators.hyena import CgcgConfig, HyenaMROperator, HyenaMixer
+
+    torch.manual_seed(0)
+    bs, L, g, dg = 2, 384, 4, 16
+    op = HyenaMROperator(g * dg, g, 128, CgcgConfig(cgcg_dtype=cgcg), small_init=False, device=DEV)
+    mixer = HyenaMixer(op, 3, dtype=act, device=DEV)
+    feats = torch.randn(bs, L, 3 * g * dg, device=DEV).to(act).requires_grad_(True)
+    dz = (0.1 * torch.randn(bs, L, g * dg, device=DEV)).to(act)
+    params = [op.filter.h, mixer.hyena_proj_conv.short_conv_weight]
+
+    def run(fuse):
+        mixer.fuse_medium = fuse
+        feats.grad = None
+        for p in params:
+            p.grad = None
+        z = mixer(feats)
+        z.backward(dz)
+        return [z.detach(), feats.grad.clone()] + [p.grad.clone() for p in params]
+
+    want = run(False)
+    from torch.profiler import ProfilerActivity, profile
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        got = run(True)
+        torch.cuda.synchronize()
+    for a, b, n in zip(got, want, ("z", "dfeatures", "dw", "dwf")):
+        assert a.dtype == b.dtype, n
+        if n == "dw":
+            assert_close(a, b, 2e-5, n)
+        else:
+            assert torch.equal(a, b), n
+    big = [e.key for e in prof.key_averages() if "mfma_il" in e.key or "dwconv" in e.key]
+    assert len(big) == 3, big
