@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the gated chunked causal convolution on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--only] [--all] [--kernels]
 
 A step is one pass of the hot path over one batch of synthetic input that is already
 resident in HBM: forward, plus backward for the forward+backward workloads.  The default
@@ -384,6 +384,70 @@ def cpu_baseline(wl, budget_s=20.0):
     }
 
 
+# (label, layout, bs, L, g, dg, hl, tensor dtype, filter dtype) of the single-kernel table (--kernels)
+KERNEL_TABLE = (
+    ("mfma bf16 hl=128, 7B", "sep", 2, 8192, 256, 16, 128, torch.bfloat16, torch.bfloat16),
+    ("mfma interleaved bf16 hl=128, 7B", "il", 2, 8192, 256, 16, 128, torch.bfloat16, torch.bfloat16),
+    ("mfma fp32 hl=128, 7B", "sep", 2, 8192, 256, 16, 128, torch.float32, torch.float32),
+    ("mfma interleaved fp32 hl=128, 7B", "il", 2, 8192, 256, 16, 128, torch.float32, torch.float32),
+    ("mfma bf16 tensors + fp32 filter hl=128, 7B", "sep", 2, 8192, 256, 16, 128, torch.bfloat16, torch.float32),
+    ("mfma interleaved bf16 tensors + fp32 filter hl=128, 7B", "il", 2, 8192, 256, 16, 128, torch.bfloat16, torch.float32),
+    ("mfma bf16 hl=128, 40B", "sep", 1, 32768, 512, 16, 128, torch.bfloat16, torch.bfloat16),
+    ("window bf16 hl=7, 40B", "sep", 1, 32768, 512, 16, 7, torch.bfloat16, torch.bfloat16),
+    ("window interleaved bf16 hl=7, 40B", "il", 1, 32768, 512, 16, 7, torch.bfloat16, torch.bfloat16),
+    ("window bf16 hl=7, 7B", "sep", 2, 8192, 256, 16, 7, torch.bfloat16, torch.bfloat16),
+    ("window fp32 hl=7, 7B", "sep", 2, 8192, 256, 16, 7, torch.float32, torch.float32),
+    ("window interleaved fp32 hl=7, 7B", "il", 2, 8192, 256, 16, 7, torch.float32, torch.float32),
+)
+
+
+def kernel_table(device, n=30, nsets=4):
+    """Forward and backward kernel of the gated entry points alone: each launch between two HIP events that the
+    runtime stamps at its start and end (gcg_time_next_kernel), inputs rotated over `nsets` sets, mean of n."""
+    rows = []
+    for label, layout, bs, L, g, dg, hl, dt, fdt in KERNEL_TABLE:
+        gen = torch.Generator(device=device).manual_seed(1)
+        sets = []
+        for _ in range(nsets):
+            feat = torch.randn(bs, L, g, dg, 3, generator=gen, device=device).to(dt)
+            dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen, device=device)).to(dt)
+            h = (torch.randn(g, 1, hl, generator=gen, device=device) / hl ** 0.5).to(fdt)
+            if layout == "sep":
+                C, B, x = (feat[..., j].contiguous() for j in range(3))
+                sets.append((x, B, C, dy, h))
+            else:
+                sets.append((feat, dy, h))
+        if layout == "sep":
+            fwd = lambda s: _lib.fwd(s[0], s[1], s[2], s[4])                    # noqa: E731
+            bwd = lambda s: _lib.bwd(s[3], s[0], s[1], s[2], s[4])              # noqa: E731
+        else:
+            fwd = lambda s: _lib.fwd_interleaved(s[0], s[2])                    # noqa: E731
+            bwd = lambda s: _lib.bwd_interleaved(s[1], s[0], s[2])              # noqa: E731
+        t0 = time.perf_counter()
+        i = 0
+        while i < 8 or time.perf_counter() - t0 < SETTLE_S:
+            fwd(sets[i % nsets]), bwd(sets[i % nsets])
+            torch.cuda.synchronize()
+            i += 1
+        kf, kb = KernelEvents(n), KernelEvents(n)
+        for i in range(n):
+            s = sets[i % nsets]
+            _lib.time_next_kernel(*kf.pairs[i])
+            fwd(s)
+            _lib.time_next_kernel(*kb.pairs[i])
+            bwd(s)
+        torch.cuda.synchronize()
+        fms, bms = kf.mean_ms(), kb.mean_ms()
+        kf.close(), kb.close()
+        nbytes = bs * L * g * dg * dy.element_size()
+        rows.append({"kernel": label, "shape": [bs, L, g, dg], "hl": hl,
+                     "fwd_us": fms * 1e3, "fwd_gbs": 4 * nbytes / fms / 1e6, "fwd_hbm_frac": 4 * nbytes / fms / 1e6 / HBM_PEAK_GBS,
+                     "bwd_us": bms * 1e3, "bwd_gbs": 7 * nbytes / bms / 1e6, "bwd_hbm_frac": 7 * nbytes / bms / 1e6 / HBM_PEAK_GBS})
+        del sets
+        torch.cuda.empty_cache()
+    return rows
+
+
 def main():
     global KEEP_INTERMEDIATES, SETTLE_S
     ap = argparse.ArgumentParser()
@@ -401,6 +465,9 @@ def main():
                     help="also time the step replayed from a captured HIP graph (launch-bound shapes)")
     ap.add_argument("--settle", type=float, default=SETTLE_S,
                     help="seconds of untimed steps before the warm-up steps, so that clocks have settled (0: none)")
+    ap.add_argument("--kernels", action="store_true",
+                    help="print the single-kernel table instead (forward and backward kernel of the gated entry "
+                         "points alone at the 7B and 40B layer shapes, one JSON line) and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, so a counter profile of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -417,6 +484,11 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     _lib.load()
+
+    if args.kernels:
+        print(json.dumps({"single_kernels": kernel_table(device, n=max(10, args.steps)), "unit": "us, GB/s of algorithmic "
+                          "bytes (4 tensors forward, 7 backward), fraction of 8 TB/s"}), flush=True)
+        return
 
     wl = WORKLOADS[args.workload]
     res = time_workload(wl, device, args.steps, args.warmup, graph=args.graph)
