@@ -292,10 +292,15 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
  * in 10^5 by one unit in the last place).
  *   raw  (bs, L, g, dg, 3)   wf  (3 * g * dg, 1, kf), tensors' type   h  (g, 1, hl)   y  out, (bs, L, g, dg)
  * Forward: reads raw, writes y -- 4 N s of memory traffic instead of 10 N s.
- * Backward: one kernel recomputes the features from raw and writes their gradient into dfeat_scratch
- * ((bs, L, g, dg, 3), caller's memory, contents on return unspecified), then the featurizer's own backward
- * turns it into draw and dwf: the traffic of the two-call chain (16 N s), but nothing of size 3 N is kept
- * between forward and backward.
+ * Backward, 16-bit tensors with arithmetic in their own type: one kernel goes from dy and raw to draw, dwf and dh --
+ * the features are made again from raw, their gradient is handed from the operator's part to the featurizer's
+ * part inside the workgroup and never stored: 7 N s of memory traffic (dy and raw in, draw out) instead of the two-call
+ * chain's 16 N s.  draw and dh are the chain's bit for bit (bf16), dwf up to the order in which partial sums are added.
+ * Other types (fp32 arithmetic): one kernel recomputes the features and writes their gradient into dfeat_scratch
+ * ((bs, L, g, dg, 3), caller's memory, contents on return unspecified), then the featurizer's own backward turns
+ * it into draw and dwf -- the chain's traffic, but nothing of size 3 N is kept between forward and backward.
+ * gcg_mixer_mr_bwd_scratch_bytes(...) says how large dfeat_scratch has to be: 0 (it may then be NULL) where the
+ * one-kernel backward runs, the size of raw otherwise.
  *   draw  out, (bs, L, g, dg, 3)   dwf  out, (3 * g * dg, 1, kf)   dh  out, (g, 1, hl), filter's type
  *   workspace  gcg_mixer_mr_bwd_workspace_bytes(...) bytes, 256-byte aligned
  * Matrix-core kernels with full-length filters only: 98 <= hl <= 128, dg % 16 == 0, kf <= 3, 16-byte aligned
@@ -305,6 +310,8 @@ GCG_API int gcg_mixer_mr_fwd(const void *raw, const void *wf, const void *h, voi
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
             int32_t dtype, void *stream);
 GCG_API size_t gcg_mixer_mr_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t kf, int32_t dtype);
+GCG_API size_t gcg_mixer_mr_bwd_scratch_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
             int32_t kf, int32_t dtype);
 GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, const void *h,
             void *draw, void *dwf, void *dh, void *dfeat_scratch,

@@ -35,7 +35,7 @@ EXPORTS = (
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
-    "gcg_mixer_mr_fwd", "gcg_mixer_mr_bwd_workspace_bytes", "gcg_mixer_mr_bwd", "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
+    "gcg_mixer_mr_fwd", "gcg_mixer_mr_bwd_workspace_bytes", "gcg_mixer_mr_bwd_scratch_bytes", "gcg_mixer_mr_bwd", "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
     "gcg_fwd_decay", "gcg_bwd_decay", "gcg_fwd_interleaved_decay", "gcg_bwd_interleaved_decay",
 )
 
@@ -104,6 +104,8 @@ def load() -> ctypes.CDLL:
         lib.gcg_mixer_mr_fwd.restype = ctypes.c_int
         lib.gcg_mixer_mr_bwd_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32, i32]
         lib.gcg_mixer_mr_bwd_workspace_bytes.restype = sz
+        lib.gcg_mixer_mr_bwd_scratch_bytes.argtypes = [i64, i64, i32, i32, i32, i32, i32]
+        lib.gcg_mixer_mr_bwd_scratch_bytes.restype = sz
         lib.gcg_mixer_mr_bwd.argtypes = [vp] * 9 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_mixer_mr_bwd.restype = ctypes.c_int
         lib.gcg_fwd_time_major.argtypes = [vp] * 5 + [i64, i64, i32, i32, i32, i32, vp]
@@ -540,8 +542,8 @@ def mixer_mr_fwd(raw, wf, h):
 
 
 def mixer_mr_bwd(dy, raw, wf, h):
-    """(draw, dwf, dh) of mixer_mr_fwd from the projection output alone: the features are recomputed, their
-    gradient lives in a scratch tensor for the duration of the call."""
+    """(draw, dwf, dh) of mixer_mr_fwd from the projection output alone: the features are recomputed; their
+    gradient stays inside the kernel (16-bit arithmetic) or lives in a scratch tensor for the duration of the call."""
     _require_gpu(raw)
     if TORCH_OPS:
         return torch.ops.gcg.mixer_mr_bwd(dy, raw, wf, h)
@@ -558,9 +560,11 @@ def mixer_mr_bwd(dy, raw, wf, h):
         check(-2, "gcg_mixer_mr_bwd_workspace_bytes")
     with _on_device(raw.device):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
-        scratch = torch.empty_like(raw)
+        sbytes = lib.gcg_mixer_mr_bwd_scratch_bytes(bs, L, g, dg, hl, kf, code)
+        scratch = torch.empty(sbytes, dtype=torch.uint8, device=raw.device)
         rc = lib.gcg_mixer_mr_bwd(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
-                                  dwf.data_ptr(), dh.data_ptr(), scratch.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg,
+                                  dwf.data_ptr(), dh.data_ptr(), scratch.data_ptr() if sbytes else None, ws.data_ptr(),
+                                  nbytes, bs, L, g, dg,
                                   hl, kf, code, torch.cuda.current_stream().cuda_stream)
     check(rc, "gcg_mixer_mr_bwd")
     return draw, dwf, dh

@@ -562,7 +562,18 @@ GCG_API size_t gcg_mixer_mr_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g
     if (kf <= 0 || make_dims(bs, L, g, dg, hl, dtype, &dm, true)) return 0;
     if (!gcg::mfma_feat_supported(dtype, dm, kf)) return 0;
     if (make_dims(bs, L, 3 * g * dg, 1, kf, plain_tensor_code(dtype), &df) || !gcg::dwconv_supported(df)) return 0;
-    return up256(gcg::mfma_feat_bwd_workspace(dtype, dm)) + up256(gcg::dwconv_bwd_workspace(df));
+    const size_t chain = up256(gcg::mfma_feat_bwd_workspace(dtype, dm)) + up256(gcg::dwconv_bwd_workspace(df));
+    const size_t fused = gcg::mixer_mr_fused_supported(dtype, dm, kf) ? up256(gcg::mixer_mr_fused_workspace(dm, kf)) : 0;
+    return chain > fused ? chain : fused;
+}
+
+GCG_API size_t gcg_mixer_mr_bwd_scratch_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+                                              int32_t dtype)
+{
+    gcg::Dims dm;
+    if (kf <= 0 || make_dims(bs, L, g, dg, hl, dtype, &dm, true)) return 0;
+    if (gcg::mixer_mr_fused_supported(dtype, dm, kf)) return 0;
+    return (size_t)(3 * bs * L * dm.d) * (dtype == GCG_F32 ? 4 : 2);
 }
 
 GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf,
@@ -570,13 +581,17 @@ GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, co
                              int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
 {
     TimerScope timer_scope;
-    if (!dy || !raw || !wf || !h || !draw || !dwf || !dh || !dfeat_scratch || kf <= 0) return GCG_ERR_BAD_ARG;
+    if (!dy || !raw || !wf || !h || !draw || !dwf || !dh || kf <= 0) return GCG_ERR_BAD_ARG;
     gcg::Dims dm, df;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     dm.es = 3;
     dm.keep_out = 1;
-    if (!all_aligned16({dy, raw, draw, dfeat_scratch}) || !gcg::mfma_feat_supported(dtype, dm, kf)) return GCG_ERR_UNSUPPORTED;
+    const bool fused = gcg::mixer_mr_fused_supported(dtype, dm, kf);
+    if (!fused && !dfeat_scratch) return GCG_ERR_BAD_ARG;
+    if (!all_aligned16({dy, raw, draw}) || (!fused && !all_aligned16({dfeat_scratch})) ||
+        !gcg::mfma_feat_supported(dtype, dm, kf))
+        return GCG_ERR_UNSUPPORTED;
     rc = make_dims(bs, L, 3 * g * dg, 1, kf, plain_tensor_code(dtype), &df);
     if (rc) return rc;
     if (!gcg::dwconv_supported(df)) return GCG_ERR_UNSUPPORTED;
@@ -585,6 +600,8 @@ GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, co
     rc = check_device();
     if (rc) return rc;
     hipStream_t st = (hipStream_t)stream;
+    if (fused)
+        return finish(gcg::mixer_mr_fused_bwd_launch(dtype, dy, raw, wf, kf, h, draw, dwf, dh, workspace, dm, st));
     void *ws2 = (char *)workspace + up256(gcg::mfma_feat_bwd_workspace(dtype, dm));
     int e = gcg::mfma_il_bwd_feat_launch(dtype, dy, raw, wf, kf, h, dfeat_scratch, dh, workspace, dm, st);
     if (e) return finish(e);

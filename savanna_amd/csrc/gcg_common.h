@@ -302,6 +302,12 @@ int mfma_il_fwd_feat_launch(int dtype, const void *raw, const void *wfeat, int k
 int mfma_il_bwd_feat_launch(int dtype, const void *dy, const void *raw, const void *wfeat, int kf, const void *h,
                             void *dfeat, void *dh, void *ws, const Dims &dm, hipStream_t st);
 
+// the whole backward of featurizer -> Hyena-MR operator in one kernel (no gradient of the features in memory)
+bool mixer_mr_fused_supported(int dtype, const Dims &dm, int kf);
+size_t mixer_mr_fused_workspace(const Dims &dm, int kf);
+int mixer_mr_fused_bwd_launch(int dtype, const void *dy, const void *raw, const void *wfeat, int kf, const void *h,
+                              void *draw, void *dwf, void *dh, void *ws, const Dims &dm, hipStream_t st);
+
 // ungated short causal depthwise convolution (the featurizer), (bs, L, g, dg) channel-fastest
 bool dwconv_supported(const Dims &dm);
 int dwconv_fwd_launch(int dtype, const void *x, const void *w, void *y, const Dims &dm, hipStream_t st);

@@ -546,9 +546,12 @@ std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd(const Tensor &dy, const Tensor &
     const int code = gated_code(raw, h);
     const size_t nbytes = gcg_mixer_mr_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code);
     Tensor ws = workspace(nbytes, raw, "gcg_mixer_mr_bwd_workspace_bytes");
-    Tensor scratch = at::empty_like(raw);      // gradient of the featurized features, for the duration of the call
+    // gradient of the featurized features, for the duration of the call (not needed where one kernel does it all)
+    const size_t sbytes = gcg_mixer_mr_bwd_scratch_bytes(bs, L, g, dg, hl, kf, code);
+    Tensor scratch = at::empty({(int64_t)sbytes}, raw.options().dtype(at::kByte));
     check_rc(gcg_mixer_mr_bwd(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
-                              dwf.data_ptr(), dh.data_ptr(), scratch.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl,
+                              dwf.data_ptr(), dh.data_ptr(), scratch.numel() ? scratch.data_ptr() : nullptr,
+                              ws.data_ptr(), nbytes, bs, L, g, dg, hl,
                               kf, code, stream_of(raw)),
              "gcg_mixer_mr_bwd");
     return {draw, dwf, dh};

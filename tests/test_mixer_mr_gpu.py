@@ -21,6 +21,8 @@ SHAPES = [
     (1, 2049, 20, 16, 98, 3),
     (2, 40, 2, 32, 128, 1),       # one tap: the featurizer scales its channels
     (1, 700, 17, 16, 128, 3),     # d = 272
+    (1, 3000, 3, 64, 128, 3),     # a filter group as wide as a workgroup's channel block
+    (2, 4100, 8, 16, 128, 3),     # runs of more than a hundred steps
 ]
 TYPES = [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.float32, torch.float32),
          (torch.bfloat16, torch.float32)]
@@ -75,8 +77,11 @@ def test_against_oracle_and_chain(gcg_lib, bs, L, g, dg, hl, kf, dtype, filt):
     assert_close(dwf, dwf_ref, TOL_DH[dtype], "dwf")
     # the two-call chain: same arithmetic on the same values
     exact = dtype != torch.float16       # (f16: the featurizer's taps are summed in another grouping in the two kernels)
+    one_kernel = filt == dtype and dtype != torch.float32      # the backward that never stores the gradient of the features
     for a, b, n in zip((y, draw, dwf, dh), chain(rd, wd, hd, dyd), ("y", "draw", "dwf", "dh")):
-        if exact and n != "dh":
+        if n == "dwf" and one_kernel:
+            assert_close(a, b, TOL_DH[dtype], n)                # its partial sums are taken over other pieces of the rows
+        elif exact and n != "dh":
             assert torch.equal(a, b), n
         elif n == "dh":
             assert_close(a, b, 1e-6 if filt == torch.float32 else TOL_DH[filt], n)     # other run lengths, other order of partial sums
@@ -97,7 +102,8 @@ def test_refused_shapes(gcg_lib):
 @pytest.mark.parametrize("act,cgcg", [(torch.bfloat16, "bfloat16"), (torch.float32, "float32"), (torch.bfloat16, "float32")])
 def test_hyena_mixer_keeps_no_featurized_tensor(gcg_lib, act, cgcg):
     """HyenaMixer with a Hyena-MR operator: same output and gradients with and without the featurized tensor,
-    and the fused path runs three kernels (forward; backward; featurizer backward) plus its small reductions."""
+    and the fused path runs two large kernels (16-bit arithmetic; three with fp32 arithmetic, where the featurizer's
+    backward is a kernel of its own) plus its small reductions."""
     from savanna_amd.operators.hyena import CgcgConfig, HyenaMROperator, HyenaMixer
 
     torch.manual_seed(0)
@@ -126,7 +132,9 @@ def test_hyena_mixer_keeps_no_featurized_tensor(gcg_lib, act, cgcg):
         assert a.dtype == b.dtype, n
         if n == "dw":
             assert_close(a, b, 2e-5, n)
+        elif n == "dwf" and cgcg == "bfloat16":
+            assert_close(a, b, TOL_DH[act], n)
         else:
             assert torch.equal(a, b), n
-    big = [e.key for e in prof.key_averages() if "mfma_il" in e.key or "dwconv" in e.key]
-    assert len(big) == 3, big
+    big = [e.key for e in prof.key_averages() if "mfma_il" in e.key or "dwconv" in e.key or "mixer_mr" in e.key]
+    assert len(big) == (2 if cgcg == "bfloat16" else 3), big
