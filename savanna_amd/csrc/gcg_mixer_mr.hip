@@ -4,27 +4,30 @@
 // features is rounded like the operator's backward would have stored it and handed on through LDS to the
 // featurizer's backward.  Per element the kernel moves 7 values (dy and 3 of raw in, 3 of d raw out).
 //
-// All of that is vector arithmetic on row pieces; the banded-Toeplitz products are a small part.  A workgroup
-// therefore splits its eight waves by role, one wave of each kind per SIMD:
+// Nearly all of that is vector arithmetic on row pieces, and a SIMD issues one vector or matrix instruction at a
+// time, so the instruction count is what bounds the kernel.  A workgroup splits its eight waves by role, one wave
+// of each kind per SIMD, so that neither kind holds the other's registers (Toeplitz tiles, operand rings and
+// filter-gradient tiles on one side; rows in flight, taps, queues and accumulators on the other) and both fit
+// two waves per SIMD:
 //   memory waves (0..3)  own the rows: a lane holds 4 consecutive time rows of 2 channels -- one 12-byte piece
 //                        (C0 B0 | x0 C1 | B1 x1) per row, 384 contiguous bytes per row across 32 lanes -- loads
-//                        them, makes features, products and gradients, and stores d raw;
-//   matrix waves (4..7)  own 16 channels each: operand tiles from LDS, the products y2 = T u, du = T' g2 and the
-//                        filter-gradient tiles, results back to LDS.
-// Neither kind holds the other's registers (Toeplitz tiles, operand rings and gradient tiles on one side; rows
-// in flight, taps, queues and accumulators on the other), so both fit two waves per SIMD.
+//                        them, makes features, operands and the gradient of the features, and accumulates d wf;
+//   matrix waves (4..7)  own 16 channels each for the products y2 = T u, du = T' g2 and the filter-gradient tiles
+//                        (operands from LDS, results to LDS), and in the row layout turn the gradient of the
+//                        features into d raw and store it.
 //
-// Step k of a run (32 rows x 64 channels) between its two barriers:
-//   before the first   memory: gradient of the features of step k-1 from y2, du (LDS) -> LDS slot, d wf
-//                              accumulation; x, B of step k from the raw ring -> u(k); g2(k+4) -> ring
-//   between            matrix: operands of u(k), g2(k+4), 20 products -> y2(k), du(k), 9 filter-gradient products
-//                      memory: d raw of step k-1 from the gradient slot (rows two back, which need the two rows
-//                              after them) -> memory; rows of step k+5 arrive -> raw ring, C and g2 of that step;
-//                              rows of step k+6 requested
-// The raw rows wait in an LDS ring (6 steps) from their arrival, 5 steps ahead for the anti-causal product, to
-// the step after their own, where d wf needs them again; dy waits in registers.  A run goes one step beyond its
-// end (products only, nothing accumulated) because its last two rows of d raw need the first two gradient rows
-// of the next run.
+// Step k of a run (32 rows x 64 channels) has two barriers:
+//   before the first   memory: gradient of the features of step k-1 from y2, du (LDS) -> LDS; x, B of step k from
+//                              the raw ring -> u(k); g2(k+4) -> ring
+//                      matrix: d raw of step k-2 from the gradient rows in LDS (its rows two back, which need the
+//                              two rows after them) -> memory
+//   between the two    matrix: operands of u(k), g2(k+4), 20 products -> y2(k), du(k), 9 filter-gradient products
+//                      memory: rows of step k+5 arrive -> C and g2 of that step, raw ring; rows of step k+7
+//                              requested; d wf of step k-1
+// The raw rows wait in an LDS ring (7 steps) from their arrival, 5 steps ahead for the anti-causal product, to
+// the step after their own, where d wf needs them again; dy waits in registers; the gradient rows of two steps
+// are in LDS at a time.  A run goes one step beyond its end (products only, nothing accumulated) because its last
+// two rows of d raw need the first two gradient rows of the next run.
 #include "gcg_il_tile.h"
 #include "gcg_rowvec.h"
 
@@ -41,7 +44,7 @@ template <typename T> struct MixGeo {
     static constexpr int XW = 4, MW = 4, NT = 64 * (XW + MW);
     static constexpr int NK = 5, ND = 2 * NK - 1;
     static constexpr int CB = 16 * XW;                          // channels per workgroup
-    static constexpr int UROW = M::urow(CB), YROW = CB * 4 + 16;
+    static constexpr int UROW = CB * 2 + 16, YROW = CB * 4 + 16;    // LDS rows of u / g2 and of y2 / du (padded)
     static constexpr int LPR = CB / 2;                          // row lanes per row
     static constexpr int NR = 4, NG = STEP / NR;                // rows per lane, row groups
     static constexpr int NH = MR_KF - 1;                        // rows before a lane's own that its features need
@@ -55,8 +58,9 @@ template <typename T> struct MixGeo {
     static constexpr int OFF_Y = OFF_G + NK * STEP * UROW;
     static constexpr int OFF_D = OFF_Y + STEP * YROW;
     static constexpr int OFF_RAW = OFF_D + STEP * YROW;
-    static constexpr int OFF_DF = OFF_RAW + RAW_SLOTS * SLOT;   // gradient rows of one step, and two sets of the NH rows before
-    static constexpr int LDS_BYTES = OFF_DF + PRE + 2 * PRE_BYTES;
+    static constexpr int OFF_DF = OFF_RAW + RAW_SLOTS * SLOT;   // gradient rows of two steps, then three sets of a step's last NH rows
+    static constexpr int OFF_DFP = OFF_DF + 2 * PRE;
+    static constexpr int LDS_BYTES = OFF_DFP + 3 * PRE_BYTES;
     static constexpr int OFF_H = OFF_DF;                        // filter tables: read before the first gradient rows are written
     static constexpr int OFF_P = OFF_RAW;                       // tail: gradient tiles, then the d wf accumulators
     static constexpr int OFF_W = OFF_P + XW * ND * 1024;
@@ -133,6 +137,35 @@ template <typename T> __device__ __forceinline__ u32x3 values_piece(const float 
 {
     return u32x3{MT<T>::pack2(v[0], v[1]), MT<T>::pack2(v[2], v[3]), MT<T>::pack2(v[4], v[5])};
 }
+// a.lo * b.lo + a.hi * b.hi + c on packed 16-bit pairs (the sum may differ from two fused multiply-adds in the
+// last place of fp32: used where partial sums are added in another order anyway)
+template <typename T> __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c);
+template <> __device__ __forceinline__ float dot2<bf16_t>(uint32_t a, uint32_t b, float c)
+{
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    return __builtin_amdgcn_fdot2_f32_bf16(x, y, c, false);
+}
+template <> __device__ __forceinline__ float dot2<f16_t>(uint32_t a, uint32_t b, float c)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    h2 x, y;
+    __builtin_memcpy(&x, &a, 4);
+    __builtin_memcpy(&y, &b, 4);
+    return __builtin_amdgcn_fdot2(x, y, c, false);
+}
+// the low (high) halves of two dwords as one pair: first dword's in the low half
+__device__ __forceinline__ uint32_t pair_lo(uint32_t first, uint32_t second)
+{
+    return __builtin_amdgcn_perm(second, first, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t pair_hi(uint32_t first, uint32_t second)
+{
+    return __builtin_amdgcn_perm(second, first, 0x07060302u);
+}
+
 // one feature value: the featurizer kernel's order of summation (oldest sample first, fp32)
 __device__ __forceinline__ float feat_sum(const float (&tap)[MR_KF][6], const float (&rv)[MR_KF - 1 + 4][6], int k, int v)
 {
@@ -222,12 +255,13 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
         for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
         unsigned char *y_wr = y_st + j * YROW + (16 * xw + 4 * q) * 4;
         unsigned char *d_wr = d_st + (15 - j) * YROW + (16 * xw + 4 * q) * 4;      // columns come out reversed
-        // d raw
+        // d raw, from the gradient rows the memory waves leave in LDS, two steps behind the products
         const win_t wdr = make_window(draw + 3 * (b * L + T0) * d, 3 * (T1 - T0) * row_bytes);
-        uint32_t dr_b = 3u * step_base(s_lo, T0);      // of step k-1
+        uint32_t dr_b = 3u * step_base(s_lo, T0);      // of step k-2
         const unsigned char *df_own = df_rg + own_off;
-        const unsigned char *df_halo = df_rg + (rr ? halo_off : G::PRE + a * 24);
-        int pre = 0;                                    // which set of "rows before" step k-1 reads (row group 0 only)
+        const unsigned char *df_halo = rr ? df_rg + halo_off : smem + G::OFF_DFP + a * 24;
+        int dfb = 0;                                    // which of the two sets of gradient rows step k-2 lies in
+        int dfp = 2 * G::PRE_BYTES;                     // where the NH rows before step k-2 lie (row group 0 only)
         u32x3 dro[NR];                                  // the rows of d raw stored last
 #pragma unroll
         for (int r = 0; r < NR; ++r) dro[r] = u32x3{0u, 0u, 0u};
@@ -235,12 +269,41 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
         // While step k runs in phase ph:  Au[(ph - i + NK) % NK] is the u operand of step k-i,
         // Ag[(ph + i) % NK] the time-reversed g2 operand of step k+i (ring slot (ph + i) % NK).
         int64_t k = k_first;
-        while (k <= s_end) {
+        while (k <= s_end + 1) {
 #pragma unroll
             for (int ph = 0; ph < NK; ++ph) {
-                if (k <= s_end) {
+                if (k <= s_end + 1) {
+                    if (k - 2 >= s_lo) {
+                        // d raw of rows NR*rr-NH .. NR*rr+NR-NH-1 of step k-2: each needs the gradient rows from its own on
+                        u32x3 pg[NH + NR];
+                        halo_pieces(lds_load_halo(df_halo + (rr ? dfb : dfp)), pg);
+                        blk_pieces(lds_load_blk(df_own + dfb), pg + NH);
+                        float gv[NH + NR][NV];
+#pragma unroll
+                        for (int i = 0; i < NH + NR; ++i) piece_values<T>(pg[i], gv[i]);
+                        // The stored rows keep registers of their own until here, one step later: a register that is
+                        // written again while its store is still on the way makes the wave wait for that store.
+#pragma unroll
+                        for (int i = 0; i < NR; ++i) asm volatile("" ::"v"(dro[i][0]), "v"(dro[i][1]), "v"(dro[i][2]));
+#pragma unroll
+                        for (int i = 0; i < NR; ++i) {
+                            float o[NV];
+#pragma unroll
+                            for (int v = 0; v < NV; ++v) {
+                                float acc = 0.f;             // the featurizer backward's order: nearest row first
+#pragma unroll
+                                for (int m = KF - 1; m >= 0; --m) acc = fmaf(tap[m][v], gv[i + KF - 1 - m][v], acc);
+                                o[v] = acc;
+                            }
+                            dro[i] = values_piece<T>(o);
+                        }
+#pragma unroll
+                        for (int i = 0; i < NR; ++i) stw12(wdr, lane_raw + dr_b + 3u * (uint32_t)i * rb, dro[i]);
+                        dr_b += 3u * step_b;
+                        dfb ^= G::PRE;
+                        dfp = dfp == 2 * G::PRE_BYTES ? 0 : dfp + G::PRE_BYTES;
+                    }
                     __syncthreads();
-                    const bool have_prev = k > s_lo;          // the gradient rows of step k-1 lie in LDS
                     if (k < s_end) {
                         const int slot_new = (ph + NK - 1) % NK;
                         Au[ph] = M::load_operand(u_rm, UROW, xw, j, q, false);
@@ -273,35 +336,6 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
                                 }
                             }
                         }
-                    }
-                    if (have_prev) {
-                        // d raw of rows NR*rr-NH .. NR*rr+NR-NH-1 of step k-1: each needs the gradient rows from its own on
-                        u32x3 pg[NH + NR];
-                        halo_pieces(lds_load_halo(df_halo + (rr ? 0 : pre)), pg);
-                        blk_pieces(lds_load_blk(df_own), pg + NH);
-                        float gv[NH + NR][NV];
-#pragma unroll
-                        for (int i = 0; i < NH + NR; ++i) piece_values<T>(pg[i], gv[i]);
-                        // The stored rows keep registers of their own until here, one step later: a register that is
-                        // written again while its store is still on the way makes the wave wait for that store.
-#pragma unroll
-                        for (int i = 0; i < NR; ++i) asm volatile("" ::"v"(dro[i][0]), "v"(dro[i][1]), "v"(dro[i][2]));
-#pragma unroll
-                        for (int i = 0; i < NR; ++i) {
-                            float o[NV];
-#pragma unroll
-                            for (int v = 0; v < NV; ++v) {
-                                float acc = 0.f;             // the featurizer backward's order: nearest row first
-#pragma unroll
-                                for (int m = KF - 1; m >= 0; --m) acc = fmaf(tap[m][v], gv[i + KF - 1 - m][v], acc);
-                                o[v] = acc;
-                            }
-                            dro[i] = values_piece<T>(o);
-                        }
-#pragma unroll
-                        for (int i = 0; i < NR; ++i) stw12(wdr, lane_raw + dr_b + 3u * (uint32_t)i * rb, dro[i]);
-                        dr_b += 3u * step_b;
-                        pre ^= G::PRE_BYTES;
                     }
                     __syncthreads();
                     ++k;
@@ -346,7 +380,7 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
     const unsigned char *y_rd = y_st + NR * rr * YROW + 8 * a;
     const unsigned char *d_rd = d_st + NR * rr * YROW + 8 * a;
     unsigned char *raw_own = raw_rg + own_off, *raw_halo = raw_rg + halo_off;
-    unsigned char *df_own = df_rg + own_off, *df_pre = df_rg + G::PRE + a * 24;
+    unsigned char *df_own = df_rg + own_off, *df_last = smem + G::OFF_DFP + a * 24;
 
     // rows of a step: the NH rows before the lane's own, its NR rows, and dy of those
     struct Rows { u32x3 p[NH + NR]; uint32_t dy[NR]; };
@@ -424,11 +458,12 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
     int rs = 0;                       // byte offset of the raw ring slot of step k
     int ra = NK * G::SLOT;            // ... of step k+NK, which arrives during step k (two slots behind step k)
     int gs = (NK - 1) * STEP * UROW;  // byte offset of the g2 ring slot of step k+NK-1
-    int pre = G::PRE_BYTES;           // which set of "rows before" the last row group writes for the step after k-1
+    int dfb = 0;                      // which of the two sets of gradient rows step k-1 goes into
+    int dfp = 0;                      // where the last row group leaves its last NH rows of step k-1 for the step after
 
     // One step.  PREV: step k-1 has products (gradient of its features); DWF: it also counts for d wf (it lies
-    // inside the run); MAKE: step k gets its u and step k+NK-1 its g2.  The three variants are separate
-    // straight-line bodies, so that within each the LDS reads can all be requested before the first use.
+    // inside the run); MAKE: step k gets its u and step k+NK-1 its g2.  The variants are separate straight-line
+    // bodies, so that within each the LDS reads can all be requested before the first use.
     auto iter = [&](auto prev_c, auto dwf_c, auto make_c, Rows &in) {
         constexpr bool PREV = decltype(prev_c)::value, DWF = decltype(dwf_c)::value, MAKE = decltype(make_c)::value;
         const int rs_prev = rs ? rs - G::SLOT : RING_END;
@@ -457,9 +492,10 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
                 o[3] = dv[1] * y2v[i].y; o[4] = duv[i].y * xv[1]; o[5] = duv[i].y * Bv[1];
                 po[i] = values_piece<T>(o);
             }
-            lds_store_blk(df_own, pieces_blk(po));
-            if (rr == G::NG - 1) lds_store_halo(df_pre + pre, pieces_halo(po + NR - NH));
-            pre ^= G::PRE_BYTES;
+            lds_store_blk(df_own + dfb, pieces_blk(po));
+            if (rr == G::NG - 1) lds_store_halo(df_last + dfp, pieces_halo(po + NR - NH));
+            dfb ^= G::PRE;
+            dfp = dfp == 2 * G::PRE_BYTES ? 0 : dfp + G::PRE_BYTES;
         }
         if constexpr (MAKE) {
             // x, B of step k -> u; g2 of step k+NK-1 -> ring
@@ -489,22 +525,32 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
         raw_b += step_b;
         dy_b += step_b;
         if constexpr (DWF) {
-            // d wf: each gradient row of step k-1 with the raw rows its feature was made of
+            // d wf: each gradient row of step k-1 with the raw rows its feature was made of, two rows per product:
+            // value v of rows (i, i+1) of the gradient with value v of rows (i+m, i+m+1)
             u32x3 prp[NH + NR];
             halo_pieces(lds_load_halo(raw_halo + rs_prev), prp);
             blk_pieces(lds_load_blk(raw_own + rs_prev), prp + NH);
-            float rv[NH + NR][NV];
+            uint32_t rp[NH + NR - 1][NV], gp[NR / 2][NV];
 #pragma unroll
-            for (int i = 0; i < NH + NR; ++i) piece_values<T>(prp[i], rv[i]);
+            for (int i = 0; i < NH + NR - 1; ++i)
 #pragma unroll
-            for (int i = 0; i < NR; ++i) {
-                float gv[NV];
-                piece_values<T>(po[i], gv);
+                for (int c = 0; c < 3; ++c) {
+                    rp[i][2 * c] = pair_lo(prp[i][c], prp[i + 1][c]);
+                    rp[i][2 * c + 1] = pair_hi(prp[i][c], prp[i + 1][c]);
+                }
+#pragma unroll
+            for (int i = 0; i < NR / 2; ++i)
+#pragma unroll
+                for (int c = 0; c < 3; ++c) {
+                    gp[i][2 * c] = pair_lo(po[2 * i][c], po[2 * i + 1][c]);
+                    gp[i][2 * c + 1] = pair_hi(po[2 * i][c], po[2 * i + 1][c]);
+                }
+#pragma unroll
+            for (int i = 0; i < NR / 2; ++i)
 #pragma unroll
                 for (int m = 0; m < KF; ++m)
 #pragma unroll
-                    for (int v = 0; v < NV; ++v) dwa[m][v] = fmaf(gv[v], rv[i + m][v], dwa[m][v]);
-            }
+                    for (int v = 0; v < NV; ++v) dwa[m][v] = dot2<T>(gp[i][v], rp[2 * i + m][v], dwa[m][v]);
         }
         rs = rs == RING_END ? 0 : rs + G::SLOT;
         ra = ra == RING_END ? 0 : ra + G::SLOT;
@@ -533,11 +579,12 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
             iter(yes, yes, yes, in0);
             odd = true;
         }
-        if (odd) iter(yes, no, no, in1);                    // the step beyond the run gives its gradient rows
+        if (odd) iter(yes, no, no, in1);                        // the step beyond the run gives its gradient rows
         else iter(yes, no, no, in0);
+        __syncthreads();                                    // one more step of the matrix waves: d raw lags two steps
+        __syncthreads();
     }
-
-    // d wf: the row groups' sums, then one partial row per run
+    // d wf: the row groups' sums, then one partial row per run (the first barrier is the one of the matrix waves' tail)
     float *wacc = (float *)(smem + G::OFF_W);
 #pragma unroll
     for (int m = 0; m < KF; ++m)
