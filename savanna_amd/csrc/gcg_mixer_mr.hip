@@ -450,9 +450,9 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
     for (int m = 0; m < KF; ++m)
 #pragma unroll
         for (int v = 0; v < NV; ++v) dwa[m][v] = 0.f;
-    uint32_t xk[NR], Bk[NR];          // x, B of the step whose products are under way
+    float xk[NR][2], Bk[NR][2];       // x, B of the step whose products are under way
 #pragma unroll
-    for (int r = 0; r < NR; ++r) { xk[r] = 0u; Bk[r] = 0u; }
+    for (int r = 0; r < NR; ++r) { xk[r][0] = xk[r][1] = 0.f; Bk[r][0] = Bk[r][1] = 0.f; }
 
     constexpr int RING_END = (G::RAW_SLOTS - 1) * G::SLOT;
     int rs = 0;                       // byte offset of the raw ring slot of step k
@@ -484,12 +484,10 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
             // gradient of the features of step k-1 -> LDS, where the matrix waves turn it into d raw
 #pragma unroll
             for (int i = 0; i < NR; ++i) {
-                float dv[2], xv[2], Bv[2], o[NV];
+                float dv[2], o[NV];
                 M::unpack2(dq[0][i], dv[0], dv[1]);
-                M::unpack2(xk[i], xv[0], xv[1]);
-                M::unpack2(Bk[i], Bv[0], Bv[1]);
-                o[0] = dv[0] * y2v[i].x; o[1] = duv[i].x * xv[0]; o[2] = duv[i].x * Bv[0];
-                o[3] = dv[1] * y2v[i].y; o[4] = duv[i].y * xv[1]; o[5] = duv[i].y * Bv[1];
+                o[0] = dv[0] * y2v[i].x; o[1] = duv[i].x * xk[i][0]; o[2] = duv[i].x * Bk[i][0];
+                o[3] = dv[1] * y2v[i].y; o[4] = duv[i].y * xk[i][1]; o[5] = duv[i].y * Bk[i][1];
                 po[i] = values_piece<T>(o);
             }
             lds_store_blk(df_own + dfb, pieces_blk(po));
@@ -504,12 +502,10 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
             for (int i = 0; i < NH + NR; ++i) piece_values<T>(prc[i], rv[i]);
 #pragma unroll
             for (int i = 0; i < NR; ++i) {
-                Bk[i] = M::pack2(feat_sum(tap, rv, i, 1), feat_sum(tap, rv, i, 4));
-                xk[i] = M::pack2(feat_sum(tap, rv, i, 2), feat_sum(tap, rv, i, 5));
-                float x0, x1, B0, B1;
-                M::unpack2(xk[i], x0, x1);
-                M::unpack2(Bk[i], B0, B1);
-                *(uint32_t *)(u_own + i * UROW) = M::pack2(x0 * B0, x1 * B1);
+                // rounded to the tensors' type like the featurizer's output, then kept as fp32 for the gradient
+                M::unpack2(M::pack2(feat_sum(tap, rv, i, 1), feat_sum(tap, rv, i, 4)), Bk[i][0], Bk[i][1]);
+                M::unpack2(M::pack2(feat_sum(tap, rv, i, 2), feat_sum(tap, rv, i, 5)), xk[i][0], xk[i][1]);
+                *(uint32_t *)(u_own + i * UROW) = M::pack2(xk[i][0] * Bk[i][0], xk[i][1] * Bk[i][1]);
                 *(uint32_t *)(g_own + gs + i * UROW) = g2n[i];
             }
         }
