@@ -547,6 +547,8 @@ GCG_API int gcg_mixer_mr_fwd(const void *raw, const void *wf, const void *h, voi
     if (!all_aligned16({raw, y}) || !gcg::mfma_feat_supported(dtype, dm, kf)) return GCG_ERR_UNSUPPORTED;
     rc = check_device();
     if (rc) return rc;
+    if (gcg::mixer_mr_fused_supported(dtype, dm, kf))
+        return finish(gcg::mixer_mr_fused_fwd_launch(dtype, raw, wf, kf, h, y, dm, (hipStream_t)stream));
     return finish(gcg::mfma_il_fwd_feat_launch(dtype, raw, wf, kf, h, y, dm, (hipStream_t)stream));
 }
 

@@ -305,6 +305,8 @@ int mfma_il_bwd_feat_launch(int dtype, const void *dy, const void *raw, const vo
 // the whole backward of featurizer -> Hyena-MR operator in one kernel (no gradient of the features in memory)
 bool mixer_mr_fused_supported(int dtype, const Dims &dm, int kf);
 size_t mixer_mr_fused_workspace(const Dims &dm, int kf);
+int mixer_mr_fused_fwd_launch(int dtype, const void *raw, const void *wfeat, int kf, const void *h, void *y,
+                              const Dims &dm, hipStream_t st);
 int mixer_mr_fused_bwd_launch(int dtype, const void *dy, const void *raw, const void *wfeat, int kf, const void *h,
                               void *draw, void *dwf, void *dh, void *ws, const Dims &dm, hipStream_t st);
 

@@ -510,6 +510,7 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
             }
         }
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);           // what follows runs beside the matrix waves' products, not before them
         // The rows of step k+NK arrive (the ring slot two behind step k).  They are taken up before anything else is
         // sent to memory, so that waiting for them does not wait for younger accesses; then the rows of step
         // k+NK+2 are requested into the same registers.
@@ -600,6 +601,200 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
     }
 }
 
+// ---------------------------------------------------------------------------- forward
+// The same division of labour for y = C * (T u), u = x * B, with the features made from the projection output on
+// the way.  The forward has no ring to keep and few registers per wave, so a workgroup takes sixteen waves and 128
+// channels: rows of 768 bytes in, 256 bytes out (with 64 channels and two workgroups per CU, 130 us at the 7B shape
+// against 118: the 128-byte pieces of y are what costs).  Step k (32 rows):
+//   before the first barrier   memory: u(k) (made during the step before) -> LDS; y of step k-1 = C * y2 -> memory
+//   between the two            matrix: operand of u(k), 10 products -> y2(k)
+//                              memory: the rows of step k+1 arrive -> its features, u and C; rows of step k+3 requested
+template <typename T> struct MixFwdGeo {
+    typedef MT<T> M;
+    static_assert(!M::SPLIT && M::ES == 2, "16-bit tensors with 16-bit arithmetic operands");
+    static constexpr int XW = 8, MW = 8, NT = 64 * (XW + MW);
+    static constexpr int NK = 5;
+    static constexpr int CB = 16 * XW;
+    static constexpr int UROW = CB * 2 + 16, YROW = CB * 4 + 16;
+    static constexpr int LPR = CB / 2, NR = 4, NH = MR_KF - 1;
+    static constexpr int OFF_U = 0;
+    static constexpr int OFF_Y = OFF_U + STEP * UROW;
+    static constexpr int OFF_H = OFF_Y;                         // filter tables: read before the first y2 tile is written
+    static constexpr int LDS_BYTES = OFF_Y + STEP * YROW;
+    static_assert(XW * HTAB * 2 <= STEP * YROW, "filter tables fit");
+};
+
+template <typename T>
+__global__ __launch_bounds__(MixFwdGeo<T>::NT) void mixer_mr_fwd_kernel(const T *__restrict__ raw, const T *__restrict__ h,
+                                                                       const T *__restrict__ wfeat, int kf,
+                                                                       T *__restrict__ y, Dims dm, MfmaPlan pl)
+{
+    typedef MT<T> M;
+    typedef typename M::op_t op_t;
+    typedef typename M::hraw_t hraw_t;
+    typedef MixFwdGeo<T> G;
+    constexpr int NK = G::NK, MW = G::MW, CB = G::CB, UROW = G::UROW, YROW = G::YROW;
+    constexpr int LPR = G::LPR, NR = G::NR, NH = G::NH, KF = MR_KF, NV = 6;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[G::LDS_BYTES];
+    unsigned char *u_rm = smem + G::OFF_U, *y_st = smem + G::OFF_Y;
+    hraw_t *htab = (hraw_t *)(smem + G::OFF_H);
+
+    const int64_t wg_id = xcd_contiguous_id(blockIdx.x, gridDim.x);
+    int64_t wg = wg_id;
+    const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
+    const int seg = (int)(wg % pl.nseg);
+    const int64_t b = wg / pl.nseg;
+    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
+    const int64_t d = dm.d, L = dm.L;
+    const int64_t c0 = (int64_t)cb * CB;
+    const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
+    const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
+    const int64_t k_first = s_lo - (NK - 1);                    // u of the NK-1 steps before the run is made again
+
+    if (w >= MW) {
+        // ------------------------------------------------------------------ matrix waves
+        const int xw = w - MW, j = l & 15, q = l >> 4;
+        hraw_t hv[HTAB / 64];
+        load_taps<T>(dm, h, (c0 + 16 * xw < d) ? (c0 + 16 * xw) / dm.dg : 0, l, hv);
+        store_taps(htab + xw * HTAB, l, hv);
+        __syncthreads();
+        typename M::wop_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step k-i
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            W0[i] = M::toeplitz(htab + xw * HTAB, 32 * i, j, q);
+            W1[i] = M::toeplitz(htab + xw * HTAB, 32 * i + 16, j, q);
+        }
+        __syncthreads();      // the filter tables have been read: their place becomes the y2 tile
+        op_t Au[NK];
+#pragma unroll
+        for (int i = 0; i < NK; ++i) Au[i] = M::zero_op();
+        unsigned char *y_wr = y_st + j * YROW + (16 * xw + 4 * q) * 4;
+        int64_t k = k_first;
+        while (k <= s_hi) {
+#pragma unroll
+            for (int ph = 0; ph < NK; ++ph) {
+                if (k <= s_hi) {
+                    __syncthreads();
+                    if (k < s_hi) {
+                        Au[ph] = M::load_operand(u_rm, UROW, xw, j, q, false);
+                        if (k >= s_lo) {
+                            f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                            for (int i = 0; i < NK; ++i) {
+                                acc0 = M::mfma(Au[(ph - i + NK) % NK], W0[i], acc0);
+                                acc1 = M::mfma(Au[(ph - i + NK) % NK], W1[i], acc1);
+                            }
+                            *(f32x4 *)y_wr = acc0;
+                            *(f32x4 *)(y_wr + 16 * YROW) = acc1;
+                        }
+                    }
+                    __syncthreads();
+                    ++k;
+                }
+            }
+        }
+        return;
+    }
+
+    // ---------------------------------------------------------------------- memory waves
+    const int rr = tid / LPR, a = tid % LPR;        // rows NR*rr .. NR*rr+3, channels c0 + 2a, 2a+1
+    const bool cvalid = c0 + 2 * a < d;
+    const int64_t row_bytes = d * 2;
+    const int64_t T0 = s_lo * STEP, T1 = s_hi * STEP < L ? s_hi * STEP : L;
+    const int64_t t0 = k_first * STEP > 0 ? k_first * STEP : 0;
+    const int64_t tf = t0 - NH > 0 ? t0 - NH : 0;
+    const win_t wraw = make_window(raw + 3 * (b * L + tf) * d, 3 * (T1 - tf) * row_bytes);
+    const win_t wy = make_window(y + (b * L + T0) * d, (T1 - T0) * row_bytes);
+    const uint32_t rb = (uint32_t)row_bytes, bad = cvalid ? 0u : WIN_OFF, step_b = (uint32_t)STEP * rb;
+    const uint32_t col_b = (uint32_t)((c0 + 2 * a) * 2);
+    const uint32_t lane_raw = 3u * ((uint32_t)(NR * rr - NH) * rb + col_b) + bad;      // row NR*rr-NH of a step
+    const uint32_t lane_y = (uint32_t)(NR * rr) * rb + col_b + bad;                     // row NR*rr
+    auto step_base = [&](int64_t step, int64_t origin) { return (uint32_t)((step * STEP - origin) * row_bytes); };
+    float tap[KF][NV];
+    load_feat_taps<T, KF, NV>(wfeat, cvalid ? 3 * (c0 + 2 * a) : 0, kf, tap);
+    unsigned char *u_own = u_rm + NR * rr * UROW + 4 * a;
+    const unsigned char *y_rd = y_st + NR * rr * YROW + 8 * a;
+
+    struct Rows { u32x3 p[NH + NR]; };
+    auto fetch = [&](Rows &r, uint32_t raw_base) {
+#pragma unroll
+        for (int i = 0; i < NH + NR; ++i) r.p[i] = ldw12(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb));
+    };
+    uint32_t un[NR], cn[NR];          // u and C of the step that arrived last
+    // what arrived rows bring: the features, rounded like the featurizer's output, and with them u and C
+    auto arrive = [&](const Rows &r) {
+        float rv[NH + NR][NV];
+#pragma unroll
+        for (int i = 0; i < NH + NR; ++i) piece_values<T>(r.p[i], rv[i]);
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            float x0, x1, B0, B1;
+            cn[i] = M::pack2(feat_sum(tap, rv, i, 0), feat_sum(tap, rv, i, 3));
+            M::unpack2(M::pack2(feat_sum(tap, rv, i, 1), feat_sum(tap, rv, i, 4)), B0, B1);
+            M::unpack2(M::pack2(feat_sum(tap, rv, i, 2), feat_sum(tap, rv, i, 5)), x0, x1);
+            un[i] = M::pack2(x0 * B0, x1 * B1);
+        }
+#pragma unroll
+        for (int i = 0; i < NR; ++i) asm volatile("" : "+v"(un[i]), "+v"(cn[i]));     // made here, not after younger loads
+        __builtin_amdgcn_sched_barrier(0);
+    };
+
+    uint32_t raw_b = step_base(k_first, tf);        // of the step requested next
+    Rows in0, in1;                                   // rows on the way, requested two steps before they are taken up
+    fetch(in0, raw_b);
+    raw_b += step_b;
+    fetch(in1, raw_b);
+    raw_b += step_b;
+    __syncthreads();
+    __syncthreads();
+    arrive(in0);                                     // step k_first
+    fetch(in0, raw_b);
+    raw_b += step_b;
+
+    uint32_t cp[NR], yo[NR];          // C of the step whose products are under way; the rows of y stored last
+#pragma unroll
+    for (int i = 0; i < NR; ++i) { cp[i] = 0u; yo[i] = 0u; }
+    uint32_t y_b = step_base(s_lo, T0);              // of step k-1
+
+    auto iter = [&](int64_t k, Rows &in) {
+        if (k < s_hi) {
+#pragma unroll
+            for (int i = 0; i < NR; ++i) *(uint32_t *)(u_own + i * UROW) = un[i];
+        }
+        if (k > s_lo) {
+            // y of step k-1
+            float2 y2v[NR];
+#pragma unroll
+            for (int i = 0; i < NR; ++i) y2v[i] = *(const float2 *)(y_rd + i * YROW);
+#pragma unroll
+            for (int i = 0; i < NR; ++i) asm volatile("" ::"v"(yo[i]));       // (stored a step ago: see the backward)
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                float c0v, c1v;
+                M::unpack2(cp[i], c0v, c1v);
+                yo[i] = M::pack2(c0v * y2v[i].x, c1v * y2v[i].y);
+            }
+#pragma unroll
+            for (int i = 0; i < NR; ++i) stw4(wy, lane_y + y_b + (uint32_t)i * rb, yo[i]);
+            y_b += step_b;
+        }
+#pragma unroll
+        for (int i = 0; i < NR; ++i) cp[i] = cn[i];
+        __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);           // what follows runs beside the matrix waves' products, not before them
+        arrive(in);                                  // step k+1
+        fetch(in, raw_b);                            // step k+3
+        raw_b += step_b;
+        __syncthreads();
+    };
+    int64_t k = k_first;
+    for (; k + 1 <= s_hi; k += 2) {
+        iter(k, in1);
+        iter(k + 1, in0);
+    }
+    if (k <= s_hi) iter(k, in1);
+}
+
 } // namespace
 
 // ---------------------------------------------------------------------------- launch
@@ -639,6 +834,29 @@ int bwd_t(const void *dy, const void *raw, const void *wfeat, int kf, const void
 }
 
 } // namespace
+
+namespace {
+MfmaPlan mixer_fwd_plan(const Dims &dm)
+{
+    return plan(dm, MixFwdGeo<bf16_t>::XW, 16, MixFwdGeo<bf16_t>::XW, 2);
+}
+template <typename T>
+int fwd_t(const void *raw, const void *wfeat, int kf, const void *h, void *y, const Dims &dm, hipStream_t st)
+{
+    const MfmaPlan p = mixer_fwd_plan(dm);
+    if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    return launch_main(mixer_mr_fwd_kernel<T>, dim3((unsigned)p.nwg), dim3(MixFwdGeo<T>::NT), st, (const T *)raw,
+                       (const T *)h, (const T *)wfeat, kf, (T *)y, dm, p);
+}
+} // namespace
+
+int mixer_mr_fused_fwd_launch(int dtype, const void *raw, const void *wfeat, int kf, const void *h, void *y,
+                              const Dims &dm, hipStream_t st)
+{
+    if (dtype == GCG_BF16) return fwd_t<bf16_t>(raw, wfeat, kf, h, y, dm, st);
+    if (dtype == GCG_F16) return fwd_t<f16_t>(raw, wfeat, kf, h, y, dm, st);
+    return (int)hipErrorInvalidValue;
+}
 
 // 16-bit tensors with arithmetic in their own type, filters of 98..128 taps, a featurizer of at most 3
 bool mixer_mr_fused_supported(int dtype, const Dims &dm, int kf)
