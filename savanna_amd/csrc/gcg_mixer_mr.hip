@@ -175,12 +175,67 @@ __device__ __forceinline__ float feat_sum(const float (&tap)[MR_KF][6], const fl
     return acc;
 }
 
+// Tail of the backward, run by every wave: the workgroup that finishes a channel block's last run adds the block's
+// partial sums of dh and d wf in a fixed order (so the results do not depend on which workgroup that is) and writes
+// the gradients; without pl.fuse_dh two small launches do it.
+template <typename T>
+__device__ __forceinline__ void mixer_bwd_finish(const float *ws, const float *wsf, T *__restrict__ dh,
+                                                 T *__restrict__ dwf, const Dims &dm, const MfmaPlan &pl, int cb, int kf)
+{
+    typedef MixGeo<T> G;
+    if (!pl.fuse_dh) return;
+    const int tid = threadIdx.x;
+    __shared__ unsigned int is_last;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // every wave's partials have completed ...
+    __syncthreads();                                         // ... before thread 0 takes the ticket
+    if (tid == 0) {
+        unsigned int *tk = dh_tickets + pl.slot * DH_UNITS + cb;
+        const unsigned int arrivals = (unsigned int)(dm.bs * pl.nseg);
+        const unsigned int mine = atomicAdd(tk, 1u) + 1u;
+        is_last = (mine == arrivals);
+        if (mine == arrivals) __hip_atomic_store(tk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last) return;
+    const int64_t np = dm.bs * pl.nseg;
+    {
+        const int gpc = G::CB / dm.dg, bpg = dm.dg / 16;   // filter groups per channel block, 16-channel blocks per group
+        const int row = dm.fw ? dm.lc : dm.hl;              // taps per group in the output
+        for (int idx = tid; idx < gpc * row; idx += G::NT) {
+            const int gl = idx / row, k = idx % row;
+            const int64_t grp = (int64_t)cb * gpc + gl;
+            if (grp >= dm.g) continue;
+            if (k >= dm.hl) {                                // the parameter's taps beyond the filter in use
+                ((float *)dh)[grp * row + k] = 0.f;
+                continue;
+            }
+            const int lag = dm.hl - 1 - k;
+            float sum = 0.f;
+            for (int64_t p = 0; p < np; ++p)
+                for (int kk = 0; kk < bpg; ++kk)
+                    sum += __hip_atomic_load(ws + ((p * pl.ncb + cb) * G::XW + gl * bpg + kk) * 128 + lag, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+            store_dh<T>(dh, dm, grp, k, sum);
+        }
+    }
+    const int64_t nf = 3 * dm.d;
+    for (int idx = tid; idx < kf * 3 * G::CB; idx += G::NT) {
+        const int kk = idx / (3 * G::CB), col = idx % (3 * G::CB);
+        const int64_t f = (int64_t)cb * 3 * G::CB + col;
+        if (f >= nf) continue;
+        float sum = 0.f;
+        for (int64_t p = 0; p < np; ++p)
+            sum += __hip_atomic_load(wsf + ((size_t)kk * np + p) * nf + f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        Elem<T>::store(dwf + f * kf + kk, sum);
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ raw,
                                                                     const T *__restrict__ h, const T *__restrict__ wfeat,
                                                                     int kf, T *__restrict__ draw, T *__restrict__ dh,
-                                                                    float *__restrict__ ws, float *__restrict__ wsf,
-                                                                    Dims dm, MfmaPlan pl)
+                                                                    T *__restrict__ dwf, float *__restrict__ ws,
+                                                                    float *__restrict__ wsf, Dims dm, MfmaPlan pl)
 {
     typedef MT<T> M;
     typedef typename M::op_t op_t;
@@ -358,9 +413,10 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
                     for (int jj = 0; jj + r < 16; ++jj) sum += pt[d0 * 256 + (jj + r) * 16 + jj];
                 if (d0 + 1 < ND)
                     for (int ii = 0; ii < r; ++ii) sum += pt[(d0 + 1) * 256 + ii * 16 + ii + 16 - r];
-                out[lag] = sum;
+                __hip_atomic_store(out + lag, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
+        mixer_bwd_finish<T>(ws, wsf, dh, dwf, dm, pl, cb, kf);
         return;
     }
 
@@ -597,8 +653,9 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
         float sum = 0.f;
 #pragma unroll
         for (int r = 0; r < G::NG; ++r) sum += wacc[(m * G::NG + r) * (LPR * NV) + col];
-        wsf[((size_t)kk * nprow + prow) * (3 * d) + f] = sum;
+        __hip_atomic_store(wsf + ((size_t)kk * nprow + prow) * (3 * d) + f, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
+    mixer_bwd_finish<T>(ws, wsf, dh, dwf, dm, pl, cb, kf);
 }
 
 // ---------------------------------------------------------------------------- forward
@@ -803,7 +860,9 @@ namespace {
 MfmaPlan mixer_plan(const Dims &dm)
 {
     MfmaPlan p = plan(dm, MixGeo<bf16_t>::XW, 16, MixGeo<bf16_t>::XW, 2);
-    p.fuse_dh = 0;
+    // the kernel adds the partials itself when a filter group lies within one channel block
+    static const int fuse = env_int("GCG_MFMA_FUSE_DH", 1);    // tuning override: 0 = always separate launches
+    p.fuse_dh = fuse && MixGeo<bf16_t>::CB % dm.dg == 0 && p.ncb <= DH_UNITS;
     return p;
 }
 
@@ -818,13 +877,14 @@ int bwd_t(const void *dy, const void *raw, const void *wfeat, int kf, const void
           void *ws, const Dims &dm, hipStream_t st)
 {
     typedef MixGeo<T> G;
-    const MfmaPlan p = mixer_plan(dm);
+    MfmaPlan p = mixer_plan(dm);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
+    if (p.fuse_dh) p.slot = next_dh_slot();
     float *ws_dh = (float *)ws;
     float *ws_f = ws_dh + (size_t)p.nwg * G::XW * 128;
     int e = launch_main(mixer_mr_bwd_kernel<T>, dim3((unsigned)p.nwg), dim3(G::NT), st, (const T *)dy, (const T *)raw,
-                        (const T *)h, (const T *)wfeat, kf, (T *)draw, (T *)dh, ws_dh, ws_f, dm, p);
-    if (e) return e;
+                        (const T *)h, (const T *)wfeat, kf, (T *)draw, (T *)dh, (T *)dwf, ws_dh, ws_f, dm, p);
+    if (e || p.fuse_dh) return e;
     const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st, (const float *)ws_dh,
                      (T *)dh, dm, p);

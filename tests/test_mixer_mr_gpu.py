@@ -89,6 +89,28 @@ def test_against_oracle_and_chain(gcg_lib, bs, L, g, dg, hl, kf, dtype, filt):
             assert (a == b).float().mean().item() > 0.99 and torch.allclose(a.float(), b.float(), rtol=2e-3, atol=1e-3), n
 
 
+def test_full_size_against_chain(gcg_lib):
+    """The 7B layer shape (B=2, L=8192, D=4096, bf16): the one-kernel forward and backward against the chain of four
+    kernels on the same values -- y, d raw and dh bit for bit, d wf up to the order of its partial sums."""
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    bs, L, g, dg, hl, kf = 2, 8192, 256, 16, 128, 3
+    raw = torch.randn(bs, L, g, dg, 3, generator=gen, device=DEV).to(torch.bfloat16)
+    wf = (torch.randn(3 * g * dg, 1, kf, generator=gen, device=DEV) / kf ** 0.5).to(torch.bfloat16)
+    h = (torch.randn(g, 1, hl, generator=gen, device=DEV) / hl ** 0.5).to(torch.bfloat16)
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen, device=DEV)).to(torch.bfloat16)
+    y = _lib.mixer_mr_fwd(raw, wf, h)
+    draw, dwf, dh = _lib.mixer_mr_bwd(dy, raw, wf, h)
+    y_c, draw_c, dwf_c, dh_c = chain(raw, wf, h, dy)
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_c), "y"
+    assert torch.equal(draw, draw_c), "draw"
+    assert_close(dh, dh_c, TOL_DH[torch.bfloat16], "dh")
+    assert (dh == dh_c).float().mean().item() > 0.99, "dh"
+    assert_close(dwf, dwf_c, TOL_DH[torch.bfloat16], "dwf")
+    # every row of d raw was written: rows at run ends and at the sequence end take the other code paths
+    assert torch.isfinite(draw.float()).all() and draw[:, -2:].float().abs().sum() > 0 and draw[:, 4094:4098].float().abs().sum() > 0
+
+
 def test_refused_shapes(gcg_lib):
     raw, wf, h, dy = (t.to(DEV) for t in make(1, 64, 2, 16, 64, 3, torch.bfloat16, torch.bfloat16))
     with pytest.raises(RuntimeError, match="not supported"):
