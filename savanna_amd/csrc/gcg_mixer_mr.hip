@@ -71,6 +71,22 @@ template <typename T> struct MixGeo {
     static_assert(OFF_RAW % 16 == 0 && SLOT % 16 == 0 && BLK % 16 == 0, "16-byte LDS accesses");
 };
 
+// Accesses without the streaming hint: the rows before a lane's own are its neighbour's rows, requested by both, and
+// read twice from memory when the first request marks them for early eviction (measured: forward 116 -> 107 us,
+// backward 4 % faster; for the stores it makes no difference in the backward and 3 us in the forward).
+__device__ __forceinline__ u32x3 ldw12_cached(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b96(w, (int)off, 0, 0);
+}
+__device__ __forceinline__ uint32_t ldw4_cached(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b32(w, (int)off, 0, 0);
+}
+__device__ __forceinline__ void stw4_cached(win_t w, uint32_t off, uint32_t v)
+{
+    __builtin_amdgcn_raw_buffer_store_b32(v, w, (int)off, 0, 0);
+}
+
 struct Blk { uint4 w[3]; };       // four 12-byte pieces
 struct Halo { uint2 w[3]; };      // two 12-byte pieces
 
@@ -442,9 +458,9 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
     struct Rows { u32x3 p[NH + NR]; uint32_t dy[NR]; };
     auto fetch = [&](Rows &r, uint32_t raw_base, uint32_t dy_base) {
 #pragma unroll
-        for (int i = 0; i < NH + NR; ++i) r.p[i] = ldw12(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb));
+        for (int i = 0; i < NH + NR; ++i) r.p[i] = ldw12_cached(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb));
 #pragma unroll
-        for (int i = 0; i < NR; ++i) r.dy[i] = ldw4(wdy, lane_dy + dy_base + (uint32_t)i * rb);
+        for (int i = 0; i < NR; ++i) r.dy[i] = ldw4_cached(wdy, lane_dy + dy_base + (uint32_t)i * rb);
     };
 
     uint32_t dq[NK + 1][NR];          // dy of the steps between arrival and their own gradient, oldest first
@@ -775,7 +791,7 @@ __global__ __launch_bounds__(MixFwdGeo<T>::NT) void mixer_mr_fwd_kernel(const T 
     struct Rows { u32x3 p[NH + NR]; };
     auto fetch = [&](Rows &r, uint32_t raw_base) {
 #pragma unroll
-        for (int i = 0; i < NH + NR; ++i) r.p[i] = ldw12(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb));
+        for (int i = 0; i < NH + NR; ++i) r.p[i] = ldw12_cached(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb));
     };
     uint32_t un[NR], cn[NR];          // u and C of the step that arrived last
     // what arrived rows bring: the features, rounded like the featurizer's output, and with them u and C
@@ -832,7 +848,7 @@ __global__ __launch_bounds__(MixFwdGeo<T>::NT) void mixer_mr_fwd_kernel(const T 
                 yo[i] = M::pack2(c0v * y2v[i].x, c1v * y2v[i].y);
             }
 #pragma unroll
-            for (int i = 0; i < NR; ++i) stw4(wy, lane_y + y_b + (uint32_t)i * rb, yo[i]);
+            for (int i = 0; i < NR; ++i) stw4_cached(wy, lane_y + y_b + (uint32_t)i * rb, yo[i]);
             y_b += step_b;
         }
 #pragma unroll
