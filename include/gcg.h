@@ -320,6 +320,24 @@ GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, co
             int32_t dtype, void *stream);
 
 /*
+ * The same with the Hyena-MR filter formed inside the kernels, as in gcg_fwd_decay / gcg_bwd_decay: h = F(w * decay)
+ * cut to hl taps (ExplicitSingleDecayFilter.filter, savanna/model/operators/hyena/parametrization/explicit.py:68-75,
+ * and the cast of hyena.py:499-503), dw the gradient of the parameter w.  A Hyena-MR layer's convolutional part --
+ * filter, featurizer, operator -- is then one launch each way.
+ *   w, decay  (g, l_cache) fp32   dw  out, (g, l_cache) fp32, zero beyond hl
+ * Workspace and scratch sizes: gcg_mixer_mr_bwd_workspace_bytes, gcg_mixer_mr_bwd_scratch_bytes.
+ */
+GCG_API int gcg_mixer_mr_fwd_decay(const void *raw, const void *wf, const float *w, const float *decay,
+            int32_t l_cache, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+GCG_API int gcg_mixer_mr_bwd_decay(const void *dy, const void *raw, const void *wf, const float *w,
+            const float *decay, int32_t l_cache, void *draw, void *dwf, float *dw, void *dfeat_scratch,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+
+/*
  * Explicit decayed filter of Hyena-MR, ready for gcg_fwd, in one launch.
  * Replaces ExplicitSingleDecayFilter.filter (savanna/model/operators/hyena/parametrization/
  * explicit.py:68-75: h = self.h[:, :L] * self.decay[:, :L]) with L = min(hyena_mr_len, seq_len),

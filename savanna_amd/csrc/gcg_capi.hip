@@ -535,14 +535,39 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
 
 // ---- featurizer and Hyena-MR operator: the forward in one pass
 
+namespace {
+int mixer_mr_fwd_dims(const void *raw, const void *wf, const void *h, void *y, gcg::Dims &dm, int kf, int dtype,
+                      void *stream);
+}
+
 GCG_API int gcg_mixer_mr_fwd(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L, int32_t g,
                              int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
 {
     TimerScope timer_scope;
     if (!raw || !wf || !h || !y || kf <= 0) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    const int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
+    return mixer_mr_fwd_dims(raw, wf, h, y, dm, kf, dtype, stream);
+}
+
+GCG_API int gcg_mixer_mr_fwd_decay(const void *raw, const void *wf, const float *w, const float *decay, int32_t l_cache,
+                                   void *y, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+                                   int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!raw || !wf || !y || kf <= 0) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    const int rc = decay_dims(bs, L, g, dg, hl, dtype, w, decay, l_cache, &dm);
+    if (rc) return rc;
+    return mixer_mr_fwd_dims(raw, wf, nullptr, y, dm, kf, dtype, stream);
+}
+
+namespace {
+int mixer_mr_fwd_dims(const void *raw, const void *wf, const void *h, void *y, gcg::Dims &dm, int kf, int dtype,
+                      void *stream)
+{
+    int rc = 0;
     dm.es = 3;
     if (!all_aligned16({raw, y}) || !gcg::mfma_feat_supported(dtype, dm, kf)) return GCG_ERR_UNSUPPORTED;
     rc = check_device();
@@ -551,6 +576,7 @@ GCG_API int gcg_mixer_mr_fwd(const void *raw, const void *wf, const void *h, voi
         return finish(gcg::mixer_mr_fused_fwd_launch(dtype, raw, wf, kf, h, y, dm, (hipStream_t)stream));
     return finish(gcg::mfma_il_fwd_feat_launch(dtype, raw, wf, kf, h, y, dm, (hipStream_t)stream));
 }
+} // namespace
 
 namespace {
 int plain_tensor_code(int dtype) { return dtype == GCG_BF16_F32 ? GCG_BF16 : dtype == GCG_F16_F32 ? GCG_F16 : dtype; }
@@ -578,15 +604,47 @@ GCG_API size_t gcg_mixer_mr_bwd_scratch_bytes(int64_t bs, int64_t L, int32_t g, 
     return (size_t)(3 * bs * L * dm.d) * (dtype == GCG_F32 ? 4 : 2);
 }
 
+namespace {
+int mixer_mr_bwd_dims(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf, void *dh,
+                      void *dfeat_scratch, void *workspace, size_t workspace_bytes, gcg::Dims &dm, int kf, int dtype,
+                      void *stream);
+}
+
 GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf,
                              void *dh, void *dfeat_scratch, void *workspace, size_t workspace_bytes, int64_t bs,
                              int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
 {
     TimerScope timer_scope;
     if (!dy || !raw || !wf || !h || !draw || !dwf || !dh || kf <= 0) return GCG_ERR_BAD_ARG;
-    gcg::Dims dm, df;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    gcg::Dims dm;
+    const int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
+    return mixer_mr_bwd_dims(dy, raw, wf, h, draw, dwf, dh, dfeat_scratch, workspace, workspace_bytes, dm, kf, dtype, stream);
+}
+
+GCG_API int gcg_mixer_mr_bwd_decay(const void *dy, const void *raw, const void *wf, const float *w, const float *decay,
+                                   int32_t l_cache, void *draw, void *dwf, float *dw, void *dfeat_scratch,
+                                   void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg,
+                                   int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !raw || !wf || !draw || !dwf || !dw || kf <= 0) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    const int rc = decay_dims(bs, L, g, dg, hl, dtype, w, decay, l_cache, &dm);
+    if (rc) return rc;
+    return mixer_mr_bwd_dims(dy, raw, wf, nullptr, draw, dwf, dw, dfeat_scratch, workspace, workspace_bytes, dm, kf, dtype,
+                             stream);
+}
+
+namespace {
+int mixer_mr_bwd_dims(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf, void *dh,
+                      void *dfeat_scratch, void *workspace, size_t workspace_bytes, gcg::Dims &dm, int kf, int dtype,
+                      void *stream)
+{
+    gcg::Dims df;
+    const int64_t bs = dm.bs, L = dm.L;
+    const int32_t g = dm.g, dg = dm.dg, hl = dm.hl;
+    int rc = 0;
     dm.es = 3;
     dm.keep_out = 1;
     const bool fused = gcg::mixer_mr_fused_supported(dtype, dm, kf);
@@ -609,6 +667,7 @@ GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, co
     if (e) return finish(e);
     return finish(gcg::dwconv_bwd_launch(plain_tensor_code(dtype), dfeat_scratch, raw, wf, draw, dwf, ws2, df, st));
 }
+} // namespace
 
 // ---- explicit decayed filter (Hyena-MR parametrization)
 

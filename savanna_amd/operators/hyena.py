@@ -334,6 +334,26 @@ class _FeaturizedGateConvGate(torch.autograd.Function):
         return _lib.mixer_mr_bwd(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, h)
 
 
+class _FeaturizedDecayedGateConvGate(torch.autograd.Function):
+    """_FeaturizedGateConvGate with the filter F(w * decay)[:, :hl] formed inside the kernels, F the cast to ``filt``
+    (ExplicitSingleDecayFilter.filter, explicit.py:68-75; hyena.py:499-503): a Hyena-MR layer's convolutional
+    part is one kernel each way, and the backward returns the gradient of the filter parameter itself."""
+
+    @staticmethod
+    def forward(ctx, raw, wf, w, decay, hl, filt):
+        raw, wf, w, decay = (t if t.is_contiguous() else t.contiguous() for t in (raw, wf, w, decay))
+        ctx.save_for_backward(raw, wf, w, decay)
+        ctx.hl, ctx.filt = hl, filt
+        return _lib.mixer_mr_fwd_decay(raw, wf, w, decay, hl, filt)
+
+    @staticmethod
+    def backward(ctx, dz):
+        raw, wf, w, decay = ctx.saved_tensors
+        draw, dwf, dw = _lib.mixer_mr_bwd_decay(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, w, decay,
+                                                ctx.hl, ctx.filt)
+        return draw, dwf, dw, None, None, None
+
+
 class HyenaMixer(nn.Module):
     """The convolutional part of ParallelSequenceMixer.forward for the hyena operators
     (savanna/model/block.py:865-890): featurizer conv on the projected features, interleaved split,
@@ -344,7 +364,8 @@ class HyenaMixer(nn.Module):
     feature channel) the two convolutions run as one kernel each way (``fuse_short``); the result
     differs from the two-kernel chain by the rounding of fp32 sums only.  With a full-length Hyena-MR filter
     (98 to 128 taps) and a featurizer of at most 3 taps the featurized tensor is never stored (``fuse_medium``):
-    the operator's kernels make its rows from the projection output, forward and backward, with the chain's results."""
+    the operator's kernels make its rows from the projection output, forward and backward, with the chain's results,
+    and form the decayed filter themselves where the operator allows it (``HyenaMROperator.fuse_filter``)."""
 
     def __init__(self, operator: _CgcgOperatorBase, short_conv_L: int = 3, dtype=torch.float32, device=None,
                  fuse_short: bool = True, fuse_medium: bool = True):
@@ -362,8 +383,17 @@ class HyenaMixer(nn.Module):
     def forward(self, features: torch.Tensor) -> torch.Tensor:
         op = self.mixer
         bs, seqlen, d3 = features.shape
-        h = op._filter(seqlen)
         conv = self.hyena_proj_conv
+        fused = op._filter_in_kernel(seqlen, op.num_groups, op.group_dim, features.dtype, features)
+        if (fused is not None and self.fuse_medium and conv.group_dim == 1 and
+                _lib.mixer_mr_supported(op.group_dim, fused[0], conv.kernel_size, features)):
+            g, dg = op.num_groups, op.group_dim
+            assert d3 == 3 * g * dg
+            z = _FeaturizedDecayedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3),
+                                                     conv.short_conv_weight.to(features.dtype), op.filter.h,
+                                                     op.filter.decay, fused[0], fused[1])
+            return z.reshape(bs, seqlen, g * dg)
+        h = op._filter(seqlen)
         if (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and
                 _lib.mixer_mr_supported(op.group_dim, h.shape[-1], conv.kernel_size, features) and
                 (op.cgcg_dtype == features.dtype or op._fp32_inside(features.dtype, features))):

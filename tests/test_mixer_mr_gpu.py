@@ -111,6 +111,26 @@ def test_full_size_against_chain(gcg_lib):
     assert torch.isfinite(draw.float()).all() and draw[:, -2:].float().abs().sum() > 0 and draw[:, 4094:4098].float().abs().sum() > 0
 
 
+@pytest.mark.parametrize("dtype,filt", TYPES)
+@pytest.mark.parametrize("bs,L,g,dg,hl,kf,lc", [(2, 700, 6, 16, 128, 3, 160), (1, 3000, 3, 64, 128, 3, 128),
+                                                (2, 1100, 5, 32, 100, 2, 128)])
+def test_filter_formed_in_the_kernels(gcg_lib, bs, L, g, dg, hl, kf, lc, dtype, filt):
+    """gcg_mixer_mr_fwd_decay / _bwd_decay against the explicit-filter entry points given h = F(w * decay)[:, :hl]
+    from gcg_filter_decay_fwd, and dw against gcg_filter_decay_bwd of their dh: bit for bit."""
+    raw, wf, _, dy = (t.to(DEV) for t in make(bs, L, g, dg, hl, kf, dtype, filt, seed=5))
+    gen = torch.Generator().manual_seed(6)
+    w = (torch.randn(g, lc, generator=gen) / lc ** 0.5).to(DEV)
+    decay = torch.exp(-torch.logspace(0, 2, g)[:, None] * torch.linspace(0, 1, lc)[None]).to(DEV)
+    y = _lib.mixer_mr_fwd_decay(raw, wf, w, decay, hl, filt)
+    draw, dwf, dw = _lib.mixer_mr_bwd_decay(dy, raw, wf, w, decay, hl, filt)
+    h = _lib.filter_decay_fwd(w, decay, hl, filt)
+    assert torch.equal(y, _lib.mixer_mr_fwd(raw, wf, h))
+    draw2, dwf2, dh2 = _lib.mixer_mr_bwd(dy, raw, wf, h)
+    torch.cuda.synchronize()
+    assert torch.equal(draw, draw2) and torch.equal(dwf, dwf2)
+    assert dw.shape == w.shape and torch.equal(dw, _lib.filter_decay_bwd(dh2, decay))
+
+
 def test_refused_shapes(gcg_lib):
     raw, wf, h, dy = (t.to(DEV) for t in make(1, 64, 2, 16, 64, 3, torch.bfloat16, torch.bfloat16))
     with pytest.raises(RuntimeError, match="not supported"):
@@ -160,3 +180,6 @@ def test_hyena_mixer_keeps_no_featurized_tensor(gcg_lib, act, cgcg):
             assert torch.equal(a, b), n
     big = [e.key for e in prof.key_averages() if "mfma_il" in e.key or "dwconv" in e.key or "mixer_mr" in e.key]
     assert len(big) == (2 if cgcg == "bfloat16" else 3), big
+    if cgcg == "bfloat16":       # filter, featurizer and operator: nothing else of the library's is launched
+        ours = [e.key for e in prof.key_averages() if "gcg::" in e.key and e.device_time_total > 0]
+        assert len(ours) == 2 and all("mixer_mr" in k for k in ours), ours
