@@ -448,6 +448,103 @@ def kernel_table(device, n=30, nsets=4):
     return rows
 
 
+class BoardSensors:
+    """Shader clock and board power of card 0 from sysfs (pp_dpm_sclk, hwmon power1_input), sampled by a thread."""
+
+    def __init__(self, period_s=0.05):
+        import glob
+        import threading
+        dev = "/sys/class/drm/card0/device"
+        power = sorted(glob.glob(dev + "/hwmon/hwmon*/power1_input") + glob.glob(dev + "/hwmon/hwmon*/power1_average"))
+        self.paths = {"sclk": dev + "/pp_dpm_sclk", "power": power[0] if power else None}
+        self.period_s, self.samples, self.stop = period_s, [], False
+        self.thread = threading.Thread(target=self._poll, daemon=True)
+        self.thread.start()
+
+    def _read(self):
+        out = {}
+        try:
+            cur = [ln for ln in open(self.paths["sclk"]).read().splitlines() if ln.rstrip().endswith("*")]
+            out["sclk_mhz"] = float(cur[0].split(":")[1].strip().rstrip("*").strip().lower().replace("mhz", ""))
+        except (OSError, IndexError, ValueError):
+            out["sclk_mhz"] = None
+        try:
+            out["power_w"] = int(open(self.paths["power"]).read()) / 1e6
+        except (OSError, TypeError, ValueError):
+            out["power_w"] = None
+        return out
+
+    def _poll(self):
+        while not self.stop:
+            self.samples.append((time.perf_counter(), self._read()))
+            time.sleep(self.period_s)
+
+    def between(self, t0, t1):
+        """Median reading over [t0, t1) (perf_counter times)."""
+        rows = [r for t, r in self.samples if t0 <= t < t1]
+        out = {}
+        for key in ("sclk_mhz", "power_w"):
+            v = sorted(r[key] for r in rows if r[key] is not None)
+            out[key] = v[len(v) // 2] if v else None
+        return out
+
+    def close(self):
+        self.stop = True
+        self.thread.join()
+
+
+def power_table(device, secs=2.0):
+    """Each kernel of the Hyena-MR paths launched back to back for `secs` seconds at the 7B and 40B layer shapes:
+    median time per call (HIP events around groups of five) with the shader clock and board power meanwhile."""
+    sensors = BoardSensors()
+    rows = []
+    for shape_name, bs, L, g, dg in (("7B", 2, 8192, 256, 16), ("40B", 1, 32768, 512, 16)):
+        gen = torch.Generator(device=device).manual_seed(1)
+        sets = []
+        for _ in range(2):
+            feat = torch.randn(bs, L, g, dg, 3, generator=gen, device=device).to(torch.bfloat16)
+            dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen, device=device)).to(torch.bfloat16)
+            sets.append((feat, dy))
+        x, B, C = (torch.randn(bs, L, g, dg, generator=gen, device=device).to(torch.bfloat16) for _ in range(3))
+        h = (torch.randn(g, 1, 128, generator=gen, device=device) / 128 ** 0.5).to(torch.bfloat16)
+        hs = (torch.randn(g, 1, 7, generator=gen, device=device) / 7 ** 0.5).to(torch.bfloat16)
+        wf = (torch.randn(3 * g * dg, 1, 3, generator=gen, device=device) / 3 ** 0.5).to(torch.bfloat16)
+        calls = (
+            ("gcg_fwd hl=128", lambda s: _lib.fwd(x, B, C, h)),
+            ("gcg_bwd hl=128", lambda s: _lib.bwd(s[1], x, B, C, h)),
+            ("gcg_fwd_interleaved hl=128", lambda s: _lib.fwd_interleaved(s[0], h)),
+            ("gcg_bwd_interleaved hl=128", lambda s: _lib.bwd_interleaved(s[1], s[0], h)),
+            ("gcg_mixer_mr_fwd", lambda s: _lib.mixer_mr_fwd(s[0], wf, h)),
+            ("gcg_mixer_mr_bwd", lambda s: _lib.mixer_mr_bwd(s[1], s[0], wf, h)),
+            ("gcg_bwd hl=7", lambda s: _lib.bwd(s[1], x, B, C, hs)),
+        )
+        for name, fn in calls:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            groups, i = [], 0
+            while time.perf_counter() - t0 < secs:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(5):
+                    fn(sets[i % 2])
+                    i += 1
+                e1.record()
+                torch.cuda.synchronize()
+                groups.append(e0.elapsed_time(e1) / 5 * 1e3)
+            t1 = time.perf_counter()
+            late = sorted(groups[len(groups) // 2:])           # the second half: clocks and power have settled
+            rows.append({"kernel": name, "shape": shape_name, "us": late[len(late) // 2], "us_min": late[0],
+                         "us_max": late[-1], **sensors.between(t0 + 0.5 * (t1 - t0), t1)})
+        del sets, x, B, C
+        torch.cuda.empty_cache()
+    time.sleep(0.5)
+    t_idle = time.perf_counter()
+    time.sleep(0.5)
+    idle = sensors.between(t_idle, time.perf_counter())
+    sensors.close()
+    return {"kernels": rows, "idle": idle}
+
+
 def main():
     global KEEP_INTERMEDIATES, SETTLE_S
     ap = argparse.ArgumentParser()
@@ -468,6 +565,9 @@ def main():
     ap.add_argument("--kernels", action="store_true",
                     help="print the single-kernel table instead (forward and backward kernel of the gated entry "
                          "points alone at the 7B and 40B layer shapes, one JSON line) and exit")
+    ap.add_argument("--power", action="store_true",
+                    help="print shader clock and board power (sysfs) under each Hyena-MR kernel launched back to "
+                         "back, with the time per call, as one JSON line, and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, so a counter profile of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -488,6 +588,11 @@ def main():
     if args.kernels:
         print(json.dumps({"single_kernels": kernel_table(device, n=max(10, args.steps)), "unit": "us, GB/s of algorithmic "
                           "bytes (4 tensors forward, 7 backward), fraction of 8 TB/s"}), flush=True)
+        return
+
+    if args.power:
+        print(json.dumps({"power": power_table(device), "unit": "us per call (median, min, max of the settled half), "
+                          "MHz, W"}), flush=True)
         return
 
     wl = WORKLOADS[args.workload]
