@@ -521,9 +521,27 @@ def _check_mixer_mr(raw, wf, h):
         raise ValueError("raw, wf and h must be on one device")
 
 
+def _aligned16(t) -> bool:
+    """16-byte alignment of a tensor's first element.  While torch.compile traces there is no address to look at
+    and the answer is yes: the choice of kernels is then part of the graph, and the entry points themselves
+    refuse a misaligned tensor with an error."""
+    if torch.compiler.is_compiling():
+        return True
+    return t.data_ptr() % 16 == 0
+
+
+def _all_aligned16(tensors, skip_strided=False) -> bool:
+    for t in tensors:                      # (a plain loop: torch.compile traces it)
+        if skip_strided and not t.is_contiguous():
+            continue
+        if not _aligned16(t):
+            return False
+    return True
+
+
 def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors) -> bool:
     """Whether gcg_mixer_mr_fwd / _bwd take these sizes (matrix-core kernels, full-length filter, short featurizer)."""
-    return 98 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and all(t.data_ptr() % 16 == 0 for t in tensors)
+    return 98 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and _all_aligned16(tensors)
 
 
 def mixer_mr_fwd(raw, wf, h):
@@ -625,7 +643,7 @@ def mixer_mr_bwd_decay(dy, raw, wf, w, decay, hl: int, filt: torch.dtype):
 
 def time_major_supported(dg: int, hl: int, *tensors) -> bool:
     """Whether gcg_fwd_time_major / gcg_bwd_time_major take these sizes (register-window kernels)."""
-    return hl <= 8 and dg % 4 == 0 and all(t.is_contiguous() and t.data_ptr() % 16 == 0 for t in tensors)
+    return hl <= 8 and dg % 4 == 0 and all(t.is_contiguous() for t in tensors) and _all_aligned16(tensors)
 
 
 def fwd_time_major(x, B, C, h):
@@ -675,7 +693,7 @@ def decay_supported(g: int, dg: int, hl: int, *tensors) -> bool:
     """Whether the *_decay entry points take these sizes: matrix-core kernels only
     (hl <= 128, dg a multiple of 16, 16-byte aligned tensors; a tensor that is not contiguous is
     copied or read through its interleaved source before it reaches them)."""
-    return hl <= 128 and dg % 16 == 0 and all(t.data_ptr() % 16 == 0 for t in tensors if t.is_contiguous())
+    return hl <= 128 and dg % 16 == 0 and _all_aligned16(tensors, skip_strided=True)
 
 
 def _decay_code(t: torch.Tensor, filt: torch.dtype) -> int:

@@ -44,6 +44,18 @@ def test_meta_shapes_on_fake_gpu_tensors(gcg_lib):
         hh = torch.ops.gcg.filter_decay_fwd(p, p, 64, torch.float16)
         assert hh.shape == (g, 1, 64) and hh.dtype == torch.float16
         assert torch.ops.gcg.filter_decay_bwd(hh, p).shape == p.shape
+        # Hyena-MR mixer (featurizer + operator), with the filter given and with the filter formed in the kernels
+        assert torch.ops.gcg.mixer_mr_fwd(feat, wf, h).shape == x.shape
+        draw, dwf, dh = torch.ops.gcg.mixer_mr_bwd(x, feat, wf, h)
+        assert draw.shape == feat.shape and dwf.shape == wf.shape and dh.shape == h.shape
+        y = torch.ops.gcg.mixer_mr_fwd_decay(feat, wf, p, p, 128, torch.bfloat16)
+        assert y.shape == x.shape and y.dtype == x.dtype
+        draw, dwf, dw = torch.ops.gcg.mixer_mr_bwd_decay(x, feat, wf, p, p, 128, torch.bfloat16)
+        assert draw.shape == feat.shape and dwf.shape == wf.shape and dw.shape == p.shape and dw.dtype == torch.float32
+        y = torch.ops.gcg.fwd_interleaved_decay(feat, p, p, 128, torch.bfloat16)
+        assert y.shape == x.shape
+        dfeat, dw = torch.ops.gcg.bwd_interleaved_decay(x, feat, p, p, 128, torch.bfloat16)
+        assert dfeat.shape == feat.shape and dw.shape == p.shape
 
 
 def test_meta_implementations_check_arguments(gcg_lib):

@@ -71,6 +71,17 @@ def test_library_opcheck(gcg_lib):
     torch.library.opcheck(torch.ops.gcg.fwd_interleaved, (feat, h), test_utils=checks)
     torch.library.opcheck(torch.ops.gcg.bwd_interleaved, (dy, feat, h), test_utils=checks)
     torch.library.opcheck(torch.ops.gcg.fwd_out, (x, B, C, h, torch.empty_like(x)), test_utils=checks)
+    # the Hyena-MR mixer operators, with the filter given and formed in the kernels
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(1, 130, 2, 16, 128, torch.bfloat16))
+    feat = torch.stack([C, B, x], dim=-1).contiguous()
+    wf = (torch.randn(3 * 2 * 16, 1, 3, device=DEV) / 3 ** 0.5).to(torch.bfloat16)
+    w = torch.randn(2, 128, device=DEV) / 128 ** 0.5
+    decay = torch.rand(2, 128, device=DEV)
+    torch.library.opcheck(torch.ops.gcg.mixer_mr_fwd, (feat, wf, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_mr_bwd, (dy, feat, wf, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_mr_fwd_decay, (feat, wf, w, decay, 128, torch.bfloat16), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_mr_bwd_decay, (dy, feat, wf, w, decay, 128, torch.bfloat16),
+                          test_utils=checks)
 
 
 def _grads(fn, tensors, dy):
@@ -108,3 +119,35 @@ def test_compile_fullgraph_interleaved(gcg_lib):
     compiled = _grads(torch.compile(op, fullgraph=True, backend="aot_eager"), (feat, h), dy)
     for name, a, b in zip(("y", "dfeat", "dh"), eager, compiled):
         assert torch.equal(a, b), name
+
+
+@pytest.mark.parametrize("kind", ["mr", "se"])
+def test_compile_fullgraph_hyena_mixer(gcg_lib, kind):
+    """HyenaMixer (featurizer conv, split, operator; for Hyena-MR with the filter formed in the kernel) traced by
+    torch.compile without a graph break: output and every gradient equal to eager."""
+    from savanna_amd.operators.hyena import CgcgConfig, HyenaMixer, HyenaMROperator, HyenaSEOperator
+
+    torch.manual_seed(3)
+    bs, L, g, dg = 2, 384, 4, 16
+    cfg = CgcgConfig(cgcg_dtype="bfloat16")
+    op = (HyenaMROperator(g * dg, g, 128, cfg, small_init=False, device=DEV) if kind == "mr"
+          else HyenaSEOperator(g * dg, g * dg, 7, cfg, device=DEV))
+    mixer = HyenaMixer(op, 3, dtype=torch.bfloat16, device=DEV)
+    feats = torch.randn(bs, L, 3 * g * dg, device=DEV).to(torch.bfloat16).requires_grad_(True)
+    dz = (0.1 * torch.randn(bs, L, g * dg, device=DEV)).to(torch.bfloat16)
+    params = list(mixer.parameters())
+
+    def run(fn):
+        feats.grad = None
+        for p in params:
+            p.grad = None
+        z = fn(feats)
+        z.backward(dz)
+        return [z.detach(), feats.grad.clone()] + [p.grad.clone() for p in params]
+
+    eager = run(mixer)
+    torch._dynamo.reset()
+    compiled = run(torch.compile(mixer, fullgraph=True, backend="aot_eager"))
+    assert len(eager) == len(compiled) == 2 + len(params)
+    for i, (a, b) in enumerate(zip(eager, compiled)):
+        assert torch.equal(a, b), i
