@@ -303,8 +303,9 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
  * one-kernel backward runs, the size of raw otherwise.
  *   draw  out, (bs, L, g, dg, 3)   dwf  out, (3 * g * dg, 1, kf)   dh  out, (g, 1, hl), filter's type
  *   workspace  gcg_mixer_mr_bwd_workspace_bytes(...) bytes, 256-byte aligned
- * Matrix-core kernels with full-length filters only: 98 <= hl <= 128, dg % 16 == 0, kf <= 3, 16-byte aligned
- * tensors; otherwise GCG_ERR_UNSUPPORTED (use the two calls).  dtype: any, GCG_BF16_F32 / GCG_F16_F32 included.
+ * Matrix-core kernels only: hl <= 128, dg % 16 == 0, kf <= 3, 16-byte aligned tensors; otherwise
+ * GCG_ERR_UNSUPPORTED (use the two calls).  The kernels are laid out for filters of 98 to 128 taps (five slices of
+ * the banded matrix); a shorter filter leaves the far slices zero and costs the same time.  dtype: any, GCG_BF16_F32 / GCG_F16_F32 included.
  */
 GCG_API int gcg_mixer_mr_fwd(const void *raw, const void *wf, const void *h, void *y,
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,

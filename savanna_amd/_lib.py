@@ -540,8 +540,9 @@ def _all_aligned16(tensors, skip_strided=False) -> bool:
 
 
 def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors) -> bool:
-    """Whether gcg_mixer_mr_fwd / _bwd take these sizes (matrix-core kernels, full-length filter, short featurizer)."""
-    return 98 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and _all_aligned16(tensors)
+    """Whether gcg_mixer_mr_fwd / _bwd take these sizes (matrix-core kernels, filters of up to 128 taps
+    -- those of at most 8 are the fused Hyena-SE kernels' -- and a featurizer of at most 3)."""
+    return 9 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and _all_aligned16(tensors)
 
 
 def mixer_mr_fwd(raw, wf, h):

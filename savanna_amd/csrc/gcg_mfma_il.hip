@@ -630,7 +630,8 @@ size_t mfma_feat_bwd_workspace(int dtype, const Dims &dm)
 
 bool mfma_feat_supported(int dtype, const Dims &dm, int kf)
 {
-    return kf >= 1 && kf <= FEAT_KF && nk_for(dm.hl) == 5 && mfma_supported(dtype, dm);
+    // (the kernels walk five slices of the banded matrix whatever hl is: a shorter filter leaves the far ones zero)
+    return kf >= 1 && kf <= FEAT_KF && mfma_supported(dtype, dm);
 }
 
 int mfma_il_fwd_feat_launch(int dtype, const void *raw, const void *wfeat, int kf, const void *h, void *y,

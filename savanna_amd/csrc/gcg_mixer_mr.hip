@@ -934,7 +934,7 @@ int mixer_mr_fused_fwd_launch(int dtype, const void *raw, const void *wfeat, int
     return (int)hipErrorInvalidValue;
 }
 
-// 16-bit tensors with arithmetic in their own type, filters of 98..128 taps, a featurizer of at most 3
+// 16-bit tensors with arithmetic in their own type, filters of up to 128 taps, a featurizer of at most 3
 bool mixer_mr_fused_supported(int dtype, const Dims &dm, int kf)
 {
     static const int off = env_int("GCG_MIXER_MR_FUSED", 1) == 0;      // tuning override: 0 = the two-kernel backward

@@ -362,8 +362,8 @@ class HyenaMixer(nn.Module):
 
     With a short operator filter (Hyena-SE: at most 8 taps, featurizer of at most 4, one filter per
     feature channel) the two convolutions run as one kernel each way (``fuse_short``); the result
-    differs from the two-kernel chain by the rounding of fp32 sums only.  With a full-length Hyena-MR filter
-    (98 to 128 taps) and a featurizer of at most 3 taps the featurized tensor is never stored (``fuse_medium``):
+    differs from the two-kernel chain by the rounding of fp32 sums only.  With a Hyena-MR filter
+    (9 to 128 taps) and a featurizer of at most 3 taps the featurized tensor is never stored (``fuse_medium``):
     the operator's kernels make its rows from the projection output, forward and backward, with the chain's results,
     and form the decayed filter themselves where the operator allows it (``HyenaMROperator.fuse_filter``)."""
 

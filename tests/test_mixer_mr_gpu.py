@@ -23,6 +23,10 @@ SHAPES = [
     (1, 700, 17, 16, 128, 3),     # d = 272
     (1, 3000, 3, 64, 128, 3),     # a filter group as wide as a workgroup's channel block
     (2, 4100, 8, 16, 128, 3),     # runs of more than a hundred steps
+    (2, 900, 6, 16, 64, 3),       # shorter filters (hyena_mr_len 64 in some configurations): the far slices are zero
+    (1, 1300, 4, 32, 33, 2),
+    (2, 500, 5, 16, 9, 3),
+    (1, 200, 3, 16, 97, 3),
 ]
 TYPES = [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.float32, torch.float32),
          (torch.bfloat16, torch.float32)]
@@ -132,13 +136,14 @@ def test_filter_formed_in_the_kernels(gcg_lib, bs, L, g, dg, hl, kf, lc, dtype, 
 
 
 def test_refused_shapes(gcg_lib):
-    raw, wf, h, dy = (t.to(DEV) for t in make(1, 64, 2, 16, 64, 3, torch.bfloat16, torch.bfloat16))
+    raw, wf, h, dy = (t.to(DEV) for t in make(1, 64, 2, 8, 64, 3, torch.bfloat16, torch.bfloat16))
     with pytest.raises(RuntimeError, match="not supported"):
-        _lib.mixer_mr_fwd(raw, wf, h)                      # short filter: fewer slices than the fused kernels walk
+        _lib.mixer_mr_fwd(raw, wf, h)                      # groups of 8 channels: less than a matrix tile
     raw, wf, h, dy = (t.to(DEV) for t in make(1, 64, 2, 16, 128, 4, torch.bfloat16, torch.bfloat16))
     with pytest.raises(RuntimeError, match="not supported"):
         _lib.mixer_mr_bwd(dy, raw, wf, h)                  # four featurizer taps
-    assert not _lib.mixer_mr_supported(16, 64, 3) and not _lib.mixer_mr_supported(16, 128, 4) and _lib.mixer_mr_supported(16, 128, 3)
+    assert not _lib.mixer_mr_supported(8, 64, 3) and not _lib.mixer_mr_supported(16, 128, 4) and _lib.mixer_mr_supported(16, 128, 3)
+    assert _lib.mixer_mr_supported(16, 64, 3) and not _lib.mixer_mr_supported(16, 7, 3)      # (Hyena-SE filters: gcg_mixer_se_*)
 
 
 @pytest.mark.parametrize("act,cgcg", [(torch.bfloat16, "bfloat16"), (torch.float32, "float32"), (torch.bfloat16, "float32")])
