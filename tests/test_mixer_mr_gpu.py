@@ -27,6 +27,10 @@ SHAPES = [
     (1, 1300, 4, 32, 33, 2),
     (2, 500, 5, 16, 9, 3),
     (1, 200, 3, 16, 97, 3),
+    (1, 20, 2, 16, 20, 3),        # sequences shorter than a step of 32 rows (the operator cuts hl to the length)
+    (2, 31, 3, 16, 9, 3),
+    (1, 33, 2, 16, 33, 1),
+    (3, 9, 1, 16, 9, 2),
 ]
 TYPES = [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16), (torch.float32, torch.float32),
          (torch.bfloat16, torch.float32)]
