@@ -118,6 +118,8 @@ class Op:
                 t["raw"] = raw.contiguous().requires_grad_(True)
                 t["wf"] = wf.to(wl.dtype).to(device).requires_grad_(True)
                 t["h"] = t["h"].requires_grad_(True)
+            elif wl.layout == "planar":
+                t["feat"] = torch.stack([t.pop("v"), t.pop("q"), t.pop("k")], dim=2).contiguous()
             elif wl.layout != "separate":
                 # kernel names: C = v, B = q, x = k
                 t["feat"] = torch.stack([t.pop("v"), t.pop("q"), t.pop("k")], dim=-1).contiguous()
@@ -186,6 +188,10 @@ class Op:
             y = _lib.fwd_interleaved(feat, h)
             if self.backward:
                 _lib.bwd_interleaved(t["dy"], feat, h)
+        elif self.layout == "planar":
+            y = _lib.fwd_planar(feat, h)
+            if self.backward:
+                _lib.bwd_planar(t["dy"], feat, h)
         else:
             C, B, x = (feat[..., i].contiguous() for i in range(3))     # cgcg/interface.py:51-54
             _, _, y = _lib.fwd(x, B, C, h)
@@ -644,7 +650,8 @@ def main():
         # the rows next to the hot path: the operator fed from the interleaved projected features, the
         # featurizer conv, and the two chained through autograd
         extra = {}
-        for name in ("mr_fwdbwd_7b_interleaved", "se_fwdbwd_40b_interleaved", "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b",
+        for name in ("mr_fwdbwd_7b_interleaved", "se_fwdbwd_40b_interleaved", "mr_fwdbwd_7b_planar", "se_fwdbwd_40b_planar",
+                     "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b",
                      "mixer_fwdbwd_7b_fused", "mixer_fwd_7b", "mixer_fwd_7b_fused", "mixer_se_fwdbwd_40b",
                      "mixer_se_fwdbwd_40b_fused"):
             r = time_workload(WORKLOADS[name], device, max(10, args.steps // 2), 4)

@@ -204,6 +204,26 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
             int32_t dtype, int32_t algo, int32_t flags, void *stream);
 
 /*
+ * The gated convolution on planar projected features: one (bs, L, 3, g, dg) tensor whose rows hold the three
+ * operands side by side, [..., 0, :, :] = C (post-gate, x1), [..., 1, :, :] = B (pre-gate, x2), [..., 2, :, :] = x (v)
+ * -- the split without interleaving of savanna/model/block.py:881-884 ("b l (p g dg) -> b l p g dg", kept for
+ * checkpoints trained with interleave_projections = false).  The reference gathers the three strided views into
+ * contiguous tensors (kernels/triton_src/cgcg/interface.py:51-54) and autograd re-assembles the gradient; here
+ * the kernels read the thirds of the rows in place and write dfeat (same layout) directly.
+ *   feat, dfeat  (bs, L, 3, g, dg)   h, dh  (g, 1, hl)   y, dy  (bs, L, g, dg)
+ * Same values as gcg_fwd / gcg_bwd on the gathered operands.  dtype: any, GCG_BF16_F32 / GCG_F16_F32 included.
+ * Workspace: gcg_bwd_workspace_bytes(...) with the same algo.
+ */
+GCG_API int gcg_fwd_planar(const void *feat, const void *h, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, int32_t algo, void *stream);
+GCG_API int gcg_bwd_planar(const void *dy, const void *feat, const void *h,
+            void *dfeat, void *dh,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+            int32_t dtype, int32_t algo, void *stream);
+
+/*
  * Short causal depthwise convolution without gates: the featurizer that the hyena blocks apply to
  * the projected features before splitting them.
  * Replaces ParallelCausalDepthwiseConv1d.forward (savanna/model/operators/hyena/hyena.py:136-181,

@@ -31,7 +31,7 @@ GCG_BF16_F32, GCG_F16_F32 = 3, 4       # 16-bit tensors, fp32 filter and arithme
 EXPORTS = (
     "gcg_strerror", "gcg_last_hip_error", "gcg_time_next_kernel", "gcg_version", "gcg_fwd",
     "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_bwd_static", "gcg_select_algo",
-    "gcg_fwd_interleaved", "gcg_bwd_interleaved",
+    "gcg_fwd_interleaved", "gcg_bwd_interleaved", "gcg_fwd_planar", "gcg_bwd_planar",
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
@@ -84,6 +84,10 @@ def load() -> ctypes.CDLL:
         lib.gcg_fwd_interleaved.restype = ctypes.c_int
         lib.gcg_bwd_interleaved.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, i32, i32, vp]
         lib.gcg_bwd_interleaved.restype = ctypes.c_int
+        lib.gcg_fwd_planar.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_fwd_planar.restype = ctypes.c_int
+        lib.gcg_bwd_planar.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_bwd_planar.restype = ctypes.c_int
         lib.gcg_dwconv_fwd.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_dwconv_fwd.restype = ctypes.c_int
         lib.gcg_dwconv_bwd_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32]
@@ -344,6 +348,62 @@ def bwd_interleaved(dy, feat, h, algo=ALGO_AUTO, keep_output=False):
                                      ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, a,
                                      KEEP_OUTPUT if keep_output else 0, st)
     check(rc, "gcg_bwd_interleaved")
+    return dfeat, dh
+
+
+def _check_planar(feat, h):
+    if feat.dim() != 5 or feat.shape[2] != 3 or not feat.is_contiguous():
+        raise ValueError("feat must be a contiguous (bs, L, 3, g, dg) tensor")
+    if h.dim() != 3 or h.shape[0] != feat.shape[3] or h.shape[1] != 1 or not h.is_contiguous():
+        raise ValueError("h must be a contiguous (g, 1, hl) tensor")
+    gated_code(feat, h)
+    if h.device != feat.device:
+        raise ValueError("feat and h must share dtype and device")
+
+
+def fwd_planar(feat, h, algo=ALGO_AUTO):
+    """y (bs, L, g, dg) for planar features feat (bs, L, 3, g, dg): feat[:, :, 0] = C, [:, :, 1] = B, [:, :, 2] = x,
+    the thirds of each row read in place (block.py:881-884, the split without interleaving)."""
+    _require_gpu(feat)
+    if TORCH_OPS:
+        return torch.ops.gcg.fwd_planar(feat, h, algo_code(algo))
+    lib = load()
+    _check_planar(feat, h)
+    bs, L, _, g, dg = feat.shape
+    y = torch.empty(bs, L, g, dg, dtype=feat.dtype, device=feat.device)
+    if y.numel() == 0:
+        return y
+    with _on_device(feat.device):
+        rc = lib.gcg_fwd_planar(feat.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg, h.shape[-1],
+                                gated_code(feat, h), algo_code(algo), torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_fwd_planar")
+    return y
+
+
+def bwd_planar(dy, feat, h, algo=ALGO_AUTO):
+    """(dfeat, dh): dfeat has feat's layout, dfeat[:, :, 0] = dC, [:, :, 1] = dB, [:, :, 2] = dx."""
+    _require_gpu(feat)
+    if TORCH_OPS:
+        return torch.ops.gcg.bwd_planar(dy, feat, h, algo_code(algo))
+    lib = load()
+    _check_planar(feat, h)
+    bs, L, _, g, dg = feat.shape
+    hl = h.shape[-1]
+    if dy.shape != (bs, L, g, dg) or dy.dtype != feat.dtype or not dy.is_contiguous():
+        raise ValueError("dy must be a contiguous (bs, L, g, dg) tensor of feat's dtype")
+    dfeat, dh = torch.empty_like(feat), torch.empty_like(h)
+    if dy.numel() == 0:
+        return dfeat, dh.zero_()
+    code, a = gated_code(feat, h), algo_code(algo)
+    nbytes = lib.gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, a)
+    if nbytes == 0:
+        raise GcgError("gcg_bwd_workspace_bytes: arguments rejected")
+    with _on_device(feat.device):
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=feat.device)
+        rc = lib.gcg_bwd_planar(dy.data_ptr(), feat.data_ptr(), h.data_ptr(), dfeat.data_ptr(), dh.data_ptr(),
+                                ws.data_ptr(), nbytes, bs, L, g, dg, hl, code, a,
+                                torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_bwd_planar")
     return dfeat, dh
 
 

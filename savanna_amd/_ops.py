@@ -36,4 +36,5 @@ OP_NAMES = (
     "fwd", "fwd_full", "fwd_out", "bwd", "fwd_interleaved", "bwd_interleaved", "dwconv_fwd", "dwconv_bwd",
     "mixer_se_fwd", "mixer_se_bwd", "filter_decay_fwd", "filter_decay_bwd",
     "mixer_mr_fwd", "mixer_mr_bwd", "mixer_mr_fwd_decay", "mixer_mr_bwd_decay", "fwd_time_major", "bwd_time_major", "fwd_decay", "bwd_decay", "fwd_interleaved_decay", "bwd_interleaved_decay",
+    "fwd_planar", "bwd_planar",
 )

@@ -40,7 +40,7 @@ int make_dims(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t 
     const bool mixed = dtype == GCG_BF16_F32 || dtype == GCG_F16_F32;
     if (!plain && !(mixed && mixed_ok)) return GCG_ERR_BAD_ARG;
     dm->bs = bs; dm->L = L; dm->g = g; dm->dg = dg; dm->hl = hl; dm->d = (int64_t)g * dg; dm->es = 1; dm->keep_out = 0;
-    dm->fw = dm->fdecay = nullptr; dm->lc = 0; dm->tmajor = 0;
+    dm->fw = dm->fdecay = nullptr; dm->lc = 0; dm->tmajor = 0; dm->planar = 0;
     return GCG_OK;
 }
 
@@ -308,6 +308,69 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
         return finish(gcg::window_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
     case GCG_ALGO_MFMA:
         return finish(gcg::mfma_il_bwd_launch(dtype, dy, feat, h, dfeat, dh, workspace, dm, st));
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
+// ---- planar operands: the thirds (C | B | x) of the rows of one (bs, L, 3 * g * dg) tensor, read in place
+
+namespace {
+const void *plane(const void *base, int k, int64_t d, int dtype)
+{
+    return (const char *)base + (size_t)k * d * (dtype == GCG_F32 ? 4 : 2);
+}
+void *plane_out(void *base, int k, int64_t d, int dtype) { return (char *)base + (size_t)k * d * (dtype == GCG_F32 ? 4 : 2); }
+} // namespace
+
+GCG_API int gcg_fwd_planar(const void *feat, const void *h, void *y, int64_t bs, int64_t L, int32_t g, int32_t dg,
+                           int32_t hl, int32_t dtype, int32_t algo, void *stream)
+{
+    TimerScope timer_scope;
+    if (!feat || !h || !y) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    if (rc) return rc;
+    dm.planar = 1;
+    const void *C = feat, *B = plane(feat, 1, dm.d, dtype), *x = plane(feat, 2, dm.d, dtype);
+    const int a = resolve_algo(algo, dtype, dm, false, all_aligned16({C, B, x, y}));
+    if (a < 0) return a;
+    rc = check_device();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (a) {
+    case GCG_ALGO_DIRECT: return finish(gcg::direct_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
+    case GCG_ALGO_WINDOW: return finish(gcg::window_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
+    case GCG_ALGO_MFMA:   return finish(gcg::mfma_fwd_launch(dtype, x, B, C, h, y, nullptr, nullptr, dm, st));
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
+GCG_API int gcg_bwd_planar(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *workspace,
+                           size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                           int32_t dtype, int32_t algo, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !feat || !h || !dfeat || !dh) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    if (rc) return rc;
+    dm.planar = 1;
+    const void *C = feat, *B = plane(feat, 1, dm.d, dtype), *x = plane(feat, 2, dm.d, dtype);
+    void *dC = dfeat, *dB = plane_out(dfeat, 1, dm.d, dtype), *dx = plane_out(dfeat, 2, dm.d, dtype);
+    const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, C, B, x, dC, dB, dx}));
+    if (a < 0) return a;
+    const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    hipStream_t st = (hipStream_t)stream;
+    switch (a) {
+    case GCG_ALGO_DIRECT:
+        return finish(gcg::direct_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    case GCG_ALGO_WINDOW:
+        return finish(gcg::window_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
+    case GCG_ALGO_MFMA:
+        return finish(gcg::mfma_bwd_launch(dtype, dy, x, B, C, h, dx, dB, dC, dh, workspace, dm, st));
     }
     return GCG_ERR_BAD_ARG;
 }

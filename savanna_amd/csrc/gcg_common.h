@@ -218,6 +218,10 @@ struct Dims {
     // Time-major operands (register-window kernels, separate tensors): x, B, C and dx, dB, dC are laid out
     // (L, bs, g, dg) -- the rows of one batch entry lie bs * d elements apart -- while y and dy stay (bs, L, g, dg).
     int32_t tmajor;
+    // Planar features (the split without interleaving, block.py:881-884): x, B, C are the thirds of the rows of one
+    // (bs, L, 3 * d) tensor -- C = base, B = base + d, x = base + 2 d elements, rows 3 * d elements apart -- and
+    // dC, dB, dx the thirds of its gradient; y and dy stay (bs, L, g, dg).  Separate-tensor kernels only (es = 1).
+    int32_t planar;
 };
 
 constexpr int kWave = 64;

@@ -39,6 +39,7 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(const T *__restrict__ x
     const bool cvalid = c < d;
     const int hl = dm.hl;
     const int64_t es = dm.es;   // element stride of x, B, C (3 when they are interleaved in one tensor)
+    const int64_t pad = dm.planar ? 2 * dm.d : 0;   // planar features: the three lie side by side in rows of 3 * d
     const int64_t t0 = tt * TT;
     typedef typename Filt<T>::type FT;           // element type of the filter
     const FT *hg = (const FT *)h + (cvalid ? (c / dm.dg) : 0) * hl;
@@ -58,8 +59,8 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(const T *__restrict__ x
             const int64_t time = base + row;
             float v = 0.f;
             if (time >= 0 && time < L && c0 + cc < d) {
-                const int64_t off = (b * L + time) * d + c0 + cc;
-                v = ld(B, off * es) * ld(x, off * es);
+                const int64_t off = (b * L + time) * d + c0 + cc, ioff = off * es + (b * L + time) * pad;
+                v = ld(B, ioff) * ld(x, ioff);
             }
             us[row][cc] = v;
         }
@@ -86,10 +87,10 @@ __global__ __launch_bounds__(256) void direct_fwd_kernel(const T *__restrict__ x
     for (int r = 0; r < RB; ++r) {
         const int64_t t = t0 + r0 + r;
         if (t < L) {
-            const int64_t o = (b * L + t) * d + c;
+            const int64_t o = (b * L + t) * d + c, io = o * es + (b * L + t) * pad;
             if (y2) Elem<T>::store(y2 + o, acc[r]);
-            if (bx) Elem<T>::store(bx + o, ld(B, o * es) * ld(x, o * es));
-            Elem<T>::store(y + o, ld(C, o * es) * acc[r]);
+            if (bx) Elem<T>::store(bx + o, ld(B, io) * ld(x, io));
+            Elem<T>::store(y + o, ld(C, io) * acc[r]);
         }
     }
 }
@@ -127,6 +128,7 @@ __global__ __launch_bounds__(256) void direct_bwd_kernel(const T *__restrict__ d
     const bool cvalid = c < d;
     const int hl = dm.hl, dg = dm.dg;
     const int64_t es = dm.es;   // element stride of x, B, C, dx, dB, dC
+    const int64_t pad = dm.planar ? 2 * dm.d : 0;   // planar features and gradient: rows of 3 * d
     typedef typename Filt<T>::type FT;           // element type of the filter
     const FT *hg = (const FT *)h + (cvalid ? (c / dg) : 0) * hl;
     const int64_t g0 = c0 / dg;                                            // first group in this tile
@@ -160,15 +162,15 @@ __global__ __launch_bounds__(256) void direct_bwd_kernel(const T *__restrict__ d
                 int64_t time = ubase + row;
                 float v = 0.f;
                 if (time >= 0 && time < L && cok) {
-                    const int64_t off = (b * L + time) * d + c0 + cc;
-                    v = ld(B, off * es) * ld(x, off * es);
+                    const int64_t off = (b * L + time) * d + c0 + cc, ioff = off * es + (b * L + time) * pad;
+                    v = ld(B, ioff) * ld(x, ioff);
                 }
                 us[row][cc] = v;
                 time = gbase + row;
                 v = 0.f;
                 if (time < L && cok) {
-                    const int64_t off = (b * L + time) * d + c0 + cc;
-                    v = ld(dy, off) * ld(C, off * es);
+                    const int64_t off = (b * L + time) * d + c0 + cc, ioff = off * es + (b * L + time) * pad;
+                    v = ld(dy, off) * ld(C, ioff);
                 }
                 gs[row][cc] = v;
             }
@@ -230,10 +232,10 @@ __global__ __launch_bounds__(256) void direct_bwd_kernel(const T *__restrict__ d
             for (int r = 0; r < RB; ++r) {
                 const int64_t t = t0 + r0 + r;
                 if (t < L) {
-                    const int64_t o = (b * L + t) * d + c;
-                    Elem<T>::store(dC + o * es, ld(dy, o) * y2a[r]);
-                    Elem<T>::store(dx + o * es, dua[r] * ld(B, o * es));
-                    Elem<T>::store(dB + o * es, dua[r] * ld(x, o * es));
+                    const int64_t o = (b * L + t) * d + c, io = o * es + (b * L + t) * pad;
+                    Elem<T>::store(dC + io, ld(dy, o) * y2a[r]);
+                    Elem<T>::store(dx + io, dua[r] * ld(B, io));
+                    Elem<T>::store(dB + io, dua[r] * ld(x, io));
                 }
             }
         }

@@ -28,7 +28,8 @@ namespace {
 
 // ---------------------------------------------------------------------------- forward
 // EXTRA: also write the convolution before the post-gate (y2o) and the pre-gate product (bxo).
-template <typename T, int NK, int NW, bool EXTRA>
+// PL: x, B, C are the thirds of the rows of one (bs, L, 3 d) tensor (Dims::planar): their rows lie 3 d elements apart.
+template <typename T, int NK, int NW, bool EXTRA, bool PL = false>
 __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__ x, const T *__restrict__ B,
                                                        const T *__restrict__ C, const T *__restrict__ h,
                                                        T *__restrict__ y, T *__restrict__ y2o,
@@ -68,11 +69,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
     const int64_t row_bytes = d * ES, win_bytes = (t1 - t0) * row_bytes;
     const int64_t origin = (b * L + t0) * d;
-    const win_t wx = make_window(x + origin, win_bytes), wB = make_window(B + origin, win_bytes);
-    const win_t wC = make_window(C + origin, win_bytes), wy = make_window(y + origin, win_bytes);
+    constexpr int IM = PL ? 3 : 1;                  // row stride of x, B, C in rows of y
+    const win_t wx = make_window(x + IM * origin, IM * win_bytes), wB = make_window(B + IM * origin, IM * win_bytes);
+    const win_t wC = make_window(C + IM * origin, IM * win_bytes), wy = make_window(y + origin, win_bytes);
     const win_t wy2 = make_window(EXTRA && y2o ? y2o + origin : y + origin, EXTRA && y2o ? win_bytes : 0);
     const win_t wbx = make_window(EXTRA && bxo ? bxo + origin : y + origin, EXTRA && bxo ? win_bytes : 0);
     const uint32_t lane_off = (uint32_t)(r * row_bytes + (c0 + 8 * a) * ES) + (c0 + 8 * a < d ? 0u : WIN_OFF);
+    const uint32_t lane_in = PL ? (uint32_t)(r * IM * row_bytes + (c0 + 8 * a) * ES) + (c0 + 8 * a < d ? 0u : WIN_OFF) : lane_off;
     auto step_off = [&](int64_t s) { return (uint32_t)((s * STEP - t0) * row_bytes); };
 
     op_t A[NK];            // A[(ph - i + NK) % NK]: operand of step s-i while step s runs in phase ph
@@ -99,14 +102,14 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     if constexpr (NK > 1) {
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
-            const uint32_t o = lane_off + step_off(s_lo - i);
+            const uint32_t o = lane_in + IM * step_off(s_lo - i);
             lx[i - 1] = ldw_row<T>(wx, o);
             lB[i - 1] = ldw_row<T>(wB, o);
         }
     }
     Row<T> xr, Br, Cr;
     auto fetch = [&](int64_t s, Row<T> &xo, Row<T> &Bo, Row<T> &Co) {
-        const uint32_t o = lane_off + step_off(s);
+        const uint32_t o = lane_in + IM * step_off(s);
         xo = ldw_row<T>(wx, o);
         Bo = ldw_row<T>(wB, o);
         Co = ldw_row<T>(wC, o);
@@ -205,7 +208,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 // (one 32-deep product contracts 16 channels x 2 row halves), lag = 16*delta + i - j.  At the
 // end the diagonals of the P tiles are summed in a fixed order into per-wave partials in
 // the workspace, and a second kernel adds the partials in a fixed order.
-template <typename T, int NK, int NW>
+// PL: x, B, C and dx, dB, dC are thirds of the rows of (bs, L, 3 d) tensors (Dims::planar).
+template <typename T, int NK, int NW, bool PL = false>
 __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                        const T *__restrict__ B, const T *__restrict__ C,
                                                        const T *__restrict__ h, T *__restrict__ dx,
@@ -260,11 +264,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     const int64_t t2 = (s_hi + NK - 1) * STEP < L ? (s_hi + NK - 1) * STEP : L;
     const int64_t row_bytes = d * ES, origin = (b * L + t0) * d;
     const int64_t near_bytes = (t1 - t0) * row_bytes, far_bytes = (t2 - t0) * row_bytes;
-    const win_t wx = make_window(x + origin, near_bytes), wB = make_window(B + origin, near_bytes);
-    const win_t wdy = make_window(dy + origin, far_bytes), wC = make_window(C + origin, far_bytes);
-    const win_t wdx = make_window(dx + origin, near_bytes), wdB = make_window(dB + origin, near_bytes);
-    const win_t wdC = make_window(dC + origin, near_bytes);
+    constexpr int IM = PL ? 3 : 1;                  // row stride of x, B, C, dx, dB, dC in rows of dy
+    const win_t wx = make_window(x + IM * origin, IM * near_bytes), wB = make_window(B + IM * origin, IM * near_bytes);
+    const win_t wdy = make_window(dy + origin, far_bytes), wC = make_window(C + IM * origin, IM * far_bytes);
+    const win_t wdx = make_window(dx + IM * origin, IM * near_bytes), wdB = make_window(dB + IM * origin, IM * near_bytes);
+    const win_t wdC = make_window(dC + IM * origin, IM * near_bytes);
     const uint32_t lane_off = (uint32_t)(r * row_bytes + (c0 + 8 * a) * ES) + (c0 + 8 * a < d ? 0u : WIN_OFF);
+    const uint32_t lane_in = PL ? (uint32_t)(r * IM * row_bytes + (c0 + 8 * a) * ES) + (c0 + 8 * a < d ? 0u : WIN_OFF) : lane_off;
     auto step_off = [&](int64_t sg) { return (uint32_t)((sg * STEP - t0) * row_bytes); };
 
     // While step s runs in phase ph:  Au[(ph - i + NK) % NK] is the u operand of step s-i,
@@ -295,11 +301,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
 
     // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the windows)
     auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
-        const uint32_t o = lane_off + step_off(sg), o2 = lane_off + step_off(sg + NK - 1);
+        const uint32_t o = lane_in + IM * step_off(sg), o2 = lane_off + step_off(sg + NK - 1);
         xo = ldw_row<T>(wx, o);
         Bo = ldw_row<T>(wB, o);
         dyo = ldw_row<T>(wdy, o2);
-        Co = ldw_row<T>(wC, o2);
+        Co = ldw_row<T>(wC, PL ? lane_in + IM * step_off(sg + NK - 1) : o2);
     };
 
     // Lead-in: u of the NK-1 steps before the segment and g2 of its first NK-1 steps, i.e. the
@@ -402,7 +408,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                 }
                 __syncthreads();
                 {
-                    const uint32_t o = lane_off + step_off(s);
+                    const uint32_t o = lane_in + IM * step_off(s);
                     {
                         const f32x4 p0 = *(const f32x4 *)y_rd;
                         const f32x4 p1 = *(const f32x4 *)(y_rd + 16);
@@ -448,6 +454,13 @@ int fwd_launch(const void *x, const void *B, const void *C, const void *h, void 
     // from d = 8192 on.  (The backward is 3 % faster XCD-contiguous at every width.)
     static const int order = env_int("GCG_MFMA_FWD_ORDER", -1);   // tuning override: 0 round-robin, 1 XCD-contiguous
     p.xcd = order >= 0 ? (order != 0) : (p.ncb >= 32);
+    if constexpr (NK == 5) {
+        // planar operands: instantiated for the five-slice walk only (fwd_t sends every filter length there)
+        if (dm.planar)
+            return (y2 || bx) ? (int)hipErrorInvalidValue
+                              : launch_main((mfma_fwd_kernel<T, NK, NW, false, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+                                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
+    }
     if (y2 || bx)
         e = launch_main((mfma_fwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)y, (T *)y2, (T *)bx, dm, p);
@@ -473,7 +486,7 @@ template <typename T>
 int fwd_t(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
           const Dims &dm, hipStream_t st)
 {
-    switch (nk_for(dm.hl)) {
+    switch (dm.planar ? 5 : nk_for(dm.hl)) {
     case 1: return fwd_nk<T, 1>(x, B, C, h, y, y2, bx, dm, st);
     case 2: return fwd_nk<T, 2>(x, B, C, h, y, y2, bx, dm, st);
     case 3: return fwd_nk<T, 3>(x, B, C, h, y, y2, bx, dm, st);
@@ -515,9 +528,19 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
     MfmaPlan p = plan_bwd(dm, MT<T>::SPLIT, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (p.fuse_dh) p.slot = next_dh_slot();
-    e = launch_main((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
-                       (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
-                       (T *)dh, (float *)ws, dm, p);
+    bool launched = false;
+    if constexpr (NK == 5) {
+        if (dm.planar) {        // instantiated for the five-slice walk only (bwd_t sends every filter length there)
+            e = launch_main((mfma_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
+                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
+                            (T *)dh, (float *)ws, dm, p);
+            launched = true;
+        }
+    }
+    if (!launched)
+        e = launch_main((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
+                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
+                        (T *)dh, (float *)ws, dm, p);
     if (e || p.fuse_dh) return e;
     const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
@@ -539,7 +562,7 @@ template <typename T>
 int bwd_t(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
           void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    switch (nk_for(dm.hl)) {
+    switch (dm.planar ? 5 : nk_for(dm.hl)) {
     case 1: return bwd_nk<T, 1>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     case 2: return bwd_nk<T, 2>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
     case 3: return bwd_nk<T, 3>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);

@@ -197,6 +197,54 @@ std::tuple<Tensor, Tensor> bwd_interleaved(const Tensor &dy, const Tensor &feat,
     return {dfeat, dh};
 }
 
+// ---- gated convolution on the planar features tensor (bs, L, 3, g, dg) ---------------------------
+
+void check_planar(const Tensor &feat, const Tensor &h)
+{
+    TORCH_CHECK(feat.dim() == 5 && feat.size(2) == 3 && feat.is_contiguous(),
+                "gcg: feat must be a contiguous (bs, L, 3, g, dg) tensor");
+    TORCH_CHECK(h.dim() == 3 && h.size(0) == feat.size(3) && h.size(1) == 1 && h.is_contiguous(),
+                "gcg: h must be a contiguous (g, 1, hl) tensor");
+    TORCH_CHECK(h.device() == feat.device(), "gcg: feat and h must be on one device");
+    (void)gated_code(feat, h);
+}
+
+Tensor fwd_planar(const Tensor &feat, const Tensor &h, int64_t algo)
+{
+    require_gpu(feat, "feat");
+    check_planar(feat, h);
+    DeviceGuard guard(feat.device());
+    Tensor y = at::empty({feat.size(0), feat.size(1), feat.size(3), feat.size(4)}, feat.options());
+    if (y.numel() == 0) return y;
+    check_rc(gcg_fwd_planar(feat.data_ptr(), h.data_ptr(), y.data_ptr(), feat.size(0), feat.size(1),
+                            (int32_t)feat.size(3), (int32_t)feat.size(4), (int32_t)h.size(2), gated_code(feat, h),
+                            (int32_t)algo, stream_of(feat)),
+             "gcg_fwd_planar");
+    return y;
+}
+
+std::tuple<Tensor, Tensor> bwd_planar(const Tensor &dy, const Tensor &feat, const Tensor &h, int64_t algo)
+{
+    require_gpu(feat, "feat");
+    check_planar(feat, h);
+    TORCH_CHECK(dy.dim() == 4 && dy.size(0) == feat.size(0) && dy.size(1) == feat.size(1) && dy.size(2) == feat.size(3) &&
+                    dy.size(3) == feat.size(4) && dy.scalar_type() == feat.scalar_type() && dy.device() == feat.device() &&
+                    dy.is_contiguous(),
+                "gcg: dy must be a contiguous (bs, L, g, dg) tensor of feat's dtype and device");
+    DeviceGuard guard(feat.device());
+    Tensor dfeat = at::empty_like(feat), dh = at::empty_like(h);
+    if (dy.numel() == 0) return {dfeat, dh.zero_()};
+    const int64_t bs = feat.size(0), L = feat.size(1);
+    const int32_t g = (int32_t)feat.size(3), dg = (int32_t)feat.size(4), hl = (int32_t)h.size(2);
+    const int code = gated_code(feat, h);
+    const size_t nbytes = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, code, (int32_t)algo);
+    Tensor ws = workspace(nbytes, feat, "gcg_bwd_workspace_bytes");
+    check_rc(gcg_bwd_planar(dy.data_ptr(), feat.data_ptr(), h.data_ptr(), dfeat.data_ptr(), dh.data_ptr(), ws.data_ptr(),
+                            nbytes, bs, L, g, dg, hl, code, (int32_t)algo, stream_of(feat)),
+             "gcg_bwd_planar");
+    return {dfeat, dh};
+}
+
 // ---- featurizer convolution -------------------------------------------------------------------
 
 void check_dwconv(const Tensor &x, const Tensor &w)
@@ -648,6 +696,17 @@ std::tuple<Tensor, Tensor> bwd_interleaved_meta(const Tensor &dy, const Tensor &
     (void)dy;
     return {at::empty_like(feat), at::empty_like(h)};
 }
+Tensor fwd_planar_meta(const Tensor &feat, const Tensor &h, int64_t)
+{
+    check_planar(feat, h);
+    return at::empty({feat.size(0), feat.size(1), feat.size(3), feat.size(4)}, feat.options());
+}
+std::tuple<Tensor, Tensor> bwd_planar_meta(const Tensor &dy, const Tensor &feat, const Tensor &h, int64_t)
+{
+    check_planar(feat, h);
+    (void)dy;
+    return {at::empty_like(feat), at::empty_like(h)};
+}
 Tensor dwconv_fwd_meta(const Tensor &x, const Tensor &w, bool)
 {
     check_dwconv(x, w);
@@ -775,6 +834,8 @@ TORCH_LIBRARY(gcg, m)
     m.def("bwd(Tensor dy, Tensor x, Tensor B, Tensor C, Tensor h, int algo=0) -> (Tensor, Tensor, Tensor, Tensor)");
     m.def("fwd_interleaved(Tensor feat, Tensor h, int algo=0) -> Tensor");
     m.def("bwd_interleaved(Tensor dy, Tensor feat, Tensor h, int algo=0, bool keep_output=False) -> (Tensor, Tensor)");
+    m.def("fwd_planar(Tensor feat, Tensor h, int algo=0) -> Tensor");
+    m.def("bwd_planar(Tensor dy, Tensor feat, Tensor h, int algo=0) -> (Tensor, Tensor)");
     m.def("dwconv_fwd(Tensor x, Tensor w, bool keep_output=False) -> Tensor");
     m.def("dwconv_bwd(Tensor dy, Tensor x, Tensor w) -> (Tensor, Tensor)");
     m.def("mixer_se_fwd(Tensor raw, Tensor wf, Tensor h) -> Tensor");
@@ -804,6 +865,8 @@ TORCH_LIBRARY_IMPL(gcg, CUDA, m)
     m.impl("bwd", &bwd);
     m.impl("fwd_interleaved", &fwd_interleaved);
     m.impl("bwd_interleaved", &bwd_interleaved);
+    m.impl("fwd_planar", &fwd_planar);
+    m.impl("bwd_planar", &bwd_planar);
     m.impl("dwconv_fwd", &dwconv_fwd);
     m.impl("dwconv_bwd", &dwconv_bwd);
     m.impl("mixer_se_fwd", &mixer_se_fwd);
@@ -830,6 +893,8 @@ TORCH_LIBRARY_IMPL(gcg, Meta, m)
     m.impl("bwd", &bwd_meta);
     m.impl("fwd_interleaved", &fwd_interleaved_meta);
     m.impl("bwd_interleaved", &bwd_interleaved_meta);
+    m.impl("fwd_planar", &fwd_planar_meta);
+    m.impl("bwd_planar", &bwd_planar_meta);
     m.impl("dwconv_fwd", &dwconv_fwd_meta);
     m.impl("dwconv_bwd", &dwconv_bwd_meta);
     m.impl("mixer_se_fwd", &mixer_se_fwd_meta);

@@ -106,8 +106,9 @@ __global__ __launch_bounds__(256) void window_fwd_kernel(const T *__restrict__ x
     const int64_t origin = (b * L + t0) * d, rows = t_end - t0;
     // time-major inputs: the rows of this batch entry lie bs rows apart (a window then spans the other
     // entries' rows in between, which no offset of this lane reaches)
-    const int64_t in_origin = dm.tmajor ? (t0 * dm.bs + b) * d : origin;
-    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow * (uint32_t)(dm.tmajor ? dm.bs : 1);   // bytes per row: outputs, inputs
+    // planar inputs: the thirds of rows of 3 d elements (a window then spans the other thirds in between as well)
+    const int64_t in_origin = dm.tmajor ? (t0 * dm.bs + b) * d : dm.planar ? 3 * origin : origin;
+    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow * (uint32_t)(dm.tmajor ? dm.bs : dm.planar ? 3 : 1);   // bytes per row: outputs, inputs
     const win_t wx = make_window((PK ? C : x) + IS * in_origin, rows * irow);
     const win_t wB = make_window(B + in_origin, PK ? 0 : rows * irow), wC = make_window(C + in_origin, PK ? 0 : rows * irow);
     const win_t wy = make_window(y + origin, rows * orow);
@@ -235,9 +236,10 @@ __global__ __launch_bounds__(256) void window_bwd_kernel(const T *__restrict__ d
     const int64_t t_far = t_stop < L ? t_stop : L;
     const int64_t origin = (b * L + t0) * d;
     // time-major x, B, C, dx, dB, dC: the rows of this batch entry lie bs rows apart
-    const int64_t in_origin = dm.tmajor ? (t0 * dm.bs + b) * d : origin;
-    const int64_t out_origin = dm.tmajor ? (t_start * dm.bs + b) * d : (b * L + t_start) * d;
-    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow * (uint32_t)(dm.tmajor ? dm.bs : 1);
+    // (planar x, B, C, dx, dB, dC: the thirds of rows of 3 d elements)
+    const int64_t in_origin = dm.tmajor ? (t0 * dm.bs + b) * d : dm.planar ? 3 * origin : origin;
+    const int64_t out_origin = dm.tmajor ? (t_start * dm.bs + b) * d : (b * L + t_start) * d * (dm.planar ? 3 : 1);
+    const uint32_t orow = (uint32_t)(d * ES), irow = IS * orow * (uint32_t)(dm.tmajor ? dm.bs : dm.planar ? 3 : 1);
     // PK: wx is the interleaved tensor and reaches as far as dy (C is part of it)
     const win_t wx = make_window((PK ? C : x) + IS * in_origin, ((PK ? t_far : t_end) - t0) * irow);
     const win_t wB = make_window(B + in_origin, PK ? 0 : (t_end - t0) * irow);
@@ -399,7 +401,7 @@ WinPlan plan(const Dims &dm, int v)
     static const char *env = getenv("GCG_WINDOW_ROWS");   // tuning override: rows per lane, a multiple of 8
     if (env && atoi(env) >= 8 && atoi(env) % 8 == 0) p.ts = atoi(env);
     // the rows of a run, its halo and an interleaved fp32 row width must fit one tensor window
-    while (p.ts > 8 && (int64_t)(p.ts + 2 * RING) * 3 * dm.d * 4 * (dm.tmajor ? dm.bs : 1) > WIN_MAX_BYTES) p.ts >>= 1;
+    while (p.ts > 8 && (int64_t)(p.ts + 2 * RING) * 3 * dm.d * 4 * (dm.tmajor ? dm.bs : 1) > WIN_MAX_BYTES) p.ts >>= 1;   // (planar rows are 3 d wide too)
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);
     p.nthreads = dm.bs * p.nseg * p.nvec;       // workspace slots (one per lane with work)
     p.threads = p.nvec >= 256 ? 256 : ((p.nvec + 63) / 64) * 64;   // narrow tensors: fewer idle lanes
@@ -495,7 +497,8 @@ int bwd_hl(const void *dy, const void *x, const void *B, const void *C, const vo
 bool window_supported(const Dims &dm)
 {
     return dm.hl <= RING && dm.dg % 4 == 0 && (int64_t)dm.g * dm.hl <= 0x7fffffffLL &&
-           (int64_t)(3 * RING) * 3 * dm.d * 4 * (dm.tmajor ? dm.bs : 1) <= WIN_MAX_BYTES && !(dm.tmajor && dm.es == 3);
+           (int64_t)(3 * RING) * 3 * dm.d * 4 * (dm.tmajor ? dm.bs : 1) <= WIN_MAX_BYTES && !(dm.tmajor && dm.es == 3) &&
+           !(dm.planar && (dm.es == 3 || dm.tmajor));
 }
 
 int window_fwd_launch(int dtype, const void *x, const void *B, const void *C, const void *h, void *y,

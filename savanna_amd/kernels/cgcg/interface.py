@@ -46,6 +46,32 @@ def interleaved_source(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor):
     return torch.as_strided(C, (bs, L, g, dg, 3), want + (1,), o)
 
 
+def planar_source(x: torch.Tensor, B: torch.Tensor, C: torch.Tensor):
+    """The (bs, L, 3, g, dg) tensor whose thirds [:, :, 0], [:, :, 1], [:, :, 2] are C, B, x, or None.
+
+    The split without interleaving (savanna/model/block.py:881-884,
+    ``rearrange(features, "b l (p g dg) -> b l p g dg", p=3).unbind(dim=2)`` -> x1, x2, v, passed on as C, B, x;
+    interleave_projections = false) hands the operator three views whose rows lie 3 * g * dg elements apart.
+    """
+    if not (x.shape == B.shape == C.shape and x.dim() == 4 and x.dtype == B.dtype == C.dtype):
+        return None
+    if not (x.device == B.device == C.device):
+        return None
+    bs, L, g, dg = x.shape
+    d = g * dg
+    want = (L * 3 * d, 3 * d, dg, 1)
+    for t in (x, B, C):
+        if any(n > 1 and st != w for n, st, w in zip(t.shape, t.stride(), want)):
+            return None
+    base = C.untyped_storage().data_ptr()
+    if x.untyped_storage().data_ptr() != base or B.untyped_storage().data_ptr() != base:
+        return None
+    o = C.storage_offset()
+    if B.storage_offset() != o + d or x.storage_offset() != o + 2 * d:
+        return None
+    return torch.as_strided(C, (bs, L, 3, g, dg), (L * 3 * d, 3 * d, d, dg, 1), o)
+
+
 class TwoPassChunkedGateConvGate(torch.autograd.Function):
     """y = C * conv(B * x, h); saves only the four inputs (the reference also saves
     Bx and y2, interface.py:79 -- here they are recomputed in the backward kernel)."""
@@ -59,17 +85,20 @@ class TwoPassChunkedGateConvGate(torch.autograd.Function):
         ctx.input_shape = (bs, seqlen, g, dg)
         # (under torch.compile the storage test cannot be traced: compiled callers that hold the features tensor
         # call two_pass_chunked_gate_conv_gate_interleaved)
-        feat = interleaved_source(x, B, C) if x.numel() > 0 and not torch.compiler.is_compiling() else None
+        tracing = torch.compiler.is_compiling()
+        feat = interleaved_source(x, B, C) if x.numel() > 0 and not tracing else None
         ctx.interleaved = feat is not None
-        if feat is not None:
-            # three views of one interleaved buffer: no gathers, one fused read
+        planar = planar_source(x, B, C) if feat is None and x.numel() > 0 and g * dg > 1 and not tracing else None
+        ctx.planar = planar is not None
+        if feat is not None or planar is not None:
+            # three views of one buffer (interleaved elements, or the thirds of its rows): no gathers
             assert h.dim() == 3 and h.shape[0] == g and h.shape[1] == 1, "h must be (g, 1, hl)"
             if schedule != "default":
                 raise NotImplementedError("Skip persistent for now") if schedule == "persistent" else \
                     ValueError(f"schedule {schedule} not implemented")
             h = _contig(h)
-            y = _lib.fwd_interleaved(feat, h)
-            ctx.save_for_backward(feat, h)
+            y = _lib.fwd_interleaved(feat, h) if feat is not None else _lib.fwd_planar(planar, h)
+            ctx.save_for_backward(feat if feat is not None else planar, h)
             return y
         x, B, C, h = _contig(x), _contig(B), _contig(C), _contig(h)
         _, _, y = two_pass_fwd_grouped(x, B, C, h, autotune=fwd_autotune, schedule=schedule,
@@ -83,6 +112,10 @@ class TwoPassChunkedGateConvGate(torch.autograd.Function):
             feat, h = ctx.saved_tensors
             dfeat, dh = _lib.bwd_interleaved(_contig(dy), feat, h)
             return (dfeat[..., 2], dfeat[..., 1], dfeat[..., 0], dh) + (None,) * 10
+        if ctx.planar:
+            feat, h = ctx.saved_tensors
+            dfeat, dh = _lib.bwd_planar(_contig(dy), feat, h)
+            return (dfeat[:, :, 2], dfeat[:, :, 1], dfeat[:, :, 0], dh) + (None,) * 10
         x, B, C, h = ctx.saved_tensors
         bs, seqlen, g, dg = ctx.input_shape
         dx, dB, dC, dh = two_pass_bwd_refactor(dy=_contig(dy), x=x, B=B, C=C, h=h,
@@ -150,6 +183,35 @@ def two_pass_chunked_gate_conv_gate_interleaved(features: torch.Tensor, h: torch
     assert features.numel() == bs * seqlen * g * dg * 3, "features must hold 3*g*dg values per position"
     assert h.dim() == 3 and h.shape[0] == g and h.shape[1] == 1, "h must be (g, 1, hl)"
     return InterleavedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3), h, keep_dfeatures)
+
+
+class PlanarGateConvGate(torch.autograd.Function):
+    """The same operator on the planar features tensor (bs, L, 3, g, dg) itself: the kernels read the thirds of each
+    row in place and the backward writes the gradient in the same layout."""
+
+    @staticmethod
+    def forward(ctx, feat, h):
+        feat, h = _contig(feat), _contig(h)
+        ctx.save_for_backward(feat, h)
+        return _lib.fwd_planar(feat, h)
+
+    @staticmethod
+    def backward(ctx, dy):
+        feat, h = ctx.saved_tensors
+        return _lib.bwd_planar(_contig(dy), feat, h)
+
+
+def two_pass_chunked_gate_conv_gate_planar(features: torch.Tensor, h: torch.Tensor,
+                                           bs: int, seqlen: int, g: int, dg: int) -> torch.Tensor:
+    """y = x1 * conv(x2 * v, h) for projected features laid out "(p g dg)" with p = (x1, x2, v) slowest, i.e. the
+    tensor savanna/model/block.py:881-884 splits when interleave_projections is off.
+
+    features: (bs, seqlen, 3*g*dg) or (bs, seqlen, 3, g, dg); h: (g, 1, hl).  Returns (bs, seqlen, g, dg).
+    Equivalent to ``two_pass_chunked_gate_conv_gate(x=v, B=x2, C=x1, h=h, ...)`` on the split views.
+    """
+    assert features.numel() == bs * seqlen * g * dg * 3, "features must hold 3*g*dg values per position"
+    assert h.dim() == 3 and h.shape[0] == g and h.shape[1] == 1, "h must be (g, 1, hl)"
+    return PlanarGateConvGate.apply(features.reshape(bs, seqlen, 3, g, dg), h)
 
 
 class DecayedGateConvGate(torch.autograd.Function):

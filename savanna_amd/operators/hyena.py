@@ -27,7 +27,8 @@ import torch.nn as nn
 
 from .. import _lib
 from ..kernels.cgcg.interface import (DecayedGateConvGate, InterleavedDecayedGateConvGate,
-                                       two_pass_chunked_gate_conv_gate, two_pass_chunked_gate_conv_gate_interleaved)
+                                       two_pass_chunked_gate_conv_gate, two_pass_chunked_gate_conv_gate_interleaved,
+                                       two_pass_chunked_gate_conv_gate_planar)
 from ..kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
 
 _DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "float16": torch.float16}
@@ -181,15 +182,26 @@ class _CgcgOperatorBase(nn.Module):
         """16-bit activations with ``cgcg_dtype`` float32 on the GPU: one kernel instead of casts around it."""
         return self.cgcg_dtype == torch.float32 and dtype in (torch.bfloat16, torch.float16) and t.is_cuda
 
-    def forward_features(self, features: torch.Tensor, from_featurizer: bool = False) -> torch.Tensor:
+    def forward_features(self, features: torch.Tensor, from_featurizer: bool = False,
+                         interleaved: bool = True) -> torch.Tensor:
         """The same on the projected features before their split: (b, l, 3*g*dg) laid out
         "(g dg p)" with p = (x1, x2, v) fastest (block.py:886-888) -> z: (b, l, g*dg).  The kernels
         read the tensor as it is and the backward writes its gradient in the same layout.
-        ``from_featurizer``: the gradient goes straight into the featurizer's backward (cache hint)."""
+        ``from_featurizer``: the gradient goes straight into the featurizer's backward (cache hint).
+        ``interleaved=False``: the layout is "(p g dg)", the split of block.py:881-884 for checkpoints trained
+        without interleaving; the kernels then read the thirds of each row in place."""
         dtype = features.dtype
         bs, seqlen, d3 = features.shape
         g, dg = self.num_groups, self.group_dim
         assert d3 == 3 * g * dg
+        if not interleaved:
+            h = self._filter(seqlen)
+            cast = self.cgcg_dtype != dtype and not self._fp32_inside(dtype, features)
+            if cast:
+                features = features.to(self.cgcg_dtype)
+            z = two_pass_chunked_gate_conv_gate_planar(features, h.to(self.cgcg_dtype), bs, seqlen, g, dg)
+            z = z.reshape(bs, seqlen, g * dg)
+            return z.to(dtype) if cast else z
         fused = self._filter_in_kernel(seqlen, g, dg, dtype, features)
         if fused is not None:
             hl, filt = fused
@@ -365,14 +377,16 @@ class HyenaMixer(nn.Module):
     differs from the two-kernel chain by the rounding of fp32 sums only.  With a Hyena-MR filter
     (9 to 128 taps) and a featurizer of at most 3 taps the featurized tensor is never stored (``fuse_medium``):
     the operator's kernels make its rows from the projection output, forward and backward, with the chain's results,
-    and form the decayed filter themselves where the operator allows it (``HyenaMROperator.fuse_filter``)."""
+    and form the decayed filter themselves where the operator allows it (``HyenaMROperator.fuse_filter``).
+    ``interleave_projections=False`` takes the features laid out "(p g dg)" instead (block.py:881-884)."""
 
     def __init__(self, operator: _CgcgOperatorBase, short_conv_L: int = 3, dtype=torch.float32, device=None,
-                 fuse_short: bool = True, fuse_medium: bool = True):
+                 fuse_short: bool = True, fuse_medium: bool = True, interleave_projections: bool = True):
         super().__init__()
         self.mixer = operator
         self.fuse_short = fuse_short
         self.fuse_medium = fuse_medium
+        self.interleave_projections = interleave_projections        # global_config.py:270
         self.hyena_proj_conv = CausalDepthwiseConv1d(3 * operator.hidden_size, short_conv_L, dtype=dtype, device=device)
 
     def _fusable(self, features: torch.Tensor, hl: int) -> bool:
@@ -384,6 +398,9 @@ class HyenaMixer(nn.Module):
         op = self.mixer
         bs, seqlen, d3 = features.shape
         conv = self.hyena_proj_conv
+        if not self.interleave_projections:
+            # "(p g dg)" features: featurizer kernel, then the operator on the thirds of its rows (two kernels each way)
+            return op.forward_features(conv.forward_bld(features, feeds_operator=True), interleaved=False)
         fused = op._filter_in_kernel(seqlen, op.num_groups, op.group_dim, features.dtype, features)
         if (fused is not None and self.fuse_medium and conv.group_dim == 1 and
                 _lib.mixer_mr_supported(op.group_dim, fused[0], conv.kernel_size, features)):

@@ -27,6 +27,7 @@ class Workload:
     dtype: torch.dtype
     backward: bool
     about: str
+    # "planar": q, k, v are the thirds of the rows of one (bs, L, 3, g, dg) tensor, read in place.
     # "separate": q, k, v are three contiguous tensors.  "interleaved": they are the thirds of one
     # (bs, L, g, dg, 3) projected-features tensor and the kernels read it as it is.  "gathered": same
     # features tensor, handled the way the reference does (three strided gathers before the forward,
@@ -99,6 +100,13 @@ WORKLOADS = {
     "se_fwdbwd_40b_interleaved": Workload("se_fwdbwd_40b_interleaved", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
                                           "Hyena-SE forward+backward on interleaved features, bf16, B=1 L=32768 "
                                           "D=8192 G=512 hl=7", layout="interleaved"),
+    # the same two on planar features, the split without interleaving (block.py:881-884, interleave_projections = false)
+    "mr_fwdbwd_7b_planar": Workload("mr_fwdbwd_7b_planar", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
+                                    "Hyena-MR forward+backward on planar features (the thirds of each row read in "
+                                    "place), bf16, B=2 L=8192 D=4096 G=256 hl=128", layout="planar"),
+    "se_fwdbwd_40b_planar": Workload("se_fwdbwd_40b_planar", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
+                                     "Hyena-SE forward+backward on planar features, bf16, B=1 L=32768 D=8192 G=512 "
+                                     "hl=7", layout="planar"),
     "se_fwdbwd_40b_gathered": Workload("se_fwdbwd_40b_gathered", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
                                        "the same with three gathers, separate-tensor kernels and re-assembly",
                                        layout="gathered"),

@@ -44,6 +44,10 @@ def test_meta_shapes_on_fake_gpu_tensors(gcg_lib):
         hh = torch.ops.gcg.filter_decay_fwd(p, p, 64, torch.float16)
         assert hh.shape == (g, 1, 64) and hh.dtype == torch.float16
         assert torch.ops.gcg.filter_decay_bwd(hh, p).shape == p.shape
+        planar = torch.empty(bs, L, 3, g, dg, dtype=torch.bfloat16, device="cuda")
+        assert torch.ops.gcg.fwd_planar(planar, h).shape == x.shape
+        dplanar, dh = torch.ops.gcg.bwd_planar(x, planar, h)
+        assert dplanar.shape == planar.shape and dh.shape == h.shape
         # Hyena-MR mixer (featurizer + operator), with the filter given and with the filter formed in the kernels
         assert torch.ops.gcg.mixer_mr_fwd(feat, wf, h).shape == x.shape
         draw, dwf, dh = torch.ops.gcg.mixer_mr_bwd(x, feat, wf, h)

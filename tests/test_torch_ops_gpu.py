@@ -71,6 +71,9 @@ def test_library_opcheck(gcg_lib):
     torch.library.opcheck(torch.ops.gcg.fwd_interleaved, (feat, h), test_utils=checks)
     torch.library.opcheck(torch.ops.gcg.bwd_interleaved, (dy, feat, h), test_utils=checks)
     torch.library.opcheck(torch.ops.gcg.fwd_out, (x, B, C, h, torch.empty_like(x)), test_utils=checks)
+    planar = torch.stack([C, B, x], dim=2).contiguous()
+    torch.library.opcheck(torch.ops.gcg.fwd_planar, (planar, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.bwd_planar, (dy, planar, h), test_utils=checks)
     # the Hyena-MR mixer operators, with the filter given and formed in the kernels
     x, B, C, h, dy = (t.to(DEV) for t in inputs(1, 130, 2, 16, 128, torch.bfloat16))
     feat = torch.stack([C, B, x], dim=-1).contiguous()
