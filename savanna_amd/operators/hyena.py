@@ -27,7 +27,8 @@ import torch.nn as nn
 
 from .. import _lib
 from ..kernels.cgcg.interface import (DecayedGateConvGate, InterleavedDecayedGateConvGate,
-                                       two_pass_chunked_gate_conv_gate, two_pass_chunked_gate_conv_gate_interleaved,
+                                       planar_source, two_pass_chunked_gate_conv_gate,
+                                       two_pass_chunked_gate_conv_gate_interleaved,
                                        two_pass_chunked_gate_conv_gate_planar)
 from ..kernels.cgcg.src.kernel_utils import BwdKernelConfigRefactor, FwdKernelConfigRefactor
 
@@ -238,6 +239,9 @@ class HyenaMROperator(_CgcgOperatorBase):
         hl = min(self.hyena_mr_len, L)
         if not _lib.decay_supported(g, dg, hl, *tensors):
             return None
+        if len(tensors) == 3 and not torch.compiler.is_compiling() and \
+                planar_source(tensors[2], tensors[1], tensors[0]) is not None:
+            return None         # the split without interleaving: the planar entry points take an explicit filter
         return hl, self.cgcg_dtype
 
     def _filter(self, L: int) -> torch.Tensor:

@@ -224,3 +224,31 @@ def test_mixer_without_interleaving(gcg_lib, kind):
     want = [z_ref.detach(), feats.grad.clone()] + [p.grad.clone() for p in mixer.parameters()]
     for a, b, n in zip(got, want, ["z", "d features"] + [n for n, _ in mixer.named_parameters()]):
         assert_close(a, b, 2e-2 if n != "z" else 1e-2, n)
+
+
+@pytest.mark.parametrize("kind", ["mr", "se"])
+def test_operator_modules_read_planar_views_in_place(gcg_lib, monkeypatch, kind):
+    """HyenaMROperator / HyenaSEOperator called as ParallelSequenceMixer does, on the three views of the split
+    without interleaving: the planar kernels run (no gathers), for Hyena-MR with its filter from one small launch."""
+    from savanna_amd.operators.hyena import CgcgConfig, HyenaMROperator, HyenaSEOperator
+
+    calls = {"planar": 0, "plain": 0, "decay": 0}
+    real_pl, real_p, real_d = _lib.fwd_planar, _lib.fwd, _lib.fwd_decay
+    monkeypatch.setattr(interface._lib, "fwd_planar",
+                        lambda *a, **k: (calls.__setitem__("planar", calls["planar"] + 1), real_pl(*a, **k))[1])
+    monkeypatch.setattr(interface._lib, "fwd",
+                        lambda *a, **k: (calls.__setitem__("plain", calls["plain"] + 1), real_p(*a, **k))[1])
+    monkeypatch.setattr(interface._lib, "fwd_decay",
+                        lambda *a, **k: (calls.__setitem__("decay", calls["decay"] + 1), real_d(*a, **k))[1])
+    torch.manual_seed(5)
+    bs, L, hidden, groups = 2, 256, 128, 8
+    cfg = CgcgConfig(cgcg_dtype="bfloat16")
+    op = (HyenaMROperator(hidden, groups, 128, cfg, small_init=False, device=DEV) if kind == "mr"
+          else HyenaSEOperator(hidden, groups, 7, cfg, device=DEV))
+    feats = torch.randn(bs, L, 3 * hidden, device=DEV).to(torch.bfloat16)
+    x1, x2, v = rearrange(feats, "b l (p g dg) -> b l p g dg", p=3, g=groups).unbind(dim=2)
+    z = op(x1, x2, v)
+    z_ref = op(x1.contiguous(), x2.contiguous(), v.contiguous())
+    torch.cuda.synchronize()
+    assert calls["planar"] == 1 and calls["plain"] + calls["decay"] == 1, calls
+    assert torch.equal(z, z_ref)
