@@ -303,6 +303,20 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
             int32_t dtype, void *stream);
 
 /*
+ * The same two on planar features -- the split without interleaving of savanna/model/block.py:881-884
+ * (interleave_projections = false): raw and draw are (bs, L, 3, g, dg), each row the planes C | B | x one after the
+ * other, and wf, dwf hold their 3 * g * dg filters in that channel order.  Same workspace size.
+ */
+GCG_API int gcg_mixer_se_fwd_planar(const void *raw, const void *wf, const void *h, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+GCG_API int gcg_mixer_se_bwd_planar(const void *dy, const void *raw, const void *wf, const void *h,
+            void *draw, void *dwf, void *dh,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+
+/*
  * Featurizer and Hyena-MR operator without the featurized tensor: gcg_dwconv_fwd followed by
  * gcg_fwd_interleaved as one kernel that makes every row of (C, B, x) on the way
  * (savanna/model/block.py:867-890 -> hyena.py:517-531), and a backward that needs the projection output only.

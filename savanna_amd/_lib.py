@@ -34,6 +34,7 @@ EXPORTS = (
     "gcg_fwd_interleaved", "gcg_bwd_interleaved", "gcg_fwd_planar", "gcg_bwd_planar",
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
+    "gcg_mixer_se_fwd_planar", "gcg_mixer_se_bwd_planar",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
     "gcg_mixer_mr_fwd", "gcg_mixer_mr_bwd_workspace_bytes", "gcg_mixer_mr_bwd_scratch_bytes", "gcg_mixer_mr_bwd", "gcg_mixer_mr_fwd_decay", "gcg_mixer_mr_bwd_decay", "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
     "gcg_fwd_decay", "gcg_bwd_decay", "gcg_fwd_interleaved_decay", "gcg_bwd_interleaved_decay",
@@ -100,6 +101,10 @@ def load() -> ctypes.CDLL:
         lib.gcg_mixer_se_bwd_workspace_bytes.restype = sz
         lib.gcg_mixer_se_bwd.argtypes = [vp] * 8 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_mixer_se_bwd.restype = ctypes.c_int
+        lib.gcg_mixer_se_fwd_planar.argtypes = lib.gcg_mixer_se_fwd.argtypes
+        lib.gcg_mixer_se_fwd_planar.restype = ctypes.c_int
+        lib.gcg_mixer_se_bwd_planar.argtypes = lib.gcg_mixer_se_bwd.argtypes
+        lib.gcg_mixer_se_bwd_planar.restype = ctypes.c_int
         lib.gcg_filter_decay_fwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
         lib.gcg_filter_decay_fwd.restype = ctypes.c_int
         lib.gcg_filter_decay_bwd.argtypes = [vp] * 3 + [i32, i32, i32, i32, vp]
@@ -463,10 +468,11 @@ def dwconv_bwd(dy, x, w):
     return dx, dw
 
 
-def _check_mixer_se(raw, wf, h):
-    if raw.dim() != 5 or raw.shape[-1] != 3 or not raw.is_contiguous():
-        raise ValueError("raw must be a contiguous (bs, L, g, dg, 3) tensor")
-    bs, L, g, dg, _ = raw.shape
+def _check_mixer_se(raw, wf, h, planar=False):
+    if raw.dim() != 5 or raw.shape[2 if planar else 4] != 3 or not raw.is_contiguous():
+        raise ValueError("raw must be a contiguous (bs, L, 3, g, dg) tensor" if planar
+                         else "raw must be a contiguous (bs, L, g, dg, 3) tensor")
+    g, dg = (raw.shape[3], raw.shape[4]) if planar else (raw.shape[2], raw.shape[3])
     if wf.dim() != 3 or wf.shape[0] != 3 * g * dg or wf.shape[1] != 1 or not wf.is_contiguous():
         raise ValueError("wf must be a contiguous (3 * g * dg, 1, kf) tensor")
     if h.dim() != 3 or h.shape[0] != g or h.shape[1] != 1 or not h.is_contiguous():
@@ -476,33 +482,37 @@ def _check_mixer_se(raw, wf, h):
             raise ValueError("raw, wf and h must share dtype and device")
 
 
-def mixer_se_fwd(raw, wf, h):
-    """y (bs, L, g, dg) = fwd_interleaved(dwconv_fwd(raw, wf), h) in one pass over raw (bs, L, g, dg, 3)."""
+def mixer_se_fwd(raw, wf, h, planar=False):
+    """y (bs, L, g, dg) = fwd_interleaved(dwconv_fwd(raw, wf), h) in one pass over raw (bs, L, g, dg, 3);
+    ``planar``: raw is (bs, L, 3, g, dg), the split without interleaving (block.py:881-884)."""
     _require_gpu(raw)
     if TORCH_OPS:
-        return torch.ops.gcg.mixer_se_fwd(raw, wf, h)
+        return torch.ops.gcg.mixer_se_fwd(raw, wf, h, bool(planar))
     lib = load()
-    _check_mixer_se(raw, wf, h)
-    bs, L, g, dg, _ = raw.shape
+    _check_mixer_se(raw, wf, h, planar)
+    bs, L = raw.shape[:2]
+    g, dg = (raw.shape[3], raw.shape[4]) if planar else (raw.shape[2], raw.shape[3])
     y = torch.empty(bs, L, g, dg, dtype=raw.dtype, device=raw.device)
     if y.numel() == 0:
         return y
+    fn = lib.gcg_mixer_se_fwd_planar if planar else lib.gcg_mixer_se_fwd
     with _on_device(raw.device):
         st = torch.cuda.current_stream().cuda_stream
-        rc = lib.gcg_mixer_se_fwd(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg,
-                                  h.shape[-1], wf.shape[-1], dtype_code(raw.dtype), st)
-    check(rc, "gcg_mixer_se_fwd")
+        rc = fn(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg,
+                h.shape[-1], wf.shape[-1], dtype_code(raw.dtype), st)
+    check(rc, "gcg_mixer_se_fwd_planar" if planar else "gcg_mixer_se_fwd")
     return y
 
 
-def mixer_se_bwd(dy, raw, wf, h):
+def mixer_se_bwd(dy, raw, wf, h, planar=False):
     """(draw, dwf, dh) of mixer_se_fwd."""
     _require_gpu(raw)
     if TORCH_OPS:
-        return torch.ops.gcg.mixer_se_bwd(dy, raw, wf, h)
+        return torch.ops.gcg.mixer_se_bwd(dy, raw, wf, h, bool(planar))
     lib = load()
-    _check_mixer_se(raw, wf, h)
-    bs, L, g, dg, _ = raw.shape
+    _check_mixer_se(raw, wf, h, planar)
+    bs, L = raw.shape[:2]
+    g, dg = (raw.shape[3], raw.shape[4]) if planar else (raw.shape[2], raw.shape[3])
     if dy.shape != (bs, L, g, dg) or dy.dtype != raw.dtype or not dy.is_contiguous() or dy.device != raw.device:
         raise ValueError("dy must be a contiguous (bs, L, g, dg) tensor of raw's dtype and device")
     hl, kf = h.shape[-1], wf.shape[-1]
@@ -516,10 +526,10 @@ def mixer_se_bwd(dy, raw, wf, h):
     with _on_device(raw.device):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
         st = torch.cuda.current_stream().cuda_stream
-        rc = lib.gcg_mixer_se_bwd(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
-                                  dwf.data_ptr(), dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl, kf,
-                                  code, st)
-    check(rc, "gcg_mixer_se_bwd")
+        fn = lib.gcg_mixer_se_bwd_planar if planar else lib.gcg_mixer_se_bwd
+        rc = fn(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
+                dwf.data_ptr(), dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl, kf, code, st)
+    check(rc, "gcg_mixer_se_bwd_planar" if planar else "gcg_mixer_se_bwd")
     return draw, dwf, dh
 
 

@@ -555,19 +555,52 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
 
 // ---- featurizer + Hyena-SE operator in one pass
 
-GCG_API int gcg_mixer_se_fwd(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L, int32_t g,
-                             int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+namespace {
+int mixer_se_fwd_any(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L, int32_t g,
+                     int32_t dg, int32_t hl, int32_t kf, int32_t dtype, int planar, void *stream)
 {
-    TimerScope timer_scope;
     if (!raw || !wf || !h || !y) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
     int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
     if (rc) return rc;
     if (kf <= 0) return GCG_ERR_BAD_ARG;
+    dm.planar = planar;
     if (!gcg::mixer_se_supported(dm, kf) || !all_aligned16({raw, y})) return GCG_ERR_UNSUPPORTED;
     rc = check_device();
     if (rc) return rc;
     return finish(gcg::mixer_se_fwd_launch(dtype, raw, wf, h, y, dm, kf, (hipStream_t)stream));
+}
+int mixer_se_bwd_any(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf, void *dh,
+                     void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                     int32_t kf, int32_t dtype, int planar, void *stream)
+{
+    if (!dy || !raw || !wf || !h || !draw || !dwf || !dh) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    if (rc) return rc;
+    if (kf <= 0) return GCG_ERR_BAD_ARG;
+    dm.planar = planar;
+    if (!gcg::mixer_se_supported(dm, kf) || !all_aligned16({dy, raw, draw})) return GCG_ERR_UNSUPPORTED;
+    const size_t need = gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, dtype);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
+    rc = check_device();
+    if (rc) return rc;
+    return finish(gcg::mixer_se_bwd_launch(dtype, dy, raw, wf, h, draw, dwf, dh, workspace, dm, kf, (hipStream_t)stream));
+}
+} // namespace
+
+GCG_API int gcg_mixer_se_fwd(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L, int32_t g,
+                             int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    return mixer_se_fwd_any(raw, wf, h, y, bs, L, g, dg, hl, kf, dtype, 0, stream);
+}
+
+GCG_API int gcg_mixer_se_fwd_planar(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L,
+                                    int32_t g, int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    return mixer_se_fwd_any(raw, wf, h, y, bs, L, g, dg, hl, kf, dtype, 1, stream);
 }
 
 GCG_API size_t gcg_mixer_se_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
@@ -583,17 +616,17 @@ GCG_API int gcg_mixer_se_bwd(const void *dy, const void *raw, const void *wf, co
                              int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
 {
     TimerScope timer_scope;
-    if (!dy || !raw || !wf || !h || !draw || !dwf || !dh) return GCG_ERR_BAD_ARG;
-    gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
-    if (rc) return rc;
-    if (kf <= 0) return GCG_ERR_BAD_ARG;
-    if (!gcg::mixer_se_supported(dm, kf) || !all_aligned16({dy, raw, draw})) return GCG_ERR_UNSUPPORTED;
-    const size_t need = gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, dtype);
-    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;
-    rc = check_device();
-    if (rc) return rc;
-    return finish(gcg::mixer_se_bwd_launch(dtype, dy, raw, wf, h, draw, dwf, dh, workspace, dm, kf, (hipStream_t)stream));
+    return mixer_se_bwd_any(dy, raw, wf, h, draw, dwf, dh, workspace, workspace_bytes, bs, L, g, dg, hl, kf, dtype, 0,
+                            stream);
+}
+
+GCG_API int gcg_mixer_se_bwd_planar(const void *dy, const void *raw, const void *wf, const void *h, void *draw,
+                                    void *dwf, void *dh, void *workspace, size_t workspace_bytes, int64_t bs, int64_t L,
+                                    int32_t g, int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    return mixer_se_bwd_any(dy, raw, wf, h, draw, dwf, dh, workspace, workspace_bytes, bs, L, g, dg, hl, kf, dtype, 1,
+                            stream);
 }
 
 // ---- featurizer and Hyena-MR operator: the forward in one pass

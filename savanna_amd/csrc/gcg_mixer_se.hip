@@ -72,15 +72,42 @@ template <typename T> struct Piece {
     static __device__ __forceinline__ void unpack_unit(uint32_t w, float (&f)[CH]) { Word<T>::unpack(w, f); }
 };
 
+// Planar features (PL; the split without interleaving, block.py:881-884): a row holds the planes C | B | x one after
+// the other, d elements each, instead of (C, B, x) channel by channel.  A lane's piece is then three words orow
+// bytes apart and its elements come plane by plane (at 16 bits: C0 C1 | B0 B1 | x0 x1), which is all that differs:
+// where an element sits in the piece, which feature channel it is, and how the piece is loaded and stored.
+template <bool PL, int CH> __device__ __forceinline__ constexpr int ei(int ch, int p) { return PL ? p * CH + ch : 3 * ch + p; }
+template <bool PL, int CH> __device__ __forceinline__ int64_t feat_channel(int64_t c, int e, int64_t d)
+{
+    return PL ? (int64_t)(e / CH) * d + c + e % CH : 3 * c + e;
+}
+template <bool PL> __device__ __forceinline__ u32x3 piece_load(win_t w, uint32_t off, uint32_t orow)
+{
+    if constexpr (PL)
+        return u32x3{win_load<uint32_t>(w, off), win_load<uint32_t>(w, off + orow), win_load<uint32_t>(w, off + 2 * orow)};
+    else
+        return win_load<u32x3>(w, off);
+}
+template <bool PL> __device__ __forceinline__ void piece_store(win_t w, uint32_t off, uint32_t orow, const u32x3 &v)
+{
+    if constexpr (PL) {
+        win_store(w, off, (uint32_t)v[0]);
+        win_store(w, off + orow, (uint32_t)v[1]);
+        win_store(w, off + 2 * orow, (uint32_t)v[2]);
+    } else {
+        win_store(w, off, v);
+    }
+}
+
 // taps of a lane: wfr[j][e] multiplies the raw sample j rows in the past of feature channel c3 + e,
 // hr[j] the pre-gate product j rows in the past
-template <typename T, int HL, int KF>
+template <typename T, int HL, int KF, bool PL>
 __device__ __forceinline__ void load_taps(const T *wf, const T *h, int64_t c, const Dims &dm, int kf,
                                           float (&wfr)[KF][Piece<T>::E], float (&hr)[HL])
 {
 #pragma unroll
     for (int e = 0; e < Piece<T>::E; ++e) {
-        const T *wp = wf + (3 * c + e) * kf;
+        const T *wp = wf + feat_channel<PL, Piece<T>::CH>(c, e, dm.d) * kf;
 #pragma unroll
         for (int j = 0; j < KF; ++j) wfr[j][e] = (j < kf) ? Elem<T>::load(wp + kf - 1 - j) : 0.f;
     }
@@ -122,7 +149,7 @@ __device__ __forceinline__ void featurize_packed(const float (&wfr)[KF][Piece<T>
 }
 
 // ---------------------------------------------------------------------------- forward
-template <typename T, int HL, int KF>
+template <typename T, int HL, int KF, bool PL = false>
 __global__ __launch_bounds__(256) void mixer_se_fwd_kernel(const T *__restrict__ raw, const T *__restrict__ wf,
                                                            const T *__restrict__ h, T *__restrict__ y, Dims dm,
                                                            int kf, MixPlan pl)
@@ -138,7 +165,7 @@ __global__ __launch_bounds__(256) void mixer_se_fwd_kernel(const T *__restrict__
     const int64_t L = dm.L, d = dm.d, c = (int64_t)cv * CH;
 
     float wfr[KF][E], hr[HL];
-    load_taps<T, HL, KF>(wf, h, c, dm, kf, wfr, hr);
+    load_taps<T, HL, KF, PL>(wf, h, c, dm, kf, wfr, hr);
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
@@ -146,8 +173,8 @@ __global__ __launch_bounds__(256) void mixer_se_fwd_kernel(const T *__restrict__
     const uint32_t orow = (uint32_t)(d * ES), irow = 3 * orow;
     const win_t wr = make_window(raw + 3 * (b * L + t0) * d, (t_end - t0) * irow);
     const win_t wy = make_window(y + (b * L + t_start) * d, (t_end - t_start) * orow);
-    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = 3 * lane_o;
-    auto load_raw = [&](int64_t t) { return win_load<u32x3>(wr, lane_i + (uint32_t)(t - t0) * irow); };
+    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = PL ? lane_o : 3 * lane_o;
+    auto load_raw = [&](int64_t t) { return piece_load<PL>(wr, lane_i + (uint32_t)(t - t0) * irow, orow); };
 
     float rr[4][E], ur[8][CH];
 #pragma unroll
@@ -173,7 +200,7 @@ __global__ __launch_bounds__(256) void mixer_se_fwd_kernel(const T *__restrict__
                 float f[E];
                 featurize<T, KF>(wfr, rr, (-i) & 3, f);
 #pragma unroll
-                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[ei<PL, CH>(ch, 1)] * f[ei<PL, CH>(ch, 2)];
             }
         }
     }
@@ -195,11 +222,11 @@ __global__ __launch_bounds__(256) void mixer_se_fwd_kernel(const T *__restrict__
                 featurize<T, KF>(wfr, rr, k & 3, f);
 #pragma unroll
                 for (int ch = 0; ch < CH; ++ch) {
-                    ur[k][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                    ur[k][ch] = f[ei<PL, CH>(ch, 1)] * f[ei<PL, CH>(ch, 2)];
                     float acc = 0.f;
 #pragma unroll
                     for (int j = HL - 1; j >= 0; --j) acc = fmaf(hr[j], ur[(k - j) & 7][ch], acc);
-                    out[ch] = f[3 * ch] * acc;
+                    out[ch] = f[ei<PL, CH>(ch, 0)] * acc;
                 }
                 win_store(wy, lane_o + (uint32_t)(tb + k - t_start) * orow, P::pack_unit(out));
             }
@@ -215,7 +242,7 @@ __global__ __launch_bounds__(256) void mixer_se_fwd_kernel(const T *__restrict__
 // t2 = t1 - (KF-1) leaves.  The walk therefore runs HL-1 + KF-1 rows past the run, and computes
 // d f for KF-1 rows past the run (the next run's lane computes them too; nothing is exchanged).
 // Filter gradients (dh, dwf) only take the rows of the run.
-template <typename T, int HL, int KF>
+template <typename T, int HL, int KF, bool PL = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))) void mixer_se_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ raw,
                                                            const T *__restrict__ wf, const T *__restrict__ h,
                                                            T *__restrict__ draw, float *__restrict__ ws_h,
@@ -233,7 +260,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
     const int hl = dm.hl;
 
     float wfr[KF][E], hr[HL];
-    load_taps<T, HL, KF>(wf, h, c, dm, kf, wfr, hr);
+    load_taps<T, HL, KF, PL>(wf, h, c, dm, kf, wfr, hr);
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
@@ -245,7 +272,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
     const win_t wr = make_window(raw + 3 * (b * L + t0) * d, (t_far - t0) * irow);
     const win_t wdy = make_window(dy + (b * L + t0) * d, (t_far - t0) * orow);
     const win_t wdr = make_window(draw + 3 * (b * L + t_start) * d, (t_end - t_start) * irow);
-    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = 3 * lane_o;
+    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = PL ? lane_o : 3 * lane_o;
 
     // rings, slot = row & (size-1):  rp raw rows as loaded (the featurizer's history and, HL-1 + KF-1
     // rows back, the terms of dwf), ur u, gr g2, xs / Bs f's x and B, dCs dC, dfr d f (the last four
@@ -275,7 +302,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
     {
         u32x3 hp[NH];
 #pragma unroll
-        for (int i = 1; i <= NH; ++i) hp[i - 1] = win_load<u32x3>(wr, lane_i + (uint32_t)(t_start - i - t0) * irow);
+        for (int i = 1; i <= NH; ++i) hp[i - 1] = piece_load<PL>(wr, lane_i + (uint32_t)(t_start - i - t0) * irow, orow);
 #pragma unroll
         for (int i = NH; i >= 1; --i) {
             rp[(-i) & 15] = hp[i - 1];
@@ -283,7 +310,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
                 float f[E];
                 featurize_packed<T, KF>(wfr, rp, (-i) & 15, f);
 #pragma unroll
-                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[ei<PL, CH>(ch, 1)] * f[ei<PL, CH>(ch, 2)];
             }
         }
     }
@@ -296,7 +323,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
 #pragma unroll
             for (int kk = 0; kk < BATCH; ++kk) {
                 const uint32_t row = (uint32_t)(tb + q * BATCH + kk - t0);
-                in[kk] = win_load<u32x3>(wr, lane_i + row * irow);          // zero past t_far
+                in[kk] = piece_load<PL>(wr, lane_i + row * irow, orow);     // zero past t_far
                 dyr[kk] = win_load<uint32_t>(wdy, lane_o + row * orow);
             }
 #pragma unroll
@@ -313,9 +340,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
                     const uint32_t in_run = row_mask(t < t_end);    // rows whose filter-gradient terms are ours
 #pragma unroll
                     for (int ch = 0; ch < CH; ++ch) {
-                        xv[ch] = f[3 * ch + 2];
-                        Bv[ch] = f[3 * ch + 1];
-                        gr[k & 7][ch] = dyf[ch] * f[3 * ch];
+                        xv[ch] = f[ei<PL, CH>(ch, 2)];
+                        Bv[ch] = f[ei<PL, CH>(ch, 1)];
+                        gr[k & 7][ch] = dyf[ch] * f[ei<PL, CH>(ch, 0)];
                         ur[k & 7][ch] = masked(Bv[ch] * xv[ch], live);
                     }
                     xs[k & 7] = P::pack_unit(xv);
@@ -356,9 +383,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
 #pragma unroll
                     for (int ch = 0; ch < CH; ++ch) {
                         const float duv = masked(du[ch], have);
-                        df[3 * ch] = masked(dCo[ch], have);
-                        df[3 * ch + 1] = duv * xo[ch];
-                        df[3 * ch + 2] = duv * Bo[ch];
+                        df[ei<PL, CH>(ch, 0)] = masked(dCo[ch], have);
+                        df[ei<PL, CH>(ch, 1)] = duv * xo[ch];
+                        df[ei<PL, CH>(ch, 2)] = duv * Bo[ch];
                     }
                     const u32x3 dfp = P::pack(df);
                     P::unpack(dfp, df);
@@ -386,7 +413,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
 #pragma unroll
                         for (int e = 0; e < E; ++e) dr[e] = fmaf(wfr[j][e], dfj[e], dr[e]);
                     }
-                    win_store(wdr, lane_i + (uint32_t)(t - D1 - D2 - t_start) * irow, P::pack(dr));
+                    piece_store<PL>(wdr, lane_i + (uint32_t)(t - D1 - D2 - t_start) * irow, orow, P::pack(dr));
                 }
             }
         }
@@ -399,9 +426,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE))
 #pragma unroll
     for (int j = 0; j < KF; ++j)
         if (j < kf) {
-            float *dst = ws_w + ((size_t)(kf - 1 - j) * pl.nrows + prow) * (3 * d) + 3 * c;
+            float *dst = ws_w + ((size_t)(kf - 1 - j) * pl.nrows + prow) * (3 * d) + (PL ? c : 3 * c);
 #pragma unroll
-            for (int e = 0; e < E; ++e) dst[e] = dwa[j][e];
+            for (int e = 0; e < E; ++e) dst[PL ? (int64_t)(e / CH) * d + e % CH : (int64_t)e] = dwa[j][e];
         }
 }
 
@@ -469,13 +496,13 @@ template <int HX, int HY> __device__ __forceinline__ uint32_t halves(uint32_t x,
     return __builtin_amdgcn_perm(y, x, sel);
 }
 // packed taps of a lane: Wa[e] = (tap 0 rows back, tap 1 row back), Wb[e] = (2 back, 3 back); hr as above
-template <typename T, int HL>
+template <typename T, int HL, bool PL>
 __device__ __forceinline__ void load_taps16(const T *wf, const T *h, int64_t c, const Dims &dm, int kf,
                                             uint32_t (&Wa)[6], uint32_t (&Wb)[6], float (&hr)[HL])
 {
 #pragma unroll
     for (int e = 0; e < 6; ++e) {
-        const T *wp = wf + (3 * c + e) * kf;
+        const T *wp = wf + feat_channel<PL, 2>(c, e, dm.d) * kf;
         float w[4];
 #pragma unroll
         for (int j = 0; j < 4; ++j) w[j] = (j < kf) ? Elem<T>::load(wp + kf - 1 - j) : 0.f;
@@ -505,7 +532,7 @@ __device__ __forceinline__ void featurize16(const uint32_t (&Wa)[6], const uint3
     featurize16<T>(Wa, Wb, pe_t, pe_t2, f, fp);
 }
 
-template <typename T, int HL>
+template <typename T, int HL, bool PL = false>
 __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict__ raw, const T *__restrict__ wf,
                                                              const T *__restrict__ h, T *__restrict__ y, Dims dm,
                                                              int kf, MixPlan pl)
@@ -521,7 +548,7 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
 
     uint32_t Wa[6], Wb[6];
     float hr[HL];
-    load_taps16<T, HL>(wf, h, c, dm, kf, Wa, Wb, hr);
+    load_taps16<T, HL, PL>(wf, h, c, dm, kf, Wa, Wb, hr);
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
@@ -529,8 +556,8 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
     const uint32_t orow = (uint32_t)(d * ES), irow = 3 * orow;
     const win_t wr = make_window(raw + 3 * (b * L + t0) * d, (t_end - t0) * irow);
     const win_t wy = make_window(y + (b * L + t_start) * d, (t_end - t_start) * orow);
-    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = 3 * lane_o;
-    auto load_raw = [&](int64_t t) { return win_load<u32x3>(wr, lane_i + (uint32_t)(t - t0) * irow); };
+    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = PL ? lane_o : 3 * lane_o;
+    auto load_raw = [&](int64_t t) { return piece_load<PL>(wr, lane_i + (uint32_t)(t - t0) * irow, orow); };
 
     // pe[row & 3] = pair_rows(raw[row], raw[row - 1]); ur[row & 7] = u of the row
     uint32_t pe[4][6];
@@ -558,13 +585,13 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
                 float f[6];
                 featurize16<T>(Wa, Wb, pe[(-i) & 3], pe[(-i - 2) & 3], f);
 #pragma unroll
-                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[ei<PL, CH>(ch, 1)] * f[ei<PL, CH>(ch, 2)];
             }
         }
     }
 
     // FB rows are in flight while FB are worked on
-    constexpr int FB = MIXER_BATCH_FWD16;
+    constexpr int FB = PL ? 2 * MIXER_BATCH_FWD16 : MIXER_BATCH_FWD16;     // (planar rows arrive as three small loads each)
     u32x3 in[2][FB];
 #pragma unroll
     for (int kk = 0; kk < FB; ++kk) in[0][kk] = load_raw(t_start + kk);
@@ -583,11 +610,11 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
                 featurize16<T>(Wa, Wb, pe[k & 3], pe[(k - 2) & 3], f);
 #pragma unroll
                 for (int ch = 0; ch < CH; ++ch) {
-                    ur[k & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                    ur[k & 7][ch] = f[ei<PL, CH>(ch, 1)] * f[ei<PL, CH>(ch, 2)];
                     float acc = 0.f;
 #pragma unroll
                     for (int j = HL - 1; j >= 0; --j) acc = fmaf(hr[j], ur[(k - j) & 7][ch], acc);
-                    out[ch] = f[3 * ch] * acc;
+                    out[ch] = f[ei<PL, CH>(ch, 0)] * acc;
                 }
                 win_store(wy, lane_o + (uint32_t)(tb + k - t_start) * orow, Pair<T>::pack2(out[0], out[1]));
             }
@@ -597,7 +624,7 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
 
 // The backward walk above with the featurizer's three sums done two taps (or two rows) at a time.
 // d raw lags d f by three rows whatever the filter length (the fourth tap is zero for shorter filters).
-template <typename T, int HL, int KF>
+template <typename T, int HL, int KF, bool PL = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE)))
 void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, const T *__restrict__ wf,
                            const T *__restrict__ h, T *__restrict__ draw, float *__restrict__ ws_h,
@@ -616,7 +643,7 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
 
     uint32_t Wa[6], Wb[6];
     float hr[HL];
-    load_taps16<T, HL>(wf, h, c, dm, kf, Wa, Wb, hr);
+    load_taps16<T, HL, PL>(wf, h, c, dm, kf, Wa, Wb, hr);
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
@@ -627,7 +654,7 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
     const win_t wr = make_window(raw + 3 * (b * L + t0) * d, (t_far - t0) * irow);
     const win_t wdy = make_window(dy + (b * L + t0) * d, (t_far - t0) * orow);
     const win_t wdr = make_window(draw + 3 * (b * L + t_start) * d, (t_end - t_start) * irow);
-    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = 3 * lane_o;
+    const uint32_t lane_o = (uint32_t)(c * ES), lane_i = PL ? lane_o : 3 * lane_o;
 
     // rings, slot = row & (size-1): rp raw rows as loaded; pe = pair_rows(raw[row], raw[row-1]);
     // ur u; gr g2; xs / Bs / dCs f's x, B and dC as elements of T; pd = pair_rows(d f[row-1], d f[row])
@@ -657,7 +684,7 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
     {
         u32x3 hp[NH];
 #pragma unroll
-        for (int i = 1; i <= NH; ++i) hp[i - 1] = win_load<u32x3>(wr, lane_i + (uint32_t)(t_start - i - t0) * irow);
+        for (int i = 1; i <= NH; ++i) hp[i - 1] = piece_load<PL>(wr, lane_i + (uint32_t)(t_start - i - t0) * irow, orow);
 #pragma unroll
         for (int i = NH; i >= 1; --i) {
             rp[(-i) & 15] = hp[i - 1];
@@ -666,7 +693,7 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
                 float f[E];
                 featurize16<T>(Wa, Wb, pe[(-i) & 3], pe[(-i - 2) & 3], f);
 #pragma unroll
-                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                for (int ch = 0; ch < CH; ++ch) ur[(-i) & 7][ch] = f[ei<PL, CH>(ch, 1)] * f[ei<PL, CH>(ch, 2)];
             }
         }
     }
@@ -686,7 +713,7 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
     auto fetch = [&](int slot) {
 #pragma unroll
         for (int kk = 0; kk < BATCH16; ++kk) {
-            in[slot][kk] = win_load<u32x3>(wr, vin);          // zero past t_far
+            in[slot][kk] = piece_load<PL>(wr, vin, orow);     // zero past t_far
             dyr[slot][kk] = win_load<uint32_t>(wdy, vdy);
             vin += irow;
             vdy += orow;
@@ -707,11 +734,11 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
             P::unpack_unit(dyrow, dyf);
 #pragma unroll
             for (int ch = 0; ch < CH; ++ch) {
-                gr[k & 7][ch] = dyf[ch] * f[3 * ch];
-                ur[k & 7][ch] = f[3 * ch + 1] * f[3 * ch + 2];
+                gr[k & 7][ch] = dyf[ch] * f[ei<PL, CH>(ch, 0)];
+                ur[k & 7][ch] = f[ei<PL, CH>(ch, 1)] * f[ei<PL, CH>(ch, 2)];
             }
-            xs[k & 7] = halves<0, 1>(fp[1], fp[2]);          // (x of channel 0, x of channel 1)
-            Bs[k & 7] = halves<1, 0>(fp[0], fp[2]);          // (B, B)
+            xs[k & 7] = PL ? (uint32_t)fp[2] : halves<0, 1>(fp[1], fp[2]);          // (x of channel 0, x of channel 1)
+            Bs[k & 7] = PL ? (uint32_t)fp[1] : halves<1, 0>(fp[0], fp[2]);          // (B, B)
             float y2v[CH];
 #pragma unroll
             for (int ch = 0; ch < CH; ++ch) y2v[ch] = 0.f;
@@ -746,7 +773,7 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
                 }
                 // the row (dC, dB, dx) x 2 channels, assembled from words of two channels each
                 const uint32_t pC = dCs[k1 & 7], pB = Pair<T>::pack2(dBv[0], dBv[1]), pX = Pair<T>::pack2(dxv[0], dxv[1]);
-                dfp = u32x3{halves<0, 0>(pC, pB), halves<0, 1>(pX, pC), halves<1, 1>(pB, pX)};
+                dfp = PL ? u32x3{pC, pB, pX} : u32x3{halves<0, 0>(pC, pB), halves<0, 1>(pX, pC), halves<1, 1>(pB, pX)};
             }
             pair_rows(dfprev, dfp, pd[k1 & 3]);
             dfprev = dfp;
@@ -768,7 +795,7 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
 #pragma unroll
             for (int e = 0; e < E; ++e)
                 dr[e] = Pair<T>::dot2(pd[(k1 - 2) & 3][e], Wa[e], Pair<T>::dot2(pd[k1 & 3][e], Wb[e], 0.f));
-            win_store(wdr, vout, pack6<T>(dr));
+            piece_store<PL>(wdr, vout, orow, pack6<T>(dr));
             vout += irow;
         }
     };
@@ -797,9 +824,9 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
 #pragma unroll
     for (int j = 0; j < KF; ++j)
         if (j < kf) {
-            float *dst = ws_w + ((size_t)(kf - 1 - j) * pl.nrows + prow) * (3 * d) + 3 * c;
+            float *dst = ws_w + ((size_t)(kf - 1 - j) * pl.nrows + prow) * (3 * d) + (PL ? c : 3 * c);
 #pragma unroll
-            for (int e = 0; e < E; ++e) dst[e] = dwa[j][e];
+            for (int e = 0; e < E; ++e) dst[PL ? (int64_t)(e / CH) * d + e % CH : (int64_t)e] = dwa[j][e];
         }
 }
 
@@ -834,12 +861,21 @@ int fwd_launch(const void *raw, const void *wf, const void *h, void *y, const Di
     int e = 0;
     const MixPlan p = plan(dm, Piece<T>::CH, false);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    if constexpr (sizeof(T) == 2)
-        e = launch_plain((mixer_se_fwd16_kernel<T, HL>), dim3((unsigned)p.nwg), dim3(p.threads), st, (const T *)raw,
-                           (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
-    else
-        e = launch_plain((mixer_se_fwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
-                           (const T *)raw, (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+    if constexpr (sizeof(T) == 2) {
+        if (dm.planar)
+            e = launch_plain((mixer_se_fwd16_kernel<T, HL, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)raw, (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+        else
+            e = launch_plain((mixer_se_fwd16_kernel<T, HL>), dim3((unsigned)p.nwg), dim3(p.threads), st, (const T *)raw,
+                             (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+    } else {
+        if (dm.planar)
+            e = launch_plain((mixer_se_fwd_kernel<T, HL, KF, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)raw, (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+        else
+            e = launch_plain((mixer_se_fwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)raw, (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+    }
     return e;
 }
 
@@ -852,12 +888,21 @@ int bwd_launch(const void *dy, const void *raw, const void *wf, const void *h, v
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     float *ws_h = (float *)ws;
     float *ws_w = ws_h + (size_t)dm.hl * p.nrows * p.nvec;
-    if constexpr (sizeof(T) == 2)
-        e = launch_plain((mixer_se_bwd16_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
-                           (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
-    else
-        e = launch_plain((mixer_se_bwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
-                           (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+    if constexpr (sizeof(T) == 2) {
+        if (dm.planar)
+            e = launch_plain((mixer_se_bwd16_kernel<T, HL, KF, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+        else
+            e = launch_plain((mixer_se_bwd16_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+    } else {
+        if (dm.planar)
+            e = launch_plain((mixer_se_bwd_kernel<T, HL, KF, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+        else
+            e = launch_plain((mixer_se_bwd_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+    }
     if (e) return e;
     // both filter gradients in one launch
     const ColsumJob jh{ws_h, dh, p.nrows, p.nvec, dm.dg / p.ch, dm.g, dm.hl};

@@ -292,54 +292,60 @@ std::tuple<Tensor, Tensor> dwconv_bwd(const Tensor &dy, const Tensor &x, const T
 
 // ---- featurizer + Hyena-SE operator in one pass ------------------------------------------------
 
-void check_mixer_se(const Tensor &raw, const Tensor &wf, const Tensor &h)
+// planar: raw is (bs, L, 3, g, dg) -- the planes C | B | x of each row one after the other -- instead of (bs, L, g, dg, 3)
+void check_mixer_se(const Tensor &raw, const Tensor &wf, const Tensor &h, bool planar = false)
 {
-    TORCH_CHECK(raw.dim() == 5 && raw.size(4) == 3 && raw.is_contiguous(),
-                "gcg: raw must be a contiguous (bs, L, g, dg, 3) tensor");
-    TORCH_CHECK(wf.dim() == 3 && wf.size(0) == 3 * raw.size(2) * raw.size(3) && wf.size(1) == 1 && wf.is_contiguous(),
+    TORCH_CHECK(raw.dim() == 5 && raw.size(planar ? 2 : 4) == 3 && raw.is_contiguous(),
+                planar ? "gcg: raw must be a contiguous (bs, L, 3, g, dg) tensor"
+                       : "gcg: raw must be a contiguous (bs, L, g, dg, 3) tensor");
+    const int64_t g = raw.size(planar ? 3 : 2), dg = raw.size(planar ? 4 : 3);
+    TORCH_CHECK(wf.dim() == 3 && wf.size(0) == 3 * g * dg && wf.size(1) == 1 && wf.is_contiguous(),
                 "gcg: wf must be a contiguous (3 * g * dg, 1, kf) tensor");
-    TORCH_CHECK(h.dim() == 3 && h.size(0) == raw.size(2) && h.size(1) == 1 && h.is_contiguous(),
+    TORCH_CHECK(h.dim() == 3 && h.size(0) == g && h.size(1) == 1 && h.is_contiguous(),
                 "gcg: h must be a contiguous (g, 1, hl) tensor");
     TORCH_CHECK(wf.scalar_type() == raw.scalar_type() && h.scalar_type() == raw.scalar_type() &&
                     wf.device() == raw.device() && h.device() == raw.device(),
                 "gcg: raw, wf and h must share dtype and device");
 }
 
-Tensor mixer_se_fwd(const Tensor &raw, const Tensor &wf, const Tensor &h)
+Tensor mixer_se_fwd(const Tensor &raw, const Tensor &wf, const Tensor &h, bool planar)
 {
     require_gpu(raw, "raw");
-    check_mixer_se(raw, wf, h);
+    check_mixer_se(raw, wf, h, planar);
     DeviceGuard guard(raw.device());
-    Tensor y = at::empty({raw.size(0), raw.size(1), raw.size(2), raw.size(3)}, raw.options());
+    const int64_t g = raw.size(planar ? 3 : 2), dg = raw.size(planar ? 4 : 3);
+    Tensor y = at::empty({raw.size(0), raw.size(1), g, dg}, raw.options());
     if (y.numel() == 0) return y;
-    check_rc(gcg_mixer_se_fwd(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), raw.size(0), raw.size(1),
-                              (int32_t)raw.size(2), (int32_t)raw.size(3), (int32_t)h.size(2), (int32_t)wf.size(2),
-                              dtype_code(raw.scalar_type()), stream_of(raw)),
-             "gcg_mixer_se_fwd");
+    check_rc((planar ? gcg_mixer_se_fwd_planar : gcg_mixer_se_fwd)(
+                 raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), raw.size(0), raw.size(1), (int32_t)g,
+                 (int32_t)dg, (int32_t)h.size(2), (int32_t)wf.size(2), dtype_code(raw.scalar_type()), stream_of(raw)),
+             planar ? "gcg_mixer_se_fwd_planar" : "gcg_mixer_se_fwd");
     return y;
 }
 
-std::tuple<Tensor, Tensor, Tensor> mixer_se_bwd(const Tensor &dy, const Tensor &raw, const Tensor &wf, const Tensor &h)
+std::tuple<Tensor, Tensor, Tensor> mixer_se_bwd(const Tensor &dy, const Tensor &raw, const Tensor &wf, const Tensor &h,
+                                                bool planar)
 {
     require_gpu(raw, "raw");
-    check_mixer_se(raw, wf, h);
-    TORCH_CHECK(dy.dim() == 4 && dy.sizes() == raw.sizes().slice(0, 4) && dy.scalar_type() == raw.scalar_type() &&
-                    dy.device() == raw.device() && dy.is_contiguous(),
+    check_mixer_se(raw, wf, h, planar);
+    const int32_t g = (int32_t)raw.size(planar ? 3 : 2), dg = (int32_t)raw.size(planar ? 4 : 3);
+    TORCH_CHECK(dy.dim() == 4 && dy.size(0) == raw.size(0) && dy.size(1) == raw.size(1) && dy.size(2) == g &&
+                    dy.size(3) == dg && dy.scalar_type() == raw.scalar_type() && dy.device() == raw.device() &&
+                    dy.is_contiguous(),
                 "gcg: dy must be a contiguous (bs, L, g, dg) tensor of raw's dtype and device");
     DeviceGuard guard(raw.device());
     Tensor draw = at::empty_like(raw), dwf = at::empty_like(wf), dh = at::empty_like(h);
     if (raw.numel() == 0) return {draw, dwf.zero_(), dh.zero_()};
     const int64_t bs = raw.size(0), L = raw.size(1);
-    const int32_t g = (int32_t)raw.size(2), dg = (int32_t)raw.size(3), hl = (int32_t)h.size(2),
-                  kf = (int32_t)wf.size(2);
+    const int32_t hl = (int32_t)h.size(2), kf = (int32_t)wf.size(2);
     const int code = dtype_code(raw.scalar_type());
     const size_t nbytes = gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code);
     if (nbytes == 0) check_rc(GCG_ERR_UNSUPPORTED, "gcg_mixer_se_bwd_workspace_bytes");
     Tensor ws = workspace(nbytes, raw, "gcg_mixer_se_bwd_workspace_bytes");
-    check_rc(gcg_mixer_se_bwd(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
-                              dwf.data_ptr(), dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl, kf, code,
-                              stream_of(raw)),
-             "gcg_mixer_se_bwd");
+    check_rc((planar ? gcg_mixer_se_bwd_planar : gcg_mixer_se_bwd)(
+                 dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(), dwf.data_ptr(),
+                 dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl, kf, code, stream_of(raw)),
+             planar ? "gcg_mixer_se_bwd_planar" : "gcg_mixer_se_bwd");
     return {draw, dwf, dh};
 }
 
@@ -718,15 +724,15 @@ std::tuple<Tensor, Tensor> dwconv_bwd_meta(const Tensor &dy, const Tensor &x, co
     check_like(dy, x, "dy");
     return {at::empty_like(x), at::empty_like(w)};
 }
-Tensor mixer_se_fwd_meta(const Tensor &raw, const Tensor &wf, const Tensor &h)
+Tensor mixer_se_fwd_meta(const Tensor &raw, const Tensor &wf, const Tensor &h, bool planar)
 {
-    check_mixer_se(raw, wf, h);
-    return at::empty({raw.size(0), raw.size(1), raw.size(2), raw.size(3)}, raw.options());
+    check_mixer_se(raw, wf, h, planar);
+    return at::empty({raw.size(0), raw.size(1), raw.size(planar ? 3 : 2), raw.size(planar ? 4 : 3)}, raw.options());
 }
 std::tuple<Tensor, Tensor, Tensor> mixer_se_bwd_meta(const Tensor &dy, const Tensor &raw, const Tensor &wf,
-                                                     const Tensor &h)
+                                                     const Tensor &h, bool planar)
 {
-    check_mixer_se(raw, wf, h);
+    check_mixer_se(raw, wf, h, planar);
     (void)dy;
     return {at::empty_like(raw), at::empty_like(wf), at::empty_like(h)};
 }
@@ -838,8 +844,8 @@ TORCH_LIBRARY(gcg, m)
     m.def("bwd_planar(Tensor dy, Tensor feat, Tensor h, int algo=0) -> (Tensor, Tensor)");
     m.def("dwconv_fwd(Tensor x, Tensor w, bool keep_output=False) -> Tensor");
     m.def("dwconv_bwd(Tensor dy, Tensor x, Tensor w) -> (Tensor, Tensor)");
-    m.def("mixer_se_fwd(Tensor raw, Tensor wf, Tensor h) -> Tensor");
-    m.def("mixer_se_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h) -> (Tensor, Tensor, Tensor)");
+    m.def("mixer_se_fwd(Tensor raw, Tensor wf, Tensor h, bool planar=False) -> Tensor");
+    m.def("mixer_se_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h, bool planar=False) -> (Tensor, Tensor, Tensor)");
     m.def("filter_decay_fwd(Tensor w, Tensor decay, int hl, ScalarType dtype) -> Tensor");
     m.def("filter_decay_bwd(Tensor dh, Tensor decay) -> Tensor");
     m.def("mixer_mr_fwd(Tensor raw, Tensor wf, Tensor h) -> Tensor");

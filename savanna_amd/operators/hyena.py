@@ -319,18 +319,19 @@ class CausalDepthwiseConv1d(nn.Module):
 
 class _FeaturizedShortGateConvGate(torch.autograd.Function):
     """z = gated short convolution of the featurized projection, raw (b, l, g, dg, 3) -> (b, l, g, dg),
-    in one kernel each way; the featurized tensor exists in registers only."""
+    in one kernel each way; the featurized tensor exists in registers only.  ``planar``: raw is (b, l, 3, g, dg)."""
 
     @staticmethod
-    def forward(ctx, raw, wf, h):
+    def forward(ctx, raw, wf, h, planar=False):
         raw, wf, h = (t if t.is_contiguous() else t.contiguous() for t in (raw, wf, h))
         ctx.save_for_backward(raw, wf, h)
-        return _lib.mixer_se_fwd(raw, wf, h)
+        ctx.planar = planar
+        return _lib.mixer_se_fwd(raw, wf, h, planar)
 
     @staticmethod
     def backward(ctx, dz):
         raw, wf, h = ctx.saved_tensors
-        return _lib.mixer_se_bwd(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, h)
+        return _lib.mixer_se_bwd(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, h, ctx.planar) + (None,)
 
 
 class _FeaturizedGateConvGate(torch.autograd.Function):
@@ -403,7 +404,18 @@ class HyenaMixer(nn.Module):
         bs, seqlen, d3 = features.shape
         conv = self.hyena_proj_conv
         if not self.interleave_projections:
-            # "(p g dg)" features: featurizer kernel, then the operator on the thirds of its rows (two kernels each way)
+            # "(p g dg)" features.  Hyena-SE: the fused kernels on planar pieces; otherwise the featurizer kernel,
+            # then the operator on the thirds of its rows (two kernels each way)
+            h = op._filter(seqlen)
+            if self._fusable(features, h.shape[-1]):
+                dtype = features.dtype
+                if op.cgcg_dtype != dtype:
+                    features = features.to(op.cgcg_dtype)
+                g, dg = op.num_groups, op.group_dim
+                z = _FeaturizedShortGateConvGate.apply(features.reshape(bs, seqlen, 3, g, dg),
+                                                       conv.short_conv_weight.to(op.cgcg_dtype), h.to(op.cgcg_dtype), True)
+                z = z.reshape(bs, seqlen, g * dg)
+                return z.to(dtype) if op.cgcg_dtype != dtype else z
             return op.forward_features(conv.forward_bld(features, feeds_operator=True), interleaved=False)
         fused = op._filter_in_kernel(seqlen, op.num_groups, op.group_dim, features.dtype, features)
         if (fused is not None and self.fuse_medium and conv.group_dim == 1 and

@@ -138,6 +138,10 @@ WORKLOADS = {
     "mixer_se_fwdbwd_40b_fused": Workload("mixer_se_fwdbwd_40b_fused", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
                                           "the same as one kernel each way (the featurized tensor stays in "
                                           "registers)", layout="mixer_fused"),
+    "mixer_se_fwdbwd_40b_fused_planar": Workload("mixer_se_fwdbwd_40b_fused_planar", 1, 32768, 512, 16, (7,),
+                                                 torch.bfloat16, True,
+                                                 "the same on planar features (interleave_projections = false): "
+                                                 "gcg_mixer_se_fwd_planar / _bwd_planar", layout="mixer_fused_planar"),
 }
 # the order in which the benchmark reports them
 WORKLOAD_ORDER = ("se_fwd_fp32", "mr_fwd_7b", "mr_fwdbwd_7b", "se_mr_fwdbwd_40b", "mr_fwd_1m")

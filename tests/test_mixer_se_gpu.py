@@ -206,3 +206,59 @@ def test_fused_kernels_in_a_replayed_graph(gcg_lib, dtype):
         torch.cuda.synchronize()
         for a, b, n in zip(out_g, out_e, ("y", "d raw", "dwf", "dh")):
             assert torch.equal(a, b), f"replay {it}: {n}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=lambda d: str(d)[6:])
+@pytest.mark.parametrize("bs,L,g,dg,hl,kf", SHAPES + [(2, 4096, 64, 16, 7, 3)])
+def test_planar_features_match_interleaved(gcg_lib, bs, L, g, dg, hl, kf, dtype):
+    """gcg_mixer_se_fwd_planar / _bwd_planar -- raw (bs, L, 3, g, dg), the split without interleaving of
+    block.py:881-884, with the featurizer's filters in that channel order -- give the interleaved entry points'
+    results on the same values, bit for bit (the same arithmetic on pieces loaded plane by plane)."""
+    raw, dy, wf, h = (t.to(DEV) for t in data(bs, L, g, dg, hl, kf, dtype, seed=17))
+    d = g * dg
+    raw_pl = raw.permute(0, 1, 4, 2, 3).contiguous()                                  # (bs, L, 3, g, dg)
+    wf_pl = wf.view(d, 3, 1, kf).permute(1, 0, 2, 3).reshape(3 * d, 1, kf).contiguous()    # row p * d + c <- row 3 c + p
+    y = _lib.mixer_se_fwd(raw, wf, h)
+    draw, dwf, dh = _lib.mixer_se_bwd(dy, raw, wf, h)
+    y_pl = _lib.mixer_se_fwd(raw_pl, wf_pl, h, planar=True)
+    draw_pl, dwf_pl, dh_pl = _lib.mixer_se_bwd(dy, raw_pl, wf_pl, h, planar=True)
+    torch.cuda.synchronize()
+    assert y_pl.shape == y.shape and draw_pl.shape == raw_pl.shape and dwf_pl.shape == wf.shape
+    assert torch.equal(y_pl, y)
+    assert torch.equal(draw_pl, draw.permute(0, 1, 4, 2, 3))
+    assert torch.equal(dwf_pl.view(3, d, 1, kf), dwf.view(d, 3, 1, kf).permute(1, 0, 2, 3))
+    assert torch.equal(dh_pl, dh)
+
+
+def test_hyena_mixer_planar_fused(gcg_lib):
+    """HyenaMixer(interleave_projections=False) with a Hyena-SE operator: one kernel each way, same output and
+    gradients as the two-kernel chain on the same layout up to the rounding of fp32 sums."""
+    from savanna_amd.operators.hyena import CgcgConfig, HyenaMixer, HyenaSEOperator
+
+    torch.manual_seed(2)
+    bs, L, hidden, groups = 2, 512, 128, 8
+    cfg = CgcgConfig(cgcg_dtype="bfloat16")
+    mixer = HyenaMixer(HyenaSEOperator(hidden, groups, 7, cfg, device=DEV), 3, dtype=torch.bfloat16, device=DEV,
+                       interleave_projections=False)
+    feats = torch.randn(bs, L, 3 * hidden, device=DEV).to(torch.bfloat16).requires_grad_(True)
+    dz = (0.1 * torch.randn(bs, L, hidden, device=DEV)).to(torch.bfloat16)
+    params = list(mixer.parameters())
+
+    def run(fuse):
+        mixer.fuse_short = fuse
+        feats.grad = None
+        for p in params:
+            p.grad = None
+        z = mixer(feats)
+        z.backward(dz)
+        return [z.detach(), feats.grad.clone()] + [p.grad.clone() for p in params]
+
+    want = run(False)
+    from torch.profiler import ProfilerActivity, profile
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        got = run(True)
+        torch.cuda.synchronize()
+    for a, b, n in zip(got, want, ("z", "d features", "p0", "p1")):
+        assert_close(a, b, 2e-2, n)
+    big = [e.key for e in prof.key_averages() if "mixer_se" in e.key or "dwconv" in e.key or "window" in e.key]
+    assert len(big) == 2 and all("mixer_se" in k for k in big), big
