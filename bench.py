@@ -152,7 +152,8 @@ class Op:
             fused = _FeaturizedShortGateConvGate if self.hl <= 8 else _FeaturizedGateConvGate
             y = fused.apply(raw.reshape(wl.bs, wl.L, wl.g, wl.dg, 3), wf, h)
         elif self.layout == "mixer_fused_planar":       # the same values read as (bs, L, 3, g, dg)
-            y = _FeaturizedShortGateConvGate.apply(raw.reshape(wl.bs, wl.L, 3, wl.g, wl.dg), wf, h, True)
+            fused = _FeaturizedShortGateConvGate if self.hl <= 8 else _FeaturizedGateConvGate
+            y = fused.apply(raw.reshape(wl.bs, wl.L, 3, wl.g, wl.dg), wf, h, True)
         elif self.layout == "mixer":
             f = _CausalDepthwiseConv.apply(raw.reshape(wl.bs, wl.L, 3 * wl.d, 1), wf, KEEP_INTERMEDIATES)
             y = two_pass_chunked_gate_conv_gate_interleaved(f, h, wl.bs, wl.L, wl.g, wl.dg,

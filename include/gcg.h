@@ -355,6 +355,22 @@ GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, co
             int32_t dtype, void *stream);
 
 /*
+ * The same two on planar features (interleave_projections = false, savanna/model/block.py:881-884): raw and draw
+ * are (bs, L, 3, g, dg), each row the planes C | B | x one after the other, and wf, dwf hold their filters in that
+ * channel order.  One-kernel path only: 16-bit tensors with arithmetic in their own type (GCG_BF16, GCG_F16),
+ * otherwise GCG_ERR_UNSUPPORTED (run gcg_dwconv_fwd and gcg_fwd_planar, and their backwards, instead).
+ * Workspace: gcg_mixer_mr_bwd_workspace_bytes; no scratch tensor.
+ */
+GCG_API int gcg_mixer_mr_fwd_planar(const void *raw, const void *wf, const void *h, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+GCG_API int gcg_mixer_mr_bwd_planar(const void *dy, const void *raw, const void *wf, const void *h,
+            void *draw, void *dwf, void *dh,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+
+/*
  * The same with the Hyena-MR filter formed inside the kernels, as in gcg_fwd_decay / gcg_bwd_decay: h = F(w * decay)
  * cut to hl taps (ExplicitSingleDecayFilter.filter, savanna/model/operators/hyena/parametrization/explicit.py:68-75,
  * and the cast of hyena.py:499-503), dw the gradient of the parameter w.  A Hyena-MR layer's convolutional part --

@@ -36,7 +36,8 @@ EXPORTS = (
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
     "gcg_mixer_se_fwd_planar", "gcg_mixer_se_bwd_planar",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
-    "gcg_mixer_mr_fwd", "gcg_mixer_mr_bwd_workspace_bytes", "gcg_mixer_mr_bwd_scratch_bytes", "gcg_mixer_mr_bwd", "gcg_mixer_mr_fwd_decay", "gcg_mixer_mr_bwd_decay", "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
+    "gcg_mixer_mr_fwd", "gcg_mixer_mr_bwd_workspace_bytes", "gcg_mixer_mr_bwd_scratch_bytes", "gcg_mixer_mr_bwd", "gcg_mixer_mr_fwd_decay", "gcg_mixer_mr_bwd_decay",
+    "gcg_mixer_mr_fwd_planar", "gcg_mixer_mr_bwd_planar", "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
     "gcg_fwd_decay", "gcg_bwd_decay", "gcg_fwd_interleaved_decay", "gcg_bwd_interleaved_decay",
 )
 
@@ -117,6 +118,10 @@ def load() -> ctypes.CDLL:
         lib.gcg_mixer_mr_bwd_scratch_bytes.restype = sz
         lib.gcg_mixer_mr_bwd.argtypes = [vp] * 9 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_mixer_mr_bwd.restype = ctypes.c_int
+        lib.gcg_mixer_mr_fwd_planar.argtypes = [vp] * 4 + [i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_mixer_mr_fwd_planar.restype = ctypes.c_int
+        lib.gcg_mixer_mr_bwd_planar.argtypes = [vp] * 8 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_mixer_mr_bwd_planar.restype = ctypes.c_int
         lib.gcg_mixer_mr_fwd_decay.argtypes = [vp] * 4 + [i32, vp, i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_mixer_mr_fwd_decay.restype = ctypes.c_int
         lib.gcg_mixer_mr_bwd_decay.argtypes = [vp] * 5 + [i32] + [vp] * 5 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
@@ -579,10 +584,11 @@ def filter_decay_bwd(dh, decay):
 
 
 
-def _check_mixer_mr(raw, wf, h):
-    if raw.dim() != 5 or raw.shape[-1] != 3 or not raw.is_contiguous():
-        raise ValueError("raw must be a contiguous (bs, L, g, dg, 3) tensor")
-    bs, L, g, dg, _ = raw.shape
+def _check_mixer_mr(raw, wf, h, planar=False):
+    if raw.dim() != 5 or raw.shape[2 if planar else 4] != 3 or not raw.is_contiguous():
+        raise ValueError("raw must be a contiguous (bs, L, 3, g, dg) tensor" if planar
+                         else "raw must be a contiguous (bs, L, g, dg, 3) tensor")
+    g, dg = (raw.shape[3], raw.shape[4]) if planar else (raw.shape[2], raw.shape[3])
     if wf.dim() != 3 or wf.shape[0] != 3 * g * dg or wf.shape[1] != 1 or not wf.is_contiguous() or wf.dtype != raw.dtype:
         raise ValueError("wf must be a contiguous (3 * g * dg, 1, kf) tensor of raw's dtype")
     if h.dim() != 3 or h.shape[0] != g or h.shape[1] != 1 or not h.is_contiguous():
@@ -615,34 +621,38 @@ def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors) -> bool:
     return 9 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and _all_aligned16(tensors)
 
 
-def mixer_mr_fwd(raw, wf, h):
+def mixer_mr_fwd(raw, wf, h, planar=False):
     """Featurizer conv and Hyena-MR operator in one pass: y (bs, L, g, dg) from the projection output
-    raw (bs, L, g, dg, 3), without the featurized tensor; the same values as dwconv_fwd followed by fwd_interleaved."""
+    raw (bs, L, g, dg, 3), without the featurized tensor; the same values as dwconv_fwd followed by fwd_interleaved.
+    ``planar``: raw is (bs, L, 3, g, dg), the split without interleaving (block.py:881-884); 16-bit arithmetic only."""
     _require_gpu(raw)
     if TORCH_OPS:
-        return torch.ops.gcg.mixer_mr_fwd(raw, wf, h)
+        return torch.ops.gcg.mixer_mr_fwd(raw, wf, h, bool(planar))
     lib = load()
-    _check_mixer_mr(raw, wf, h)
-    bs, L, g, dg, _ = raw.shape
+    _check_mixer_mr(raw, wf, h, planar)
+    bs, L = raw.shape[:2]
+    g, dg = (raw.shape[3], raw.shape[4]) if planar else (raw.shape[2], raw.shape[3])
     y = torch.empty(bs, L, g, dg, dtype=raw.dtype, device=raw.device)
     if y.numel() == 0:
         return y
+    fn = lib.gcg_mixer_mr_fwd_planar if planar else lib.gcg_mixer_mr_fwd
     with _on_device(raw.device):
-        rc = lib.gcg_mixer_mr_fwd(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg,
-                                  h.shape[-1], wf.shape[-1], gated_code(raw, h), torch.cuda.current_stream().cuda_stream)
-    check(rc, "gcg_mixer_mr_fwd")
+        rc = fn(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg,
+                h.shape[-1], wf.shape[-1], gated_code(raw, h), torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_mixer_mr_fwd_planar" if planar else "gcg_mixer_mr_fwd")
     return y
 
 
-def mixer_mr_bwd(dy, raw, wf, h):
+def mixer_mr_bwd(dy, raw, wf, h, planar=False):
     """(draw, dwf, dh) of mixer_mr_fwd from the projection output alone: the features are recomputed; their
     gradient stays inside the kernel (16-bit arithmetic) or lives in a scratch tensor for the duration of the call."""
     _require_gpu(raw)
     if TORCH_OPS:
-        return torch.ops.gcg.mixer_mr_bwd(dy, raw, wf, h)
+        return torch.ops.gcg.mixer_mr_bwd(dy, raw, wf, h, bool(planar))
     lib = load()
-    _check_mixer_mr(raw, wf, h)
-    bs, L, g, dg, _ = raw.shape
+    _check_mixer_mr(raw, wf, h, planar)
+    bs, L = raw.shape[:2]
+    g, dg = (raw.shape[3], raw.shape[4]) if planar else (raw.shape[2], raw.shape[3])
     hl, kf = h.shape[-1], wf.shape[-1]
     draw, dwf, dh = torch.empty_like(raw), torch.empty_like(wf), torch.empty_like(h)
     if dy.numel() == 0:
@@ -651,6 +661,14 @@ def mixer_mr_bwd(dy, raw, wf, h):
     nbytes = lib.gcg_mixer_mr_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code)
     if nbytes == 0:
         check(-2, "gcg_mixer_mr_bwd_workspace_bytes")
+    if planar:
+        with _on_device(raw.device):
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
+            rc = lib.gcg_mixer_mr_bwd_planar(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
+                                             dwf.data_ptr(), dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl, kf,
+                                             code, torch.cuda.current_stream().cuda_stream)
+        check(rc, "gcg_mixer_mr_bwd_planar")
+        return draw, dwf, dh
     with _on_device(raw.device):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
         sbytes = lib.gcg_mixer_mr_bwd_scratch_bytes(bs, L, g, dg, hl, kf, code)

@@ -647,6 +647,18 @@ GCG_API int gcg_mixer_mr_fwd(const void *raw, const void *wf, const void *h, voi
     return mixer_mr_fwd_dims(raw, wf, h, y, dm, kf, dtype, stream);
 }
 
+GCG_API int gcg_mixer_mr_fwd_planar(const void *raw, const void *wf, const void *h, void *y, int64_t bs, int64_t L,
+                                    int32_t g, int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!raw || !wf || !h || !y || kf <= 0) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    const int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    if (rc) return rc;
+    dm.planar = 1;
+    return mixer_mr_fwd_dims(raw, wf, h, y, dm, kf, dtype, stream);
+}
+
 GCG_API int gcg_mixer_mr_fwd_decay(const void *raw, const void *wf, const float *w, const float *decay, int32_t l_cache,
                                    void *y, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
                                    int32_t dtype, void *stream)
@@ -664,8 +676,9 @@ int mixer_mr_fwd_dims(const void *raw, const void *wf, const void *h, void *y, g
                       void *stream)
 {
     int rc = 0;
-    dm.es = 3;
+    dm.es = dm.planar ? 1 : 3;
     if (!all_aligned16({raw, y}) || !gcg::mfma_feat_supported(dtype, dm, kf)) return GCG_ERR_UNSUPPORTED;
+    if (dm.planar && !gcg::mixer_mr_fused_supported(dtype, dm, kf)) return GCG_ERR_UNSUPPORTED;   // one-kernel path only
     rc = check_device();
     if (rc) return rc;
     if (gcg::mixer_mr_fused_supported(dtype, dm, kf))
@@ -718,6 +731,19 @@ GCG_API int gcg_mixer_mr_bwd(const void *dy, const void *raw, const void *wf, co
     return mixer_mr_bwd_dims(dy, raw, wf, h, draw, dwf, dh, dfeat_scratch, workspace, workspace_bytes, dm, kf, dtype, stream);
 }
 
+GCG_API int gcg_mixer_mr_bwd_planar(const void *dy, const void *raw, const void *wf, const void *h, void *draw,
+                                    void *dwf, void *dh, void *workspace, size_t workspace_bytes, int64_t bs, int64_t L,
+                                    int32_t g, int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !raw || !wf || !h || !draw || !dwf || !dh || kf <= 0) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    const int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
+    if (rc) return rc;
+    dm.planar = 1;
+    return mixer_mr_bwd_dims(dy, raw, wf, h, draw, dwf, dh, nullptr, workspace, workspace_bytes, dm, kf, dtype, stream);
+}
+
 GCG_API int gcg_mixer_mr_bwd_decay(const void *dy, const void *raw, const void *wf, const float *w, const float *decay,
                                    int32_t l_cache, void *draw, void *dwf, float *dw, void *dfeat_scratch,
                                    void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g, int32_t dg,
@@ -741,9 +767,10 @@ int mixer_mr_bwd_dims(const void *dy, const void *raw, const void *wf, const voi
     const int64_t bs = dm.bs, L = dm.L;
     const int32_t g = dm.g, dg = dm.dg, hl = dm.hl;
     int rc = 0;
-    dm.es = 3;
+    dm.es = dm.planar ? 1 : 3;
     dm.keep_out = 1;
     const bool fused = gcg::mixer_mr_fused_supported(dtype, dm, kf);
+    if (dm.planar && !fused) return GCG_ERR_UNSUPPORTED;          // one-kernel path only
     if (!fused && !dfeat_scratch) return GCG_ERR_BAD_ARG;
     if (!all_aligned16({dy, raw, draw}) || (!fused && !all_aligned16({dfeat_scratch})) ||
         !gcg::mfma_feat_supported(dtype, dm, kf))

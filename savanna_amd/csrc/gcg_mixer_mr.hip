@@ -87,6 +87,54 @@ __device__ __forceinline__ void stw4_cached(win_t w, uint32_t off, uint32_t v)
     __builtin_amdgcn_raw_buffer_store_b32(v, w, (int)off, 0, 0);
 }
 
+// Planar features (PL; Dims::planar, the split without interleaving of block.py:881-884): a row holds the planes
+// C | B | x one after the other, d elements each.  A lane's piece is then three words one plane apart, and its six
+// values come plane by plane, C0 C1 | B0 B1 | x0 x1, instead of C0 B0 | x0 C1 | B1 x1.  That changes where a value
+// sits in a piece (vi), which feature channel it is (feature_channel), and how a piece is loaded and stored; the
+// rings, the featurizer's sums and the pairing of rows treat the six values alike.
+template <bool PL> __device__ __forceinline__ constexpr int vi(int ch, int p) { return PL ? 2 * p + ch : 3 * ch + p; }
+template <bool PL> __device__ __forceinline__ int64_t feature_channel(int64_t c, int v, int64_t d)
+{
+    return PL ? (int64_t)(v / 2) * d + c + v % 2 : 3 * c + v;
+}
+// off: the piece's offset in an interleaved row, or that of its first word in a planar one; plane: bytes of a plane
+template <bool PL> __device__ __forceinline__ u32x3 piece_load_cached(win_t w, uint32_t off, uint32_t plane)
+{
+    if constexpr (PL)
+        return u32x3{ldw4_cached(w, off), ldw4_cached(w, off + plane), ldw4_cached(w, off + 2 * plane)};
+    else
+        return ldw12_cached(w, off);
+}
+template <bool PL> __device__ __forceinline__ void piece_store(win_t w, uint32_t off, uint32_t plane, const u32x3 &v)
+{
+    if constexpr (PL) {
+        stw4(w, off, v[0]);
+        stw4(w, off + plane, v[1]);
+        stw4(w, off + 2 * plane, v[2]);
+    } else {
+        stw12(w, off, v);
+    }
+}
+// taps of a lane's six feature channels, oldest sample first, zero-padded in front to KF taps
+template <typename T, int KF, bool PL>
+__device__ __forceinline__ void lane_feat_taps(const T *wfeat, int64_t c, bool valid, int64_t d, int kf, float (&tap)[KF][6])
+{
+    if constexpr (PL) {
+#pragma unroll
+        for (int v = 0; v < 6; ++v) {
+            const T *wp = wfeat + (valid ? feature_channel<true>(c, v, d) : 0) * kf;
+#pragma unroll
+            for (int m = 0; m < KF; ++m) {
+                const int kk = m - (KF - kf);                // index into the kf taps of the filter
+                const float t = Elem<T>::load(wp + (kk >= 0 ? kk : 0));
+                tap[m][v] = kk >= 0 ? t : 0.f;
+            }
+        }
+    } else {
+        load_feat_taps<T, KF, 6>(wfeat, valid ? 3 * c : 0, kf, tap);
+    }
+}
+
 struct Blk { uint4 w[3]; };       // four 12-byte pieces
 struct Halo { uint2 w[3]; };      // two 12-byte pieces
 
@@ -194,7 +242,7 @@ __device__ __forceinline__ float feat_sum(const float (&tap)[MR_KF][6], const fl
 // Tail of the backward, run by every wave: the workgroup that finishes a channel block's last run adds the block's
 // partial sums of dh and d wf in a fixed order (so the results do not depend on which workgroup that is) and writes
 // the gradients; without pl.fuse_dh two small launches do it.
-template <typename T>
+template <typename T, bool PL>
 __device__ __forceinline__ void mixer_bwd_finish(const float *ws, const float *wsf, T *__restrict__ dh,
                                                  T *__restrict__ dwf, const Dims &dm, const MfmaPlan &pl, int cb, int kf)
 {
@@ -237,8 +285,9 @@ __device__ __forceinline__ void mixer_bwd_finish(const float *ws, const float *w
     const int64_t nf = 3 * dm.d;
     for (int idx = tid; idx < kf * 3 * G::CB; idx += G::NT) {
         const int kk = idx / (3 * G::CB), col = idx % (3 * G::CB);
-        const int64_t f = (int64_t)cb * 3 * G::CB + col;
-        if (f >= nf) continue;
+        // the block's feature channels: 3 * CB consecutive ones, or CB of each plane
+        const int64_t f = PL ? (int64_t)(col / G::CB) * dm.d + (int64_t)cb * G::CB + col % G::CB : (int64_t)cb * 3 * G::CB + col;
+        if (PL ? (int64_t)cb * G::CB + col % G::CB >= dm.d : f >= nf) continue;
         float sum = 0.f;
         for (int64_t p = 0; p < np; ++p)
             sum += __hip_atomic_load(wsf + ((size_t)kk * np + p) * nf + f, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -246,7 +295,7 @@ __device__ __forceinline__ void mixer_bwd_finish(const float *ws, const float *w
     }
 }
 
-template <typename T>
+template <typename T, bool PL = false>
 __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ raw,
                                                                     const T *__restrict__ h, const T *__restrict__ wfeat,
                                                                     int kf, T *__restrict__ draw, T *__restrict__ dh,
@@ -292,10 +341,11 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
     // stores are dropped, and lanes whose channels lie beyond the tensor add WIN_OFF.
     const uint32_t rb = (uint32_t)row_bytes, bad = cvalid ? 0u : WIN_OFF, step_b = (uint32_t)STEP * rb;
     const uint32_t col_b = (uint32_t)((c0 + 2 * a) * 2);
-    const uint32_t lane_raw = 3u * ((uint32_t)(NR * rr - NH) * rb + col_b) + bad;      // row NR*rr-NH of a step
+    const uint32_t lane_raw = PL ? 3u * ((uint32_t)(NR * rr - NH) * rb) + col_b + bad
+                                 : 3u * ((uint32_t)(NR * rr - NH) * rb + col_b) + bad;     // row NR*rr-NH of a step
     auto step_base = [&](int64_t step, int64_t origin) { return (uint32_t)((step * STEP - origin) * row_bytes); };
     float tap[KF][NV];
-    load_feat_taps<T, KF, NV>(wfeat, cvalid ? 3 * (c0 + 2 * a) : 0, kf, tap);
+    lane_feat_taps<T, KF, PL>(wfeat, c0 + 2 * a, cvalid, d, kf, tap);
     const int own_off = (rr * LPR + a) * G::BLK;                                   // own rows in a slot
     const int halo_off = rr ? ((rr - 1) * LPR + a) * G::BLK + 24 : G::PRE + a * 24;    // the NH rows before them
 
@@ -369,7 +419,7 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
                             dro[i] = values_piece<T>(o);
                         }
 #pragma unroll
-                        for (int i = 0; i < NR; ++i) stw12(wdr, lane_raw + dr_b + 3u * (uint32_t)i * rb, dro[i]);
+                        for (int i = 0; i < NR; ++i) piece_store<PL>(wdr, lane_raw + dr_b + 3u * (uint32_t)i * rb, rb, dro[i]);
                         dr_b += 3u * step_b;
                         dfb ^= G::PRE;
                         dfp = dfp == 2 * G::PRE_BYTES ? 0 : dfp + G::PRE_BYTES;
@@ -432,7 +482,7 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
                 __hip_atomic_store(out + lag, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        mixer_bwd_finish<T>(ws, wsf, dh, dwf, dm, pl, cb, kf);
+        mixer_bwd_finish<T, PL>(ws, wsf, dh, dwf, dm, pl, cb, kf);
         return;
     }
 
@@ -458,7 +508,7 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
     struct Rows { u32x3 p[NH + NR]; uint32_t dy[NR]; };
     auto fetch = [&](Rows &r, uint32_t raw_base, uint32_t dy_base) {
 #pragma unroll
-        for (int i = 0; i < NH + NR; ++i) r.p[i] = ldw12_cached(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb));
+        for (int i = 0; i < NH + NR; ++i) r.p[i] = piece_load_cached<PL>(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb), rb);
 #pragma unroll
         for (int i = 0; i < NR; ++i) r.dy[i] = ldw4_cached(wdy, lane_dy + dy_base + (uint32_t)i * rb);
     };
@@ -478,7 +528,7 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
             float c0r, c1r, d0, d1;
-            M::unpack2(M::pack2(feat_sum(tap, rv, i, 0), feat_sum(tap, rv, i, 3)), c0r, c1r);
+            M::unpack2(M::pack2(feat_sum(tap, rv, i, vi<PL>(0, 0)), feat_sum(tap, rv, i, vi<PL>(1, 0))), c0r, c1r);
             M::unpack2(r.dy[i], d0, d1);
             g2n[i] = M::pack2(d0 * c0r, d1 * c1r);
         }
@@ -558,8 +608,8 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
             for (int i = 0; i < NR; ++i) {
                 float dv[2], o[NV];
                 M::unpack2(dq[0][i], dv[0], dv[1]);
-                o[0] = dv[0] * y2v[i].x; o[1] = duv[i].x * xk[i][0]; o[2] = duv[i].x * Bk[i][0];
-                o[3] = dv[1] * y2v[i].y; o[4] = duv[i].y * xk[i][1]; o[5] = duv[i].y * Bk[i][1];
+                o[vi<PL>(0, 0)] = dv[0] * y2v[i].x; o[vi<PL>(0, 1)] = duv[i].x * xk[i][0]; o[vi<PL>(0, 2)] = duv[i].x * Bk[i][0];
+                o[vi<PL>(1, 0)] = dv[1] * y2v[i].y; o[vi<PL>(1, 1)] = duv[i].y * xk[i][1]; o[vi<PL>(1, 2)] = duv[i].y * Bk[i][1];
                 po[i] = values_piece<T>(o);
             }
             lds_store_blk(df_own + dfb, pieces_blk(po));
@@ -575,8 +625,8 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
 #pragma unroll
             for (int i = 0; i < NR; ++i) {
                 // rounded to the tensors' type like the featurizer's output, then kept as fp32 for the gradient
-                M::unpack2(M::pack2(feat_sum(tap, rv, i, 1), feat_sum(tap, rv, i, 4)), Bk[i][0], Bk[i][1]);
-                M::unpack2(M::pack2(feat_sum(tap, rv, i, 2), feat_sum(tap, rv, i, 5)), xk[i][0], xk[i][1]);
+                M::unpack2(M::pack2(feat_sum(tap, rv, i, vi<PL>(0, 1)), feat_sum(tap, rv, i, vi<PL>(1, 1))), Bk[i][0], Bk[i][1]);
+                M::unpack2(M::pack2(feat_sum(tap, rv, i, vi<PL>(0, 2)), feat_sum(tap, rv, i, vi<PL>(1, 2))), xk[i][0], xk[i][1]);
                 *(uint32_t *)(u_own + i * UROW) = M::pack2(xk[i][0] * Bk[i][0], xk[i][1] * Bk[i][1]);
                 *(uint32_t *)(g_own + gs + i * UROW) = g2n[i];
             }
@@ -664,14 +714,15 @@ __global__ __launch_bounds__(MixGeo<T>::NT) void mixer_mr_bwd_kernel(const T *__
     for (int idx = tid; idx < KF * LPR * NV; idx += 64 * MW) {
         const int m = idx / (LPR * NV), col = idx % (LPR * NV);
         const int kk = m - (KF - kf);                           // index into the kf taps of the filter
-        const int64_t f = 3 * c0 + col;
-        if (kk < 0 || f >= 3 * d) continue;
+        // column a * NV + v: value v of the lane that owns channels c0 + 2a, 2a+1
+        const int64_t f = PL ? feature_channel<true>(c0 + 2 * (col / NV), col % NV, d) : 3 * c0 + col;
+        if (kk < 0 || (PL ? c0 + 2 * (col / NV) + (col % NV) % 2 >= d : f >= 3 * d)) continue;
         float sum = 0.f;
 #pragma unroll
         for (int r = 0; r < G::NG; ++r) sum += wacc[(m * G::NG + r) * (LPR * NV) + col];
         __hip_atomic_store(wsf + ((size_t)kk * nprow + prow) * (3 * d) + f, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    mixer_bwd_finish<T>(ws, wsf, dh, dwf, dm, pl, cb, kf);
+    mixer_bwd_finish<T, PL>(ws, wsf, dh, dwf, dm, pl, cb, kf);
 }
 
 // ---------------------------------------------------------------------------- forward
@@ -697,7 +748,7 @@ template <typename T> struct MixFwdGeo {
     static_assert(XW * HTAB * 2 <= STEP * YROW, "filter tables fit");
 };
 
-template <typename T>
+template <typename T, bool PL = false>
 __global__ __launch_bounds__(MixFwdGeo<T>::NT) void mixer_mr_fwd_kernel(const T *__restrict__ raw, const T *__restrict__ h,
                                                                        const T *__restrict__ wfeat, int kf,
                                                                        T *__restrict__ y, Dims dm, MfmaPlan pl)
@@ -780,18 +831,19 @@ __global__ __launch_bounds__(MixFwdGeo<T>::NT) void mixer_mr_fwd_kernel(const T 
     const win_t wy = make_window(y + (b * L + T0) * d, (T1 - T0) * row_bytes);
     const uint32_t rb = (uint32_t)row_bytes, bad = cvalid ? 0u : WIN_OFF, step_b = (uint32_t)STEP * rb;
     const uint32_t col_b = (uint32_t)((c0 + 2 * a) * 2);
-    const uint32_t lane_raw = 3u * ((uint32_t)(NR * rr - NH) * rb + col_b) + bad;      // row NR*rr-NH of a step
+    const uint32_t lane_raw = PL ? 3u * ((uint32_t)(NR * rr - NH) * rb) + col_b + bad
+                                 : 3u * ((uint32_t)(NR * rr - NH) * rb + col_b) + bad;     // row NR*rr-NH of a step
     const uint32_t lane_y = (uint32_t)(NR * rr) * rb + col_b + bad;                     // row NR*rr
     auto step_base = [&](int64_t step, int64_t origin) { return (uint32_t)((step * STEP - origin) * row_bytes); };
     float tap[KF][NV];
-    load_feat_taps<T, KF, NV>(wfeat, cvalid ? 3 * (c0 + 2 * a) : 0, kf, tap);
+    lane_feat_taps<T, KF, PL>(wfeat, c0 + 2 * a, cvalid, d, kf, tap);
     unsigned char *u_own = u_rm + NR * rr * UROW + 4 * a;
     const unsigned char *y_rd = y_st + NR * rr * YROW + 8 * a;
 
     struct Rows { u32x3 p[NH + NR]; };
     auto fetch = [&](Rows &r, uint32_t raw_base) {
 #pragma unroll
-        for (int i = 0; i < NH + NR; ++i) r.p[i] = ldw12_cached(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb));
+        for (int i = 0; i < NH + NR; ++i) r.p[i] = piece_load_cached<PL>(wraw, lane_raw + 3u * (raw_base + (uint32_t)i * rb), rb);
     };
     uint32_t un[NR], cn[NR];          // u and C of the step that arrived last
     // what arrived rows bring: the features, rounded like the featurizer's output, and with them u and C
@@ -802,9 +854,9 @@ __global__ __launch_bounds__(MixFwdGeo<T>::NT) void mixer_mr_fwd_kernel(const T 
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
             float x0, x1, B0, B1;
-            cn[i] = M::pack2(feat_sum(tap, rv, i, 0), feat_sum(tap, rv, i, 3));
-            M::unpack2(M::pack2(feat_sum(tap, rv, i, 1), feat_sum(tap, rv, i, 4)), B0, B1);
-            M::unpack2(M::pack2(feat_sum(tap, rv, i, 2), feat_sum(tap, rv, i, 5)), x0, x1);
+            cn[i] = M::pack2(feat_sum(tap, rv, i, vi<PL>(0, 0)), feat_sum(tap, rv, i, vi<PL>(1, 0)));
+            M::unpack2(M::pack2(feat_sum(tap, rv, i, vi<PL>(0, 1)), feat_sum(tap, rv, i, vi<PL>(1, 1))), B0, B1);
+            M::unpack2(M::pack2(feat_sum(tap, rv, i, vi<PL>(0, 2)), feat_sum(tap, rv, i, vi<PL>(1, 2))), x0, x1);
             un[i] = M::pack2(x0 * B0, x1 * B1);
         }
 #pragma unroll
@@ -898,8 +950,13 @@ int bwd_t(const void *dy, const void *raw, const void *wfeat, int kf, const void
     if (p.fuse_dh) p.slot = next_dh_slot();
     float *ws_dh = (float *)ws;
     float *ws_f = ws_dh + (size_t)p.nwg * G::XW * 128;
-    int e = launch_main(mixer_mr_bwd_kernel<T>, dim3((unsigned)p.nwg), dim3(G::NT), st, (const T *)dy, (const T *)raw,
-                        (const T *)h, (const T *)wfeat, kf, (T *)draw, (T *)dh, (T *)dwf, ws_dh, ws_f, dm, p);
+    int e = dm.planar
+                ? launch_main((mixer_mr_bwd_kernel<T, true>), dim3((unsigned)p.nwg), dim3(G::NT), st, (const T *)dy,
+                              (const T *)raw, (const T *)h, (const T *)wfeat, kf, (T *)draw, (T *)dh, (T *)dwf, ws_dh, ws_f,
+                              dm, p)
+                : launch_main((mixer_mr_bwd_kernel<T>), dim3((unsigned)p.nwg), dim3(G::NT), st, (const T *)dy,
+                              (const T *)raw, (const T *)h, (const T *)wfeat, kf, (T *)draw, (T *)dh, (T *)dwf, ws_dh, ws_f,
+                              dm, p);
     if (e || p.fuse_dh) return e;
     const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st, (const float *)ws_dh,
@@ -921,7 +978,10 @@ int fwd_t(const void *raw, const void *wfeat, int kf, const void *h, void *y, co
 {
     const MfmaPlan p = mixer_fwd_plan(dm);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    return launch_main(mixer_mr_fwd_kernel<T>, dim3((unsigned)p.nwg), dim3(MixFwdGeo<T>::NT), st, (const T *)raw,
+    if (dm.planar)
+        return launch_main((mixer_mr_fwd_kernel<T, true>), dim3((unsigned)p.nwg), dim3(MixFwdGeo<T>::NT), st,
+                           (const T *)raw, (const T *)h, (const T *)wfeat, kf, (T *)y, dm, p);
+    return launch_main((mixer_mr_fwd_kernel<T>), dim3((unsigned)p.nwg), dim3(MixFwdGeo<T>::NT), st, (const T *)raw,
                        (const T *)h, (const T *)wfeat, kf, (T *)y, dm, p);
 }
 } // namespace

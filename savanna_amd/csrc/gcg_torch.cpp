@@ -558,14 +558,17 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> bwd_time_major(const Tensor &dy, cons
 
 // ---- featurizer and Hyena-MR operator without the featurized tensor ----------------------------
 
-void check_mixer_mr(const Tensor &raw, const Tensor &wf, const Tensor &h)
+// planar: raw is (bs, L, 3, g, dg) -- the planes C | B | x of each row one after the other -- instead of (bs, L, g, dg, 3)
+void check_mixer_mr(const Tensor &raw, const Tensor &wf, const Tensor &h, bool planar = false)
 {
-    TORCH_CHECK(raw.dim() == 5 && raw.size(4) == 3 && raw.is_contiguous(),
-                "gcg: raw must be a contiguous (bs, L, g, dg, 3) tensor");
-    TORCH_CHECK(wf.dim() == 3 && wf.size(0) == 3 * raw.size(2) * raw.size(3) && wf.size(1) == 1 && wf.is_contiguous() &&
+    TORCH_CHECK(raw.dim() == 5 && raw.size(planar ? 2 : 4) == 3 && raw.is_contiguous(),
+                planar ? "gcg: raw must be a contiguous (bs, L, 3, g, dg) tensor"
+                       : "gcg: raw must be a contiguous (bs, L, g, dg, 3) tensor");
+    const int64_t g = raw.size(planar ? 3 : 2), dg = raw.size(planar ? 4 : 3);
+    TORCH_CHECK(wf.dim() == 3 && wf.size(0) == 3 * g * dg && wf.size(1) == 1 && wf.is_contiguous() &&
                     wf.scalar_type() == raw.scalar_type(),
                 "gcg: wf must be a contiguous (3 * g * dg, 1, kf) tensor of raw's dtype");
-    TORCH_CHECK(h.dim() == 3 && h.size(0) == raw.size(2) && h.size(1) == 1 && h.is_contiguous(),
+    TORCH_CHECK(h.dim() == 3 && h.size(0) == g && h.size(1) == 1 && h.is_contiguous(),
                 "gcg: h must be a contiguous (g, 1, hl) tensor");
     TORCH_CHECK(wf.device() == raw.device() && h.device() == raw.device(), "gcg: raw, wf and h must be on one device");
     (void)gated_code(raw, h);
@@ -625,35 +628,46 @@ std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd_decay(const Tensor &dy, const Te
     return {draw, dwf, dw};
 }
 
-Tensor mixer_mr_fwd(const Tensor &raw, const Tensor &wf, const Tensor &h)
+Tensor mixer_mr_fwd(const Tensor &raw, const Tensor &wf, const Tensor &h, bool planar)
 {
     require_gpu(raw, "raw");
-    check_mixer_mr(raw, wf, h);
+    check_mixer_mr(raw, wf, h, planar);
     DeviceGuard guard(raw.device());
-    Tensor y = at::empty({raw.size(0), raw.size(1), raw.size(2), raw.size(3)}, raw.options());
+    const int64_t g = raw.size(planar ? 3 : 2), dg = raw.size(planar ? 4 : 3);
+    Tensor y = at::empty({raw.size(0), raw.size(1), g, dg}, raw.options());
     if (y.numel() == 0) return y;
-    check_rc(gcg_mixer_mr_fwd(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), raw.size(0), raw.size(1),
-                              (int32_t)raw.size(2), (int32_t)raw.size(3), (int32_t)h.size(2), (int32_t)wf.size(2),
-                              gated_code(raw, h), stream_of(raw)),
-             "gcg_mixer_mr_fwd");
+    check_rc((planar ? gcg_mixer_mr_fwd_planar : gcg_mixer_mr_fwd)(
+                 raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), raw.size(0), raw.size(1), (int32_t)g,
+                 (int32_t)dg, (int32_t)h.size(2), (int32_t)wf.size(2), gated_code(raw, h), stream_of(raw)),
+             planar ? "gcg_mixer_mr_fwd_planar" : "gcg_mixer_mr_fwd");
     return y;
 }
 
-std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd(const Tensor &dy, const Tensor &raw, const Tensor &wf, const Tensor &h)
+std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd(const Tensor &dy, const Tensor &raw, const Tensor &wf, const Tensor &h,
+                                                bool planar)
 {
     require_gpu(raw, "raw");
-    check_mixer_mr(raw, wf, h);
-    TORCH_CHECK(dy.dim() == 4 && dy.sizes() == raw.sizes().slice(0, 4) && dy.scalar_type() == raw.scalar_type() &&
-                    dy.device() == raw.device() && dy.is_contiguous(),
+    check_mixer_mr(raw, wf, h, planar);
+    const int32_t g = (int32_t)raw.size(planar ? 3 : 2), dg = (int32_t)raw.size(planar ? 4 : 3);
+    TORCH_CHECK(dy.dim() == 4 && dy.size(0) == raw.size(0) && dy.size(1) == raw.size(1) && dy.size(2) == g &&
+                    dy.size(3) == dg && dy.scalar_type() == raw.scalar_type() && dy.device() == raw.device() &&
+                    dy.is_contiguous(),
                 "gcg: dy must be a contiguous (bs, L, g, dg) tensor of raw's dtype and device");
     DeviceGuard guard(raw.device());
     Tensor draw = at::empty_like(raw), dwf = at::empty_like(wf), dh = at::empty_like(h);
     if (dy.numel() == 0) return {draw, dwf.zero_(), dh.zero_()};
     const int64_t bs = raw.size(0), L = raw.size(1);
-    const int32_t g = (int32_t)raw.size(2), dg = (int32_t)raw.size(3), hl = (int32_t)h.size(2), kf = (int32_t)wf.size(2);
+    const int32_t hl = (int32_t)h.size(2), kf = (int32_t)wf.size(2);
     const int code = gated_code(raw, h);
     const size_t nbytes = gcg_mixer_mr_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code);
     Tensor ws = workspace(nbytes, raw, "gcg_mixer_mr_bwd_workspace_bytes");
+    if (planar) {
+        check_rc(gcg_mixer_mr_bwd_planar(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), h.data_ptr(), draw.data_ptr(),
+                                         dwf.data_ptr(), dh.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl, kf, code,
+                                         stream_of(raw)),
+                 "gcg_mixer_mr_bwd_planar");
+        return {draw, dwf, dh};
+    }
     // gradient of the featurized features, for the duration of the call (not needed where one kernel does it all)
     const size_t sbytes = gcg_mixer_mr_bwd_scratch_bytes(bs, L, g, dg, hl, kf, code);
     Tensor scratch = at::empty({(int64_t)sbytes}, raw.options().dtype(at::kByte));
@@ -816,15 +830,15 @@ std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd_decay_meta(const Tensor &dy, con
     return {at::empty_like(raw), at::empty_like(wf), at::empty_like(w)};
 }
 
-Tensor mixer_mr_fwd_meta(const Tensor &raw, const Tensor &wf, const Tensor &h)
+Tensor mixer_mr_fwd_meta(const Tensor &raw, const Tensor &wf, const Tensor &h, bool planar)
 {
-    check_mixer_mr(raw, wf, h);
-    return at::empty({raw.size(0), raw.size(1), raw.size(2), raw.size(3)}, raw.options());
+    check_mixer_mr(raw, wf, h, planar);
+    return at::empty({raw.size(0), raw.size(1), raw.size(planar ? 3 : 2), raw.size(planar ? 4 : 3)}, raw.options());
 }
 std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd_meta(const Tensor &dy, const Tensor &raw, const Tensor &wf,
-                                                     const Tensor &h)
+                                                     const Tensor &h, bool planar)
 {
-    check_mixer_mr(raw, wf, h);
+    check_mixer_mr(raw, wf, h, planar);
     (void)dy;
     return {at::empty_like(raw), at::empty_like(wf), at::empty_like(h)};
 }
@@ -848,8 +862,8 @@ TORCH_LIBRARY(gcg, m)
     m.def("mixer_se_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h, bool planar=False) -> (Tensor, Tensor, Tensor)");
     m.def("filter_decay_fwd(Tensor w, Tensor decay, int hl, ScalarType dtype) -> Tensor");
     m.def("filter_decay_bwd(Tensor dh, Tensor decay) -> Tensor");
-    m.def("mixer_mr_fwd(Tensor raw, Tensor wf, Tensor h) -> Tensor");
-    m.def("mixer_mr_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h) -> (Tensor, Tensor, Tensor)");
+    m.def("mixer_mr_fwd(Tensor raw, Tensor wf, Tensor h, bool planar=False) -> Tensor");
+    m.def("mixer_mr_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h, bool planar=False) -> (Tensor, Tensor, Tensor)");
     m.def("mixer_mr_fwd_decay(Tensor raw, Tensor wf, Tensor w, Tensor decay, int hl, ScalarType filt) -> Tensor");
     m.def("mixer_mr_bwd_decay(Tensor dy, Tensor raw, Tensor wf, Tensor w, Tensor decay, int hl, ScalarType filt)"
           " -> (Tensor, Tensor, Tensor)");

@@ -337,18 +337,20 @@ class _FeaturizedShortGateConvGate(torch.autograd.Function):
 class _FeaturizedGateConvGate(torch.autograd.Function):
     """z = gated Hyena-MR convolution of the featurized projection, raw (b, l, g, dg, 3) -> (b, l, g, dg), without
     the featurized tensor: the forward makes its rows on the way, the backward recomputes them from raw and hands
-    their gradient to the featurizer's backward inside the same call.  Only raw, wf and h are saved."""
+    their gradient to the featurizer's backward inside the same call.  Only raw, wf and h are saved.
+    ``planar``: raw is (b, l, 3, g, dg)."""
 
     @staticmethod
-    def forward(ctx, raw, wf, h):
+    def forward(ctx, raw, wf, h, planar=False):
         raw, wf, h = (t if t.is_contiguous() else t.contiguous() for t in (raw, wf, h))
         ctx.save_for_backward(raw, wf, h)
-        return _lib.mixer_mr_fwd(raw, wf, h)
+        ctx.planar = planar
+        return _lib.mixer_mr_fwd(raw, wf, h, planar)
 
     @staticmethod
     def backward(ctx, dz):
         raw, wf, h = ctx.saved_tensors
-        return _lib.mixer_mr_bwd(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, h)
+        return _lib.mixer_mr_bwd(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, h, ctx.planar) + (None,)
 
 
 class _FeaturizedDecayedGateConvGate(torch.autograd.Function):
@@ -416,6 +418,13 @@ class HyenaMixer(nn.Module):
                                                        conv.short_conv_weight.to(op.cgcg_dtype), h.to(op.cgcg_dtype), True)
                 z = z.reshape(bs, seqlen, g * dg)
                 return z.to(dtype) if op.cgcg_dtype != dtype else z
+            if (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and op.cgcg_dtype == features.dtype and
+                    features.dtype in (torch.bfloat16, torch.float16) and
+                    _lib.mixer_mr_supported(op.group_dim, h.shape[-1], conv.kernel_size, features)):
+                g, dg = op.num_groups, op.group_dim
+                z = _FeaturizedGateConvGate.apply(features.reshape(bs, seqlen, 3, g, dg),
+                                                  conv.short_conv_weight.to(features.dtype), h.to(op.cgcg_dtype), True)
+                return z.reshape(bs, seqlen, g * dg)
             return op.forward_features(conv.forward_bld(features, feeds_operator=True), interleaved=False)
         fused = op._filter_in_kernel(seqlen, op.num_groups, op.group_dim, features.dtype, features)
         if (fused is not None and self.fuse_medium and conv.group_dim == 1 and

@@ -120,6 +120,9 @@ WORKLOADS = {
     "mixer_fwdbwd_7b_fused": Workload("mixer_fwdbwd_7b_fused", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
                                       "the same without the featurized tensor: the operator's kernels make its rows "
                                       "from the projection output, forward and backward", layout="mixer_fused"),
+    "mixer_fwdbwd_7b_fused_planar": Workload("mixer_fwdbwd_7b_fused_planar", 2, 8192, 256, 16, (128,), torch.bfloat16,
+                                             True, "the same on planar features (interleave_projections = false): "
+                                             "gcg_mixer_mr_fwd_planar / _bwd_planar", layout="mixer_fused_planar"),
     "mixer_fwd_7b": Workload("mixer_fwd_7b", 2, 8192, 256, 16, (128,), torch.bfloat16, False,
                              "featurizer conv + Hyena-MR on interleaved features, forward only (prefill), bf16, "
                              "B=2 L=8192 D=4096 G=256 hl=128", layout="mixer"),

@@ -192,3 +192,89 @@ def test_hyena_mixer_keeps_no_featurized_tensor(gcg_lib, act, cgcg):
     if cgcg == "bfloat16":       # filter, featurizer and operator: nothing else of the library's is launched
         ours = [e.key for e in prof.key_averages() if "gcg::" in e.key and e.device_time_total > 0]
         assert len(ours) == 2 and all("mixer_mr" in k for k in ours), ours
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("bs,L,g,dg,hl,kf", SHAPES)
+def test_planar_features_match_interleaved(gcg_lib, bs, L, g, dg, hl, kf, dtype):
+    """gcg_mixer_mr_fwd_planar / _bwd_planar -- raw (bs, L, 3, g, dg), the split without interleaving of
+    block.py:881-884, with the featurizer's filters in that channel order -- give the interleaved entry points'
+    results on the same values, bit for bit (the same arithmetic on pieces loaded plane by plane)."""
+    raw, wf, h, dy = (t.to(DEV) for t in make(bs, L, g, dg, hl, kf, dtype, dtype, seed=23))
+    d = g * dg
+    raw_pl = raw.permute(0, 1, 4, 2, 3).contiguous()                                          # (bs, L, 3, g, dg)
+    wf_pl = wf.view(d, 3, 1, kf).permute(1, 0, 2, 3).reshape(3 * d, 1, kf).contiguous()       # row p * d + c <- row 3 c + p
+    y = _lib.mixer_mr_fwd(raw, wf, h)
+    draw, dwf, dh = _lib.mixer_mr_bwd(dy, raw, wf, h)
+    y_pl = _lib.mixer_mr_fwd(raw_pl, wf_pl, h, planar=True)
+    draw_pl, dwf_pl, dh_pl = _lib.mixer_mr_bwd(dy, raw_pl, wf_pl, h, planar=True)
+    torch.cuda.synchronize()
+    assert y_pl.shape == y.shape and draw_pl.shape == raw_pl.shape and dwf_pl.shape == wf.shape
+    assert torch.equal(y_pl, y)
+    assert torch.equal(draw_pl, draw.permute(0, 1, 4, 2, 3))
+    assert torch.equal(dwf_pl.view(3, d, 1, kf), dwf.view(d, 3, 1, kf).permute(1, 0, 2, 3))
+    assert torch.equal(dh_pl, dh)
+
+
+def test_planar_full_size(gcg_lib):
+    """The same at the 7B layer shape."""
+    bs, L, g, dg, hl, kf = 2, 8192, 256, 16, 128, 3
+    gen = torch.Generator(device=DEV).manual_seed(3)
+    raw = torch.randn(bs, L, g, dg, 3, generator=gen, device=DEV).to(torch.bfloat16)
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen, device=DEV)).to(torch.bfloat16)
+    wf = (torch.randn(3 * g * dg, 1, kf, generator=gen, device=DEV) / kf ** 0.5).to(torch.bfloat16)
+    h = (torch.randn(g, 1, hl, generator=gen, device=DEV) / hl ** 0.5).to(torch.bfloat16)
+    d = g * dg
+    raw_pl = raw.permute(0, 1, 4, 2, 3).contiguous()
+    wf_pl = wf.view(d, 3, 1, kf).permute(1, 0, 2, 3).reshape(3 * d, 1, kf).contiguous()
+    y = _lib.mixer_mr_fwd(raw, wf, h)
+    draw, dwf, dh = _lib.mixer_mr_bwd(dy, raw, wf, h)
+    y_pl = _lib.mixer_mr_fwd(raw_pl, wf_pl, h, planar=True)
+    draw_pl, dwf_pl, dh_pl = _lib.mixer_mr_bwd(dy, raw_pl, wf_pl, h, planar=True)
+    torch.cuda.synchronize()
+    assert torch.equal(y_pl, y) and torch.equal(draw_pl, draw.permute(0, 1, 4, 2, 3)) and torch.equal(dh_pl, dh)
+    assert torch.equal(dwf_pl.view(3, d, 1, kf), dwf.view(d, 3, 1, kf).permute(1, 0, 2, 3))
+
+
+def test_planar_refused_for_fp32_arithmetic(gcg_lib):
+    raw, wf, h, dy = (t.to(DEV) for t in make(1, 64, 2, 16, 128, 3, torch.float32, torch.float32))
+    with pytest.raises(RuntimeError, match="not supported"):
+        _lib.mixer_mr_fwd(raw.permute(0, 1, 4, 2, 3).contiguous(), wf, h, planar=True)
+
+
+def test_hyena_mixer_planar_fused(gcg_lib):
+    """HyenaMixer(interleave_projections=False) with a Hyena-MR operator: one kernel each way, same output and
+    gradients as the two-kernel chain on the same layout."""
+    from savanna_amd.operators.hyena import CgcgConfig, HyenaMROperator, HyenaMixer
+
+    torch.manual_seed(0)
+    bs, L, g, dg = 2, 384, 4, 16
+    op = HyenaMROperator(g * dg, g, 128, CgcgConfig(cgcg_dtype="bfloat16"), small_init=False, device=DEV)
+    mixer = HyenaMixer(op, 3, dtype=torch.bfloat16, device=DEV, interleave_projections=False)
+    feats = torch.randn(bs, L, 3 * g * dg, device=DEV).to(torch.bfloat16).requires_grad_(True)
+    dz = (0.1 * torch.randn(bs, L, g * dg, device=DEV)).to(torch.bfloat16)
+    params = [op.filter.h, mixer.hyena_proj_conv.short_conv_weight]
+
+    def run(fuse):
+        mixer.fuse_medium = fuse
+        feats.grad = None
+        for p in params:
+            p.grad = None
+        z = mixer(feats)
+        z.backward(dz)
+        return [z.detach(), feats.grad.clone()] + [p.grad.clone() for p in params]
+
+    want = run(False)
+    from torch.profiler import ProfilerActivity, profile
+    with profile(activities=[ProfilerActivity.CUDA]) as prof:
+        got = run(True)
+        torch.cuda.synchronize()
+    for a, b, n in zip(got, want, ("z", "dfeatures", "dw", "dwf")):
+        if n == "dw":
+            assert_close(a, b, 2e-5, n)
+        elif n == "dwf":
+            assert_close(a, b, TOL_DH[torch.bfloat16], n)
+        else:
+            assert torch.equal(a, b), n
+    big = [e.key for e in prof.key_averages() if "mfma" in e.key or "dwconv" in e.key or "mixer_mr" in e.key]
+    assert len(big) == 2 and all("mixer_mr" in k for k in big), big

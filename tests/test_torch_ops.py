@@ -45,6 +45,12 @@ def test_meta_shapes_on_fake_gpu_tensors(gcg_lib):
         assert hh.shape == (g, 1, 64) and hh.dtype == torch.float16
         assert torch.ops.gcg.filter_decay_bwd(hh, p).shape == p.shape
         planar = torch.empty(bs, L, 3, g, dg, dtype=torch.bfloat16, device="cuda")
+        assert torch.ops.gcg.mixer_mr_fwd(planar, wf, h, True).shape == x.shape
+        assert torch.ops.gcg.mixer_se_fwd(planar, wf, h7, True).shape == x.shape
+        dpl, dwf_pl, dh_pl = torch.ops.gcg.mixer_mr_bwd(x, planar, wf, h, True)
+        assert dpl.shape == planar.shape and dwf_pl.shape == wf.shape and dh_pl.shape == h.shape
+        dpl, dwf_pl, dh_pl = torch.ops.gcg.mixer_se_bwd(x, planar, wf, h7, True)
+        assert dpl.shape == planar.shape and dwf_pl.shape == wf.shape and dh_pl.shape == h7.shape
         assert torch.ops.gcg.fwd_planar(planar, h).shape == x.shape
         dplanar, dh = torch.ops.gcg.bwd_planar(x, planar, h)
         assert dplanar.shape == planar.shape and dh.shape == h.shape
