@@ -195,6 +195,37 @@ def test_interleaved_views_are_recognised_on_the_host():
     assert src is not None and src.data_ptr() == big[1:].data_ptr()
 
 
+def test_planar_views_are_recognised_on_the_host():
+    """The split without interleaving (block.py:881-884) gives three views whose rows lie 3 d elements apart;
+    the autograd boundary must find their buffer, and only then."""
+    import torch
+    from einops import rearrange
+
+    from savanna_amd.kernels.cgcg.interface import planar_source
+
+    g, dg = 4, 16
+    d = g * dg
+    feats = torch.randn(2, 5, 3 * d)
+    x1, x2, v = rearrange(feats, "b l (p g dg) -> b l p g dg", p=3, g=g).unbind(dim=2)
+    src = planar_source(x=v, B=x2, C=x1)
+    assert src is not None and src.shape == (2, 5, 3, g, dg) and src.data_ptr() == feats.data_ptr()
+    assert torch.equal(src[:, :, 0], x1) and torch.equal(src[:, :, 1], x2) and torch.equal(src[:, :, 2], v)
+    # wrong order, gathered copies, a padded row, the interleaved split, separate tensors: not recognised
+    assert planar_source(x=x1, B=x2, C=v) is None
+    assert planar_source(x=v.contiguous(), B=x2, C=x1) is None
+    padded = torch.randn(2, 5, 3 * d + 8)[:, :, 8:]
+    p1, p2, pv = rearrange(padded, "b l (p g dg) -> b l p g dg", p=3, g=g).unbind(dim=2)
+    assert planar_source(x=pv, B=p2, C=p1) is None
+    q1, q2, qv = rearrange(feats, "b l (g dg p) -> b l g p dg", p=3, g=g).unbind(dim=3)
+    assert planar_source(x=qv, B=q2, C=q1) is None
+    assert planar_source(x=torch.randn(2, 5, g, dg), B=torch.randn(2, 5, g, dg), C=torch.randn(2, 5, g, dg)) is None
+    # an offset into a larger buffer is fine
+    big = torch.randn(3, 5, 3 * d)
+    b1, b2, bv = rearrange(big[1:], "b l (p g dg) -> b l p g dg", p=3, g=g).unbind(dim=2)
+    src = planar_source(x=bv, B=b2, C=b1)
+    assert src is not None and src.data_ptr() == big[1:].data_ptr()
+
+
 def test_workspace_sizing_runs_on_the_host_for_any_shape(gcg_lib):
     """The *_workspace_bytes entry points are host arithmetic (launch plans): every shape, also a
     tensor narrower than a lane's vector, must give a 256-byte multiple or 0 -- never trap."""
