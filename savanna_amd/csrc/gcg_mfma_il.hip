@@ -239,7 +239,6 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     const int j = l & 15, q = l >> 4;               // matrix layout
     const int64_t d = dm.d, L = dm.L;
     const int64_t c0 = (int64_t)cb * CB;
-    const int hl = dm.hl;
     const bool wave_valid = c0 + 16 * w < d;
 
     const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
