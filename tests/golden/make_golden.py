@@ -84,9 +84,50 @@ def mixer_se_case():
     print("mixer_se_bf16_small written")
 
 
+def mixer_mr_case():
+    """The convolutional part of a Hyena-MR layer as the reference chains it, in float64 with its bf16 tensors
+    emulated: the decayed filter h = (w * decay)[:, :hl] cast to the tensors' type
+    (savanna/model/operators/hyena/parametrization/explicit.py:68-75, hyena.py:440-441, :499-503), the featurizer
+    conv and interleaved split as in mixer_se_case (block.py:867-890), and y = x1 * conv(x2 * v, h)
+    (hyena.py:517-531 -> ref_fwd.py:109-129).  The gradient of the filter is stored in the filter's type before
+    it reaches w, as autograd of the cast does."""
+    import torch.nn.functional as F
+    from einops import rearrange
+
+    bs, L, g, dg, hl, lc, K, dtype = 2, 300, 3, 16, 128, 160, 3, torch.bfloat16
+    D = g * dg
+    gen = torch.Generator().manual_seed(0)
+    raw = torch.randn(bs, L, 3 * D, generator=gen).to(dtype).double().requires_grad_(True)
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen)).to(dtype).double()
+    wf = (torch.randn(3 * D, 1, K, generator=gen) / K ** 0.5).to(dtype).double().requires_grad_(True)
+    w = (torch.randn(g, lc, generator=gen) / lc ** 0.5).float().double().requires_grad_(True)
+    decay = torch.exp(-torch.logspace(0, 2, g)[:, None] * torch.linspace(0, 1, lc)[None]).float().double()
+    hfull = (w * decay)[:, :hl]
+    h = hfull + (hfull.to(dtype).double() - hfull).detach()       # the cast to the tensors' type
+    h.register_hook(lambda gr: gr.to(dtype).double())             # whose gradient is stored in that type
+    h = h[:, None]
+    u = raw.permute(0, 2, 1)
+    f = F.conv1d(F.pad(u, (K - 1, 0)), wf, bias=None, stride=1, padding=0, groups=3 * D)[..., :L].permute(0, 2, 1)
+    f = f + (f.to(dtype).double() - f).detach()
+    f.register_hook(lambda gr: gr.to(dtype).double())
+    x1, x2, v = rearrange(f, "b l (g dg p) -> b l g p dg", p=3, g=g).unbind(dim=3)
+    y = oracle.gcg_fwd_ref_torch(v.contiguous(), x2.contiguous(), x1.contiguous(), h)
+    y.backward(dy)
+    np.savez_compressed(
+        os.path.join(HERE, "mixer_mr_bf16_small.npz"),
+        raw=raw.detach().reshape(bs, L, g, dg, 3).float().numpy(), dy=dy.float().numpy(),
+        wf=wf.detach().float().numpy(), w=w.detach().float().numpy(), decay=decay.float().numpy(),
+        h=h.detach().float().numpy(), hl=np.array(hl), y=y.detach().numpy(),
+        draw=raw.grad.reshape(bs, L, g, dg, 3).numpy(), dwf=wf.grad.numpy(), dw=w.grad.numpy(),
+        dtype=np.array(str(dtype)),
+    )
+    print("mixer_mr_bf16_small written")
+
+
 def main():
     featurizer_case()
     mixer_se_case()
+    mixer_mr_case()
     for name, (bs, L, g, dg, hl, dtype) in CASES.items():
         gen = torch.Generator().manual_seed(0)
         x, B, C, dy = (torch.randn(bs, L, g, dg, generator=gen).to(dtype).double() for _ in range(4))

@@ -17,18 +17,19 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ALL = sorted(glob.glob(os.path.join(HERE, "golden", "*.npz")))
 FEAT = [f for f in ALL if os.path.basename(f).startswith("featurizer")]           # the ungated featurizer conv
 MIXER = [f for f in ALL if os.path.basename(f).startswith("mixer_se")]            # featurizer + Hyena-SE operator
-FILES = [f for f in ALL if f not in FEAT and f not in MIXER]                      # the gated operator
+MIXER_MR = [f for f in ALL if os.path.basename(f).startswith("mixer_mr")]         # featurizer + Hyena-MR operator, decayed filter
+FILES = [f for f in ALL if f not in FEAT and f not in MIXER and f not in MIXER_MR]   # the gated operator
 DT = {"torch.float32": torch.float32, "torch.bfloat16": torch.bfloat16, "torch.float16": torch.float16}
 
 
 def load(path):
     z = np.load(path, allow_pickle=False)
-    t = {k: torch.from_numpy(z[k]) for k in z.files if k != "dtype"}
+    t = {k: torch.from_numpy(z[k]) for k in z.files if k != "dtype"}     # (0-d arrays, e.g. hl, become 0-d tensors)
     return t, DT[str(z["dtype"])]
 
 
 def test_fixtures_present():
-    assert len(FILES) >= 4 and len(FEAT) >= 1 and len(MIXER) >= 1
+    assert len(FILES) >= 4 and len(FEAT) >= 1 and len(MIXER) >= 1 and len(MIXER_MR) >= 1
 
 
 @pytest.mark.parametrize("path", FILES, ids=[os.path.basename(f) for f in FILES])
@@ -140,3 +141,56 @@ def test_hip_mixer_reproduces_golden(gcg_lib, path):
     assert_close(draw, t["draw"], 2 * TOL[dtype], "d raw")
     assert_close(dwf, t["dwf"], 2 * TOL_DH[dtype], "dwf")
     assert_close(dh, t["dh"], TOL_DH[dtype], "dh")
+
+
+def _dw_from_dh(dh, t, dtype):
+    """Gradient of the filter parameter from the gradient of the filter: through the cast to the tensors' type
+    (stored in that type) and the product with the decay, zero beyond the taps in use."""
+    hl = int(t["hl"])
+    dw = torch.zeros_like(t["w"])
+    dw[:, :hl] = dh[:, 0].to(dtype).float() * t["decay"][:, :hl]
+    return dw
+
+
+@pytest.mark.parametrize("path", MIXER_MR, ids=[os.path.basename(f) for f in MIXER_MR])
+def test_c_oracle_chain_reproduces_mixer_mr_golden(path):
+    """The Hyena-MR layer's chain written with F.conv1d, rearrange / unbind and autograd in float64 (decayed filter,
+    featurizer, operator) against the oracle applied twice on the fixture's filter, and the filter as
+    (w * decay)[:, :hl] rounded to the tensors' type."""
+    t, dtype = load(path)
+    hl = int(t["hl"])
+    h = (t["w"] * t["decay"])[:, :hl].to(dtype).float()[:, None]
+    assert torch.equal(h, t["h"])
+    y, draw, dwf, dh = _chain_with_oracle(t, dtype)
+    assert_close(y, t["y"], TOL[dtype], "y")
+    assert_close(draw, t["draw"], TOL[dtype], "d raw")
+    assert_close(dwf, t["dwf"], TOL_DH[dtype], "dwf")
+    assert_close(_dw_from_dh(dh, t, dtype), t["dw"], TOL_DH[dtype], "dw")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layout", ["interleaved", "planar"])
+@pytest.mark.parametrize("path", MIXER_MR, ids=[os.path.basename(f) for f in MIXER_MR])
+def test_hip_mixer_mr_reproduces_golden(gcg_lib, path, layout):
+    """gcg_mixer_mr_fwd_decay / _bwd_decay (filter formed in the kernels) and, on the planar layout of the same
+    values, gcg_mixer_mr_fwd_planar / _bwd_planar with the fixture's filter."""
+    t, dtype = load(path)
+    hl = int(t["hl"])
+    dev = {k: (v.to(dtype) if k not in ("w", "decay", "hl") else v).to("cuda:0") for k, v in t.items()}
+    if layout == "interleaved":
+        y = _lib.mixer_mr_fwd_decay(dev["raw"], dev["wf"], dev["w"], dev["decay"], hl, dtype)
+        draw, dwf, dw = _lib.mixer_mr_bwd_decay(dev["dy"], dev["raw"], dev["wf"], dev["w"], dev["decay"], hl, dtype)
+    else:
+        bs, L, g, dg, _ = t["raw"].shape
+        d = g * dg
+        raw_pl = dev["raw"].permute(0, 1, 4, 2, 3).contiguous()
+        wf_pl = dev["wf"].view(d, 3, 1, -1).permute(1, 0, 2, 3).reshape(3 * d, 1, -1).contiguous()
+        y = _lib.mixer_mr_fwd(raw_pl, wf_pl, dev["h"], planar=True)
+        draw_pl, dwf_pl, dh = _lib.mixer_mr_bwd(dev["dy"], raw_pl, wf_pl, dev["h"], planar=True)
+        draw = draw_pl.permute(0, 1, 3, 4, 2)
+        dwf = dwf_pl.view(3, d, 1, -1).permute(1, 0, 2, 3).reshape(3 * d, 1, -1)
+        dw = _dw_from_dh(dh.float().cpu(), t, dtype)
+    assert_close(y, t["y"], TOL[dtype], "y")
+    assert_close(draw, t["draw"], 2 * TOL[dtype], "d raw")
+    assert_close(dwf, t["dwf"], 2 * TOL_DH[dtype], "dwf")
+    assert_close(dw, t["dw"], TOL_DH[dtype], "dw")
