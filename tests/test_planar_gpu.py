@@ -252,3 +252,27 @@ def test_operator_modules_read_planar_views_in_place(gcg_lib, monkeypatch, kind)
     torch.cuda.synchronize()
     assert calls["planar"] == 1 and calls["plain"] + calls["decay"] == 1, calls
     assert torch.equal(z, z_ref)
+
+
+@pytest.mark.parametrize("act", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("hl,algo", [(128, "mfma"), (64, "mfma"), (7, "window"), (7, "direct")])
+def test_planar_with_fp32_arithmetic(gcg_lib, act, hl, algo):
+    """16-bit planar features with an fp32 filter (fp32 arithmetic inside, cgcg_dtype float32 on 16-bit activations):
+    the same results as on gathered copies."""
+    bs, L, g, dg = 2, 700, 5, 16
+    x, B, C, h, dy = inputs(bs, L, g, dg, hl, act, seed=8, dy_scale=0.1)
+    h = h.float()
+    xd, Bd, Cd, hd, dyd = (t.to(DEV) for t in (x, B, C, h, dy))
+    feat = pack(xd, Bd, Cd)
+    y = _lib.fwd_planar(feat, hd, algo=algo)
+    dfeat, dh = _lib.bwd_planar(dyd, feat, hd, algo=algo)
+    _, _, y_p = _lib.fwd(xd, Bd, Cd, hd, algo=algo)
+    dx, dB, dC, dh_p = _lib.bwd(dyd, xd, Bd, Cd, hd, algo=algo)
+    torch.cuda.synchronize()
+    assert y.dtype == act and dh.dtype == torch.float32
+    assert torch.equal(y, y_p)
+    assert torch.equal(dfeat[:, :, 0], dC) and torch.equal(dfeat[:, :, 1], dB) and torch.equal(dfeat[:, :, 2], dx)
+    if same_kernel_family(hl, algo):
+        assert torch.equal(dh, dh_p)
+    else:
+        assert_close(dh, dh_p, 2e-5, "dh")
