@@ -212,8 +212,6 @@ GCG_API int gcg_bwd_interleaved(const void *dy, const void *feat, const void *h,
  * the kernels read the thirds of the rows in place and write dfeat (same layout) directly.
  *   feat, dfeat  (bs, L, 3, g, dg)   h, dh  (g, 1, hl)   y, dy  (bs, L, g, dg)
  * Same values as gcg_fwd / gcg_bwd on the gathered operands.  dtype: any, GCG_BF16_F32 / GCG_F16_F32 included.
- * The three planes count as three tensors for the alignment rule of the kernel families: where g * dg elements are
- * not a multiple of 16 bytes, GCG_ALGO_AUTO takes the direct kernels.
  * Workspace: gcg_bwd_workspace_bytes(...) with the same algo.
  */
 GCG_API int gcg_fwd_planar(const void *feat, const void *h, void *y,

@@ -332,7 +332,8 @@ GCG_API int gcg_fwd_planar(const void *feat, const void *h, void *y, int64_t bs,
     if (rc) return rc;
     dm.planar = 1;
     const void *C = feat, *B = plane(feat, 1, dm.d, dtype), *x = plane(feat, 2, dm.d, dtype);
-    const int a = resolve_algo(algo, dtype, dm, false, all_aligned16({C, B, x, y}));
+    // (the planes themselves lie d elements apart: a multiple of the kernels' vector width wherever a family takes the shape)
+    const int a = resolve_algo(algo, dtype, dm, false, all_aligned16({feat, y}));
     if (a < 0) return a;
     rc = check_device();
     if (rc) return rc;
@@ -357,7 +358,7 @@ GCG_API int gcg_bwd_planar(const void *dy, const void *feat, const void *h, void
     dm.planar = 1;
     const void *C = feat, *B = plane(feat, 1, dm.d, dtype), *x = plane(feat, 2, dm.d, dtype);
     void *dC = dfeat, *dB = plane_out(dfeat, 1, dm.d, dtype), *dx = plane_out(dfeat, 2, dm.d, dtype);
-    const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, C, B, x, dC, dB, dx}));
+    const int a = resolve_algo(algo, dtype, dm, true, all_aligned16({dy, feat, dfeat}));
     if (a < 0) return a;
     const size_t need = gcg_bwd_workspace_bytes(bs, L, g, dg, hl, dtype, a);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return GCG_ERR_WORKSPACE;

@@ -276,3 +276,19 @@ def test_planar_with_fp32_arithmetic(gcg_lib, act, hl, algo):
         assert torch.equal(dh, dh_p)
     else:
         assert_close(dh, dh_p, 2e-5, "dh")
+
+
+@pytest.mark.parametrize("bs,L,g,dg,hl,dtype", [(3, 2106, 25, 4, 3, torch.bfloat16), (2, 31, 15, 4, 5, torch.float16),
+                                                (2, 1000, 23, 4, 7, torch.float16), (1, 300, 31, 4, 6, torch.float32)])
+def test_planes_eight_bytes_apart(gcg_lib, bs, L, g, dg, hl, dtype):
+    """d * element size not a multiple of 16: the planes are only 8-byte aligned, which the register-window kernels
+    take (their rows are no better aligned on separate tensors of that width): same kernels, same results."""
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(bs, L, g, dg, hl, dtype, seed=3, dy_scale=0.1))
+    feat = pack(x, B, C)
+    y = _lib.fwd_planar(feat, h, algo="window")
+    dfeat, dh = _lib.bwd_planar(dy, feat, h, algo="window")
+    _, _, y_p = _lib.fwd(x, B, C, h, algo="window")
+    dx, dB, dC, dh_p = _lib.bwd(dy, x, B, C, h, algo="window")
+    torch.cuda.synchronize()
+    assert torch.equal(y, y_p) and torch.equal(dh, dh_p)
+    assert torch.equal(dfeat[:, :, 0], dC) and torch.equal(dfeat[:, :, 1], dB) and torch.equal(dfeat[:, :, 2], dx)
