@@ -445,7 +445,9 @@ int fwd_launch(const void *x, const void *B, const void *C, const void *h, void 
 {
     int e = 0;
     // 16-bit: ~112 registers, 4 waves per SIMD; fp32: ~200 registers, 2 waves per SIMD
-    MfmaPlan p = plan(dm, NW, 16, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
+    // runs down to 4 steps: on a tensor too small to fill the machine otherwise (a tensor-parallel rank's share, d = 1024)
+    // more, shorter runs beat the lead-in they replay (35 -> 24 us at (1, 8192, 1024)); large tensors never get there
+    MfmaPlan p = plan(dm, NW, 4, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     // Workgroup order.  With 32 or more channel blocks per row the XCD-contiguous order gives an XCD whole rows;
     // with fewer, dealing the blocks round-robin measured 3-5 % faster in the forward (d = 2048, 4096) and the same

@@ -474,7 +474,7 @@ template <typename T, int NK, int NW>
 int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
 {
     int e = 0;
-    MfmaPlan p = plan(dm, NW, 16, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
+    MfmaPlan p = plan(dm, NW, 4, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     // Workgroup order: dealing the channel blocks to the XCDs round-robin measured 3-4 % faster than XCD-contiguous
     // runs on interleaved operands at every width (d = 4096: 102.5 against 105.4 us, d = 8192: 376 against 389 us,
@@ -491,7 +491,7 @@ constexpr int FEAT_KF = 3;
 template <typename T, int NW>
 int fwd_feat_launch(const void *raw, const void *wfeat, int kf, const void *h, void *y, const Dims &dm, hipStream_t st)
 {
-    MfmaPlan p = plan(dm, NW, 16, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
+    MfmaPlan p = plan(dm, NW, 4, MT<T>::SPLIT ? 8 : 16, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     static const int order = env_int("GCG_MFMA_FWD_ORDER", -1);
     p.xcd = order >= 0 ? (order != 0) : 0;

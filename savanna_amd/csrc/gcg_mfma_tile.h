@@ -592,6 +592,8 @@ MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu, int elem_
     // steps plus its lead-in; e.g. 192 columns on 256 slots are better cut in 4 (3 rounds of 68
     // steps) than in 2 (2 rounds of 132), and 128 columns in 2 (one round of 132).
     const int64_t cols = dm.bs * p.ncb, slots = (int64_t)cu_count() * wg_per_cu;
+    static const int min_forced = env_int("GCG_MFMA_MIN_STEPS", 0);         // tuning override: shortest run considered
+    if (min_forced > 0) min_steps = min_forced;
     int64_t max_seg = p.nsteps / min_steps;
     if (max_seg < 1) max_seg = 1;
     const int64_t lead = (dm.hl + 30) / 32 < 4 ? (dm.hl + 30) / 32 : 4;     // NK - 1 steps replayed by a later segment

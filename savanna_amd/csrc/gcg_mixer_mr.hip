@@ -971,7 +971,7 @@ int bwd_t(const void *dy, const void *raw, const void *wfeat, int kf, const void
 namespace {
 MfmaPlan mixer_fwd_plan(const Dims &dm)
 {
-    return plan(dm, MixFwdGeo<bf16_t>::XW, 16, MixFwdGeo<bf16_t>::XW, 2);
+    return plan(dm, MixFwdGeo<bf16_t>::XW, 4, MixFwdGeo<bf16_t>::XW, 2);
 }
 template <typename T>
 int fwd_t(const void *raw, const void *wfeat, int kf, const void *h, void *y, const Dims &dm, hipStream_t st)
