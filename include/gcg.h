@@ -387,6 +387,16 @@ GCG_API int gcg_mixer_mr_bwd_decay(const void *dy, const void *raw, const void *
             void *workspace, size_t workspace_bytes,
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
             int32_t dtype, void *stream);
+/* Both at once: planar features and the filter formed in the kernels (one-kernel path only, no scratch tensor). */
+GCG_API int gcg_mixer_mr_fwd_planar_decay(const void *raw, const void *wf, const float *w, const float *decay,
+            int32_t l_cache, void *y,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
+GCG_API int gcg_mixer_mr_bwd_planar_decay(const void *dy, const void *raw, const void *wf, const float *w,
+            const float *decay, int32_t l_cache, void *draw, void *dwf, float *dw,
+            void *workspace, size_t workspace_bytes,
+            int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+            int32_t dtype, void *stream);
 
 /*
  * Explicit decayed filter of Hyena-MR, ready for gcg_fwd, in one launch.

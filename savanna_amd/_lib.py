@@ -37,7 +37,7 @@ EXPORTS = (
     "gcg_mixer_se_fwd_planar", "gcg_mixer_se_bwd_planar",
     "gcg_filter_decay_fwd", "gcg_filter_decay_bwd",
     "gcg_mixer_mr_fwd", "gcg_mixer_mr_bwd_workspace_bytes", "gcg_mixer_mr_bwd_scratch_bytes", "gcg_mixer_mr_bwd", "gcg_mixer_mr_fwd_decay", "gcg_mixer_mr_bwd_decay",
-    "gcg_mixer_mr_fwd_planar", "gcg_mixer_mr_bwd_planar", "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
+    "gcg_mixer_mr_fwd_planar", "gcg_mixer_mr_bwd_planar", "gcg_mixer_mr_fwd_planar_decay", "gcg_mixer_mr_bwd_planar_decay", "gcg_fwd_time_major", "gcg_bwd_time_major_workspace_bytes", "gcg_bwd_time_major",
     "gcg_fwd_decay", "gcg_bwd_decay", "gcg_fwd_interleaved_decay", "gcg_bwd_interleaved_decay",
 )
 
@@ -118,6 +118,10 @@ def load() -> ctypes.CDLL:
         lib.gcg_mixer_mr_bwd_scratch_bytes.restype = sz
         lib.gcg_mixer_mr_bwd.argtypes = [vp] * 9 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_mixer_mr_bwd.restype = ctypes.c_int
+        lib.gcg_mixer_mr_fwd_planar_decay.argtypes = [vp] * 4 + [i32, vp, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_mixer_mr_fwd_planar_decay.restype = ctypes.c_int
+        lib.gcg_mixer_mr_bwd_planar_decay.argtypes = [vp] * 5 + [i32] + [vp] * 4 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
+        lib.gcg_mixer_mr_bwd_planar_decay.restype = ctypes.c_int
         lib.gcg_mixer_mr_fwd_planar.argtypes = [vp] * 4 + [i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_mixer_mr_fwd_planar.restype = ctypes.c_int
         lib.gcg_mixer_mr_bwd_planar.argtypes = [vp] * 8 + [sz, i64, i64, i32, i32, i32, i32, i32, vp]
@@ -681,33 +685,35 @@ def mixer_mr_bwd(dy, raw, wf, h, planar=False):
     return draw, dwf, dh
 
 
-def mixer_mr_fwd_decay(raw, wf, w, decay, hl: int, filt: torch.dtype):
+def mixer_mr_fwd_decay(raw, wf, w, decay, hl: int, filt: torch.dtype, planar=False):
     """mixer_mr_fwd with the filter F(w * decay)[:, :hl] formed inside the kernel (w, decay: (g, l_cache) fp32)."""
     _require_gpu(raw)
     if TORCH_OPS:
-        return torch.ops.gcg.mixer_mr_fwd_decay(raw, wf, w, decay, hl, filt)
+        return torch.ops.gcg.mixer_mr_fwd_decay(raw, wf, w, decay, hl, filt, bool(planar))
     lib = load()
     _check_filter_params(w, decay)
-    bs, L, g, dg, _ = raw.shape
+    bs, L = raw.shape[:2]
+    g, dg = (raw.shape[3], raw.shape[4]) if planar else (raw.shape[2], raw.shape[3])
     y = torch.empty(bs, L, g, dg, dtype=raw.dtype, device=raw.device)
     if y.numel() == 0:
         return y
+    fn = lib.gcg_mixer_mr_fwd_planar_decay if planar else lib.gcg_mixer_mr_fwd_decay
     with _on_device(raw.device):
-        rc = lib.gcg_mixer_mr_fwd_decay(raw.data_ptr(), wf.data_ptr(), w.data_ptr(), decay.data_ptr(), w.shape[1],
-                                        y.data_ptr(), bs, L, g, dg, hl, wf.shape[-1], _decay_code(raw, filt),
-                                        torch.cuda.current_stream().cuda_stream)
-    check(rc, "gcg_mixer_mr_fwd_decay")
+        rc = fn(raw.data_ptr(), wf.data_ptr(), w.data_ptr(), decay.data_ptr(), w.shape[1], y.data_ptr(), bs, L, g, dg,
+                hl, wf.shape[-1], _decay_code(raw, filt), torch.cuda.current_stream().cuda_stream)
+    check(rc, "gcg_mixer_mr_fwd_planar_decay" if planar else "gcg_mixer_mr_fwd_decay")
     return y
 
 
-def mixer_mr_bwd_decay(dy, raw, wf, w, decay, hl: int, filt: torch.dtype):
+def mixer_mr_bwd_decay(dy, raw, wf, w, decay, hl: int, filt: torch.dtype, planar=False):
     """(draw, dwf, dw) of mixer_mr_fwd_decay; dw is the gradient of the filter parameter w."""
     _require_gpu(raw)
     if TORCH_OPS:
-        return torch.ops.gcg.mixer_mr_bwd_decay(dy, raw, wf, w, decay, hl, filt)
+        return torch.ops.gcg.mixer_mr_bwd_decay(dy, raw, wf, w, decay, hl, filt, bool(planar))
     lib = load()
     _check_filter_params(w, decay)
-    bs, L, g, dg, _ = raw.shape
+    bs, L = raw.shape[:2]
+    g, dg = (raw.shape[3], raw.shape[4]) if planar else (raw.shape[2], raw.shape[3])
     kf = wf.shape[-1]
     draw, dwf, dw = torch.empty_like(raw), torch.empty_like(wf), torch.empty_like(w)
     if dy.numel() == 0:
@@ -718,13 +724,19 @@ def mixer_mr_bwd_decay(dy, raw, wf, w, decay, hl: int, filt: torch.dtype):
         check(-2, "gcg_mixer_mr_bwd_workspace_bytes")
     with _on_device(raw.device):
         ws = torch.empty(nbytes, dtype=torch.uint8, device=raw.device)
-        sbytes = lib.gcg_mixer_mr_bwd_scratch_bytes(bs, L, g, dg, hl, kf, code)
-        scratch = torch.empty(sbytes, dtype=torch.uint8, device=raw.device)
-        rc = lib.gcg_mixer_mr_bwd_decay(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), w.data_ptr(), decay.data_ptr(),
-                                        w.shape[1], draw.data_ptr(), dwf.data_ptr(), dw.data_ptr(),
-                                        scratch.data_ptr() if sbytes else None, ws.data_ptr(), nbytes, bs, L, g, dg, hl,
-                                        kf, code, torch.cuda.current_stream().cuda_stream)
-    check(rc, "gcg_mixer_mr_bwd_decay")
+        st = torch.cuda.current_stream().cuda_stream
+        if planar:
+            rc = lib.gcg_mixer_mr_bwd_planar_decay(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), w.data_ptr(),
+                                                   decay.data_ptr(), w.shape[1], draw.data_ptr(), dwf.data_ptr(),
+                                                   dw.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg, hl, kf, code, st)
+        else:
+            sbytes = lib.gcg_mixer_mr_bwd_scratch_bytes(bs, L, g, dg, hl, kf, code)
+            scratch = torch.empty(sbytes, dtype=torch.uint8, device=raw.device)
+            rc = lib.gcg_mixer_mr_bwd_decay(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), w.data_ptr(), decay.data_ptr(),
+                                            w.shape[1], draw.data_ptr(), dwf.data_ptr(), dw.data_ptr(),
+                                            scratch.data_ptr() if sbytes else None, ws.data_ptr(), nbytes, bs, L, g, dg, hl,
+                                            kf, code, st)
+    check(rc, "gcg_mixer_mr_bwd_planar_decay" if planar else "gcg_mixer_mr_bwd_decay")
     return draw, dwf, dw
 
 

@@ -672,6 +672,19 @@ GCG_API int gcg_mixer_mr_fwd_decay(const void *raw, const void *wf, const float 
     return mixer_mr_fwd_dims(raw, wf, nullptr, y, dm, kf, dtype, stream);
 }
 
+GCG_API int gcg_mixer_mr_fwd_planar_decay(const void *raw, const void *wf, const float *w, const float *decay,
+                                          int32_t l_cache, void *y, int64_t bs, int64_t L, int32_t g, int32_t dg,
+                                          int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!raw || !wf || !y || kf <= 0) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    const int rc = decay_dims(bs, L, g, dg, hl, dtype, w, decay, l_cache, &dm);
+    if (rc) return rc;
+    dm.planar = 1;
+    return mixer_mr_fwd_dims(raw, wf, nullptr, y, dm, kf, dtype, stream);
+}
+
 namespace {
 int mixer_mr_fwd_dims(const void *raw, const void *wf, const void *h, void *y, gcg::Dims &dm, int kf, int dtype,
                       void *stream)
@@ -757,6 +770,20 @@ GCG_API int gcg_mixer_mr_bwd_decay(const void *dy, const void *raw, const void *
     if (rc) return rc;
     return mixer_mr_bwd_dims(dy, raw, wf, nullptr, draw, dwf, dw, dfeat_scratch, workspace, workspace_bytes, dm, kf, dtype,
                              stream);
+}
+
+GCG_API int gcg_mixer_mr_bwd_planar_decay(const void *dy, const void *raw, const void *wf, const float *w,
+                                          const float *decay, int32_t l_cache, void *draw, void *dwf, float *dw,
+                                          void *workspace, size_t workspace_bytes, int64_t bs, int64_t L, int32_t g,
+                                          int32_t dg, int32_t hl, int32_t kf, int32_t dtype, void *stream)
+{
+    TimerScope timer_scope;
+    if (!dy || !raw || !wf || !draw || !dwf || !dw || kf <= 0) return GCG_ERR_BAD_ARG;
+    gcg::Dims dm;
+    const int rc = decay_dims(bs, L, g, dg, hl, dtype, w, decay, l_cache, &dm);
+    if (rc) return rc;
+    dm.planar = 1;
+    return mixer_mr_bwd_dims(dy, raw, wf, nullptr, draw, dwf, dw, nullptr, workspace, workspace_bytes, dm, kf, dtype, stream);
 }
 
 namespace {

@@ -574,50 +574,63 @@ void check_mixer_mr(const Tensor &raw, const Tensor &wf, const Tensor &h, bool p
     (void)gated_code(raw, h);
 }
 
-void check_mixer_mr_decay(const Tensor &raw, const Tensor &wf, const Tensor &w, const Tensor &decay, int64_t hl)
+void check_mixer_mr_decay(const Tensor &raw, const Tensor &wf, const Tensor &w, const Tensor &decay, int64_t hl,
+                          bool planar = false)
 {
-    TORCH_CHECK(raw.dim() == 5 && raw.size(4) == 3 && raw.is_contiguous(),
-                "gcg: raw must be a contiguous (bs, L, g, dg, 3) tensor");
-    TORCH_CHECK(wf.dim() == 3 && wf.size(0) == 3 * raw.size(2) * raw.size(3) && wf.size(1) == 1 && wf.is_contiguous() &&
+    TORCH_CHECK(raw.dim() == 5 && raw.size(planar ? 2 : 4) == 3 && raw.is_contiguous(),
+                planar ? "gcg: raw must be a contiguous (bs, L, 3, g, dg) tensor"
+                       : "gcg: raw must be a contiguous (bs, L, g, dg, 3) tensor");
+    const int64_t g = raw.size(planar ? 3 : 2), dg = raw.size(planar ? 4 : 3);
+    TORCH_CHECK(wf.dim() == 3 && wf.size(0) == 3 * g * dg && wf.size(1) == 1 && wf.is_contiguous() &&
                     wf.scalar_type() == raw.scalar_type() && wf.device() == raw.device(),
                 "gcg: wf must be a contiguous (3 * g * dg, 1, kf) tensor of raw's dtype and device");
-    check_decay(w, decay, hl, raw.size(2), raw);
+    check_decay(w, decay, hl, g, raw);
 }
 
 Tensor mixer_mr_fwd_decay(const Tensor &raw, const Tensor &wf, const Tensor &w, const Tensor &decay, int64_t hl,
-                          at::ScalarType filt)
+                          at::ScalarType filt, bool planar)
 {
     require_gpu(raw, "raw");
-    check_mixer_mr_decay(raw, wf, w, decay, hl);
+    check_mixer_mr_decay(raw, wf, w, decay, hl, planar);
     const int code = gated_code_for(raw.scalar_type(), filt);
     DeviceGuard guard(raw.device());
-    Tensor y = at::empty({raw.size(0), raw.size(1), raw.size(2), raw.size(3)}, raw.options());
+    const int64_t g = raw.size(planar ? 3 : 2), dg = raw.size(planar ? 4 : 3);
+    Tensor y = at::empty({raw.size(0), raw.size(1), g, dg}, raw.options());
     if (y.numel() == 0) return y;
-    check_rc(gcg_mixer_mr_fwd_decay(raw.data_ptr(), wf.data_ptr(), (const float *)w.data_ptr(),
-                                    (const float *)decay.data_ptr(), (int32_t)w.size(1), y.data_ptr(), raw.size(0),
-                                    raw.size(1), (int32_t)raw.size(2), (int32_t)raw.size(3), (int32_t)hl,
-                                    (int32_t)wf.size(2), code, stream_of(raw)),
-             "gcg_mixer_mr_fwd_decay");
+    check_rc((planar ? gcg_mixer_mr_fwd_planar_decay : gcg_mixer_mr_fwd_decay)(
+                 raw.data_ptr(), wf.data_ptr(), (const float *)w.data_ptr(), (const float *)decay.data_ptr(),
+                 (int32_t)w.size(1), y.data_ptr(), raw.size(0), raw.size(1), (int32_t)g, (int32_t)dg, (int32_t)hl,
+                 (int32_t)wf.size(2), code, stream_of(raw)),
+             planar ? "gcg_mixer_mr_fwd_planar_decay" : "gcg_mixer_mr_fwd_decay");
     return y;
 }
 
 std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd_decay(const Tensor &dy, const Tensor &raw, const Tensor &wf,
                                                       const Tensor &w, const Tensor &decay, int64_t hl,
-                                                      at::ScalarType filt)
+                                                      at::ScalarType filt, bool planar)
 {
     require_gpu(raw, "raw");
-    check_mixer_mr_decay(raw, wf, w, decay, hl);
-    TORCH_CHECK(dy.dim() == 4 && dy.sizes() == raw.sizes().slice(0, 4) && dy.scalar_type() == raw.scalar_type() &&
-                    dy.device() == raw.device() && dy.is_contiguous(),
+    check_mixer_mr_decay(raw, wf, w, decay, hl, planar);
+    const int32_t g = (int32_t)raw.size(planar ? 3 : 2), dg = (int32_t)raw.size(planar ? 4 : 3), kf = (int32_t)wf.size(2);
+    TORCH_CHECK(dy.dim() == 4 && dy.size(0) == raw.size(0) && dy.size(1) == raw.size(1) && dy.size(2) == g &&
+                    dy.size(3) == dg && dy.scalar_type() == raw.scalar_type() && dy.device() == raw.device() &&
+                    dy.is_contiguous(),
                 "gcg: dy must be a contiguous (bs, L, g, dg) tensor of raw's dtype and device");
     const int code = gated_code_for(raw.scalar_type(), filt);
     DeviceGuard guard(raw.device());
     Tensor draw = at::empty_like(raw), dwf = at::empty_like(wf), dw = at::empty_like(w);
     if (dy.numel() == 0) return {draw, dwf.zero_(), dw.zero_()};
     const int64_t bs = raw.size(0), L = raw.size(1);
-    const int32_t g = (int32_t)raw.size(2), dg = (int32_t)raw.size(3), kf = (int32_t)wf.size(2);
     const size_t nbytes = gcg_mixer_mr_bwd_workspace_bytes(bs, L, g, dg, (int32_t)hl, kf, code);
     Tensor ws = workspace(nbytes, raw, "gcg_mixer_mr_bwd_workspace_bytes");
+    if (planar) {
+        check_rc(gcg_mixer_mr_bwd_planar_decay(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), (const float *)w.data_ptr(),
+                                               (const float *)decay.data_ptr(), (int32_t)w.size(1), draw.data_ptr(),
+                                               dwf.data_ptr(), (float *)dw.data_ptr(), ws.data_ptr(), nbytes, bs, L, g, dg,
+                                               (int32_t)hl, kf, code, stream_of(raw)),
+                 "gcg_mixer_mr_bwd_planar_decay");
+        return {draw, dwf, dw};
+    }
     const size_t sbytes = gcg_mixer_mr_bwd_scratch_bytes(bs, L, g, dg, (int32_t)hl, kf, code);
     Tensor scratch = at::empty({(int64_t)sbytes}, raw.options().dtype(at::kByte));
     check_rc(gcg_mixer_mr_bwd_decay(dy.data_ptr(), raw.data_ptr(), wf.data_ptr(), (const float *)w.data_ptr(),
@@ -814,17 +827,17 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> bwd_time_major_meta(const Tensor &dy,
 }
 
 Tensor mixer_mr_fwd_decay_meta(const Tensor &raw, const Tensor &wf, const Tensor &w, const Tensor &decay, int64_t hl,
-                               at::ScalarType filt)
+                               at::ScalarType filt, bool planar)
 {
-    check_mixer_mr_decay(raw, wf, w, decay, hl);
+    check_mixer_mr_decay(raw, wf, w, decay, hl, planar);
     (void)gated_code_for(raw.scalar_type(), filt);
-    return at::empty({raw.size(0), raw.size(1), raw.size(2), raw.size(3)}, raw.options());
+    return at::empty({raw.size(0), raw.size(1), raw.size(planar ? 3 : 2), raw.size(planar ? 4 : 3)}, raw.options());
 }
 std::tuple<Tensor, Tensor, Tensor> mixer_mr_bwd_decay_meta(const Tensor &dy, const Tensor &raw, const Tensor &wf,
                                                            const Tensor &w, const Tensor &decay, int64_t hl,
-                                                           at::ScalarType filt)
+                                                           at::ScalarType filt, bool planar)
 {
-    check_mixer_mr_decay(raw, wf, w, decay, hl);
+    check_mixer_mr_decay(raw, wf, w, decay, hl, planar);
     (void)dy;
     (void)gated_code_for(raw.scalar_type(), filt);
     return {at::empty_like(raw), at::empty_like(wf), at::empty_like(w)};
@@ -864,9 +877,10 @@ TORCH_LIBRARY(gcg, m)
     m.def("filter_decay_bwd(Tensor dh, Tensor decay) -> Tensor");
     m.def("mixer_mr_fwd(Tensor raw, Tensor wf, Tensor h, bool planar=False) -> Tensor");
     m.def("mixer_mr_bwd(Tensor dy, Tensor raw, Tensor wf, Tensor h, bool planar=False) -> (Tensor, Tensor, Tensor)");
-    m.def("mixer_mr_fwd_decay(Tensor raw, Tensor wf, Tensor w, Tensor decay, int hl, ScalarType filt) -> Tensor");
-    m.def("mixer_mr_bwd_decay(Tensor dy, Tensor raw, Tensor wf, Tensor w, Tensor decay, int hl, ScalarType filt)"
-          " -> (Tensor, Tensor, Tensor)");
+    m.def("mixer_mr_fwd_decay(Tensor raw, Tensor wf, Tensor w, Tensor decay, int hl, ScalarType filt, bool planar=False)"
+          " -> Tensor");
+    m.def("mixer_mr_bwd_decay(Tensor dy, Tensor raw, Tensor wf, Tensor w, Tensor decay, int hl, ScalarType filt,"
+          " bool planar=False) -> (Tensor, Tensor, Tensor)");
     m.def("fwd_time_major(Tensor x, Tensor B, Tensor C, Tensor h) -> Tensor");
     m.def("bwd_time_major(Tensor dy, Tensor x, Tensor B, Tensor C, Tensor h) -> (Tensor, Tensor, Tensor, Tensor)");
     m.def("fwd_decay(Tensor x, Tensor B, Tensor C, Tensor w, Tensor decay, int hl, ScalarType filt) -> Tensor");

@@ -359,18 +359,18 @@ class _FeaturizedDecayedGateConvGate(torch.autograd.Function):
     part is one kernel each way, and the backward returns the gradient of the filter parameter itself."""
 
     @staticmethod
-    def forward(ctx, raw, wf, w, decay, hl, filt):
+    def forward(ctx, raw, wf, w, decay, hl, filt, planar=False):
         raw, wf, w, decay = (t if t.is_contiguous() else t.contiguous() for t in (raw, wf, w, decay))
         ctx.save_for_backward(raw, wf, w, decay)
-        ctx.hl, ctx.filt = hl, filt
-        return _lib.mixer_mr_fwd_decay(raw, wf, w, decay, hl, filt)
+        ctx.hl, ctx.filt, ctx.planar = hl, filt, planar
+        return _lib.mixer_mr_fwd_decay(raw, wf, w, decay, hl, filt, planar)
 
     @staticmethod
     def backward(ctx, dz):
         raw, wf, w, decay = ctx.saved_tensors
         draw, dwf, dw = _lib.mixer_mr_bwd_decay(dz if dz.is_contiguous() else dz.contiguous(), raw, wf, w, decay,
-                                                ctx.hl, ctx.filt)
-        return draw, dwf, dw, None, None, None
+                                                ctx.hl, ctx.filt, ctx.planar)
+        return draw, dwf, dw, None, None, None, None
 
 
 class HyenaMixer(nn.Module):
@@ -406,8 +406,17 @@ class HyenaMixer(nn.Module):
         bs, seqlen, d3 = features.shape
         conv = self.hyena_proj_conv
         if not self.interleave_projections:
-            # "(p g dg)" features.  Hyena-SE: the fused kernels on planar pieces; otherwise the featurizer kernel,
-            # then the operator on the thirds of its rows (two kernels each way)
+            # "(p g dg)" features.  The fused kernels on planar pieces where they take the shape; otherwise the
+            # featurizer kernel, then the operator on the thirds of its rows (two kernels each way)
+            fused = op._filter_in_kernel(seqlen, op.num_groups, op.group_dim, features.dtype, features)
+            if (fused is not None and self.fuse_medium and conv.group_dim == 1 and op.cgcg_dtype == features.dtype and
+                    features.dtype in (torch.bfloat16, torch.float16) and
+                    _lib.mixer_mr_supported(op.group_dim, fused[0], conv.kernel_size, features)):
+                g, dg = op.num_groups, op.group_dim
+                z = _FeaturizedDecayedGateConvGate.apply(features.reshape(bs, seqlen, 3, g, dg),
+                                                         conv.short_conv_weight.to(features.dtype), op.filter.h,
+                                                         op.filter.decay, fused[0], fused[1], True)
+                return z.reshape(bs, seqlen, g * dg)
             h = op._filter(seqlen)
             if self._fusable(features, h.shape[-1]):
                 dtype = features.dtype

@@ -137,6 +137,16 @@ def test_filter_formed_in_the_kernels(gcg_lib, bs, L, g, dg, hl, kf, lc, dtype, 
     torch.cuda.synchronize()
     assert torch.equal(draw, draw2) and torch.equal(dwf, dwf2)
     assert dw.shape == w.shape and torch.equal(dw, _lib.filter_decay_bwd(dh2, decay))
+    if dtype == filt and dtype != torch.float32:
+        # and on planar features (one-kernel path: 16-bit arithmetic)
+        d = g * dg
+        raw_pl = raw.permute(0, 1, 4, 2, 3).contiguous()
+        wf_pl = wf.view(d, 3, 1, kf).permute(1, 0, 2, 3).reshape(3 * d, 1, kf).contiguous()
+        y_pl = _lib.mixer_mr_fwd_decay(raw_pl, wf_pl, w, decay, hl, filt, planar=True)
+        draw_pl, dwf_pl, dw_pl = _lib.mixer_mr_bwd_decay(dy, raw_pl, wf_pl, w, decay, hl, filt, planar=True)
+        torch.cuda.synchronize()
+        assert torch.equal(y_pl, y) and torch.equal(draw_pl, draw.permute(0, 1, 4, 2, 3)) and torch.equal(dw_pl, dw)
+        assert torch.equal(dwf_pl.view(3, d, 1, kf), dwf.view(d, 3, 1, kf).permute(1, 0, 2, 3))
 
 
 def test_refused_shapes(gcg_lib):
@@ -278,3 +288,5 @@ def test_hyena_mixer_planar_fused(gcg_lib):
             assert torch.equal(a, b), n
     big = [e.key for e in prof.key_averages() if "mfma" in e.key or "dwconv" in e.key or "mixer_mr" in e.key]
     assert len(big) == 2 and all("mixer_mr" in k for k in big), big
+    ours = [e.key for e in prof.key_averages() if "gcg::" in e.key and e.device_time_total > 0]
+    assert len(ours) == 2, ours               # the filter is formed in the kernels on this layout too
