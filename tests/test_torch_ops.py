@@ -51,6 +51,9 @@ def test_meta_shapes_on_fake_gpu_tensors(gcg_lib):
         assert dpl.shape == planar.shape and dwf_pl.shape == wf.shape and dh_pl.shape == h.shape
         dpl, dwf_pl, dh_pl = torch.ops.gcg.mixer_se_bwd(x, planar, wf, h7, True)
         assert dpl.shape == planar.shape and dwf_pl.shape == wf.shape and dh_pl.shape == h7.shape
+        assert torch.ops.gcg.mixer_mr_fwd_decay(planar, wf, p, p, 128, torch.bfloat16, True).shape == x.shape
+        dpl, dwf_pl, dw_pl = torch.ops.gcg.mixer_mr_bwd_decay(x, planar, wf, p, p, 128, torch.bfloat16, True)
+        assert dpl.shape == planar.shape and dwf_pl.shape == wf.shape and dw_pl.shape == p.shape
         assert torch.ops.gcg.fwd_planar(planar, h).shape == x.shape
         dplanar, dh = torch.ops.gcg.bwd_planar(x, planar, h)
         assert dplanar.shape == planar.shape and dh.shape == h.shape
