@@ -10,7 +10,11 @@ from savanna_amd import _lib, _ops, two_pass_chunked_gate_conv_gate
 from savanna_amd.kernels.cgcg.interface import two_pass_chunked_gate_conv_gate_interleaved
 from savanna_amd.kernels.cgcg.src.kernel_utils import FwdKernelConfigRefactor
 
-pytestmark = pytest.mark.gpu
+import os
+
+# with GCG_BINDING=ctypes the operators are deliberately not registered: there is nothing here to test then
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(os.environ.get("GCG_BINDING") == "ctypes", reason="GCG_BINDING=ctypes: no torch operators")]
 
 DEV = "cuda:0"
 CFG = FwdKernelConfigRefactor(CHUNK_SIZE=128, BLOCK_D=16, THREADBLOCK_SWIZZLE="row")
