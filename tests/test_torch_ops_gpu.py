@@ -2,6 +2,8 @@
 (torch operators and ctypes), torch.library's own operator checks, and torch.compile(fullgraph=True) of the
 reference-compatible entry point against eager (the reference compiles its filter, explicit.py:71, so callers of
 this path are traced)."""
+import os
+
 import pytest
 import torch
 
@@ -9,8 +11,6 @@ from helpers import TOL, TOL_DH, assert_close, inputs, oracle_bwd, oracle_fwd
 from savanna_amd import _lib, _ops, two_pass_chunked_gate_conv_gate
 from savanna_amd.kernels.cgcg.interface import two_pass_chunked_gate_conv_gate_interleaved
 from savanna_amd.kernels.cgcg.src.kernel_utils import FwdKernelConfigRefactor
-
-import os
 
 # with GCG_BINDING=ctypes the operators are deliberately not registered: there is nothing here to test then
 pytestmark = [pytest.mark.gpu,
