@@ -290,3 +290,45 @@ def test_hyena_mixer_planar_fused(gcg_lib):
     assert len(big) == 2 and all("mixer_mr" in k for k in big), big
     ours = [e.key for e in prof.key_averages() if "gcg::" in e.key and e.device_time_total > 0]
     assert len(ours) == 2, ours               # the filter is formed in the kernels on this layout too
+
+
+@pytest.mark.parametrize("planar", [False, True], ids=["interleaved", "planar"])
+def test_graph_replays_match_eager(gcg_lib, planar):
+    """The fused forward and backward (explicit filter and filter formed in the kernels) recorded in a HIP graph: three
+    replays on fresh data, with eager launches of the same kernels between them (the backward's arrival counters
+    and partial sums are shared by every launch), each replay equal to eager bit for bit."""
+    bs, L, g, dg, hl, kf, lc = 2, 2100, 6, 16, 128, 3, 128
+    raw, wf, h, dy = (t.to(DEV) for t in make(bs, L, g, dg, hl, kf, torch.bfloat16, torch.bfloat16, seed=11))
+    if planar:
+        raw = raw.permute(0, 1, 4, 2, 3).contiguous()
+    gen = torch.Generator().manual_seed(12)
+    w = (torch.randn(g, lc, generator=gen) / lc ** 0.5).to(DEV)
+    decay = torch.exp(-torch.logspace(0, 2, g)[:, None] * torch.linspace(0, 1, lc)[None]).to(DEV)
+
+    def step(raw_, dy_):
+        y = _lib.mixer_mr_fwd(raw_, wf, h, planar=planar)
+        draw, dwf, dh = _lib.mixer_mr_bwd(dy_, raw_, wf, h, planar=planar)
+        y2 = _lib.mixer_mr_fwd_decay(raw_, wf, w, decay, hl, torch.bfloat16, planar=planar)
+        draw2, dwf2, dw = _lib.mixer_mr_bwd_decay(dy_, raw_, wf, w, decay, hl, torch.bfloat16, planar=planar)
+        return y, draw, dwf, dh, y2, draw2, dwf2, dw
+
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):                      # warm-up on the capture stream
+        step(raw, dy)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs_g = step(raw, dy)
+    names = ("y", "d raw", "dw featurizer", "dh", "y decay", "d raw decay", "dw featurizer decay", "dw")
+    for it in range(3):
+        fresh_raw, fresh_dy = torch.randn_like(raw), 0.1 * torch.randn_like(dy)
+        raw.copy_(fresh_raw)
+        dy.copy_(fresh_dy)
+        graph.replay()
+        torch.cuda.synchronize()
+        outs_e = step(fresh_raw, fresh_dy)
+        torch.cuda.synchronize()
+        for a, b, n in zip(outs_g, outs_e, names):
+            assert torch.equal(a, b), f"replay {it}: {n}"
