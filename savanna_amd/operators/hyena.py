@@ -398,6 +398,11 @@ class HyenaMixer(nn.Module):
 
     def _fusable(self, features: torch.Tensor, hl: int) -> bool:
         conv, op = self.hyena_proj_conv, self.mixer
+        if op.cgcg_dtype != features.dtype and op._fp32_inside(features.dtype, features):
+            # 16-bit features into fp32 arithmetic: the featurizer's output is rounded to 16 bits before the operator
+            # (hyena.py:812-816 casts after the conv), which the two-kernel chain does without a cast and the
+            # one-kernel form could only do on fp32 copies of the features
+            return False
         return (self.fuse_short and features.is_cuda and hl <= 8 and conv.kernel_size <= 4 and conv.group_dim == 1
                 and op.group_dim % 2 == 0)
 

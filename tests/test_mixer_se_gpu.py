@@ -262,3 +262,47 @@ def test_hyena_mixer_planar_fused(gcg_lib):
         assert_close(a, b, 2e-2, n)
     big = [e.key for e in prof.key_averages() if "mixer_se" in e.key or "dwconv" in e.key or "window" in e.key]
     assert len(big) == 2 and all("mixer_se" in k for k in big), big
+
+
+@pytest.mark.parametrize("planar", [False, True], ids=["interleaved", "planar"])
+def test_hyena_mixer_16_bit_features_fp32_arithmetic(gcg_lib, planar):
+    """bf16 activations with cgcg_dtype float32 (the default, global_config.py:404): the featurizer's output is
+    rounded to bf16 before the operator's casts (block.py:873, hyena.py:812-816), so the mixer runs the featurizer
+    kernel and the operator on 16-bit tensors with fp32 arithmetic -- no fp32 copy of the features, and the same
+    values as the reference's chain written with torch ops."""
+    import torch.nn.functional as F
+
+    from savanna_amd.operators.hyena import CgcgConfig, HyenaMixer, HyenaSEOperator
+
+    torch.manual_seed(8)
+    bs, L, hidden, groups, hl, kf = 2, 500, 128, 8, 7, 3
+    dg = hidden // groups
+    mixer = HyenaMixer(HyenaSEOperator(hidden, groups, hl, CgcgConfig(cgcg_dtype="float32"), device=DEV), kf,
+                       dtype=torch.bfloat16, device=DEV, interleave_projections=not planar)
+    feats = torch.randn(bs, L, 3 * hidden, device=DEV).to(torch.bfloat16)
+    dz = (0.1 * torch.randn(bs, L, hidden, device=DEV)).to(torch.bfloat16)
+    assert not mixer._fusable(feats, hl)
+    x = feats.clone().requires_grad_(True)
+    z = mixer(x)
+    z.backward(dz)
+    assert z.dtype == torch.bfloat16 and x.grad.dtype == torch.bfloat16
+    got = (z, x.grad, mixer.hyena_proj_conv.short_conv_weight.grad.clone(), mixer.mixer.short_conv_weight.grad.clone())
+
+    # the reference's chain: conv on (B, 3D, L) in bf16, split, casts to fp32, gated conv, cast back
+    xr = feats.clone().requires_grad_(True)
+    wf = mixer.hyena_proj_conv.short_conv_weight.detach().clone().requires_grad_(True)
+    h = mixer.mixer.short_conv_weight.detach().clone().requires_grad_(True)
+    f = F.conv1d(F.pad(xr.transpose(1, 2), (kf - 1, 0)), wf.to(torch.bfloat16), groups=3 * hidden).transpose(1, 2)
+    if planar:
+        x1, x2, v = f.reshape(bs, L, 3, groups, dg).unbind(2)
+    else:
+        x1, x2, v = f.reshape(bs, L, groups, dg, 3).unbind(4)
+    u = (v.float() * x2.float()).reshape(bs, L, hidden).transpose(1, 2)
+    y = F.conv1d(F.pad(u, (hl - 1, 0)), h.float().repeat_interleave(dg, 0), groups=hidden).transpose(1, 2)
+    zr = (x1.float().reshape(bs, L, hidden) * y).to(torch.bfloat16)
+    zr.backward(dz)
+    torch.cuda.synchronize()
+    assert_close(got[0], zr, TOL[torch.bfloat16], "z")
+    assert_close(got[1], xr.grad, 2 * TOL[torch.bfloat16], "d features")
+    assert_close(got[2], wf.grad, TOL_DH[torch.bfloat16], "d featurizer weight")
+    assert_close(got[3], h.grad, TOL_DH[torch.bfloat16], "d operator weight")
