@@ -270,6 +270,47 @@ def test_run_short_hyena_in_place(gcg_lib, seqlen, bs, g, dg, hl, dtype):
     assert torch.equal(dev[3].grad, dh2)
 
 
+def test_time_major_64bit_offsets(gcg_lib):
+    """(seqlen, bs, g, dg) operands of 2^31 elements each (seqlen 2^18, bs 2, 4096 channels, bf16): a filter that
+    delays by two rows makes every output a product of input elements, so a wrapped offset fails an exact comparison."""
+    seqlen, bs, g, dg, hl, s_ = 1 << 18, 2, 256, 16, 7, 2
+    dt = torch.bfloat16
+    gen = torch.Generator(device=DEV)
+    tensors = []
+    for i in range(4):                                  # x, B, C (seqlen, bs, g, dg); dy (bs, seqlen, g, dg)
+        t = torch.empty((seqlen, bs, g, dg) if i < 3 else (bs, seqlen, g, dg), dtype=dt, device=DEV)
+        flat = t.view(-1)
+        for k, o in enumerate(range(0, flat.numel(), 1 << 28)):
+            gen.manual_seed(500 + 10 * i + k)
+            flat[o:o + (1 << 28)].normal_(generator=gen)
+        tensors.append(t)
+    x, B, C, dy = tensors
+    h = torch.zeros(g, 1, hl, dtype=dt, device=DEV)
+    h[:, 0, hl - 1 - s_] = 1.0
+    y = _lib.fwd_time_major(x, B, C, h)           # (bs, seqlen, g, dg)
+    torch.cuda.synchronize()
+    u = x.float() * B.float()                           # exact in fp32; these kernels keep it there
+    want = torch.zeros_like(x)
+    want[s_:] = (C[s_:].float() * u[:-s_]).to(dt)
+    assert torch.equal(y, want.permute(1, 0, 2, 3)), "y"
+    del y
+    dx, dB, dC, dh = _lib.bwd_time_major(dy, x, B, C, h)
+    torch.cuda.synchronize()
+    assert torch.isfinite(dh.float()).all()
+    dyt = dy.permute(1, 0, 2, 3)
+    want.zero_()
+    want[s_:] = (dyt[s_:].float() * u[:-s_]).to(dt)
+    assert torch.equal(dC, want), "dC"
+    del u
+    g2 = dyt.float() * C.float()
+    want.zero_()
+    want[:-s_] = (g2[s_:] * x[:-s_].float()).to(dt)
+    assert torch.equal(dB, want), "dB"
+    want.zero_()
+    want[:-s_] = (g2[s_:] * B[:-s_].float()).to(dt)
+    assert torch.equal(dx, want), "dx"
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 def test_decayed_filter_in_one_launch(gcg_lib, dtype):
     """gcg_filter_decay_fwd / _bwd against the expression of explicit.py:68-75 followed by the
