@@ -163,3 +163,47 @@ def test_long_context_64bit_offsets(gcg_lib):
         x, B, C = (inp[n][:, lo:t1].index_select(2, idx).float().cpu() for n in ("k", "q", "v"))
         ref = oracle.gcg_fwd_oracle(x, B, C, inp["h"].index_select(0, idx).float().cpu())
         assert_close(y[:, t0:t1].index_select(2, idx), ref[:, t0 - lo:], TOL[wl.dtype], f"y rows {t0}..{t1}")
+
+
+@pytest.mark.parametrize("layout", ["separate", "interleaved"])
+def test_short_filter_64bit_offsets(gcg_lib, layout):
+    """The register-window kernels (Hyena-SE, 7 taps) on B=1, L=2^19, D=4096 in bf16: 2^31 elements per tensor,
+    3 * 2^31 in the interleaved one.  A filter that delays by two rows makes every output a product of input
+    elements (these kernels keep B*x and dy*C in fp32), compared exactly on the whole tensors."""
+    bs, L, g, dg, hl, s_ = 1, 1 << 19, 256, 16, 7, 2
+    dt = torch.bfloat16
+    gen = torch.Generator(device=DEV)
+    feat = torch.empty(bs, L, g, dg, 3, dtype=dt, device=DEV)
+    dy = torch.empty(bs, L, g, dg, dtype=dt, device=DEV)
+    for k, t0 in enumerate(range(0, L, 1 << 16)):
+        gen.manual_seed(700 + k)
+        feat[:, t0:t0 + (1 << 16)].normal_(generator=gen)
+        dy[:, t0:t0 + (1 << 16)].normal_(generator=gen)
+    h = torch.zeros(g, 1, hl, dtype=dt, device=DEV)
+    h[:, 0, hl - 1 - s_] = 1.0
+    C, B, x = feat.unbind(-1)
+    if layout == "separate":
+        x, B, C = x.contiguous(), B.contiguous(), C.contiguous()
+        _, _, y = _lib.fwd(x, B, C, h)
+        dx, dB, dC, dh = _lib.bwd(dy, x, B, C, h)
+    else:
+        y = _lib.fwd_interleaved(feat, h)
+        dfeat, dh = _lib.bwd_interleaved(dy, feat, h)
+        dC, dB, dx = dfeat.unbind(-1)
+    torch.cuda.synchronize()
+    assert torch.isfinite(dh.float()).all()
+    u = x.float() * B.float()
+    want = torch.zeros_like(dy)
+    want[:, s_:] = (C[:, s_:].float() * u[:, :-s_]).to(dt)
+    assert torch.equal(y, want), "y"
+    want.zero_()
+    want[:, s_:] = (dy[:, s_:].float() * u[:, :-s_]).to(dt)
+    assert torch.equal(dC, want), "dC"
+    del u
+    g2 = dy.float() * C.float()
+    want.zero_()
+    want[:, :-s_] = (g2[:, s_:] * x[:, :-s_].float()).to(dt)
+    assert torch.equal(dB, want), "dB"
+    want.zero_()
+    want[:, :-s_] = (g2[:, s_:] * B[:, :-s_].float()).to(dt)
+    assert torch.equal(dx, want), "dx"
