@@ -165,7 +165,7 @@ def test_long_context_64bit_offsets(gcg_lib):
         assert_close(y[:, t0:t1].index_select(2, idx), ref[:, t0 - lo:], TOL[wl.dtype], f"y rows {t0}..{t1}")
 
 
-@pytest.mark.parametrize("layout", ["separate", "interleaved"])
+@pytest.mark.parametrize("layout", ["separate", "interleaved", "direct"])
 def test_short_filter_64bit_offsets(gcg_lib, layout):
     """The register-window kernels (Hyena-SE, 7 taps) on B=1, L=2^19, D=4096 in bf16: 2^31 elements per tensor,
     3 * 2^31 in the interleaved one.  A filter that delays by two rows makes every output a product of input
@@ -182,10 +182,11 @@ def test_short_filter_64bit_offsets(gcg_lib, layout):
     h = torch.zeros(g, 1, hl, dtype=dt, device=DEV)
     h[:, 0, hl - 1 - s_] = 1.0
     C, B, x = feat.unbind(-1)
-    if layout == "separate":
+    if layout != "interleaved":
+        algo = "window" if layout == "separate" else "direct"      # direct: the general fallback kernels
         x, B, C = x.contiguous(), B.contiguous(), C.contiguous()
-        _, _, y = _lib.fwd(x, B, C, h)
-        dx, dB, dC, dh = _lib.bwd(dy, x, B, C, h)
+        _, _, y = _lib.fwd(x, B, C, h, algo=algo)
+        dx, dB, dC, dh = _lib.bwd(dy, x, B, C, h, algo=algo)
     else:
         y = _lib.fwd_interleaved(feat, h)
         dfeat, dh = _lib.bwd_interleaved(dy, feat, h)
