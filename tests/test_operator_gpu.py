@@ -120,6 +120,34 @@ def test_runs_on_the_callers_stream(gcg_lib):
         assert torch.equal(a, b)
 
 
+def test_backward_launches_overlap_on_streams(gcg_lib):
+    """Backward launches in flight on four streams at once (each with its own inputs, outputs and workspace): every
+    launch counts its workgroups' arrivals on a set of counters of its own, so each result equals the one computed
+    alone, bit for bit -- the operator's kernel and the one-kernel Hyena-MR mixer."""
+    bs, L, g, dg, hl, kf = 2, 4096, 16, 16, 128, 3
+    dt = torch.bfloat16
+    n = 4
+    gen = torch.Generator(device=DEV).manual_seed(21)
+    rnd = lambda *shape: torch.randn(*shape, device=DEV, generator=gen).to(dt)
+    sets = [[rnd(bs, L, g, dg) for _ in range(4)] for _ in range(n)]                 # x, B, C, dy
+    raws = [rnd(bs, L, g, dg, 3) for _ in range(n)]
+    h = (torch.randn(g, 1, hl, device=DEV, generator=gen) / hl ** 0.5).to(dt)
+    wf = (torch.randn(3 * g * dg, 1, kf, device=DEV, generator=gen) / kf ** 0.5).to(dt)
+    alone = [(_lib.bwd(s[3], s[0], s[1], s[2], h), _lib.mixer_mr_bwd(s[3], r, wf, h)) for s, r in zip(sets, raws)]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(n)]
+    for rep in range(5):
+        got = []
+        for st, s, r in zip(streams, sets, raws):
+            with torch.cuda.stream(st):
+                got.append((_lib.bwd(s[3], s[0], s[1], s[2], h), _lib.mixer_mr_bwd(s[3], r, wf, h)))
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(got, alone)):
+            for fam in range(2):
+                for t, (u, v) in enumerate(zip(a[fam], b[fam])):
+                    assert torch.equal(u, v), f"repeat {rep}, stream {i}, family {fam}, output {t}"
+
+
 @pytest.mark.parametrize("hl,dtype", [(7, torch.float32), (128, torch.bfloat16)])
 def test_graph_capture_and_replay(gcg_lib, hl, dtype):
     """The launch-bound small shapes are what a HIP graph is for: forward and backward are
