@@ -128,8 +128,9 @@ def test_compile_fullgraph_interleaved(gcg_lib):
         assert torch.equal(a, b), name
 
 
-@pytest.mark.parametrize("kind", ["mr", "se"])
-def test_compile_fullgraph_hyena_mixer(gcg_lib, kind):
+@pytest.mark.parametrize("planar", [False, True], ids=["interleaved", "planar"])
+@pytest.mark.parametrize("kind", ["mr", "se", "se-grouped"])
+def test_compile_fullgraph_hyena_mixer(gcg_lib, kind, planar):
     """HyenaMixer (featurizer conv, split, operator; for Hyena-MR with the filter formed in the kernel) traced by
     torch.compile without a graph break: output and every gradient equal to eager."""
     from savanna_amd.operators.hyena import CgcgConfig, HyenaMixer, HyenaMROperator, HyenaSEOperator
@@ -138,8 +139,8 @@ def test_compile_fullgraph_hyena_mixer(gcg_lib, kind):
     bs, L, g, dg = 2, 384, 4, 16
     cfg = CgcgConfig(cgcg_dtype="bfloat16")
     op = (HyenaMROperator(g * dg, g, 128, cfg, small_init=False, device=DEV) if kind == "mr"
-          else HyenaSEOperator(g * dg, g * dg, 7, cfg, device=DEV))
-    mixer = HyenaMixer(op, 3, dtype=torch.bfloat16, device=DEV)
+          else HyenaSEOperator(g * dg, g * dg if kind == "se" else g, 7, cfg, device=DEV))
+    mixer = HyenaMixer(op, 3, dtype=torch.bfloat16, device=DEV, interleave_projections=not planar)
     feats = torch.randn(bs, L, 3 * g * dg, device=DEV).to(torch.bfloat16).requires_grad_(True)
     dz = (0.1 * torch.randn(bs, L, g * dg, device=DEV)).to(torch.bfloat16)
     params = list(mixer.parameters())
