@@ -89,6 +89,38 @@ def test_library_opcheck(gcg_lib):
     torch.library.opcheck(torch.ops.gcg.mixer_mr_fwd_decay, (feat, wf, w, decay, 128, torch.bfloat16), test_utils=checks)
     torch.library.opcheck(torch.ops.gcg.mixer_mr_bwd_decay, (dy, feat, wf, w, decay, 128, torch.bfloat16),
                           test_utils=checks)
+    pl, wf_pl = feat.permute(0, 1, 4, 2, 3).contiguous(), wf        # planar flag (the filters' order is immaterial here)
+    torch.library.opcheck(torch.ops.gcg.mixer_mr_fwd, (pl, wf_pl, h, True), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_mr_bwd, (dy, pl, wf_pl, h, True), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_mr_fwd_decay, (pl, wf_pl, w, decay, 128, torch.bfloat16, True), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_mr_bwd_decay, (dy, pl, wf_pl, w, decay, 128, torch.bfloat16, True),
+                          test_utils=checks)
+    # the filter alone and inside the operator's kernels
+    torch.library.opcheck(torch.ops.gcg.filter_decay_fwd, (w, decay, 128, torch.bfloat16), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.filter_decay_bwd, (torch.randn(2, 1, 128, device=DEV), decay), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.fwd_decay, (x, B, C, w, decay, 128, torch.bfloat16), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.bwd_decay, (dy, x, B, C, w, decay, 128, torch.bfloat16), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.fwd_interleaved_decay, (feat, w, decay, 128, torch.bfloat16), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.bwd_interleaved_decay, (dy, feat, w, decay, 128, torch.bfloat16), test_utils=checks)
+    # the featurizer, the Hyena-SE mixer (both layouts) and time-major operands
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(1, 130, 2, 16, 7, torch.bfloat16))
+    feat = torch.stack([C, B, x], dim=-1).contiguous()
+    flat = feat.view(1, 130, 3 * 2 * 16, 1)
+    torch.library.opcheck(torch.ops.gcg.dwconv_fwd, (flat, wf), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.dwconv_bwd, (flat, flat, wf), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_se_fwd, (feat, wf, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_se_bwd, (dy, feat, wf, h), test_utils=checks)
+    pl = feat.permute(0, 1, 4, 2, 3).contiguous()
+    torch.library.opcheck(torch.ops.gcg.mixer_se_fwd, (pl, wf, h, True), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.mixer_se_bwd, (dy, pl, wf, h, True), test_utils=checks)
+    xt, Bt, Ct = (t.permute(1, 0, 2, 3).contiguous() for t in (x, B, C))
+    torch.library.opcheck(torch.ops.gcg.fwd_time_major, (xt, Bt, Ct, h), test_utils=checks)
+    torch.library.opcheck(torch.ops.gcg.bwd_time_major, (dy, xt, Bt, Ct, h), test_utils=checks)
+    checked = {"fwd", "fwd_full", "bwd", "fwd_interleaved", "bwd_interleaved", "fwd_out", "fwd_planar", "bwd_planar",
+               "mixer_mr_fwd", "mixer_mr_bwd", "mixer_mr_fwd_decay", "mixer_mr_bwd_decay", "filter_decay_fwd",
+               "filter_decay_bwd", "fwd_decay", "bwd_decay", "fwd_interleaved_decay", "bwd_interleaved_decay", "dwconv_fwd",
+               "dwconv_bwd", "mixer_se_fwd", "mixer_se_bwd", "fwd_time_major", "bwd_time_major"}
+    assert checked == set(_ops.OP_NAMES)                # a new operator gets its check here
 
 
 def _grads(fn, tensors, dy):
