@@ -277,6 +277,9 @@ GCG_API int gcg_dwconv_bwd(const void *dy, const void *x, const void *w, void *d
  *
  * The result equals that of the two calls it replaces up to the rounding of the fp32 sums (the
  * taps are added in another order).
+ * dtype GCG_BF16_F32 / GCG_F16_F32: raw, wf, y (and dy, draw, dwf) are 16-bit, h and dh are fp32 -- cgcg_dtype
+ * float32 on 16-bit activations (hyena.py:812-816, :842-843) without the casts: f is rounded to 16 bits as the
+ * featurizer stores it, the operator's taps and arithmetic are fp32, y is rounded once.
  * Supported: hl <= 8, kf <= 4, dg even, 16-byte aligned tensors; otherwise GCG_ERR_UNSUPPORTED.
  */
 GCG_API int gcg_mixer_se_fwd(const void *raw, const void *wf, const void *h, void *y,

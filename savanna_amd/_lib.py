@@ -486,9 +486,9 @@ def _check_mixer_se(raw, wf, h, planar=False):
         raise ValueError("wf must be a contiguous (3 * g * dg, 1, kf) tensor")
     if h.dim() != 3 or h.shape[0] != g or h.shape[1] != 1 or not h.is_contiguous():
         raise ValueError("h must be a contiguous (g, 1, hl) tensor")
-    for t in (wf, h):
-        if t.dtype != raw.dtype or t.device != raw.device:
-            raise ValueError("raw, wf and h must share dtype and device")
+    if wf.dtype != raw.dtype or wf.device != raw.device or h.device != raw.device:
+        raise ValueError("raw and wf must share dtype, and raw, wf and h their device")
+    gated_code(raw, h)          # h of raw's dtype, or fp32 with 16-bit raw (fp32 arithmetic)
 
 
 def mixer_se_fwd(raw, wf, h, planar=False):
@@ -508,7 +508,7 @@ def mixer_se_fwd(raw, wf, h, planar=False):
     with _on_device(raw.device):
         st = torch.cuda.current_stream().cuda_stream
         rc = fn(raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), bs, L, g, dg,
-                h.shape[-1], wf.shape[-1], dtype_code(raw.dtype), st)
+                h.shape[-1], wf.shape[-1], gated_code(raw, h), st)
     check(rc, "gcg_mixer_se_fwd_planar" if planar else "gcg_mixer_se_fwd")
     return y
 
@@ -528,7 +528,7 @@ def mixer_se_bwd(dy, raw, wf, h, planar=False):
     draw, dwf, dh = torch.empty_like(raw), torch.empty_like(wf), torch.empty_like(h)
     if raw.numel() == 0:
         return draw, dwf.zero_(), dh.zero_()
-    code = dtype_code(raw.dtype)
+    code = gated_code(raw, h)
     nbytes = lib.gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code)
     if nbytes == 0:
         check(-2, "gcg_mixer_se_bwd_workspace_bytes")     # GCG_ERR_UNSUPPORTED

@@ -562,7 +562,7 @@ int mixer_se_fwd_any(const void *raw, const void *wf, const void *h, void *y, in
 {
     if (!raw || !wf || !h || !y) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     if (kf <= 0) return GCG_ERR_BAD_ARG;
     dm.planar = planar;
@@ -577,7 +577,7 @@ int mixer_se_bwd_any(const void *dy, const void *raw, const void *wf, const void
 {
     if (!dy || !raw || !wf || !h || !draw || !dwf || !dh) return GCG_ERR_BAD_ARG;
     gcg::Dims dm;
-    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm);
+    int rc = make_dims(bs, L, g, dg, hl, dtype, &dm, true);
     if (rc) return rc;
     if (kf <= 0) return GCG_ERR_BAD_ARG;
     dm.planar = planar;
@@ -608,7 +608,7 @@ GCG_API size_t gcg_mixer_se_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g
                                                 int32_t dtype)
 {
     gcg::Dims dm;
-    if (make_dims(bs, L, g, dg, hl, dtype, &dm) || kf <= 0 || !gcg::mixer_se_supported(dm, kf)) return 0;
+    if (make_dims(bs, L, g, dg, hl, dtype, &dm, true) || kf <= 0 || !gcg::mixer_se_supported(dm, kf)) return 0;
     return (gcg::mixer_se_bwd_workspace(dtype, dm, kf) + 255) & ~(size_t)255;
 }
 

@@ -496,8 +496,10 @@ template <int HX, int HY> __device__ __forceinline__ uint32_t halves(uint32_t x,
     return __builtin_amdgcn_perm(y, x, sel);
 }
 // packed taps of a lane: Wa[e] = (tap 0 rows back, tap 1 row back), Wb[e] = (2 back, 3 back); hr as above
-template <typename T, int HL, bool PL>
-__device__ __forceinline__ void load_taps16(const T *wf, const T *h, int64_t c, const Dims &dm, int kf,
+// (FT: element type of the operator's filter -- T, or float for fp32 arithmetic on 16-bit tensors: the taps of the
+// operator are used as fp32 values either way)
+template <typename T, int HL, bool PL, typename FT>
+__device__ __forceinline__ void load_taps16(const T *wf, const FT *h, int64_t c, const Dims &dm, int kf,
                                             uint32_t (&Wa)[6], uint32_t (&Wb)[6], float (&hr)[HL])
 {
 #pragma unroll
@@ -509,9 +511,9 @@ __device__ __forceinline__ void load_taps16(const T *wf, const T *h, int64_t c, 
         Wa[e] = Word<T>::pack(&w[0]);
         Wb[e] = Word<T>::pack(&w[2]);
     }
-    const T *hg = h + (c / dm.dg) * dm.hl;
+    const FT *hg = h + (c / dm.dg) * dm.hl;
 #pragma unroll
-    for (int j = 0; j < HL; ++j) hr[j] = (j < dm.hl) ? Elem<T>::load(hg + dm.hl - 1 - j) : 0.f;
+    for (int j = 0; j < HL; ++j) hr[j] = (j < dm.hl) ? Elem<FT>::load(hg + dm.hl - 1 - j) : 0.f;
 }
 // f of row t from pe_t = pair_rows(raw[t], raw[t-1]) and pe_t2 = pair_rows(raw[t-2], raw[t-3]), rounded to T
 // (fp: the same row as elements of T)
@@ -532,9 +534,9 @@ __device__ __forceinline__ void featurize16(const uint32_t (&Wa)[6], const uint3
     featurize16<T>(Wa, Wb, pe_t, pe_t2, f, fp);
 }
 
-template <typename T, int HL, bool PL = false>
+template <typename T, int HL, bool PL = false, typename FT = T>
 __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict__ raw, const T *__restrict__ wf,
-                                                             const T *__restrict__ h, T *__restrict__ y, Dims dm,
+                                                             const FT *__restrict__ h, T *__restrict__ y, Dims dm,
                                                              int kf, MixPlan pl)
 {
     constexpr int ES = 2, CH = 2, NH = HL - 1 + 3;
@@ -548,7 +550,7 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
 
     uint32_t Wa[6], Wb[6];
     float hr[HL];
-    load_taps16<T, HL, PL>(wf, h, c, dm, kf, Wa, Wb, hr);
+    load_taps16<T, HL, PL, FT>(wf, h, c, dm, kf, Wa, Wb, hr);
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
@@ -624,10 +626,10 @@ __global__ __launch_bounds__(256) void mixer_se_fwd16_kernel(const T *__restrict
 
 // The backward walk above with the featurizer's three sums done two taps (or two rows) at a time.
 // d raw lags d f by three rows whatever the filter length (the fourth tap is zero for shorter filters).
-template <typename T, int HL, int KF, bool PL = false>
+template <typename T, int HL, int KF, bool PL = false, typename FT = T>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MIXER_WPE)))
 void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, const T *__restrict__ wf,
-                           const T *__restrict__ h, T *__restrict__ draw, float *__restrict__ ws_h,
+                           const FT *__restrict__ h, T *__restrict__ draw, float *__restrict__ ws_h,
                            float *__restrict__ ws_w, Dims dm, int kf, MixPlan pl)
 {
     typedef Piece<T> P;
@@ -643,7 +645,7 @@ void mixer_se_bwd16_kernel(const T *__restrict__ dy, const T *__restrict__ raw, 
 
     uint32_t Wa[6], Wb[6];
     float hr[HL];
-    load_taps16<T, HL, PL>(wf, h, c, dm, kf, Wa, Wb, hr);
+    load_taps16<T, HL, PL, FT>(wf, h, c, dm, kf, Wa, Wb, hr);
 
     const int64_t t_start = (int64_t)seg * pl.ts;
     const int64_t t_end = (t_start + pl.ts < L) ? t_start + pl.ts : L;
@@ -855,7 +857,8 @@ MixPlan plan(const Dims &dm, int ch, bool backward)
 
 int lane_channels(int dtype) { return dtype == GCG_F32 ? 1 : 2; }
 
-template <typename T, int HL, int KF>
+// FT: element type of h and dh (float with 16-bit T: fp32 filter and arithmetic on 16-bit tensors)
+template <typename T, int HL, int KF, typename FT>
 int fwd_launch(const void *raw, const void *wf, const void *h, void *y, const Dims &dm, int kf, hipStream_t st)
 {
     int e = 0;
@@ -863,11 +866,11 @@ int fwd_launch(const void *raw, const void *wf, const void *h, void *y, const Di
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if constexpr (sizeof(T) == 2) {
         if (dm.planar)
-            e = launch_plain((mixer_se_fwd16_kernel<T, HL, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
-                             (const T *)raw, (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+            e = launch_plain((mixer_se_fwd16_kernel<T, HL, true, FT>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)raw, (const T *)wf, (const FT *)h, (T *)y, dm, kf, p);
         else
-            e = launch_plain((mixer_se_fwd16_kernel<T, HL>), dim3((unsigned)p.nwg), dim3(p.threads), st, (const T *)raw,
-                             (const T *)wf, (const T *)h, (T *)y, dm, kf, p);
+            e = launch_plain((mixer_se_fwd16_kernel<T, HL, false, FT>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)raw, (const T *)wf, (const FT *)h, (T *)y, dm, kf, p);
     } else {
         if (dm.planar)
             e = launch_plain((mixer_se_fwd_kernel<T, HL, KF, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
@@ -879,7 +882,7 @@ int fwd_launch(const void *raw, const void *wf, const void *h, void *y, const Di
     return e;
 }
 
-template <typename T, int HL, int KF>
+template <typename T, int HL, int KF, typename FT>
 int bwd_launch(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf, void *dh,
                void *ws, const Dims &dm, int kf, hipStream_t st)
 {
@@ -890,11 +893,11 @@ int bwd_launch(const void *dy, const void *raw, const void *wf, const void *h, v
     float *ws_w = ws_h + (size_t)dm.hl * p.nrows * p.nvec;
     if constexpr (sizeof(T) == 2) {
         if (dm.planar)
-            e = launch_plain((mixer_se_bwd16_kernel<T, HL, KF, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
-                             (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+            e = launch_plain((mixer_se_bwd16_kernel<T, HL, KF, true, FT>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)dy, (const T *)raw, (const T *)wf, (const FT *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
         else
-            e = launch_plain((mixer_se_bwd16_kernel<T, HL, KF>), dim3((unsigned)p.nwg), dim3(p.threads), st,
-                             (const T *)dy, (const T *)raw, (const T *)wf, (const T *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
+            e = launch_plain((mixer_se_bwd16_kernel<T, HL, KF, false, FT>), dim3((unsigned)p.nwg), dim3(p.threads), st,
+                             (const T *)dy, (const T *)raw, (const T *)wf, (const FT *)h, (T *)draw, ws_h, ws_w, dm, kf, p);
     } else {
         if (dm.planar)
             e = launch_plain((mixer_se_bwd_kernel<T, HL, KF, true>), dim3((unsigned)p.nwg), dim3(p.threads), st,
@@ -907,35 +910,35 @@ int bwd_launch(const void *dy, const void *raw, const void *wf, const void *h, v
     // both filter gradients in one launch
     const ColsumJob jh{ws_h, dh, p.nrows, p.nvec, dm.dg / p.ch, dm.g, dm.hl};
     const ColsumJob jw{ws_w, dwf, p.nrows, 3 * dm.d, 1, (int)(3 * dm.d), kf};
-    return launch_colsum_reduce2<T>(jh, jw, st);
+    return (launch_colsum_reduce2<FT, T>(jh, jw, st));
 }
 
-template <typename T, int KF>
+template <typename T, int KF, typename FT>
 int fwd_k(const void *raw, const void *wf, const void *h, void *y, const Dims &dm, int kf, hipStream_t st)
 {
-    if (dm.hl <= 4) return fwd_launch<T, 4, KF>(raw, wf, h, y, dm, kf, st);
-    if (dm.hl <= 7) return fwd_launch<T, 7, KF>(raw, wf, h, y, dm, kf, st);
-    return fwd_launch<T, 8, KF>(raw, wf, h, y, dm, kf, st);
+    if (dm.hl <= 4) return fwd_launch<T, 4, KF, FT>(raw, wf, h, y, dm, kf, st);
+    if (dm.hl <= 7) return fwd_launch<T, 7, KF, FT>(raw, wf, h, y, dm, kf, st);
+    return fwd_launch<T, 8, KF, FT>(raw, wf, h, y, dm, kf, st);
 }
-template <typename T>
+template <typename T, typename FT = T>
 int fwd_t(const void *raw, const void *wf, const void *h, void *y, const Dims &dm, int kf, hipStream_t st)
 {
-    return kf <= 3 ? fwd_k<T, 3>(raw, wf, h, y, dm, kf, st) : fwd_k<T, 4>(raw, wf, h, y, dm, kf, st);
+    return kf <= 3 ? fwd_k<T, 3, FT>(raw, wf, h, y, dm, kf, st) : fwd_k<T, 4, FT>(raw, wf, h, y, dm, kf, st);
 }
-template <typename T, int KF>
+template <typename T, int KF, typename FT>
 int bwd_k(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf, void *dh, void *ws,
           const Dims &dm, int kf, hipStream_t st)
 {
-    if (dm.hl <= 4) return bwd_launch<T, 4, KF>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
-    if (dm.hl <= 7) return bwd_launch<T, 7, KF>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
-    return bwd_launch<T, 8, KF>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
+    if (dm.hl <= 4) return bwd_launch<T, 4, KF, FT>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
+    if (dm.hl <= 7) return bwd_launch<T, 7, KF, FT>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
+    return bwd_launch<T, 8, KF, FT>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
 }
-template <typename T>
+template <typename T, typename FT = T>
 int bwd_t(const void *dy, const void *raw, const void *wf, const void *h, void *draw, void *dwf, void *dh, void *ws,
           const Dims &dm, int kf, hipStream_t st)
 {
-    return kf <= 3 ? bwd_k<T, 3>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st)
-                   : bwd_k<T, 4>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
+    return kf <= 3 ? bwd_k<T, 3, FT>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st)
+                   : bwd_k<T, 4, FT>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
 }
 
 } // namespace
@@ -953,6 +956,8 @@ int mixer_se_fwd_launch(int dtype, const void *raw, const void *wf, const void *
     case GCG_F32:  return fwd_t<float>(raw, wf, h, y, dm, kf, st);
     case GCG_BF16: return fwd_t<bf16_t>(raw, wf, h, y, dm, kf, st);
     case GCG_F16:  return fwd_t<f16_t>(raw, wf, h, y, dm, kf, st);
+    case GCG_BF16_F32: return fwd_t<bf16_t, float>(raw, wf, h, y, dm, kf, st);      // h in fp32
+    case GCG_F16_F32:  return fwd_t<f16_t, float>(raw, wf, h, y, dm, kf, st);
     }
     return (int)hipErrorInvalidValue;
 }
@@ -970,6 +975,8 @@ int mixer_se_bwd_launch(int dtype, const void *dy, const void *raw, const void *
     case GCG_F32:  return bwd_t<float>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
     case GCG_BF16: return bwd_t<bf16_t>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
     case GCG_F16:  return bwd_t<f16_t>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
+    case GCG_BF16_F32: return bwd_t<bf16_t, float>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);    // h, dh in fp32
+    case GCG_F16_F32:  return bwd_t<f16_t, float>(dy, raw, wf, h, draw, dwf, dh, ws, dm, kf, st);
     }
     return (int)hipErrorInvalidValue;
 }

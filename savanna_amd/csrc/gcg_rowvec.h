@@ -154,13 +154,14 @@ __global__ __launch_bounds__(256) void colsum_reduce_kernel(ColsumJob jb)
 
 // two reductions in one launch (the filter gradients of two filters from one walk): the first
 // nb0 workgroups of a grid row belong to the first; grid rows beyond a job's tap count idle
-template <typename T>
+// (T0, T1: element types of the two results)
+template <typename T0, typename T1>
 __global__ __launch_bounds__(256) void colsum_reduce2_kernel(ColsumJob j0, ColsumJob j1, int nb0)
 {
     const bool second = (int)blockIdx.x >= nb0;
-    const ColsumJob &jb = second ? j1 : j0;
-    if ((int)blockIdx.y >= jb.ntap) return;
-    colsum_reduce_block<T>(jb, second ? (int)blockIdx.x - nb0 : (int)blockIdx.x, blockIdx.y);
+    if ((int)blockIdx.y >= (second ? j1.ntap : j0.ntap)) return;
+    if (second) colsum_reduce_block<T1>(j1, (int)blockIdx.x - nb0, blockIdx.y);
+    else colsum_reduce_block<T0>(j0, (int)blockIdx.x, blockIdx.y);
 }
 
 inline unsigned colsum_blocks(int lpg, int nfilt)
@@ -179,13 +180,13 @@ inline int launch_colsum_reduce(const float *ws, T *out, int64_t nrow, int64_t n
     return e;
 }
 
-template <typename T>
+template <typename T0, typename T1 = T0>
 inline int launch_colsum_reduce2(const ColsumJob &j0, const ColsumJob &j1, hipStream_t st)
 {
     int e = 0;
     const unsigned nb0 = colsum_blocks(j0.lpg, j0.nfilt), nb1 = colsum_blocks(j1.lpg, j1.nfilt);
     const unsigned ny = (unsigned)(j0.ntap > j1.ntap ? j0.ntap : j1.ntap);
-    e = launch_plain(colsum_reduce2_kernel<T>, dim3(nb0 + nb1, ny), dim3(256), st, j0, j1, (int)nb0);
+    e = launch_plain((colsum_reduce2_kernel<T0, T1>), dim3(nb0 + nb1, ny), dim3(256), st, j0, j1, (int)nb0);
     return e;
 }
 

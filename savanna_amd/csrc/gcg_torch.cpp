@@ -303,9 +303,9 @@ void check_mixer_se(const Tensor &raw, const Tensor &wf, const Tensor &h, bool p
                 "gcg: wf must be a contiguous (3 * g * dg, 1, kf) tensor");
     TORCH_CHECK(h.dim() == 3 && h.size(0) == g && h.size(1) == 1 && h.is_contiguous(),
                 "gcg: h must be a contiguous (g, 1, hl) tensor");
-    TORCH_CHECK(wf.scalar_type() == raw.scalar_type() && h.scalar_type() == raw.scalar_type() &&
-                    wf.device() == raw.device() && h.device() == raw.device(),
-                "gcg: raw, wf and h must share dtype and device");
+    TORCH_CHECK(wf.scalar_type() == raw.scalar_type() && wf.device() == raw.device() && h.device() == raw.device(),
+                "gcg: raw and wf must share dtype, and raw, wf and h their device");
+    (void)gated_code(raw, h);       // h of raw's dtype, or fp32 with 16-bit raw (fp32 arithmetic)
 }
 
 Tensor mixer_se_fwd(const Tensor &raw, const Tensor &wf, const Tensor &h, bool planar)
@@ -318,7 +318,7 @@ Tensor mixer_se_fwd(const Tensor &raw, const Tensor &wf, const Tensor &h, bool p
     if (y.numel() == 0) return y;
     check_rc((planar ? gcg_mixer_se_fwd_planar : gcg_mixer_se_fwd)(
                  raw.data_ptr(), wf.data_ptr(), h.data_ptr(), y.data_ptr(), raw.size(0), raw.size(1), (int32_t)g,
-                 (int32_t)dg, (int32_t)h.size(2), (int32_t)wf.size(2), dtype_code(raw.scalar_type()), stream_of(raw)),
+                 (int32_t)dg, (int32_t)h.size(2), (int32_t)wf.size(2), gated_code(raw, h), stream_of(raw)),
              planar ? "gcg_mixer_se_fwd_planar" : "gcg_mixer_se_fwd");
     return y;
 }
@@ -338,7 +338,7 @@ std::tuple<Tensor, Tensor, Tensor> mixer_se_bwd(const Tensor &dy, const Tensor &
     if (raw.numel() == 0) return {draw, dwf.zero_(), dh.zero_()};
     const int64_t bs = raw.size(0), L = raw.size(1);
     const int32_t hl = (int32_t)h.size(2), kf = (int32_t)wf.size(2);
-    const int code = dtype_code(raw.scalar_type());
+    const int code = gated_code(raw, h);
     const size_t nbytes = gcg_mixer_se_bwd_workspace_bytes(bs, L, g, dg, hl, kf, code);
     if (nbytes == 0) check_rc(GCG_ERR_UNSUPPORTED, "gcg_mixer_se_bwd_workspace_bytes");
     Tensor ws = workspace(nbytes, raw, "gcg_mixer_se_bwd_workspace_bytes");

@@ -398,13 +398,27 @@ class HyenaMixer(nn.Module):
 
     def _fusable(self, features: torch.Tensor, hl: int) -> bool:
         conv, op = self.hyena_proj_conv, self.mixer
-        if op.cgcg_dtype != features.dtype and op._fp32_inside(features.dtype, features):
-            # 16-bit features into fp32 arithmetic: the featurizer's output is rounded to 16 bits before the operator
-            # (hyena.py:812-816 casts after the conv), which the two-kernel chain does without a cast and the
-            # one-kernel form could only do on fp32 copies of the features
-            return False
         return (self.fuse_short and features.is_cuda and hl <= 8 and conv.kernel_size <= 4 and conv.group_dim == 1
                 and op.group_dim % 2 == 0)
+
+    def _fused_short(self, features: torch.Tensor, h: torch.Tensor, planar: bool) -> torch.Tensor:
+        """Featurizer and Hyena-SE operator in one kernel each way.  16-bit features with ``cgcg_dtype`` float32 stay
+        16-bit: the kernels round the featurizer's output to the features' type, as the conv of block.py:873 stores
+        it before the casts of hyena.py:812-816, and keep the filter and the operator's arithmetic in fp32."""
+        op = self.mixer
+        bs, seqlen, _ = features.shape
+        g, dg = op.num_groups, op.group_dim
+        dtype = features.dtype
+        inside = op.cgcg_dtype != dtype and op._fp32_inside(dtype, features)
+        cast = op.cgcg_dtype != dtype and not inside
+        if cast:
+            features = features.to(op.cgcg_dtype)
+        shape = (bs, seqlen, 3, g, dg) if planar else (bs, seqlen, g, dg, 3)
+        z = _FeaturizedShortGateConvGate.apply(features.reshape(shape),
+                                               self.hyena_proj_conv.short_conv_weight.to(features.dtype),
+                                               h.to(op.cgcg_dtype), planar)
+        z = z.reshape(bs, seqlen, g * dg)
+        return z.to(dtype) if cast else z
 
     def forward(self, features: torch.Tensor) -> torch.Tensor:
         op = self.mixer
@@ -424,14 +438,7 @@ class HyenaMixer(nn.Module):
                 return z.reshape(bs, seqlen, g * dg)
             h = op._filter(seqlen)
             if self._fusable(features, h.shape[-1]):
-                dtype = features.dtype
-                if op.cgcg_dtype != dtype:
-                    features = features.to(op.cgcg_dtype)
-                g, dg = op.num_groups, op.group_dim
-                z = _FeaturizedShortGateConvGate.apply(features.reshape(bs, seqlen, 3, g, dg),
-                                                       conv.short_conv_weight.to(op.cgcg_dtype), h.to(op.cgcg_dtype), True)
-                z = z.reshape(bs, seqlen, g * dg)
-                return z.to(dtype) if op.cgcg_dtype != dtype else z
+                return self._fused_short(features, h, True)
             if (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and op.cgcg_dtype == features.dtype and
                     features.dtype in (torch.bfloat16, torch.float16) and
                     _lib.mixer_mr_supported(op.group_dim, h.shape[-1], conv.kernel_size, features)):
@@ -461,13 +468,5 @@ class HyenaMixer(nn.Module):
         if not self._fusable(features, h.shape[-1]):
             return op.forward_features(self.hyena_proj_conv.forward_bld(features, feeds_operator=True),
                                        from_featurizer=True)
-        dtype = features.dtype
-        if op.cgcg_dtype != dtype:
-            features = features.to(op.cgcg_dtype)
-        g, dg = op.num_groups, op.group_dim
-        assert d3 == 3 * g * dg
-        z = _FeaturizedShortGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3),
-                                               self.hyena_proj_conv.short_conv_weight.to(op.cgcg_dtype),
-                                               h.to(op.cgcg_dtype))
-        z = z.reshape(bs, seqlen, g * dg)
-        return z.to(dtype) if op.cgcg_dtype != dtype else z
+        assert d3 == 3 * op.num_groups * op.group_dim
+        return self._fused_short(features, h, False)

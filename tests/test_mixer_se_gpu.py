@@ -89,6 +89,46 @@ def test_mixer_se_fwd_bwd(gcg_lib, bs, L, g, dg, hl, kf, dtype):
             assert_close(dh, dh_c, TOL_DH[dtype], "dh vs chain")
 
 
+@pytest.mark.parametrize("planar", [False, True], ids=["interleaved", "planar"])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("bs,L,g,dg,hl,kf", SHAPES)
+def test_fp32_filter_on_16_bit_tensors(gcg_lib, bs, L, g, dg, hl, kf, dtype, planar):
+    """16-bit raw and wf with an fp32 operator filter (cgcg_dtype float32 on 16-bit activations, hyena.py:812-816):
+    the featurizer's output is rounded to the tensors' type, the operator's taps and arithmetic stay in fp32, dh
+    comes back in fp32.  Against the oracle of that chain and against the chain of kernels."""
+    raw, dy, wf, _ = data(bs, L, g, dg, hl, kf, dtype, seed=L + hl + 1)
+    h = torch.randn(g, 1, hl, generator=torch.Generator().manual_seed(L)) / hl ** 0.5          # fp32, not representable in 16 bits
+    ref = oracle_chain(raw, dy, wf, h, dtype)
+    rawd, dyd, wfd, hd = (t.to(DEV) for t in (raw, dy, wf, h))
+    if planar:
+        d = g * dg
+        raw_in = rawd.permute(0, 1, 4, 2, 3).contiguous()
+        wf_in = wfd.view(d, 3, 1, kf).permute(1, 0, 2, 3).reshape(3 * d, 1, kf).contiguous()
+    else:
+        raw_in, wf_in = rawd, wfd
+    y = _lib.mixer_se_fwd(raw_in, wf_in, hd, planar=planar)
+    draw, dwf, dh = _lib.mixer_se_bwd(dyd, raw_in, wf_in, hd, planar=planar)
+    torch.cuda.synchronize()
+    assert y.dtype == dtype and draw.dtype == dtype and dwf.dtype == dtype and dh.dtype == torch.float32
+    if planar:
+        draw = draw.permute(0, 1, 3, 4, 2)
+        dwf = dwf.view(3, g * dg, 1, kf).permute(1, 0, 2, 3).reshape(3 * g * dg, 1, kf)
+    assert_close(y, ref[0], TOL[dtype], "y")
+    assert_close(draw, ref[1], 2 * TOL[dtype], "d raw")
+    if bs * L * dg >= 256:
+        assert_close(dwf, ref[2], 2 * TOL_DH[dtype], "dwf")
+        assert_close(dh, ref[3], TOL_DH[dtype], "dh")
+    if (3 * g * dg) % 4 == 0 and dg % 4 == 0:          # what the stand-alone kernels take
+        y_c, draw_c, dwf_c, dh_c = kernel_chain(rawd, dyd, wfd, hd)
+        torch.cuda.synchronize()
+        assert dh_c.dtype == torch.float32
+        assert_close(y, y_c, TOL[dtype], "y vs chain")
+        assert (y != y_c).float().mean() < 0.02, "more than rounding separates y from the chain of kernels"
+        assert_close(draw, draw_c, TOL[dtype], "d raw vs chain")
+        if bs * L * dg >= 256:
+            assert_close(dh, dh_c, 1e-4, "dh vs chain")          # both in fp32
+
+
 def test_mixer_se_is_deterministic_and_rejects_what_it_cannot_run(gcg_lib):
     raw, dy, wf, h = (t.to(DEV) for t in data(2, 512, 8, 16, 7, 3, torch.bfloat16, seed=1))
     a, b = _lib.mixer_se_bwd(dy, raw, wf, h), _lib.mixer_se_bwd(dy, raw, wf, h)
@@ -267,9 +307,9 @@ def test_hyena_mixer_planar_fused(gcg_lib):
 @pytest.mark.parametrize("planar", [False, True], ids=["interleaved", "planar"])
 def test_hyena_mixer_16_bit_features_fp32_arithmetic(gcg_lib, planar):
     """bf16 activations with cgcg_dtype float32 (the default, global_config.py:404): the featurizer's output is
-    rounded to bf16 before the operator's casts (block.py:873, hyena.py:812-816), so the mixer runs the featurizer
-    kernel and the operator on 16-bit tensors with fp32 arithmetic -- no fp32 copy of the features, and the same
-    values as the reference's chain written with torch ops."""
+    rounded to bf16 before the operator's casts (block.py:873, hyena.py:812-816).  The one-kernel path does the
+    same on the 16-bit features with an fp32 filter and fp32 arithmetic -- no fp32 copy of the features -- and
+    gives the values of the reference's chain written with torch ops."""
     import torch.nn.functional as F
 
     from savanna_amd.operators.hyena import CgcgConfig, HyenaMixer, HyenaSEOperator
@@ -281,9 +321,10 @@ def test_hyena_mixer_16_bit_features_fp32_arithmetic(gcg_lib, planar):
                        dtype=torch.bfloat16, device=DEV, interleave_projections=not planar)
     feats = torch.randn(bs, L, 3 * hidden, device=DEV).to(torch.bfloat16)
     dz = (0.1 * torch.randn(bs, L, hidden, device=DEV)).to(torch.bfloat16)
-    assert not mixer._fusable(feats, hl)
+    assert mixer._fusable(feats, hl)
     x = feats.clone().requires_grad_(True)
     z = mixer(x)
+    assert type(z.grad_fn.next_functions[0][0]).__name__.startswith("_FeaturizedShortGateConvGate")    # below the reshape
     z.backward(dz)
     assert z.dtype == torch.bfloat16 and x.grad.dtype == torch.bfloat16
     got = (z, x.grad, mixer.hyena_proj_conv.short_conv_weight.grad.clone(), mixer.mixer.short_conv_weight.grad.clone())
