@@ -82,3 +82,46 @@ def test_every_route_gives_the_chains_values(gcg_lib, kind, planar, types, kf, d
     assert_close(got[1], xr.grad, 2 * tol, "d features")
     assert_close(got[2], wf.grad, 2 * tol_w, "d featurizer weight")
     assert_close(got[3], fp.grad, 2 * tol_w, "d filter parameter")
+
+
+@pytest.mark.parametrize("planar", [False, True], ids=["interleaved", "planar"])
+@pytest.mark.parametrize("kind", ["mr", "se"])
+def test_ways_a_training_loop_calls_the_module(gcg_lib, kind, planar):
+    """Views with a larger row stride as features and as output gradient, a second backward through a retained graph,
+    no_grad, frozen features, autocast around the call, and parameters converted to bf16: the same values each time."""
+    torch.manual_seed(0)
+    bs, L, g, dg = 2, 500, 4, 16
+    hidden = g * dg
+    cfg = CgcgConfig(cgcg_dtype="bfloat16")
+    op = (HyenaMROperator(hidden, g, 128, cfg, small_init=False, device=DEV) if kind == "mr"
+          else HyenaSEOperator(hidden, g, 7, cfg, device=DEV))
+    m = HyenaMixer(op, 3, dtype=torch.bfloat16, device=DEV, interleave_projections=not planar)
+    feats = torch.randn(bs, L, 3 * hidden + 64, device=DEV).to(torch.bfloat16)[..., :3 * hidden]
+    dz = (0.1 * torch.randn(bs, L, hidden * 2, device=DEV)).to(torch.bfloat16)[..., ::2]
+    assert not feats.is_contiguous() and not dz.is_contiguous()
+    ref_in = feats.contiguous().requires_grad_(True)
+    z_ref = m(ref_in)
+    z_ref.backward(dz, retain_graph=True)
+    g1 = ref_in.grad.clone()
+    ref_in.grad = None
+    z_ref.backward(dz)
+    assert torch.equal(ref_in.grad, g1), "second backward"
+    x = feats.detach().requires_grad_(True)
+    z = m(x)
+    assert torch.equal(z, z_ref), "features with a larger row stride"
+    z.backward(dz)
+    assert torch.equal(x.grad, g1), "their gradient"
+    with torch.no_grad():
+        assert torch.equal(m(feats), z_ref), "no_grad"
+    for p in m.parameters():
+        p.grad = None
+    m(feats.contiguous()).backward(dz)
+    assert all(p.grad is not None for p in m.parameters()), "frozen features"
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        assert torch.equal(m(feats.contiguous()), z_ref), "autocast"
+    import copy
+    m16 = copy.deepcopy(m).bfloat16()                   # every parameter in bf16: the filter is then formed by torch ops
+    z16 = m16(feats.contiguous())
+    assert_close(z16, z_ref, 3 * TOL[torch.bfloat16], "bf16 parameters")      # w and decay rounded before their product
+    z16.sum().backward()
+    assert all(p.grad is not None and p.grad.dtype == torch.bfloat16 for p in m16.parameters())
