@@ -420,53 +420,38 @@ class HyenaMixer(nn.Module):
         z = z.reshape(bs, seqlen, g * dg)
         return z.to(dtype) if cast else z
 
+    def _medium(self, features: torch.Tensor, hl: int) -> bool:
+        """Whether the one-kernel Hyena-MR mixer takes these features with a filter of ``hl`` taps.  Planar features
+        ("(p g dg)" rows) run in the one-kernel form only, which has 16-bit arithmetic."""
+        conv, op = self.hyena_proj_conv, self.mixer
+        if not (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and
+                _lib.mixer_mr_supported(op.group_dim, hl, conv.kernel_size, features)):
+            return False
+        if self.interleave_projections:
+            return op.cgcg_dtype == features.dtype or op._fp32_inside(features.dtype, features)
+        return op.cgcg_dtype == features.dtype and features.dtype in (torch.bfloat16, torch.float16)
+
     def forward(self, features: torch.Tensor) -> torch.Tensor:
-        op = self.mixer
+        op, conv = self.mixer, self.hyena_proj_conv
         bs, seqlen, d3 = features.shape
-        conv = self.hyena_proj_conv
-        if not self.interleave_projections:
-            # "(p g dg)" features.  The fused kernels on planar pieces where they take the shape; otherwise the
-            # featurizer kernel, then the operator on the thirds of its rows (two kernels each way)
-            fused = op._filter_in_kernel(seqlen, op.num_groups, op.group_dim, features.dtype, features)
-            if (fused is not None and self.fuse_medium and conv.group_dim == 1 and op.cgcg_dtype == features.dtype and
-                    features.dtype in (torch.bfloat16, torch.float16) and
-                    _lib.mixer_mr_supported(op.group_dim, fused[0], conv.kernel_size, features)):
-                g, dg = op.num_groups, op.group_dim
-                z = _FeaturizedDecayedGateConvGate.apply(features.reshape(bs, seqlen, 3, g, dg),
-                                                         conv.short_conv_weight.to(features.dtype), op.filter.h,
-                                                         op.filter.decay, fused[0], fused[1], True)
-                return z.reshape(bs, seqlen, g * dg)
-            h = op._filter(seqlen)
-            if self._fusable(features, h.shape[-1]):
-                return self._fused_short(features, h, True)
-            if (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and op.cgcg_dtype == features.dtype and
-                    features.dtype in (torch.bfloat16, torch.float16) and
-                    _lib.mixer_mr_supported(op.group_dim, h.shape[-1], conv.kernel_size, features)):
-                g, dg = op.num_groups, op.group_dim
-                z = _FeaturizedGateConvGate.apply(features.reshape(bs, seqlen, 3, g, dg),
-                                                  conv.short_conv_weight.to(features.dtype), h.to(op.cgcg_dtype), True)
-                return z.reshape(bs, seqlen, g * dg)
-            return op.forward_features(conv.forward_bld(features, feeds_operator=True), interleaved=False)
-        fused = op._filter_in_kernel(seqlen, op.num_groups, op.group_dim, features.dtype, features)
-        if (fused is not None and self.fuse_medium and conv.group_dim == 1 and
-                _lib.mixer_mr_supported(op.group_dim, fused[0], conv.kernel_size, features)):
-            g, dg = op.num_groups, op.group_dim
-            assert d3 == 3 * g * dg
-            z = _FeaturizedDecayedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3),
-                                                     conv.short_conv_weight.to(features.dtype), op.filter.h,
-                                                     op.filter.decay, fused[0], fused[1])
+        g, dg = op.num_groups, op.group_dim
+        assert d3 == 3 * g * dg
+        planar = not self.interleave_projections
+        shape = (bs, seqlen, 3, g, dg) if planar else (bs, seqlen, g, dg, 3)
+        # Hyena-MR: one kernel each way, with the decayed filter formed inside it where the operator allows that
+        fused = op._filter_in_kernel(seqlen, g, dg, features.dtype, features)
+        if fused is not None and self._medium(features, fused[0]):
+            z = _FeaturizedDecayedGateConvGate.apply(features.reshape(shape), conv.short_conv_weight.to(features.dtype),
+                                                     op.filter.h, op.filter.decay, fused[0], fused[1], planar)
             return z.reshape(bs, seqlen, g * dg)
         h = op._filter(seqlen)
-        if (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and
-                _lib.mixer_mr_supported(op.group_dim, h.shape[-1], conv.kernel_size, features) and
-                (op.cgcg_dtype == features.dtype or op._fp32_inside(features.dtype, features))):
-            g, dg = op.num_groups, op.group_dim
-            assert d3 == 3 * g * dg
-            z = _FeaturizedGateConvGate.apply(features.reshape(bs, seqlen, g, dg, 3),
-                                              conv.short_conv_weight.to(features.dtype), h.to(op.cgcg_dtype))
+        if self._medium(features, h.shape[-1]):
+            z = _FeaturizedGateConvGate.apply(features.reshape(shape), conv.short_conv_weight.to(features.dtype),
+                                              h.to(op.cgcg_dtype), planar)
             return z.reshape(bs, seqlen, g * dg)
-        if not self._fusable(features, h.shape[-1]):
-            return op.forward_features(self.hyena_proj_conv.forward_bld(features, feeds_operator=True),
-                                       from_featurizer=True)
-        assert d3 == 3 * op.num_groups * op.group_dim
-        return self._fused_short(features, h, False)
+        # Hyena-SE: one kernel each way
+        if self._fusable(features, h.shape[-1]):
+            return self._fused_short(features, h, planar)
+        # otherwise the featurizer kernel, then the operator on its output where it lies (two kernels each way)
+        return op.forward_features(conv.forward_bld(features, feeds_operator=True), from_featurizer=True,
+                                   interleaved=not planar)
