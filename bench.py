@@ -117,7 +117,7 @@ class Op:
                 wf = (torch.randn(3 * wl.d, 1, 3, generator=torch.Generator().manual_seed(i)) / 3 ** 0.5)
                 t["raw"] = raw.contiguous().requires_grad_(True)
                 t["wf"] = wf.to(wl.dtype).to(device).requires_grad_(True)
-                t["h"] = t["h"].requires_grad_(True)
+                t["h"] = (t["h"].to(wl.filt_dtype) if wl.filt_dtype else t["h"]).requires_grad_(True)
             elif wl.layout == "planar":
                 t["feat"] = torch.stack([t.pop("v"), t.pop("q"), t.pop("k")], dim=2).contiguous()
             elif wl.layout != "separate":
@@ -656,7 +656,8 @@ def main():
         for name in ("mr_fwdbwd_7b_interleaved", "se_fwdbwd_40b_interleaved", "mr_fwdbwd_7b_planar", "se_fwdbwd_40b_planar",
                      "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b",
                      "mixer_fwdbwd_7b_fused", "mixer_fwdbwd_7b_fused_planar", "mixer_fwd_7b", "mixer_fwd_7b_fused",
-                     "mixer_se_fwdbwd_40b", "mixer_se_fwdbwd_40b_fused", "mixer_se_fwdbwd_40b_fused_planar"):
+                     "mixer_se_fwdbwd_40b", "mixer_se_fwdbwd_40b_fused", "mixer_se_fwdbwd_40b_fused_planar",
+                     "mixer_se_fwdbwd_40b_fp32_arith", "mixer_se_fwdbwd_40b_fused_fp32_arith"):
             r = time_workload(WORKLOADS[name], device, max(10, args.steps // 2), 4)
             extra[name] = {k: r[k] for k in ("ms_per_step", "tokens_per_s", "step_gbs", "step_hbm_frac")}
         line["next_rows"] = extra

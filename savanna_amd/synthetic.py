@@ -39,6 +39,9 @@ class Workload:
     # F.pad + F.conv1d, permute back, interleaved split, three gathers -- around the separate-tensor
     # kernels, with autograd doing the backward of the torch part.
     layout: str = "separate"
+    # the filter's dtype where it is not the tensors': float32 with 16-bit tensors = cgcg_dtype float32 on 16-bit
+    # activations (fp32 filter, arithmetic and filter gradient; hyena.py:499-503, :812-816)
+    filt_dtype: Optional[torch.dtype] = None
 
     @property
     def d(self) -> int:
@@ -141,6 +144,13 @@ WORKLOADS = {
     "mixer_se_fwdbwd_40b_fused": Workload("mixer_se_fwdbwd_40b_fused", 1, 32768, 512, 16, (7,), torch.bfloat16, True,
                                           "the same as one kernel each way (the featurized tensor stays in "
                                           "registers)", layout="mixer_fused"),
+    "mixer_se_fwdbwd_40b_fp32_arith": Workload("mixer_se_fwdbwd_40b_fp32_arith", 1, 32768, 512, 16, (7,), torch.bfloat16,
+                                               True, "the two-kernel chain with cgcg_dtype float32 on the bf16 features "
+                                               "(fp32 filter and arithmetic inside the operator's kernels)",
+                                               layout="mixer", filt_dtype=torch.float32),
+    "mixer_se_fwdbwd_40b_fused_fp32_arith": Workload("mixer_se_fwdbwd_40b_fused_fp32_arith", 1, 32768, 512, 16, (7,),
+                                                     torch.bfloat16, True, "the same as one kernel each way",
+                                                     layout="mixer_fused", filt_dtype=torch.float32),
     "mixer_se_fwdbwd_40b_fused_planar": Workload("mixer_se_fwdbwd_40b_fused_planar", 1, 32768, 512, 16, (7,),
                                                  torch.bfloat16, True,
                                                  "the same on planar features (interleave_projections = false): "
