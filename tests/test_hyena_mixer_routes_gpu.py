@@ -52,7 +52,7 @@ def test_every_route_gives_the_chains_values(gcg_lib, kind, planar, types, kf, d
     op_kind, hl = KINDS[kind]
     act, cgcg_name = TYPES[types]
     cgcg = getattr(torch, cgcg_name)
-    torch.manual_seed(hash((kind, planar, types, kf, dg)) & 0xffff)
+    torch.manual_seed(GRID.index((kind, planar, types, kf, dg)))       # the same values in every run
     bs, L, g = 2, 333, 6
     hidden = g * dg
     cfg = CgcgConfig(cgcg_dtype=cgcg_name)
