@@ -619,9 +619,16 @@ def _all_aligned16(tensors, skip_strided=False) -> bool:
     return True
 
 
-def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors) -> bool:
+# read once, as the library reads it
+_MIXER_MR_ONE_KERNEL = os.environ.get("GCG_MIXER_MR_FUSED", "1").strip() != "0"
+
+
+def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors, planar: bool = False) -> bool:
     """Whether gcg_mixer_mr_fwd / _bwd take these sizes (matrix-core kernels, filters of up to 128 taps
-    -- those of at most 8 are the fused Hyena-SE kernels' -- and a featurizer of at most 3)."""
+    -- those of at most 8 are the fused Hyena-SE kernels' -- and a featurizer of at most 3).  ``planar``: the
+    planar entry points, which exist in the one-kernel form only (the library's GCG_MIXER_MR_FUSED=0 switches it off)."""
+    if planar and not _MIXER_MR_ONE_KERNEL:
+        return False
     return 9 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and _all_aligned16(tensors)
 
 

@@ -425,7 +425,8 @@ class HyenaMixer(nn.Module):
         ("(p g dg)" rows) run in the one-kernel form only, which has 16-bit arithmetic."""
         conv, op = self.hyena_proj_conv, self.mixer
         if not (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and
-                _lib.mixer_mr_supported(op.group_dim, hl, conv.kernel_size, features)):
+                _lib.mixer_mr_supported(op.group_dim, hl, conv.kernel_size, features,
+                                        planar=not self.interleave_projections)):
             return False
         if self.interleave_projections:
             return op.cgcg_dtype == features.dtype or op._fp32_inside(features.dtype, features)
