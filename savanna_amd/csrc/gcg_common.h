@@ -110,7 +110,11 @@ constexpr int64_t WIN_MAX_BYTES = (1ll << 31) - (1ll << 27);
 #ifndef GCG_NT
 #define GCG_NT 3                                    // bit 0: loads, bit 1: stores
 #endif
+#if defined(GCG_LD_AUX) && defined(GCG_ST_AUX)      // tuning builds: the cache-policy bits spelled out (1 sc0, 2 nt, 16 sc1)
+constexpr int WIN_NT = GCG_LD_AUX, WIN_NT_ST = GCG_ST_AUX;
+#else
 constexpr int WIN_NT = (GCG_NT & 1) ? 2 : 0, WIN_NT_ST = (GCG_NT & 2) ? 2 : 0;   // cache policy "nt"
+#endif
 
 __device__ __forceinline__ win_t make_window(const void *base, int64_t bytes)
 {
@@ -168,6 +172,16 @@ __device__ __forceinline__ void win_store(win_t w, uint32_t off, const u32x4 &v)
 {
     __builtin_amdgcn_raw_buffer_store_b128(v, w, (int)off, 0, WIN_NT_ST);
 }
+// a 16-byte store with the cache-policy bits spelled out (1 sc0, 2 nt, 16 sc1), for the kernels that measured
+// a better one than the default
+template <int AUX> __device__ __forceinline__ void win_store_policy(win_t w, uint32_t off, const u32x4 &v)
+{
+    __builtin_amdgcn_raw_buffer_store_b128(v, w, (int)off, 0, AUX);
+}
+template <int AUX> __device__ __forceinline__ u32x4 win_load_policy(win_t w, uint32_t off)
+{
+    return __builtin_amdgcn_raw_buffer_load_b128(w, (int)off, 0, AUX);
+}
 // The same without the nontemporal hint, for an output the next kernel of a chain reads back at once
 // (the featurized tensor, the gradient of the features): stored through the cache it is still
 // partly there when that kernel starts.  A kernel timed alone loses a few percent this way, which
@@ -195,6 +209,14 @@ __device__ __forceinline__ int64_t xcd_contiguous_id(int64_t id, int64_t n)
 {
 #if GCG_XCD_SWIZZLE
     if ((n & 7) == 0) return (id & 7) * (n >> 3) + (id >> 3);
+#endif
+    return id;
+}
+// the same on 32-bit indices (launches of fewer than 2^31 workgroups)
+__device__ __forceinline__ uint32_t xcd_contiguous_u32(uint32_t id, uint32_t n)
+{
+#if GCG_XCD_SWIZZLE
+    if ((n & 7u) == 0) return (id & 7u) * (n >> 3) + (id >> 3);
 #endif
     return id;
 }

@@ -26,6 +26,43 @@
 namespace gcg {
 namespace {
 
+// Per-workgroup timestamps of the 100 MHz constant clock, for builds with -DGCG_TRACE only (`make trace`):
+// thread 0 of every workgroup stamps slot k of its 16 at the marked points of both kernels.  The stamp is a
+// store through a window that only thread 0's offset falls into, so that no branch is put between a load and its use.
+#ifdef GCG_TRACE
+constexpr int TRACE_WGS = 1 << 16, TRACE_SLOTS = 16;
+__device__ unsigned long long g_trace[(size_t)TRACE_WGS * TRACE_SLOTS];
+#define TR_INIT const win_t tr_win = make_window(g_trace + (size_t)(blockIdx.x < TRACE_WGS ? blockIdx.x : 0) * TRACE_SLOTS, TRACE_SLOTS * 8)
+#define TR(k) do { const unsigned long long t_ = wall_clock64(); \
+        __builtin_amdgcn_raw_buffer_store_b64(u32x2{(uint32_t)t_, (uint32_t)(t_ >> 32)}, tr_win, \
+                                              threadIdx.x == 0 ? (k) * 8 : (int)WIN_OFF, 0, 0); } while (0)
+#else
+#define TR_INIT do { } while (0)
+#define TR(k) do { } while (0)
+#endif
+
+// Cache policy of the output stores (tuning builds may override).  Measured at the 7B layer shape, against the
+// nontemporal hint alone (92.4 and 172.1 us): forward with device-scope stores (sc1: written through the XCD's L2,
+// no dirty lines left for the end of the kernel) 90.2 us, with both hints 92.8; backward with both 171.1, with sc1 alone 179.6.
+#ifndef GCG_MFMA_FWD_ST
+#define GCG_MFMA_FWD_ST 16
+#endif
+#ifndef GCG_MFMA_BWD_ST
+#define GCG_MFMA_BWD_ST WIN_NT_ST
+#endif
+#ifndef GCG_MFMA_BWD_ST_DC
+#define GCG_MFMA_BWD_ST_DC GCG_MFMA_BWD_ST
+#endif
+#ifndef GCG_MFMA_FWD_LD
+#define GCG_MFMA_FWD_LD WIN_NT
+#endif
+#ifndef GCG_MFMA_FWD_LEAD_LD
+#define GCG_MFMA_FWD_LEAD_LD WIN_NT
+#endif
+#ifndef GCG_MFMA_BWD_LD
+#define GCG_MFMA_BWD_LD WIN_NT
+#endif
+
 // ---------------------------------------------------------------------------- forward
 // EXTRA: also write the convolution before the post-gate (y2o) and the pre-gate product (bxo).
 // PL: x, B, C are the thirds of the rows of one (bs, L, 3 d) tensor (Dims::planar): their rows lie 3 d elements apart.
@@ -48,11 +85,12 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     __shared__ __attribute__((aligned(16))) unsigned char smem[OFF_U + (LDS_WALK > LDS_LEAD ? LDS_WALK : LDS_LEAD)];
     unsigned char *u_rm = smem + OFF_U, *y_st = smem + OFF_Y;
     hraw_t (*htab)[HTAB] = (hraw_t (*)[HTAB])smem;
+    TR_INIT;
+    TR(0);
 
-    int64_t wg = pl.xcd ? xcd_contiguous_id(blockIdx.x, gridDim.x) : (int64_t)blockIdx.x;
-    const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
-    const int seg = (int)(wg % pl.nseg);
-    const int64_t b = wg / pl.nseg;
+    int cb, seg, bi;
+    wg_place(pl.xcd ? xcd_contiguous_u32(blockIdx.x, gridDim.x) : blockIdx.x, pl, cb, seg, bi);
+    const int64_t b = bi;
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
     const int r = tid / G::LPR, a = tid % G::LPR;   // row layout: row r of the step, channels 8a..8a+7
@@ -90,7 +128,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
     // order of issue, so taps requested after the rows would arrive after all of them).
     // htab[lag + 32] = h[hl-1-lag] for 0 <= lag < hl, else 0.
     hraw_t hv[HTAB / 64];
-    load_taps<T>(dm, h, (c0 + 16 * w < d) ? (c0 + 16 * w) / dm.dg : 0, l, hv);
+    load_taps<T>(dm, h, (c0 + 16 * w < d) ? fdiv((uint32_t)(cb * NW + w), pl.q_dg16) : 0, l, hv);
 
     // The operands of the NK-1 steps before the segment are rebuilt first (zero before the
     // start of the sequence).  Their rows are requested together, so the replay costs one
@@ -102,27 +140,30 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
             const uint32_t o = lane_in + IM * step_off(s_lo - i);
-            lx[i - 1] = ldw_row<T>(wx, o);
-            lB[i - 1] = ldw_row<T>(wB, o);
+            lx[i - 1] = ldw_row_policy<T, GCG_MFMA_FWD_LEAD_LD>(wx, o);
+            lB[i - 1] = ldw_row_policy<T, GCG_MFMA_FWD_LEAD_LD>(wB, o);
         }
     }
     Row<T> xr, Br, Cr;
     auto fetch = [&](int64_t s, Row<T> &xo, Row<T> &Bo, Row<T> &Co) {
         const uint32_t o = lane_in + IM * step_off(s);
-        xo = ldw_row<T>(wx, o);
-        Bo = ldw_row<T>(wB, o);
-        Co = ldw_row<T>(wC, o);
+        xo = ldw_row_policy<T, GCG_MFMA_FWD_LD>(wx, o);
+        Bo = ldw_row_policy<T, GCG_MFMA_FWD_LD>(wB, o);
+        Co = ldw_row_policy<T, GCG_MFMA_FWD_LD>(wC, o);
     };
     fetch(s_lo, xr, Br, Cr);
+    TR(1);
 
     store_taps(htab[w], l, hv);
     __syncthreads();
+    TR(2);
     typename M::wop_t W0[NK], W1[NK];   // output rows 0..15 / 16..31 of the step against input step s-i
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
         W0[i] = M::toeplitz(htab[w], 32 * i, j, q);
         W1[i] = M::toeplitz(htab[w], 32 * i + 16, j, q);
     }
+    TR(3);
 
     if constexpr (NK > 1) {
         // all lead-in tiles go to LDS together: one pair of barriers instead of NK-1
@@ -136,11 +177,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
             store_operand<T>(u_wr + (i - 1) * STEP * UROW, UROW, uf);
         }
         __syncthreads();
+        TR(4);
 #pragma unroll
         for (int i = 1; i < NK; ++i) A[NK - i] = M::load_operand(u_rm + (i - 1) * STEP * UROW, UROW, w, j, q, false);
         __syncthreads();
     }
 
+    TR(5);
     int64_t s = s_lo;
     while (s < s_hi) {
 #pragma unroll
@@ -179,7 +222,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                     unpack8<T>(Cr, Cf);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) yf[e] = Cf[e] * y2f[e];
-                    stw_row<T>(wy, o, pack8<T>(yf));
+                    stw_row_policy<T, GCG_MFMA_FWD_ST>(wy, o, pack8<T>(yf));
                     if constexpr (EXTRA) stw_row<T>(wy2, o, pack8<T>(y2f));
                 }
                 xr = xn; Br = Bn; Cr = Cn;
@@ -187,6 +230,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
             }
         }
     }
+    TR(6);
 }
 
 // --------------------------------------------------------------------------- backward
@@ -229,7 +273,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     constexpr int OFF_D = OFF_Y + STEP * YROW;              // du tile, fp32, row-major
     constexpr int OFF_H = OFF_D + STEP * YROW;              // filter tables
     constexpr int LDS_MAIN = OFF_H + NW * HTAB * (int)sizeof(hraw_t);
-    constexpr int LDS_TAIL = NW * ND * 256 * 4;             // P tiles at the end
+    constexpr int LDS_TAIL = NW * (16 * ND + 16) * 17 * 4;  // P tiles at the end (dh_finish)
     // A 4-wave workgroup at 16 bits asks for more than half of the CU's 160 KB, so that a CU holds one
     // (two on a CU, two waves per SIMD, are a third slower than one).
     constexpr int LDS_NEED = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
@@ -238,12 +282,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
     unsigned char *u_rm = smem + OFF_U, *g_rm = smem + OFF_G, *y_st = smem + OFF_Y, *d_st = smem + OFF_D;
     hraw_t *htab = (hraw_t *)(smem + OFF_H);
+    TR_INIT;
+    TR(0);
 
-    const int64_t wg_id = xcd_contiguous_id(blockIdx.x, gridDim.x);
-    int64_t wg = wg_id;
-    const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
-    const int seg = (int)(wg % pl.nseg);
-    const int64_t b = wg / pl.nseg;
+    const uint32_t wg_id = xcd_contiguous_u32(blockIdx.x, gridDim.x);
+    int cb, seg, bi;
+    wg_place(wg_id, pl, cb, seg, bi);
+    const int64_t b = bi;
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
     const int r = tid / G::LPR, a = tid % G::LPR;   // row layout: row r of the step, channels 8a..8a+7
@@ -295,15 +340,15 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     // The filter taps of this wave's group are requested before any row, so that the filter table
     // and the Toeplitz tiles are built while the rows are in flight (loads complete in order of issue).
     hraw_t hv[HTAB / 64];
-    load_taps<T>(dm, h, wave_valid ? (c0 + 16 * w) / dm.dg : 0, l, hv);
+    load_taps<T>(dm, h, wave_valid ? fdiv((uint32_t)(cb * NW + w), pl.q_dg16) : 0, l, hv);
 
     // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the windows)
     auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
         const uint32_t o = lane_in + IM * step_off(sg), o2 = lane_off + step_off(sg + NK - 1);
-        xo = ldw_row<T>(wx, o);
-        Bo = ldw_row<T>(wB, o);
-        dyo = ldw_row<T>(wdy, o2);
-        Co = ldw_row<T>(wC, PL ? lane_in + IM * step_off(sg + NK - 1) : o2);
+        xo = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wx, o);
+        Bo = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wB, o);
+        dyo = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wdy, o2);
+        Co = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wC, PL ? lane_in + IM * step_off(sg + NK - 1) : o2);
     };
 
     // Lead-in: u of the NK-1 steps before the segment and g2 of its first NK-1 steps, i.e. the
@@ -318,15 +363,18 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     }
     Row<T> xr, Br, dyr, Cr;
     fetch(s_lo, xr, Br, dyr, Cr);
+    TR(1);
 
     store_taps(htab + w * HTAB, l, hv);
     __syncthreads();
+    TR(2);
     typename M::wop_t W0[NK], W1[NK];
 #pragma unroll
     for (int i = 0; i < NK; ++i) {
         W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
         W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
     }
+    TR(3);
 
     if constexpr (NK > 1) {
 #pragma unroll
@@ -352,6 +400,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         }
     }
 
+    TR(5);
     int64_t s = s_lo;
     while (s < s_hi) {
 #pragma unroll
@@ -415,7 +464,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         unpack8<T>(dyq[ph], dyf);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = dyf[e] * y2f[e];
-                        stw_row<T>(wdC, o, pack8<T>(of));
+                        stw_row_policy<T, GCG_MFMA_BWD_ST_DC>(wdC, o, pack8<T>(of));
                     }
                     {
                         const f32x4 p0 = *(const f32x4 *)d_rd;
@@ -424,10 +473,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         float of[8];
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * Bf[e];
-                        stw_row<T>(wdx, o, pack8<T>(of));
+                        stw_row_policy<T, GCG_MFMA_BWD_ST>(wdx, o, pack8<T>(of));
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * xf[e];
-                        stw_row<T>(wdB, o, pack8<T>(of));
+                        stw_row_policy<T, GCG_MFMA_BWD_ST>(wdB, o, pack8<T>(of));
                     }
                 }
                 xr = xn; Br = Bn; dyr = dyn; Cr = Cn;
@@ -436,7 +485,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         }
     }
 
+    TR(6);
     dh_finish<T, NW, ND>(P, smem, ws, dh, dm, pl, wg_id, cb, wave_valid);
+    TR(7);
 }
 
 template <typename T, int NK, int NW>
@@ -517,6 +568,19 @@ int mfma_fwd_launch(int dtype, const void *x, const void *B, const void *C, cons
 
 bool mfma_bwd_available() { return true; }
 
+#ifdef GCG_TRACE
+} // namespace gcg
+// trace builds only: device address and size of the timestamp table (16 slots of 8 bytes per workgroup)
+extern "C" GCG_API void *gcg_trace_buffer(size_t *bytes)
+{
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(gcg::g_trace)) != hipSuccess) return nullptr;
+    if (bytes) *bytes = sizeof(gcg::g_trace);
+    return p;
+}
+namespace gcg {
+#endif
+
 namespace {
 
 
@@ -527,7 +591,7 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
     int e = 0;
     MfmaPlan p = plan_bwd(dm, MT<T>::SPLIT, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    if (p.fuse_dh) p.slot = next_dh_slot();
+    if (p.fuse_dh && (p.slot = dh_slot_for_stream(st)) < 0) p.fuse_dh = p.slot = 0;   // no ticket set: second launch
     bool launched = false;
     if constexpr (NK == 5) {
         if (dm.planar) {        // instantiated for the five-slice walk only (bwd_t sends every filter length there)

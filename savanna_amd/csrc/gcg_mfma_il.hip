@@ -217,7 +217,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     constexpr int XB_VEC = G::NT * 16 * M::RW;              // one row vector of every lane
     constexpr int XB_BYTES = XB_SLOTS * 2 * XB_VEC, H_BYTES = NW * HTAB * (int)sizeof(hraw_t);
     constexpr int LDS_MAIN = OFF_XB + (XB_BYTES > H_BYTES ? XB_BYTES : H_BYTES);
-    constexpr int LDS_TAIL = NW * ND * 256 * 4;             // P tiles at the end
+    constexpr int LDS_TAIL = NW * (16 * ND + 16) * 17 * 4;  // P tiles at the end (dh_finish)
     // a 4-wave workgroup at 16 bits asks for more than half of the CU's 160 KB, so that a CU holds one
     constexpr int LDS_NEED = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
     constexpr int LDS_ALONE = (NW == 4 && M::ES == 2) ? 82 * 1024 : 0;
@@ -542,7 +542,7 @@ int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, voi
     int e = 0;
     MfmaPlan p = plan_bwd(dm, MT<T>::SPLIT, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    if (p.fuse_dh) p.slot = next_dh_slot();
+    if (p.fuse_dh && (p.slot = dh_slot_for_stream(st)) < 0) p.fuse_dh = p.slot = 0;   // no ticket set: second launch
     if (dm.keep_out)
         e = launch_main((mfma_il_bwd_kernel<T, NK, NW, true, 0>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)dy, (const T *)feat, (const T *)h, (const T *)nullptr, 0, (T *)dfeat, (T *)dh,
@@ -578,7 +578,7 @@ int bwd_feat_t(const void *dy, const void *raw, const void *wfeat, int kf, const
 {
     MfmaPlan p = plan_bwd_nw(dm, choose_nw_bwd_feat(MT<T>::SPLIT), MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    if (p.fuse_dh) p.slot = next_dh_slot();
+    if (p.fuse_dh && (p.slot = dh_slot_for_stream(st)) < 0) p.fuse_dh = p.slot = 0;   // no ticket set: second launch
     if constexpr (!MT<T>::SPLIT) {
         if (p.nw == 8) return bwd_feat_launch<T, 8>(dy, raw, wfeat, kf, h, dfeat, dh, ws, dm, p, st);
     }

@@ -7,6 +7,7 @@
 
 #include <atomic>
 #include <cstdlib>
+#include <mutex>
 
 namespace gcg {
 namespace {
@@ -375,6 +376,23 @@ template <typename T> __device__ __forceinline__ void stw_row(win_t w, uint32_t 
 #pragma unroll
     for (int i = 0; i < MT<T>::RW; ++i) stw16(w, off + 16 * i, r.w[i]);
 }
+template <typename T, int AUX> __device__ __forceinline__ Row<T> ldw_row_policy(win_t w, uint32_t off)
+{
+    Row<T> r;
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i) {
+        const u32x4 v = win_load_policy<AUX>(w, off + 16 * i);
+        r.w[i] = make_uint4(v[0], v[1], v[2], v[3]);
+    }
+    return r;
+}
+// the same with the store's cache-policy bits given (gcg_common.h: win_store_policy)
+template <typename T, int AUX> __device__ __forceinline__ void stw_row_policy(win_t w, uint32_t off, const Row<T> &r)
+{
+#pragma unroll
+    for (int i = 0; i < MT<T>::RW; ++i)
+        win_store_policy<AUX>(w, off + 16 * i, u32x4{r.w[i].x, r.w[i].y, r.w[i].z, r.w[i].w});
+}
 
 // The filter table of a wave's group: tab[lag + HPAD] = h[hl-1-lag] for 0 <= lag < hl, else 0; lane l
 // holds entries l, l + 64, l + 128 between load_taps and store_taps.  The taps come from h, or -- decayed
@@ -422,7 +440,39 @@ template <typename T> __device__ __forceinline__ void store_dh(void *dh, const D
     else Elem<F>::store((F *)dh + grp * dm.hl + k, sum);
 }
 
-struct MfmaPlan { int ncb, nseg, steps_per_seg, nw, xcd; int64_t nsteps, nwg; int fuse_dh, slot; };
+// Exact division of a number below 2^31 by a launch constant d: n / d = (n * mul) >> sh, with
+// sh = 31 + ceil(log2 d) and mul = ceil(2^sh / d) < 2^32 (the error n * (mul * d - 2^sh) / (d * 2^sh) stays
+// below 1 / d because n * d <= 2^sh).  A workgroup finds its place in the launch with two of these instead of
+// 64-bit divisions: with sixteen waves per CU sharing one scalar unit those took over a microsecond before
+// the first load went out.
+struct FastDiv { uint32_t mul, sh; };
+inline FastDiv make_fastdiv(uint32_t d)
+{
+    int l = 0;
+    while ((1ull << l) < d) ++l;
+    FastDiv f;
+    f.sh = 31u + (uint32_t)l;
+    f.mul = (uint32_t)(((1ull << f.sh) + d - 1) / d);
+    return f;
+}
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, FastDiv f) { return (uint32_t)(((uint64_t)n * f.mul) >> f.sh); }
+
+struct MfmaPlan {
+    int ncb, nseg, steps_per_seg, nw, xcd;
+    int64_t nsteps, nwg;
+    int fuse_dh, slot;
+    FastDiv q_ncb, q_nseg, q_dg16;      // divisions by ncb, nseg and dg / 16
+};
+
+// (channel block, segment, batch row) of a workgroup from its index in the launch (below 2^31)
+__device__ __forceinline__ void wg_place(uint32_t id, const MfmaPlan &pl, int &cb, int &seg, int &b)
+{
+    const uint32_t t = fdiv(id, pl.q_ncb);
+    cb = (int)(id - t * (uint32_t)pl.ncb);
+    const uint32_t bq = fdiv(t, pl.q_nseg);
+    seg = (int)(t - bq * (uint32_t)pl.nseg);
+    b = (int)bq;
+}
 
 // Operand tile of the banded Toeplitz matrix at row offset doff = (out time) - (in time) of the
 // tile origins: element e of lane (j, q) is the tap for lag doff + j - kmap(q, e)  (MT<T>::toeplitz).
@@ -458,85 +508,156 @@ __global__ __launch_bounds__(256) void mfma_dh_reduce_kernel(const float *__rest
 // partials of its channel block, in the same fixed order whoever that is, so dh stays
 // bit-reproducible.  "Last" is decided by a ticket per channel block.  The tickets live in the
 // library image (zero when the code is loaded; the last arrival puts its ticket back to zero), in
-// DH_SLOTS sets that launches take in turn, so that launches which run at the same time on
-// different streams do not share one: a GPU executes at most one kernel per hardware queue at a
-// time and a process has at most 32 of those.
+// DH_SLOTS sets.  A set belongs to a stream (dh_slot_for_stream): launches on one stream run one
+// after the other, so two launches that may run at the same time never count on the same tickets.
 //
-// Visibility across the XCDs' separate L2 caches comes from the accesses themselves, not from
-// fences: partials are written and read with device-scope atomic stores and loads, which go
-// through to memory, and a workgroup takes its ticket only after its own partials have completed.
-// A device-scope fence instead writes back and invalidates the whole L2 of the XCD, and one per
-// workgroup cost 45 us at the end of a 175 us kernel.
+// Ordering, in the terms of the AMDGPU memory model for gfx942 / gfx950 (several XCDs, each with an L2 of its own):
+//  * partials are written with device-scope atomic stores (sc1): they are written through the XCD's L2, and the
+//    store's vmcnt slot is released only when that write has been acknowledged;
+//  * every wave then waits for vmcnt(0) -- all of its stores, the partials among them, have completed -- and the
+//    workgroup meets at a barrier: only after that does thread 0 take the ticket with a device-scope atomic add
+//    (performed where all XCDs see it).  So a workgroup that reads `arrivals` from the ticket knows that every
+//    partial of its channel block is in memory;
+//  * that workgroup invalidates what its own caches may hold (acquire fence at device scope) and reads the
+//    partials with device-scope atomic loads, which are served from beyond the XCD's L2.
+// A device-scope release fence instead (the textbook form) writes back the XCD's whole L2, dirty output rows
+// included: one per workgroup cost 45 us at the end of a 175 us kernel.
 constexpr int DH_SLOTS = 64, DH_UNITS = 1024;
 static __device__ unsigned int dh_tickets[DH_SLOTS * DH_UNITS];
 
-int next_dh_slot()
+// The ticket set of a stream, or -1 when DH_SLOTS other streams already hold one each (the caller then adds the
+// partials with a second launch), or when the stream is being captured into a graph (a replayed launch keeps the
+// set it was recorded with and would count on it whatever stream it is replayed on).
+int dh_slot_for_stream(hipStream_t st)
 {
-    static std::atomic<unsigned> n{0};
-    return (int)(n.fetch_add(1, std::memory_order_relaxed) % DH_SLOTS);
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) return -1;
+    static std::mutex mu;
+    static hipStream_t owner[DH_SLOTS];
+    static int used = 0;
+    std::lock_guard<std::mutex> lk(mu);
+    for (int i = 0; i < used; ++i)
+        if (owner[i] == st) return i;
+    if (used == DH_SLOTS) return -1;
+    owner[used] = st;
+    return used++;
+}
+
+// Arrival of a workgroup at the ticket of its channel block, after every wave has issued its partial stores.
+// Returns true in the one workgroup that arrives last (uniformly over its threads).
+__device__ __forceinline__ bool dh_arrive_last(const MfmaPlan &pl, int cb, unsigned int arrivals)
+{
+    __shared__ unsigned int is_last;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");         // this wave's stores have been acknowledged ...
+    __syncthreads();                                         // ... and so have the other waves', before the ticket is taken
+    if (threadIdx.x == 0) {
+        unsigned int *tk = dh_tickets + pl.slot * DH_UNITS + cb;
+        const unsigned int mine = __hip_atomic_fetch_add(tk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+        is_last = (mine == arrivals);
+        if (mine == arrivals) __hip_atomic_store(tk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!is_last) return false;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    return true;
+}
+
+// Sums of n partials `stride` floats apart, in index order, for two outputs at once; sixteen reads are in flight
+// together, so that the sums cost one memory latency per eight terms rather than one per term.
+__device__ __forceinline__ void dh_sum_partials2(const float *pa, const float *pb, int64_t stride, int64_t n, float &sa,
+                                                 float &sb)
+{
+    sa = sb = 0.f;
+    for (int64_t i0 = 0; i0 < n; i0 += 8) {
+        float va[8], vb[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const bool in = i0 + u < n;
+            va[u] = __hip_atomic_load(pa + (in ? (i0 + u) * stride : 0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            vb[u] = __hip_atomic_load(pb + (in ? (i0 + u) * stride : 0), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            va[u] = in ? va[u] : 0.f;
+            vb[u] = in ? vb[u] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            sa += va[u];
+            sb += vb[u];
+        }
+    }
 }
 
 // Tail of both backward kernels.  P: the wave's ND accumulator tiles, P[dl][v] = element
-// (row 4q+v, column j) of tile dl; smem: at least NW*ND*1 KB of LDS that is no longer in use.
+// (row 4q+v, column j) of tile dl; smem: at least NW*(16*ND+16)*17*4 bytes of LDS that is no longer in use.
 template <typename T, int NW, int ND>
 __device__ __forceinline__ void dh_finish(const f32x4 (&P)[ND], unsigned char *smem, float *__restrict__ ws,
                                           T *__restrict__ dh, const Dims &dm, const MfmaPlan &pl, int64_t wg_id,
                                           int cb, bool wave_valid)
 {
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, j = l & 15, q = l >> 4;
-    // diagonal sums of the P tiles -> per-wave partials, lag = 16*tile + row - column
+    // The tiles go to LDS one below the other, as one matrix of 16*ND rows (17 floats apart: the diagonal walks
+    // below then touch every bank once) followed by 16 rows of zeros.  lag = (row of the matrix) - column, so the
+    // partial for a lag is the sum over columns c of element (lag + c, c).
+    constexpr int RS = 17, ROWS = 16 * ND + 16;
     __syncthreads();
-    float *pt = (float *)smem + w * ND * 256;
+    float *pt = (float *)smem + w * ROWS * RS;
 #pragma unroll
     for (int dl = 0; dl < ND; ++dl)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) pt[dl * 256 + (4 * q + v) * 16 + j] = P[dl][v];
+        for (int v = 0; v < 4; ++v) pt[(16 * dl + 4 * q + v) * RS + j] = P[dl][v];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) pt[(16 * ND + 4 * q + v) * RS + j] = 0.f;
     __syncthreads();
     if (wave_valid) {
         float *out = ws + ((size_t)wg_id * NW + w) * 128;
-        for (int lag = l; lag < 128; lag += 64) {
-            const int d0 = lag >> 4, rr = lag & 15;
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int lag = l + 64 * half;
+            const float *d = pt + (lag < 16 * ND ? lag : 16 * ND) * RS;   // lags beyond the tiles: the rows of zeros
             float sum = 0.f;
-            if (d0 < ND)
-                for (int jj = 0; jj + rr < 16; ++jj) sum += pt[d0 * 256 + (jj + rr) * 16 + jj];
-            if (d0 + 1 < ND)
-                for (int ii = 0; ii < rr; ++ii) sum += pt[(d0 + 1) * 256 + ii * 16 + ii + 16 - rr];
+#pragma unroll
+            for (int c = 0; c < 16; ++c) sum += d[c * (RS + 1)];
             __hip_atomic_store(out + lag, sum, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     if (!pl.fuse_dh) return;       // a second launch adds the partials
 
-    __shared__ unsigned int is_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // every wave's partials have completed ...
-    __syncthreads();                                         // ... before thread 0 takes the ticket
-    if (tid == 0) {
-        unsigned int *tk = dh_tickets + pl.slot * DH_UNITS + cb;
-        const unsigned int arrivals = (unsigned int)(dm.bs * pl.nseg);
-        const unsigned int mine = atomicAdd(tk, 1u) + 1u;
-        is_last = (mine == arrivals);
-        if (mine == arrivals) __hip_atomic_store(tk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!is_last) return;
-    constexpr int CB = 16 * NW;
-    const int gpc = CB / dm.dg, bpg = dm.dg / 16;      // filter groups per channel block, 16-channel blocks per group
     const int64_t np = dm.bs * pl.nseg;
+    if (!dh_arrive_last(pl, cb, (unsigned int)np)) return;
+    constexpr int CB = 16 * NW, NT = 64 * NW;
+    const int gpc = CB / dm.dg, bpg = dm.dg / 16;      // filter groups per channel block, 16-channel blocks per group
     const int row = dm.fw ? dm.lc : dm.hl;              // taps per group in the output
-    for (int idx = tid; idx < gpc * row; idx += 64 * NW) {
-        const int gl = idx / row, k = idx % row;
-        const int64_t grp = (int64_t)cb * gpc + gl;
-        if (grp >= dm.g) continue;
-        if (k >= dm.hl) {                                // the parameter's taps beyond the filter in use
-            ((float *)dh)[grp * row + k] = 0.f;
-            continue;
+    // a thread takes outputs idx and idx + NT of the block's gpc * row together (one memory latency for both)
+    for (int idx0 = tid; idx0 < gpc * row; idx0 += 2 * NT) {
+        int gl[2], k[2];
+        bool live[2], tap[2];
+        const float *src[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int idx = idx0 + e * NT;
+            gl[e] = 0;
+            while (gl[e] + 1 < gpc && idx >= (gl[e] + 1) * row) ++gl[e];
+            k[e] = idx - gl[e] * row;
+            live[e] = idx < gpc * row && (int64_t)cb * gpc + gl[e] < dm.g;
+            tap[e] = live[e] && k[e] < dm.hl;             // else: the parameter's taps beyond the filter in use
+            // partial (p, kk) lies at ((p * ncb + cb) * NW + gl * bpg + kk) * 128 + lag
+            src[e] = ws + ((int64_t)cb * NW + (tap[e] ? gl[e] * bpg : 0)) * 128 + (tap[e] ? dm.hl - 1 - k[e] : 0);
         }
-        const int lag = dm.hl - 1 - k;
-        float sum = 0.f;
-        for (int64_t p = 0; p < np; ++p)
-            for (int kk = 0; kk < bpg; ++kk)
-                sum += __hip_atomic_load(ws + ((p * pl.ncb + cb) * NW + gl * bpg + kk) * 128 + lag, __ATOMIC_RELAXED,
-                                         __HIP_MEMORY_SCOPE_AGENT);
-        store_dh<T>(dh, dm, grp, k, sum);
+        float sum[2] = {0.f, 0.f};
+        if (bpg == 1) {
+            dh_sum_partials2(src[0], src[1], (int64_t)pl.ncb * NW * 128, np, sum[0], sum[1]);
+        } else {                                          // p-major, as the second launch adds them
+            for (int64_t p = 0; p < np; ++p)
+                for (int kk = 0; kk < bpg; ++kk)
+#pragma unroll
+                    for (int e = 0; e < 2; ++e)
+                        sum[e] += __hip_atomic_load(src[e] + (p * pl.ncb * NW + kk) * 128, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int64_t grp = (int64_t)cb * gpc + gl[e];
+            if (tap[e]) store_dh<T>(dh, dm, grp, k[e], sum[e]);
+            else if (live[e]) ((float *)dh)[grp * row + k[e]] = 0.f;
+        }
     }
 }
 
@@ -616,6 +737,9 @@ MfmaPlan plan(const Dims &dm, int nw, int min_steps, int waves_per_cu, int elem_
     p.xcd = 1;
     p.fuse_dh = 0;
     p.slot = 0;
+    p.q_ncb = make_fastdiv((uint32_t)p.ncb);
+    p.q_nseg = make_fastdiv((uint32_t)p.nseg);
+    p.q_dg16 = make_fastdiv((uint32_t)(dm.dg >= 16 ? dm.dg / 16 : 1));
     return p;
 }
 

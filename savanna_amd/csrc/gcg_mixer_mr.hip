@@ -249,18 +249,7 @@ __device__ __forceinline__ void mixer_bwd_finish(const float *ws, const float *w
     typedef MixGeo<T> G;
     if (!pl.fuse_dh) return;
     const int tid = threadIdx.x;
-    __shared__ unsigned int is_last;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // every wave's partials have completed ...
-    __syncthreads();                                         // ... before thread 0 takes the ticket
-    if (tid == 0) {
-        unsigned int *tk = dh_tickets + pl.slot * DH_UNITS + cb;
-        const unsigned int arrivals = (unsigned int)(dm.bs * pl.nseg);
-        const unsigned int mine = atomicAdd(tk, 1u) + 1u;
-        is_last = (mine == arrivals);
-        if (mine == arrivals) __hip_atomic_store(tk, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!is_last) return;
+    if (!dh_arrive_last(pl, cb, (unsigned int)(dm.bs * pl.nseg))) return;
     const int64_t np = dm.bs * pl.nseg;
     {
         const int gpc = G::CB / dm.dg, bpg = dm.dg / 16;   // filter groups per channel block, 16-channel blocks per group
@@ -947,7 +936,7 @@ int bwd_t(const void *dy, const void *raw, const void *wfeat, int kf, const void
     typedef MixGeo<T> G;
     MfmaPlan p = mixer_plan(dm);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
-    if (p.fuse_dh) p.slot = next_dh_slot();
+    if (p.fuse_dh && (p.slot = dh_slot_for_stream(st)) < 0) p.fuse_dh = p.slot = 0;   // no ticket set: second launches
     float *ws_dh = (float *)ws;
     float *ws_f = ws_dh + (size_t)p.nwg * G::XW * 128;
     int e = dm.planar
