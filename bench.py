@@ -282,10 +282,12 @@ def time_workload(wl, device, steps, warmup, graph=False):
         for op in ops:
             op.run()
     torch.cuda.synchronize()
-    # A step that carries events costs 10-15 us more than a plain one (two event records, and a timed launch is
-    # more than a kernel packet), so only a few steps of the timed region carry them; the same instrumented step
-    # is then repeated after the timed region for a steadier mean.  Both sample sets are reported.
-    n_in = min(4, steps)
+    # Instrumented steps cost time themselves: a launch that carries a pair of kernel events about 5 us, a bracket
+    # of torch events around the call about 9 us more (measured at the headline shape).  So inside the timed region
+    # two steps carry kernel events only (workloads whose dominant call is one library launch), or the bracket where
+    # the bracket is the measurement (whole-op workloads); the instrumented step is then repeated after the timed
+    # region, with both kinds of events, for a steadier mean.  Both sample sets are reported.
+    n_in = min(2, steps)
     marks = {(steps * (2 * j + 1)) // (2 * n_in): j for j in range(n_in)}       # spread over the region, not step 0
     n_after = min(16, max(4, steps))
     nsamp = n_in + n_after
@@ -297,7 +299,7 @@ def time_workload(wl, device, steps, warmup, graph=False):
         j = marks.get(k)
         for i, op in enumerate(ops):
             if i == dom and j is not None:
-                op.run(events[j], kevents.pairs[j] if kevents else None)
+                op.run(None if kevents else events[j], kevents.pairs[j] if kevents else None)
             else:
                 op.run()
     torch.cuda.synchronize()
@@ -310,7 +312,8 @@ def time_workload(wl, device, steps, warmup, graph=False):
             else:
                 op.run()
     torch.cuda.synchronize()
-    call_ms = sum(a.elapsed_time(b) for a, b in events) / nsamp      # bracket around the whole entry point
+    bracketed = events[n_in:] if kevents else events
+    call_ms = sum(a.elapsed_time(b) for a, b in bracketed) / len(bracketed)   # bracket around the whole entry point
     kern_ms = kevents.mean_ms() if kevents else None                 # the main kernel alone
     kern_ms_in = kevents.mean_ms(range(n_in)) if kevents else None
     if kevents:
