@@ -520,6 +520,7 @@ def power_table(device, secs=2.0):
         x, B, C = (torch.randn(bs, L, g, dg, generator=gen, device=device).to(torch.bfloat16) for _ in range(3))
         h = (torch.randn(g, 1, 128, generator=gen, device=device) / 128 ** 0.5).to(torch.bfloat16)
         hs = (torch.randn(g, 1, 7, generator=gen, device=device) / 7 ** 0.5).to(torch.bfloat16)
+        hf = h.float()                                    # fp32 filter: fp32 arithmetic on the bf16 tensors
         wf = (torch.randn(3 * g * dg, 1, 3, generator=gen, device=device) / 3 ** 0.5).to(torch.bfloat16)
         calls = (
             ("gcg_fwd hl=128", lambda s: _lib.fwd(x, B, C, h)),
@@ -529,6 +530,8 @@ def power_table(device, secs=2.0):
             ("gcg_mixer_mr_fwd", lambda s: _lib.mixer_mr_fwd(s[0], wf, h)),
             ("gcg_mixer_mr_bwd", lambda s: _lib.mixer_mr_bwd(s[1], s[0], wf, h)),
             ("gcg_bwd hl=7", lambda s: _lib.bwd(s[1], x, B, C, hs)),
+            ("gcg_fwd hl=128, fp32 arithmetic", lambda s: _lib.fwd(x, B, C, hf)),
+            ("gcg_bwd hl=128, fp32 arithmetic", lambda s: _lib.bwd(s[1], x, B, C, hf)),
         )
         for name, fn in calls:
             torch.cuda.synchronize()

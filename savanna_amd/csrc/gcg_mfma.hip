@@ -33,17 +33,26 @@ namespace {
 constexpr int TRACE_WGS = 1 << 16, TRACE_SLOTS = 16;
 __device__ unsigned long long g_trace[(size_t)TRACE_WGS * TRACE_SLOTS];
 #define TR_INIT const win_t tr_win = make_window(g_trace + (size_t)(blockIdx.x < TRACE_WGS ? blockIdx.x : 0) * TRACE_SLOTS, TRACE_SLOTS * 8)
-#define TR(k) do { const unsigned long long t_ = wall_clock64(); \
+// -DGCG_TRACE=1: start, walk start, walk end and end only (the forward is sensitive to more); =2: every mark
+#define TR(k) do { if (GCG_TRACE >= 2 || (k) == 0 || (k) == 5 || (k) == 6 || (k) == 7) { const unsigned long long t_ = wall_clock64(); \
         __builtin_amdgcn_raw_buffer_store_b64(u32x2{(uint32_t)t_, (uint32_t)(t_ >> 32)}, tr_win, \
-                                              threadIdx.x == 0 ? (k) * 8 : (int)WIN_OFF, 0, 0); } while (0)
+                                              threadIdx.x == 0 ? (k) * 8 : (int)WIN_OFF, 0, 0); } } while (0)
+// a stamp in slot k on the iteration for which `cond` holds (no branch: the other iterations' offsets miss the window)
+#define TR_IF(cond, k) do { if (GCG_TRACE >= 2) { const unsigned long long t_ = wall_clock64(); \
+        __builtin_amdgcn_raw_buffer_store_b64(u32x2{(uint32_t)t_, (uint32_t)(t_ >> 32)}, tr_win, \
+                                              (threadIdx.x == 0 && (cond)) ? (k) * 8 : (int)WIN_OFF, 0, 0); } } while (0)
 #else
 #define TR_INIT do { } while (0)
 #define TR(k) do { } while (0)
+#define TR_IF(cond, k) do { } while (0)
 #endif
 
 // Cache policy of the output stores (tuning builds may override).  Measured at the 7B layer shape, against the
 // nontemporal hint alone (92.4 and 172.1 us): forward with device-scope stores (sc1: written through the XCD's L2,
-// no dirty lines left for the end of the kernel) 90.2 us, with both hints 92.8; backward with both 171.1, with sc1 alone 179.6.
+// no dirty lines left for the end of the kernel) 90.2 us on 16-bit tensors (89.9 - 90.1 where the output buffer is the
+// same from call to call, 1 - 1.5 us less than the hint alone where it is not), with both hints 92.8; fp32 tensors
+// lose with it (212 -> 260 us) and keep the hint.  Backward: both hints 171.1 or 176.1 by the box, sc1 alone 179.6; the
+// hint alone stays.
 #ifndef GCG_MFMA_FWD_ST
 #define GCG_MFMA_FWD_ST 16
 #endif
@@ -189,6 +198,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
+                TR_IF(4 * (s - s_lo) == (s_hi - s_lo), 8);
+                TR_IF(4 * (s - s_lo) == 2 * (s_hi - s_lo), 9);
+                TR_IF(4 * (s - s_lo) == 3 * (s_hi - s_lo), 10);
                 // rows of the next step; past the segment they fall outside the window
                 Row<T> xn, Bn, Cn;
                 fetch(s + 1, xn, Bn, Cn);
@@ -222,7 +234,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
                     unpack8<T>(Cr, Cf);
 #pragma unroll
                     for (int e = 0; e < 8; ++e) yf[e] = Cf[e] * y2f[e];
-                    stw_row_policy<T, GCG_MFMA_FWD_ST>(wy, o, pack8<T>(yf));
+                    stw_row_policy<T, (ES == 2 ? GCG_MFMA_FWD_ST : WIN_NT_ST)>(wy, o, pack8<T>(yf));
                     if constexpr (EXTRA) stw_row<T>(wy2, o, pack8<T>(y2f));
                 }
                 xr = xn; Br = Bn; Cr = Cn;
@@ -407,6 +419,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
         for (int ph = 0; ph < NK; ++ph) {
             if (s < s_hi) {
                 const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
+                TR_IF(4 * (s - s_lo) == (s_hi - s_lo), 8);
+                TR_IF(4 * (s - s_lo) == 2 * (s_hi - s_lo), 9);
+                TR_IF(4 * (s - s_lo) == 3 * (s_hi - s_lo), 10);
                 // rows of the next iteration; past the segment they fall outside the windows
                 Row<T> xn, Bn, dyn, Cn;
                 fetch(s + 1, xn, Bn, dyn, Cn);
