@@ -284,15 +284,30 @@ STATIC_SCRATCH_BYTES = 8 << 20      # GCG_BWD_STATIC_SCRATCH_BYTES
 def bwd_static(dy, x, B, C, h, dx, dB, dC, dh, algo=ALGO_AUTO):
     """gcg_bwd_static: the backward into the caller's output tensors with the library's built-in scratch
     array instead of a workspace; nothing is allocated by the call (for callers under graph capture).
-    Calls that overlap on one GPU share the array and must be ordered by the caller."""
+    Calls that overlap on one GPU share the array and must be ordered by the caller.
+    The C entry point sees pointers only, so the tensors are checked here as gcg_bwd's binding checks them:
+    a strided or short output would be written out of bounds by the kernels."""
     lib = load()
     _require_gpu(x)
+    if x.dim() != 4:
+        raise ValueError("x must be (bs, L, g, dg)")
     bs, L, g, dg = x.shape
+    for name, t in (("x", x), ("dy", dy), ("B", B), ("C", C), ("dx", dx), ("dB", dB), ("dC", dC)):
+        if t.shape != x.shape or t.dtype != x.dtype or t.device != x.device or not t.is_contiguous():
+            raise ValueError(f"{name} must be a contiguous (bs, L, g, dg) tensor with the dtype and device of x")
+    if h.dim() != 3 or h.shape[0] != g or h.shape[1] != 1 or h.device != x.device or not h.is_contiguous():
+        raise ValueError("h must be a contiguous (g, 1, hl) tensor on the device of x")
+    if dh.shape != h.shape or dh.dtype != h.dtype or dh.device != x.device or not dh.is_contiguous():
+        raise ValueError("dh must be a contiguous tensor with the shape, dtype and device of h")
+    code = gated_code(x, h)             # raises for a filter type that does not go with the tensors'
+    if x.numel() == 0:
+        dh.zero_()
+        return
     with _on_device(x.device):
         rc = lib.gcg_bwd_static(
             dy.data_ptr(), x.data_ptr(), B.data_ptr(), C.data_ptr(), h.data_ptr(),
             dx.data_ptr(), dB.data_ptr(), dC.data_ptr(), dh.data_ptr(),
-            bs, L, g, dg, h.shape[-1], gated_code(x, h), algo_code(algo),
+            bs, L, g, dg, h.shape[-1], code, algo_code(algo),
             torch.cuda.current_stream().cuda_stream,
         )
     check(rc, "gcg_bwd_static")
@@ -619,16 +634,10 @@ def _all_aligned16(tensors, skip_strided=False) -> bool:
     return True
 
 
-# read once, as the library reads it
-_MIXER_MR_ONE_KERNEL = os.environ.get("GCG_MIXER_MR_FUSED", "1").strip() != "0"
-
-
 def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors, planar: bool = False) -> bool:
     """Whether gcg_mixer_mr_fwd / _bwd take these sizes (matrix-core kernels, filters of up to 128 taps
     -- those of at most 8 are the fused Hyena-SE kernels' -- and a featurizer of at most 3).  ``planar``: the
-    planar entry points, which exist in the one-kernel form only (the library's GCG_MIXER_MR_FUSED=0 switches it off)."""
-    if planar and not _MIXER_MR_ONE_KERNEL:
-        return False
+    planar entry points, which exist in the one-kernel form only (16-bit arithmetic)."""
     return 9 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and _all_aligned16(tensors)
 
 

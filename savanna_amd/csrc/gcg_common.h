@@ -250,6 +250,21 @@ constexpr int kWave = 64;
 
 } // namespace gcg
 
+#include <cstdlib>
+namespace gcg {
+// Tuning overrides from the environment exist in builds with -DGCG_TUNING only (A/B builds of a variant
+// against the library); the library as built by the Makefile reads no environment variable.
+inline const char *tuning_env(const char *name)
+{
+#ifdef GCG_TUNING
+    return getenv(name);
+#else
+    (void)name;
+    return nullptr;
+#endif
+}
+} // namespace gcg
+
 // Host-side launchers, one translation unit per kernel family.  Each returns a
 // hipError_t as int; none of them allocates or synchronises.
 namespace gcg {

@@ -208,7 +208,7 @@ __global__ __launch_bounds__(256) void dwconv_bwd_kernel(const T *__restrict__ d
 // 7B featurizer shape (forward 160 vs 153 us, backward 265 vs 269 us) and stays a tuning override.
 int lane_width(int dtype, const Dims &dm)
 {
-    static const char *env = getenv("GCG_DWCONV_V");       // tuning override: 4 or 8
+    static const char *env = tuning_env("GCG_DWCONV_V");       // tuning override: 4 or 8
     const int want = env ? atoi(env) : 4;
     if (dtype != GCG_F32 && want == 8 && dm.d % 8 == 0 && (dm.dg == 1 || dm.dg % 8 == 0)) return 8;
     return 4;
@@ -221,7 +221,7 @@ DwPlan plan(const Dims &dm, int V)
     p.nvec = (int)(dm.d / V);
     p.ts = 128;
     while (p.ts > 8 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
-    static const char *env = getenv("GCG_DWCONV_ROWS");     // tuning override: rows per lane, a multiple of 8
+    static const char *env = tuning_env("GCG_DWCONV_ROWS");     // tuning override: rows per lane, a multiple of 8
     if (env && atoi(env) >= 8 && atoi(env) % 8 == 0) p.ts = atoi(env);
     while (p.ts > 8 && (int64_t)(p.ts + 2 * RING) * dm.d * 4 > WIN_MAX_BYTES) p.ts >>= 1;
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);

@@ -631,10 +631,7 @@ template <typename T, int NK>
 int bwd_nk(const void *dy, const void *x, const void *B, const void *C, const void *h, void *dx, void *dB,
            void *dC, void *dh, void *ws, const Dims &dm, hipStream_t st)
 {
-    if constexpr (!MT<T>::SPLIT) {
-        if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
-    }
-    return bwd_launch<T, NK, 4>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
+    return bwd_launch<T, NK, BWD_NW>(dy, x, B, C, h, dx, dB, dC, dh, ws, dm, st);
 }
 
 template <typename T>

@@ -589,10 +589,7 @@ template <typename T, int NK>
 int bwd_nk(const void *dy, const void *feat, const void *h, void *dfeat, void *dh, void *ws, const Dims &dm,
            hipStream_t st)
 {
-    if constexpr (!MT<T>::SPLIT) {
-        if (choose_nw_bwd(dm, false) == 8) return bwd_launch<T, NK, 8>(dy, feat, h, dfeat, dh, ws, dm, st);
-    }
-    return bwd_launch<T, NK, 4>(dy, feat, h, dfeat, dh, ws, dm, st);
+    return bwd_launch<T, NK, BWD_NW>(dy, feat, h, dfeat, dh, ws, dm, st);
 }
 
 template <typename T>

@@ -675,10 +675,11 @@ int cu_count()
     return n;
 }
 
-// tuning overrides from the environment: unset or empty -> dflt; any integer, 0 included, is taken
+// tuning overrides from the environment (tuning builds only, gcg_common.h): unset or empty -> dflt; any integer,
+// 0 included, is taken
 int env_int(const char *name, int dflt)
 {
-    const char *v = getenv(name);
+    const char *v = tuning_env(name);
     if (!v || !*v) return dflt;
     char *end = nullptr;
     const long n = strtol(v, &end, 10);
@@ -748,23 +749,18 @@ int nk_for(int hl) { const int n = (hl + 30) / 32 + 1; return n > 5 ? 5 : n; }
 
 // The backward holds about twice the forward's register state per wave (two waves per SIMD at
 // most), and one wave per SIMD measured best: 4-wave workgroups, one per CU, with runs twice as
-// long (half the lead-in) take 176 us where 8-wave workgroups take 201 at (2, 8192, 4096) and 660
+// long (half the lead-in) take 176 us where 8-wave workgroups took 201 at (2, 8192, 4096) and 660
 // against 749 at (1, 32768, 8192); on interleaved operands 173 against 196 and 641 against 754.
 // Two 4-wave workgroups sharing a CU are slower than either (237 us), so the kernels' LDS
-// request keeps a CU to one.
-int choose_nw_bwd(const Dims &dm, bool fp32)
-{
-    (void)dm;
-    static const int forced = env_int("GCG_MFMA_BWD_NW", 0);   // tuning override: 4 or 8
-    if (forced == 4 || (forced == 8 && !fp32)) return forced;
-    return 4;
-}
+// request keeps a CU to one.  The 8-wave form is no longer instantiated.
+constexpr int BWD_NW = 4;
 
 // one workgroup per CU in either geometry (fp32: one wave per SIMD by its registers alone)
 MfmaPlan plan_bwd_nw(const Dims &dm, int nw, int elem_bytes);
 MfmaPlan plan_bwd(const Dims &dm, bool split, int elem_bytes)
 {
-    return plan_bwd_nw(dm, choose_nw_bwd(dm, split), elem_bytes);
+    (void)split;
+    return plan_bwd_nw(dm, BWD_NW, elem_bytes);
 }
 // The backward that recomputes the featurizer spends twice the vector instructions per row: with two waves per
 // SIMD they hide behind each other (8-wave workgroups: 220 us at the 7B shape against 263 with 4 waves).
@@ -777,9 +773,9 @@ int choose_nw_bwd_feat(bool split)
 MfmaPlan plan_bwd_nw(const Dims &dm, int nw, int elem_bytes)
 {
     MfmaPlan p = plan(dm, nw, 16, nw, elem_bytes);
-    // the kernel adds the partials itself when a filter group lies within one channel block
-    static const int fuse = env_int("GCG_MFMA_FUSE_DH", 1);    // tuning override: 0 = always a second launch
-    p.fuse_dh = fuse && (16 * nw) % dm.dg == 0 && p.ncb <= DH_UNITS;
+    // the kernel adds the partials itself when a filter group lies within one channel block (and the launch gets a
+    // ticket set, dh_slot_for_stream); otherwise a second launch does
+    p.fuse_dh = (16 * nw) % dm.dg == 0 && p.ncb <= DH_UNITS;
     return p;
 }
 

@@ -918,8 +918,7 @@ MfmaPlan mixer_plan(const Dims &dm)
 {
     MfmaPlan p = plan(dm, MixGeo<bf16_t>::XW, 16, MixGeo<bf16_t>::XW, 2);
     // the kernel adds the partials itself when a filter group lies within one channel block
-    static const int fuse = env_int("GCG_MFMA_FUSE_DH", 1);    // tuning override: 0 = always separate launches
-    p.fuse_dh = fuse && MixGeo<bf16_t>::CB % dm.dg == 0 && p.ncb <= DH_UNITS;
+    p.fuse_dh = MixGeo<bf16_t>::CB % dm.dg == 0 && p.ncb <= DH_UNITS;
     return p;
 }
 
@@ -986,8 +985,7 @@ int mixer_mr_fused_fwd_launch(int dtype, const void *raw, const void *wfeat, int
 // 16-bit tensors with arithmetic in their own type, filters of up to 128 taps, a featurizer of at most 3
 bool mixer_mr_fused_supported(int dtype, const Dims &dm, int kf)
 {
-    static const int off = env_int("GCG_MIXER_MR_FUSED", 1) == 0;      // tuning override: 0 = the two-kernel backward
-    if (off || (dtype != GCG_BF16 && dtype != GCG_F16)) return false;
+    if (dtype != GCG_BF16 && dtype != GCG_F16) return false;
     if (!mfma_feat_supported(dtype, dm, kf) || 3 * dm.d > 0x7fffffffLL) return false;
     return windows_fit(dm, mixer_plan(dm));
 }

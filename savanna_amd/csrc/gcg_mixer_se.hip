@@ -844,7 +844,7 @@ MixPlan plan(const Dims &dm, int ch, bool backward)
     // (the backward's longest ring) down to 16.
     p.ts = backward ? 512 : 1024;
     while (p.ts > 16 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
-    static const char *env = getenv("GCG_MIXER_ROWS");      // tuning override: rows per lane, a multiple of 16
+    static const char *env = tuning_env("GCG_MIXER_ROWS");      // tuning override: rows per lane, a multiple of 16
     if (env && atoi(env) >= 16 && atoi(env) % 16 == 0) p.ts = atoi(env);
     while (p.ts > 16 && (int64_t)(p.ts + 32) * 3 * dm.d * 4 > WIN_MAX_BYTES) p.ts >>= 1;
     p.nseg = (int)((dm.L + p.ts - 1) / p.ts);

@@ -398,7 +398,7 @@ WinPlan plan(const Dims &dm, int v)
     // 7B and 40B shapes for either operand layout (fewer halo rows and filter-gradient partials;
     // one step further and the machine is no longer covered)
     while (p.ts > 8 && dm.bs * ((dm.L + p.ts - 1) / p.ts) * p.nvec < 128 * 1024) p.ts >>= 1;
-    static const char *env = getenv("GCG_WINDOW_ROWS");   // tuning override: rows per lane, a multiple of 8
+    static const char *env = tuning_env("GCG_WINDOW_ROWS");   // tuning override: rows per lane, a multiple of 8
     if (env && atoi(env) >= 8 && atoi(env) % 8 == 0) p.ts = atoi(env);
     // the rows of a run, its halo and an interleaved fp32 row width must fit one tensor window
     while (p.ts > 8 && (int64_t)(p.ts + 2 * RING) * 3 * dm.d * 4 * (dm.tmajor ? dm.bs : 1) > WIN_MAX_BYTES) p.ts >>= 1;   // (planar rows are 3 d wide too)

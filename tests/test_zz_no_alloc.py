@@ -62,3 +62,67 @@ def test_sizes_beyond_the_scratch_are_rejected(gcg_lib):
     rc = gcg_lib.gcg_bwd_static(p, p, p, p, p, p, p, p, p, bs, L, g, dg, hl, code, _lib.ALGO_AUTO, None)
     assert rc == -6
     assert b"gcg_bwd_static" in gcg_lib.gcg_strerror(rc)
+
+
+def test_outputs_are_checked(gcg_lib):
+    """A strided, short or mistyped output is refused by the binding before the kernels could write past it."""
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(1, 64, 2, 16, 7, torch.bfloat16, seed=5))
+    good = [torch.empty_like(x) for _ in range(3)] + [torch.empty_like(h)]
+    _lib.bwd_static(dy, x, B, C, h, *good)
+    strided = torch.empty(1, 64, 2, 32, dtype=x.dtype, device=DEV)[..., ::2]
+    short = torch.empty(1, 32, 2, 16, dtype=x.dtype, device=DEV)
+    for bad_dx in (strided, short, torch.empty_like(x, dtype=torch.float32), torch.empty_like(x, device="cpu")):
+        with pytest.raises(ValueError, match="dx"):
+            _lib.bwd_static(dy, x, B, C, h, bad_dx, *good[1:])
+    with pytest.raises(ValueError, match="dh"):
+        _lib.bwd_static(dy, x, B, C, h, *good[:3], torch.empty(2, 1, 8, dtype=h.dtype, device=DEV))
+
+
+@pytest.mark.parametrize("algo,dtype,shape", [("mfma", torch.bfloat16, (2, 1500, 6, 16, 128)),
+                                               ("window", torch.bfloat16, (2, 2000, 8, 16, 7))])
+def test_static_backward_in_a_captured_graph(gcg_lib, algo, dtype, shape):
+    """The use the entry point is for: a first call outside the capture (it looks the scratch array up), then a call
+    recorded into a HIP graph and replayed, with eager work of the same library between the replays; every replay
+    must give gcg_bwd's bits.  Under capture the matrix-core backward adds its filter-gradient partials with a
+    second kernel instead of its ticket scheme, in the same order."""
+    bs, L, g, dg, hl = shape
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(bs, L, g, dg, hl, dtype, seed=6))
+    ref = _lib.bwd(dy, x, B, C, h, algo=algo)
+    outs = [torch.full_like(x, float("nan")) for _ in range(3)] + [torch.full_like(h, float("nan"))]
+    _lib.bwd_static(dy, x, B, C, h, *outs, algo=algo)           # outside the capture, as the header asks
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            _lib.bwd_static(dy, x, B, C, h, *outs, algo=algo)
+    torch.cuda.current_stream().wait_stream(side)
+    for replay in range(3):
+        for o in outs:
+            o.fill_(float("nan"))
+        other = _lib.bwd(dy, x, B, C, h, algo=algo)              # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, got, want, again in zip(("dx", "dB", "dC", "dh"), outs, ref, other):
+            assert torch.equal(got, want), f"replay {replay}: {name} differs from gcg_bwd"
+            assert torch.equal(again, want)
+
+
+def test_more_streams_than_ticket_sets(gcg_lib):
+    """The matrix-core backward keeps one set of arrival tickets per stream, for 64 streams; launches on further
+    streams add their filter-gradient partials with a second kernel.  Same bits either way."""
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(2, 700, 4, 16, 128, torch.bfloat16, seed=7))
+    ref = _lib.bwd(dy, x, B, C, h, algo="mfma")
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(70)]
+    results = []
+    for st in streams:
+        st.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(st):
+            results.append(_lib.bwd(dy, x, B, C, h, algo="mfma"))
+    torch.cuda.synchronize()
+    for got in results:
+        for a, b in zip(got, ref):
+            assert torch.equal(a, b)
