@@ -3,7 +3,8 @@
 // called from eager code, traced by torch.compile and captured into graphs.  Each device
 // implementation checks its arguments, allocates the outputs with torch's allocator, and
 // enqueues the C-ABI entry point on torch's current stream under a device guard; error codes
-// become exceptions.  Autograd formulas are attached on the Python side (savanna_amd/_ops.py).
+// become exceptions.  The backward formulas of the forward operators are registered on the Python side
+// (savanna_amd/_ops.py: torch.library.register_autograd), each in terms of the backward operator defined here.
 //
 // This is the counterpart of the Triton launch wrappers two_pass_fwd_grouped /
 // two_pass_bwd_refactor (savanna/kernels/triton_src/cgcg/src/fwd.py:13-233, src/bwd.py:347-474)

@@ -191,3 +191,67 @@ def test_compile_fullgraph_hyena_mixer(gcg_lib, kind, planar):
     assert len(eager) == len(compiled) == 2 + len(params)
     for i, (a, b) in enumerate(zip(eager, compiled)):
         assert torch.equal(a, b), i
+
+
+def _leaves(*ts):
+    return [t.detach().clone().requires_grad_(True) for t in ts]
+
+
+def test_forward_operators_are_differentiable(gcg_lib):
+    """A call of torch.ops.gcg.* on tensors that require grad is part of the autograd graph: the gradients are the
+    backward operator's outputs, bit for bit, and opcheck finds the registration in order."""
+    ops = torch.ops.gcg
+    x, B, C, h, dy = (t.to(DEV) for t in inputs(2, 300, 3, 16, 128, torch.bfloat16, seed=9, dy_scale=0.1))
+    feat = torch.stack([C, B, x], dim=-1).contiguous()
+    planar = torch.stack([C, B, x], dim=2).contiguous()
+    wf = (torch.randn(3 * 3 * 16, 1, 3, device=DEV) / 3 ** 0.5).to(torch.bfloat16)
+    w = torch.randn(3, 128, device=DEV) / 128 ** 0.5
+    decay = torch.rand(3, 128, device=DEV)
+    hs = h[..., :7].contiguous()
+    cases = [
+        (ops.fwd, (x, B, C, h), lambda a: ops.bwd(dy, *a)),
+        (ops.fwd_interleaved, (feat, h), lambda a: ops.bwd_interleaved(dy, *a)),
+        (ops.fwd_planar, (planar, h), lambda a: ops.bwd_planar(dy, *a)),
+        (ops.mixer_mr_fwd, (feat, wf, h), lambda a: ops.mixer_mr_bwd(dy, *a)),
+        (ops.mixer_se_fwd, (feat, wf, hs), lambda a: ops.mixer_se_bwd(dy, *a)),
+        (ops.fwd_time_major, (x.transpose(0, 1).contiguous(), B.transpose(0, 1).contiguous(),
+                              C.transpose(0, 1).contiguous(), hs), lambda a: ops.bwd_time_major(dy, *a)),
+    ]
+    for op, args, backward in cases:
+        leaves = _leaves(*args)
+        y = op(*leaves)
+        assert y.requires_grad, op
+        y.backward(dy)
+        want = backward(args)
+        for leaf, g in zip(leaves, want):
+            assert torch.equal(leaf.grad, g), op
+    # the featurizer conv (its own gradient shape) and the operators that form the filter inside the kernels
+    xs = feat.reshape(2, 300, 144, 1)
+    lx, lw = _leaves(xs, wf)
+    ops.dwconv_fwd(lx, lw).backward(xs)
+    for got, g in zip((lx.grad, lw.grad), ops.dwconv_bwd(xs, xs, wf)):
+        assert torch.equal(got, g)
+    lv = _leaves(x, B, C, w)
+    ops.fwd_decay(*lv, decay, 128, torch.bfloat16).backward(dy)
+    for leaf, g in zip(lv, ops.bwd_decay(dy, x, B, C, w, decay, 128, torch.bfloat16)):
+        assert torch.equal(leaf.grad, g)
+    lf, lw2 = _leaves(feat, w)
+    ops.fwd_interleaved_decay(lf, lw2, decay, 128, torch.bfloat16).backward(dy)
+    for got, g in zip((lf.grad, lw2.grad), ops.bwd_interleaved_decay(dy, feat, w, decay, 128, torch.bfloat16)):
+        assert torch.equal(got, g)
+    lr, lwf, lw3 = _leaves(feat, wf, w)
+    ops.mixer_mr_fwd_decay(lr, lwf, lw3, decay, 128, torch.bfloat16).backward(dy)
+    for got, g in zip((lr.grad, lwf.grad, lw3.grad), ops.mixer_mr_bwd_decay(dy, feat, wf, w, decay, 128, torch.bfloat16)):
+        assert torch.equal(got, g)
+    (lw4,) = _leaves(w)
+    dh = torch.randn(3, 1, 128, device=DEV).to(torch.bfloat16)
+    ops.filter_decay_fwd(lw4, decay, 128, torch.bfloat16).backward(dh)
+    assert torch.equal(lw4.grad, ops.filter_decay_bwd(dh, decay))
+    # the forward with optional extra outputs is not differentiable and says so
+    with pytest.raises(RuntimeError, match="not differentiable"):
+        ops.fwd_full(*_leaves(x, B, C, h), False, False)[2].backward(dy)
+    checks = ("test_schema", "test_autograd_registration", "test_faketensor")
+    torch.library.opcheck(ops.fwd, tuple(_leaves(x, B, C, h)), test_utils=checks)
+    torch.library.opcheck(ops.fwd_interleaved, tuple(_leaves(feat, h)), test_utils=checks)
+    torch.library.opcheck(ops.mixer_mr_fwd, tuple(_leaves(feat, wf, h)), test_utils=checks)
+    torch.library.opcheck(ops.dwconv_fwd, tuple(_leaves(xs, wf)), test_utils=checks)
