@@ -95,6 +95,23 @@ GCG_API int gcg_time_next_kernel(void *start_event, void *stop_event);
 GCG_API int gcg_version(void);
 
 /*
+ * Whether the entry points of a route take these sizes -- every limit they check apart from the
+ * alignment of the tensors (16 bytes), which only the call itself can see.  It has no counterpart
+ * in the reference; it is what a caller that chooses between a fused entry point and the general
+ * ones (gcg_fwd / gcg_bwd, which take any size) asks before it chooses.  kf is the featurizer's
+ * filter length for the mixer routes and ignored otherwise.  Returns 1, 0, or GCG_ERR_BAD_ARG.
+ */
+enum {
+    GCG_ROUTE_DECAY           = 1, /* gcg_fwd_decay, gcg_bwd_decay, gcg_*_interleaved_decay              */
+    GCG_ROUTE_TIME_MAJOR      = 2, /* gcg_fwd_time_major, gcg_bwd_time_major                             */
+    GCG_ROUTE_MIXER_SE        = 3, /* gcg_mixer_se_fwd / _bwd and their _planar forms                    */
+    GCG_ROUTE_MIXER_MR        = 4, /* gcg_mixer_mr_fwd / _bwd (and _decay)                               */
+    GCG_ROUTE_MIXER_MR_PLANAR = 5  /* gcg_mixer_mr_fwd_planar / _bwd_planar (and _decay): one-kernel form */
+};
+GCG_API int gcg_route_supported(int32_t route, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl,
+                        int32_t kf, int32_t dtype);
+
+/*
  * Forward.
  * Replaces two_pass_fwd_grouped(x, B, C, h, return_bx=, return_y2=)
  * (savanna/kernels/triton_src/cgcg/src/fwd.py:13-233), which launches

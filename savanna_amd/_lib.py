@@ -30,7 +30,7 @@ GCG_BF16_F32, GCG_F16_F32 = 3, 4       # 16-bit tensors, fp32 filter and arithme
 # every symbol include/gcg.h declares
 EXPORTS = (
     "gcg_strerror", "gcg_last_hip_error", "gcg_time_next_kernel", "gcg_version", "gcg_fwd",
-    "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_bwd_static", "gcg_select_algo",
+    "gcg_bwd_workspace_bytes", "gcg_bwd", "gcg_bwd_static", "gcg_select_algo", "gcg_route_supported",
     "gcg_fwd_interleaved", "gcg_bwd_interleaved", "gcg_fwd_planar", "gcg_bwd_planar",
     "gcg_dwconv_fwd", "gcg_dwconv_bwd_workspace_bytes", "gcg_dwconv_bwd",
     "gcg_mixer_se_fwd", "gcg_mixer_se_bwd_workspace_bytes", "gcg_mixer_se_bwd",
@@ -82,6 +82,8 @@ def load() -> ctypes.CDLL:
         lib.gcg_bwd_static.restype = ctypes.c_int
         lib.gcg_select_algo.argtypes = [i64, i64, i32, i32, i32, i32, i32]
         lib.gcg_select_algo.restype = ctypes.c_int
+        lib.gcg_route_supported.argtypes = [i32, i64, i64, i32, i32, i32, i32, i32]
+        lib.gcg_route_supported.restype = ctypes.c_int
         lib.gcg_fwd_interleaved.argtypes = [vp] * 3 + [i64, i64, i32, i32, i32, i32, i32, vp]
         lib.gcg_fwd_interleaved.restype = ctypes.c_int
         lib.gcg_bwd_interleaved.argtypes = [vp] * 6 + [sz, i64, i64, i32, i32, i32, i32, i32, i32, vp]
@@ -634,11 +636,29 @@ def _all_aligned16(tensors, skip_strided=False) -> bool:
     return True
 
 
-def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors, planar: bool = False) -> bool:
+ROUTE_DECAY, ROUTE_TIME_MAJOR, ROUTE_MIXER_SE, ROUTE_MIXER_MR, ROUTE_MIXER_MR_PLANAR = 1, 2, 3, 4, 5
+
+
+def route_supported(route: int, bs: int, L: int, g: int, dg: int, hl: int, kf: int, code: int) -> bool:
+    """gcg_route_supported: whether the entry points of a route take these sizes (every limit the library checks
+    apart from the tensors' alignment: filter lengths, group widths, what a tensor window can span)."""
+    if min(bs, L, g, dg, hl) <= 0:
+        return False
+    return load().gcg_route_supported(route, bs, L, g, dg, hl, kf, code) == 1
+
+
+def mixer_mr_supported(dg: int, hl: int, kf: int, *tensors, planar: bool = False, sizes=None) -> bool:
     """Whether gcg_mixer_mr_fwd / _bwd take these sizes (matrix-core kernels, filters of up to 128 taps
     -- those of at most 8 are the fused Hyena-SE kernels' -- and a featurizer of at most 3).  ``planar``: the
-    planar entry points, which exist in the one-kernel form only (16-bit arithmetic)."""
-    return 9 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and _all_aligned16(tensors)
+    planar entry points, which exist in the one-kernel form only (16-bit arithmetic).
+    ``sizes`` = (bs, L, g, dtype code): with them the library is asked as well (gcg_route_supported), which also
+    knows how far its tensor windows reach; without them only the shape rules above are applied."""
+    if not (9 <= hl <= 128 and dg % 16 == 0 and 1 <= kf <= 3 and _all_aligned16(tensors)):
+        return False
+    if sizes is None:
+        return True
+    bs, L, g, code = sizes
+    return route_supported(ROUTE_MIXER_MR_PLANAR if planar else ROUTE_MIXER_MR, bs, L, g, dg, hl, kf, code)
 
 
 def mixer_mr_fwd(raw, wf, h, planar=False):
@@ -759,8 +779,15 @@ def mixer_mr_bwd_decay(dy, raw, wf, w, decay, hl: int, filt: torch.dtype, planar
 # ---- the short-filter operator on time-major operands (seqlen, bs, g, dg) ------------------------
 
 def time_major_supported(dg: int, hl: int, *tensors) -> bool:
-    """Whether gcg_fwd_time_major / gcg_bwd_time_major take these sizes (register-window kernels)."""
-    return hl <= 8 and dg % 4 == 0 and all(t.is_contiguous() for t in tensors) and _all_aligned16(tensors)
+    """Whether gcg_fwd_time_major / gcg_bwd_time_major take these tensors (register-window kernels): the shape
+    rules, and the library's own answer for the sizes of the first tensor, (seqlen, bs, g, dg) -- its windows span
+    bs rows of memory per time row, so a large batch of wide rows is beyond them."""
+    if not (hl <= 8 and dg % 4 == 0 and all(t.is_contiguous() for t in tensors) and _all_aligned16(tensors)):
+        return False
+    if not tensors:
+        return True
+    L, bs, g, _ = tensors[0].shape
+    return route_supported(ROUTE_TIME_MAJOR, bs, L, g, dg, hl, 0, dtype_code(tensors[0].dtype))
 
 
 def fwd_time_major(x, B, C, h):
@@ -809,8 +836,14 @@ def bwd_time_major(dy, x, B, C, h):
 def decay_supported(g: int, dg: int, hl: int, *tensors) -> bool:
     """Whether the *_decay entry points take these sizes: matrix-core kernels only
     (hl <= 128, dg a multiple of 16, 16-byte aligned tensors; a tensor that is not contiguous is
-    copied or read through its interleaved source before it reaches them)."""
-    return hl <= 128 and dg % 16 == 0 and _all_aligned16(tensors, skip_strided=True)
+    copied or read through its interleaved source before it reaches them), rows no wider than a tensor window
+    of those kernels holds (the library's answer for the first tensor's (bs, L, g, dg))."""
+    if not (hl <= 128 and dg % 16 == 0 and _all_aligned16(tensors, skip_strided=True)):
+        return False
+    if not tensors or tensors[0].dim() != 4:
+        return True
+    bs, L = tensors[0].shape[:2]
+    return route_supported(ROUTE_DECAY, bs, L, g, dg, hl, 0, dtype_code(tensors[0].dtype))
 
 
 def _decay_code(t: torch.Tensor, filt: torch.dtype) -> int:

@@ -158,6 +158,42 @@ GCG_API int gcg_select_algo(int64_t bs, int64_t L, int32_t g, int32_t dg, int32_
     return resolve_algo(GCG_ALGO_AUTO, dtype, dm, backward != 0);
 }
 
+namespace {
+// the tensors' own type code of a mixed code (16-bit tensors, fp32 arithmetic)
+int plain_tensor_code(int dtype) { return dtype == GCG_BF16_F32 ? GCG_BF16 : dtype == GCG_F16_F32 ? GCG_F16 : dtype; }
+} // namespace
+
+GCG_API int gcg_route_supported(int32_t route, int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t kf,
+                                int32_t dtype)
+{
+    gcg::Dims dm;
+    const bool mixer = route == GCG_ROUTE_MIXER_SE || route == GCG_ROUTE_MIXER_MR || route == GCG_ROUTE_MIXER_MR_PLANAR;
+    if (make_dims(bs, L, g, dg, hl, dtype, &dm, true) || (mixer && kf <= 0)) return GCG_ERR_BAD_ARG;
+    switch (route) {
+    case GCG_ROUTE_DECAY:               // the filter is formed in the matrix-core kernels only
+        return gcg::mfma_supported(dtype, dm) ? 1 : 0;
+    case GCG_ROUTE_TIME_MAJOR:          // register-window kernels, whose windows span bs rows of memory per time row
+        dm.tmajor = 1;
+        return gcg::window_supported(dm) ? 1 : 0;
+    case GCG_ROUTE_MIXER_SE:
+        dm.es = 3;
+        return gcg::mixer_se_supported(dm, kf) ? 1 : 0;
+    case GCG_ROUTE_MIXER_MR: {          // one kernel each way, or the 8-wave kernels with the featurizer in front
+        dm.es = 3;
+        if (!gcg::mfma_feat_supported(dtype, dm, kf)) return 0;
+        if (gcg::mixer_mr_fused_supported(dtype, dm, kf)) return 1;
+        gcg::Dims df;                   // the two-kernel backward ends in the featurizer's own backward
+        if (make_dims(bs, L, 3 * g * dg, 1, kf, plain_tensor_code(dtype), &df)) return 0;
+        return gcg::dwconv_supported(df) ? 1 : 0;
+    }
+    case GCG_ROUTE_MIXER_MR_PLANAR:
+        dm.planar = 1;
+        dm.es = 1;
+        return gcg::mfma_feat_supported(dtype, dm, kf) && gcg::mixer_mr_fused_supported(dtype, dm, kf) ? 1 : 0;
+    }
+    return GCG_ERR_BAD_ARG;
+}
+
 GCG_API int gcg_fwd(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
             int64_t bs, int64_t L, int32_t g, int32_t dg, int32_t hl, int32_t dtype, int32_t algo,
             void *stream)
@@ -702,7 +738,6 @@ int mixer_mr_fwd_dims(const void *raw, const void *wf, const void *h, void *y, g
 } // namespace
 
 namespace {
-int plain_tensor_code(int dtype) { return dtype == GCG_BF16_F32 ? GCG_BF16 : dtype == GCG_F16_F32 ? GCG_F16 : dtype; }
 size_t up256(size_t n) { return (n + 255) & ~(size_t)255; }
 } // namespace
 

@@ -987,7 +987,8 @@ bool mixer_mr_fused_supported(int dtype, const Dims &dm, int kf)
 {
     if (dtype != GCG_BF16 && dtype != GCG_F16) return false;
     if (!mfma_feat_supported(dtype, dm, kf) || 3 * dm.d > 0x7fffffffLL) return false;
-    return windows_fit(dm, mixer_plan(dm));
+    // both launches: the forward plans its runs by itself (shorter ones), the backward by its own
+    return windows_fit(dm, mixer_plan(dm)) && windows_fit(dm, mixer_fwd_plan(dm));
 }
 
 size_t mixer_mr_fused_workspace(const Dims &dm, int kf)

@@ -420,13 +420,25 @@ class HyenaMixer(nn.Module):
         z = z.reshape(bs, seqlen, g * dg)
         return z.to(dtype) if cast else z
 
+    def _mixer_code(self, features: torch.Tensor) -> int:
+        """The library's dtype code for the mixer's call on these features: their own type, or 16-bit tensors with
+        fp32 arithmetic, or -- features cast to ``cgcg_dtype`` around the call -- that type."""
+        op = self.mixer
+        if op.cgcg_dtype == features.dtype:
+            return _lib.dtype_code(features.dtype)
+        if op._fp32_inside(features.dtype, features):
+            return _lib.GCG_BF16_F32 if features.dtype == torch.bfloat16 else _lib.GCG_F16_F32
+        return _lib.dtype_code(op.cgcg_dtype)
+
     def _medium(self, features: torch.Tensor, hl: int) -> bool:
         """Whether the one-kernel Hyena-MR mixer takes these features with a filter of ``hl`` taps.  Planar features
         ("(p g dg)" rows) run in the one-kernel form only, which has 16-bit arithmetic."""
         conv, op = self.hyena_proj_conv, self.mixer
         if not (self.fuse_medium and features.is_cuda and conv.group_dim == 1 and
                 _lib.mixer_mr_supported(op.group_dim, hl, conv.kernel_size, features,
-                                        planar=not self.interleave_projections)):
+                                        planar=not self.interleave_projections,
+                                        sizes=(features.shape[0], features.shape[1], op.num_groups,
+                                               self._mixer_code(features)))):
             return False
         if self.interleave_projections:
             return op.cgcg_dtype == features.dtype or op._fp32_inside(features.dtype, features)

@@ -267,3 +267,45 @@ def test_bench_has_no_cpu_path():
     assert r.returncode != 0
     assert "no GPU" in r.stderr + r.stdout
     assert "{" not in r.stdout
+
+
+def test_route_predicates_follow_the_library_at_its_limits(gcg_lib):
+    """gcg_route_supported answers on the host for every fused route, and the Python predicates that choose between
+    a fused entry point and the general ones return what it returns -- also where the refusal comes from how far a
+    tensor window reaches (very wide rows, a large batch of time-major rows), which the shape rules alone miss."""
+    bf16, f32, mixed = _lib.dtype_code(torch.bfloat16), _lib.dtype_code(torch.float32), _lib.GCG_BF16_F32
+    q = gcg_lib.gcg_route_supported
+    # shape rules
+    assert q(_lib.ROUTE_DECAY, 2, 8192, 256, 16, 128, 0, bf16) == 1
+    assert q(_lib.ROUTE_DECAY, 2, 8192, 256, 16, 129, 0, bf16) == 0          # longer than the matrix-core band
+    assert q(_lib.ROUTE_DECAY, 2, 8192, 256, 8, 128, 0, bf16) == 0           # groups narrower than a tile
+    assert q(_lib.ROUTE_TIME_MAJOR, 16, 8192, 48, 16, 7, 0, bf16) == 1       # the reference's run_short_hyena test shape
+    assert q(_lib.ROUTE_TIME_MAJOR, 16, 8192, 48, 16, 9, 0, bf16) == 0
+    assert q(_lib.ROUTE_MIXER_SE, 1, 32768, 512, 16, 7, 3, bf16) == 1
+    assert q(_lib.ROUTE_MIXER_SE, 1, 32768, 512, 16, 7, 5, bf16) == 0        # featurizer longer than the kernels take
+    assert q(_lib.ROUTE_MIXER_MR, 2, 8192, 256, 16, 128, 3, bf16) == 1
+    assert q(_lib.ROUTE_MIXER_MR, 2, 8192, 256, 16, 128, 3, mixed) == 1      # fp32 arithmetic: the two-kernel form
+    assert q(_lib.ROUTE_MIXER_MR_PLANAR, 2, 8192, 256, 16, 128, 3, bf16) == 1
+    assert q(_lib.ROUTE_MIXER_MR_PLANAR, 2, 8192, 256, 16, 128, 3, mixed) == 0   # planar features: one-kernel form only
+    assert q(_lib.ROUTE_MIXER_MR_PLANAR, 2, 8192, 256, 16, 128, 3, f32) == 0
+    assert q(_lib.ROUTE_MIXER_MR, 2, 8192, 256, 16, 128, 0, bf16) == -1      # a mixer route needs the featurizer's length
+    assert q(99, 2, 8192, 256, 16, 128, 3, bf16) == -1 and q(_lib.ROUTE_DECAY, 0, 8192, 256, 16, 128, 0, bf16) == -1
+    # window limits: rows too wide for the shortest run with its lead-in to fit one tensor window
+    wide_g = 1 << 17                                                        # d = 2 M channels
+    assert q(_lib.ROUTE_DECAY, 1, 4096, wide_g, 16, 128, 0, bf16) == 0
+    assert q(_lib.ROUTE_MIXER_MR, 1, 4096, wide_g, 16, 128, 3, bf16) == 0
+    assert q(_lib.ROUTE_TIME_MAJOR, 4096, 64, 4096, 16, 7, 0, bf16) == 0     # bs * d elements per time row
+    assert q(_lib.ROUTE_TIME_MAJOR, 4, 64, 4096, 16, 7, 0, bf16) == 1
+    # the predicates: same answers (meta tensors carry the shapes; alignment is not in question here)
+    def meta(*shape):
+        return torch.empty(*shape, dtype=torch.bfloat16, device="meta")
+    import unittest.mock as mock
+    with mock.patch.object(_lib, "_all_aligned16", lambda *a, **k: True):
+        assert _lib.time_major_supported(16, 7, meta(64, 4, 4096, 16))
+        assert not _lib.time_major_supported(16, 7, meta(64, 4096, 4096, 16))
+        assert _lib.decay_supported(256, 16, 128, meta(2, 8192, 256, 16))
+        assert not _lib.decay_supported(wide_g, 16, 128, meta(1, 4096, wide_g, 16))
+        assert _lib.mixer_mr_supported(16, 128, 3, sizes=(2, 8192, 256, bf16))
+        assert not _lib.mixer_mr_supported(16, 128, 3, sizes=(1, 4096, wide_g, bf16))
+        assert not _lib.mixer_mr_supported(16, 128, 3, planar=True, sizes=(2, 8192, 256, mixed))
+        assert _lib.mixer_mr_supported(16, 128, 3)                           # shape rules only, as before
