@@ -560,6 +560,103 @@ def power_table(device, secs=2.0):
     return {"kernels": rows, "idle": idle}
 
 
+TRACE_LIB = os.path.join(ROOT, "savanna_amd", "csrc", "libgcg_hip_trace.so")
+
+
+def timeline_table(device, workload="mr_fwdbwd_7b", reps=5):
+    """Per-workgroup timestamps inside the two matrix-core kernels of a separate-tensor workload: where a launch's
+    time goes (start, prologue, walk, spread between the first and the last workgroup to finish, filter-gradient
+    tail).  Uses the trace build of the library (`make -C savanna_amd/csrc trace`: libgcg_hip_trace.so, the same
+    kernels with thread 0 of every workgroup storing the 100 MHz constant clock at its start, at the start and end
+    of its walk and at its end) through the C ABI; one launch of each kernel per repetition, after warm-up, inputs
+    rotated.  Times are microseconds from the first start on the workgroup's own XCD (the XCDs' clocks are offset
+    against each other).  The stamps cost the forward about 3 us per launch (it is sensitive to any further store)
+    and the backward nothing measurable; the same launch's duration by HIP events is reported beside them."""
+    import ctypes
+    import statistics
+
+    if not os.path.exists(TRACE_LIB):
+        raise SystemExit(f"bench.py --timeline needs {TRACE_LIB}: run `make -C savanna_amd/csrc trace`")
+    wl = WORKLOADS[workload]
+    if wl.layout != "separate" or len(wl.filters) != 1:
+        raise SystemExit("--timeline takes a separate-tensor workload with one filter")
+    lib = ctypes.CDLL(TRACE_LIB)
+    vp, i64, i32 = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32
+    lib.gcg_fwd.argtypes = [vp] * 7 + [i64, i64, i32, i32, i32, i32, i32, vp]
+    lib.gcg_bwd.argtypes = [vp] * 10 + [ctypes.c_size_t, i64, i64, i32, i32, i32, i32, i32, vp]
+    lib.gcg_bwd_workspace_bytes.argtypes = [i64, i64, i32, i32, i32, i32, i32]
+    lib.gcg_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.gcg_trace_buffer.argtypes = [ctypes.POINTER(ctypes.c_size_t)]
+    lib.gcg_trace_buffer.restype = vp
+    hl = wl.filters[0]
+    code = _lib.dtype_code(wl.dtype)
+    sets = [make_inputs_device(wl.bs, wl.L, wl.g, wl.dg, hl, wl.dtype, device, seed=i, with_dy=True) for i in range(3)]
+    y, dx, dB, dC = (torch.empty_like(sets[0]["k"]) for _ in range(4))
+    dh = torch.empty_like(sets[0]["h"])
+    nws = lib.gcg_bwd_workspace_bytes(wl.bs, wl.L, wl.g, wl.dg, hl, code, 0)
+    ws = torch.empty(nws + 256, dtype=torch.uint8, device=device)
+    st = torch.cuda.current_stream().cuda_stream
+    dims = (wl.bs, wl.L, wl.g, wl.dg, hl, code, 0, st)
+
+    def fwd(t):
+        rc = lib.gcg_fwd(t["k"].data_ptr(), t["q"].data_ptr(), t["v"].data_ptr(), t["h"].data_ptr(), y.data_ptr(), None, None, *dims)
+        assert rc == 0, rc
+
+    def bwd(t):
+        rc = lib.gcg_bwd(t["dy"].data_ptr(), t["k"].data_ptr(), t["q"].data_ptr(), t["v"].data_ptr(), t["h"].data_ptr(),
+                         dx.data_ptr(), dB.data_ptr(), dC.data_ptr(), dh.data_ptr(), ws.data_ptr(), nws, *dims)
+        assert rc == 0, rc
+
+    nbytes = ctypes.c_size_t()
+    tptr = lib.gcg_trace_buffer(ctypes.byref(nbytes))
+    hip = KernelEvents(0).hip
+    hip.hipMemset.argtypes = [vp, ctypes.c_int, ctypes.c_size_t]
+    hip.hipMemcpy.argtypes = [vp, vp, ctypes.c_size_t, ctypes.c_int]
+    # workgroup counts from the library's own plan: the table is cleared, and the slots that a launch stamped are its workgroups
+    take = 4096 * 16 * 8
+    host = (ctypes.c_uint64 * (take // 8))()
+    t_end = time.perf_counter() + 0.4
+    i = 0
+    while time.perf_counter() < t_end:
+        fwd(sets[i % 3]); bwd(sets[i % 3]); i += 1
+        torch.cuda.synchronize()
+    out = {}
+    for name, run in (("forward", fwd), ("backward", bwd)):
+        rows = []
+        for rep in range(reps):
+            for k in range(4):
+                fwd(sets[(i + k) % 3]); bwd(sets[(i + k) % 3])
+            torch.cuda.synchronize()
+            assert hip.hipMemset(tptr, 0, take) == 0
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(); run(sets[(i + rep) % 3]); e1.record()
+            torch.cuda.synchronize()
+            assert hip.hipMemcpy(host, tptr, take, 2) == 0
+            import numpy as np
+            a = np.frombuffer(host, dtype=np.uint64).reshape(-1, 16).astype(np.int64)
+            a = a[a[:, 0] != 0]
+            t = a / 100.0
+            xcd = np.arange(len(t)) % 8
+            base = np.array([t[xcd == x, 0].min() for x in range(8)])
+            t = t - base[xcd][:, None]
+            last = 7 if (a[:, 7] != 0).all() else 6
+            rows.append({
+                "workgroups": int(len(t)), "event_us": e0.elapsed_time(e1) * 1e3,
+                "start_median": float(np.median(t[:, 0])), "start_last": float(t[:, 0].max()),
+                "prologue_median": float(np.median(t[:, 5] - t[:, 0])),
+                "walk_min": float((t[:, 6] - t[:, 5]).min()), "walk_median": float(np.median(t[:, 6] - t[:, 5])),
+                "walk_max": float((t[:, 6] - t[:, 5]).max()),
+                "walk_end_median": float(np.median(t[:, 6])), "walk_end_last": float(t[:, 6].max()),
+                "tail_median": float(np.median(t[:, last] - t[:, 6])), "tail_max": float((t[:, last] - t[:, 6]).max()),
+                "end_median": float(np.median(t[:, last])), "end_last": float(t[:, last].max()),
+                "walk_end_mean_by_xcd": [round(float(t[xcd == x, 6].mean()), 2) for x in range(8)],
+            })
+        out[name] = {k: (round(statistics.median(r[k] for r in rows), 2) if not isinstance(rows[0][k], list) else rows[len(rows) // 2][k])
+                     for k in rows[0]}
+        out[name]["launches"] = reps
+    return out
+
+
 def main():
     global KEEP_INTERMEDIATES, SETTLE_S
     ap = argparse.ArgumentParser()
@@ -583,6 +680,10 @@ def main():
     ap.add_argument("--power", action="store_true",
                     help="print shader clock and board power (sysfs) under each Hyena-MR kernel launched back to "
                          "back, with the time per call, as one JSON line, and exit")
+    ap.add_argument("--timeline", action="store_true",
+                    help="print per-workgroup timestamps inside the two matrix-core kernels of the workload (start, "
+                         "prologue, walk, finishing spread, filter-gradient tail) from the trace build of the library "
+                         "(make -C savanna_amd/csrc trace), as one JSON line, and exit")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy three times, so a counter profile of this "
                          "command holds a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -603,6 +704,11 @@ def main():
     if args.kernels:
         print(json.dumps({"single_kernels": kernel_table(device, n=max(10, args.steps)), "unit": "us, GB/s of algorithmic "
                           "bytes (4 tensors forward, 7 backward), fraction of 8 TB/s"}), flush=True)
+        return
+
+    if args.timeline:
+        print(json.dumps({"timeline": timeline_table(device, args.workload), "workload": args.workload,
+                          "unit": "us from the first workgroup start on the same XCD; medians over the launches"}), flush=True)
         return
 
     if args.power:

@@ -13,6 +13,13 @@
 // lane owns NR = 4 (16-bit) or 8 (fp32) rows of a 32-row step, RP = 32/NR rows apart.
 #include "gcg_il_tile.h"
 
+// Cache policy of the forward's output stores on 16-bit tensors (gcg_common.h: 2 = nontemporal, 16 = device scope:
+// written through the XCD's L2).  As in gcg_mfma.hip the device-scope store measured faster: 96.5 against 98.5 us at
+// the 7B layer shape.
+#ifndef GCG_MFMA_IL_FWD_ST
+#define GCG_MFMA_IL_FWD_ST 16
+#endif
+
 namespace gcg {
 namespace {
 
@@ -38,10 +45,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     __shared__ __attribute__((aligned(16))) unsigned char y_st[STEP * YROW];
     __shared__ hraw_t htab[NW][HTAB];
 
-    int64_t wg = pl.xcd ? xcd_contiguous_id(blockIdx.x, gridDim.x) : (int64_t)blockIdx.x;
-    const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
-    const int seg = (int)(wg % pl.nseg);
-    const int64_t b = wg / pl.nseg;
+    int cb, seg, bi;
+    wg_place(pl.xcd ? xcd_contiguous_u32(blockIdx.x, gridDim.x) : blockIdx.x, pl, cb, seg, bi);
+    const int64_t b = bi;
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
     const int rr = tid / LPR, a = tid % LPR;        // memory layout: rows row0 + KS*k, channels CH*a ..
@@ -97,7 +103,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     // The filter taps of this wave's group are requested before any row, so that the filter table and the
     // Toeplitz tiles are built while the rows are in flight (loads complete in order of issue).
     hraw_t hv[HTAB / 64];
-    load_taps<T>(dm, h, (c0 + 16 * w < d) ? (c0 + 16 * w) / dm.dg : 0, l, hv);
+    load_taps<T>(dm, h, (c0 + 16 * w < d) ? fdiv((uint32_t)(cb * NW + w), pl.q_dg16) : 0, l, hv);
 
     // A segment that starts inside the sequence first rebuilds the operands of the NK-1 steps
     // before it; their rows are requested together (one memory latency instead of NK-1) and
@@ -168,7 +174,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 #pragma unroll
                     for (int c = 0; c < CH; ++c)
                         yf[c] = Cf[CH * k + c] * *(const float *)(y_rd + KS * k * YROW + 4 * c);
-                    stw4(wy, o + k * pass_off, pack_unit<T>(yf));
+                    __builtin_amdgcn_raw_buffer_store_b32(pack_unit<T>(yf), wy, (int)(o + k * pass_off), 0,
+                                                          M::ES == 2 ? GCG_MFMA_IL_FWD_ST : WIN_NT_ST);
                 }
 #pragma unroll
                 for (int k = 0; k < NH + NR; ++k) in[k] = nx[k];
@@ -227,11 +234,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     unsigned char *u_rm = smem + OFF_U, *g_rm = smem + OFF_G, *y_st = smem + OFF_Y, *d_st = smem + OFF_D;
     hraw_t *htab = (hraw_t *)(smem + OFF_H);
 
-    const int64_t wg_id = xcd_contiguous_id(blockIdx.x, gridDim.x);
-    int64_t wg = wg_id;
-    const int cb = (int)(wg % pl.ncb); wg /= pl.ncb;
-    const int seg = (int)(wg % pl.nseg);
-    const int64_t b = wg / pl.nseg;
+    const uint32_t wg_id = xcd_contiguous_u32(blockIdx.x, gridDim.x);
+    int cb, seg, bi;
+    wg_place(wg_id, pl, cb, seg, bi);
+    const int64_t b = bi;
 
     const int tid = threadIdx.x, w = tid >> 6, l = tid & 63;
     const int rr = tid / LPR, a = tid % LPR;        // memory layout: rows row0 + KS*k, channels CH*a ..
@@ -313,7 +319,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     Row<T> dyr;
     // The filter taps of this wave's group are requested before any row (loads complete in order of issue).
     hraw_t hv[HTAB / 64];
-    load_taps<T>(dm, h, wave_valid ? (c0 + 16 * w) / dm.dg : 0, l, hv);
+    load_taps<T>(dm, h, wave_valid ? fdiv((uint32_t)(cb * NW + w), pl.q_dg16) : 0, l, hv);
 
     // Lead-in: the rows of the NK-1 steps before the segment (for u) and of its first NK-1 steps
     // (for g2, and x, B to wait in the ring), i.e. what iterations s_lo-NK+1 .. s_lo-1 would have
