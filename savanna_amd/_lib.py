@@ -639,6 +639,7 @@ def _all_aligned16(tensors, skip_strided=False) -> bool:
 ROUTE_DECAY, ROUTE_TIME_MAJOR, ROUTE_MIXER_SE, ROUTE_MIXER_MR, ROUTE_MIXER_MR_PLANAR = 1, 2, 3, 4, 5
 
 
+@torch.compiler.assume_constant_result      # sizes in, a bool out: torch.compile evaluates it while tracing
 def route_supported(route: int, bs: int, L: int, g: int, dg: int, hl: int, kf: int, code: int) -> bool:
     """gcg_route_supported: whether the entry points of a route take these sizes (every limit the library checks
     apart from the tensors' alignment: filter lengths, group widths, what a tensor window can span)."""

@@ -694,7 +694,14 @@ int choose_nw(const Dims &dm, bool fp32)
 {
     static const int forced = env_int("GCG_MFMA_NW", 0);   // tuning override: 4, 8 or 16
     if (forced == 4 || forced == 8 || (forced == 16 && !fp32)) return forced;
-    if (dm.d >= 256 && !fp32) return 16;
+    if (dm.d >= 256 && !fp32) {
+        // A tensor so small that 16-wave workgroups, one per CU, would get runs of fewer than 16 steps is better
+        // served by twice as many 8-wave workgroups (two per CU): (1, 8192, 1024) 16.9 against 22.2 us,
+        // (1, 8192, 2048) 28.6 against 34.8, (1, 4096, 4096) 28.9 against 31.9; from runs of 16 steps on the wide
+        // workgroups win again ((4, 8192, 1024) 50.4 against 52.3, (1, 8192, 4096) 51.2 against 52.7).
+        const int64_t col_steps = dm.bs * ((dm.d + 255) / 256) * ((dm.L + STEP - 1) / STEP);
+        return col_steps < 16 * (int64_t)cu_count() ? 8 : 16;
+    }
     if (dm.d >= 128) return 8;
     return 4;
 }
