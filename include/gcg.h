@@ -36,8 +36,10 @@ extern "C" {
  * call when `cgcg_dtype` ("float32", the default) differs from the activations' dtype
  * (savanna/model/operators/hyena/hyena.py:499-503 and :533-534, :805-817): the tensors
  * x, B, C, y, dy, dx, dB, dC are 16-bit, the filter h and its gradient dh are fp32, and
- * nothing is rounded to 16 bits between a load and a store -- the values are those of
- * `op(x.float(), B.float(), C.float(), h).to(bf16)` and of its autograd backward.
+ * no activation is rounded to 16 bits between a load and a store -- the values are those of
+ * `op(x.float(), B.float(), C.float(), h).to(bf16)` and of its autograd backward, with one
+ * qualification in the matrix-core kernels: the taps enter the products with 16 significant
+ * bits (2^-17 relative, far below the 16-bit outputs' own rounding; dh is not affected).
  * gcg_fwd, gcg_bwd, gcg_bwd_static, gcg_fwd_interleaved, gcg_bwd_interleaved take them
  * (every kernel family); the featurizer entry points do not (GCG_ERR_BAD_ARG). */
 enum { GCG_F32 = 0, GCG_BF16 = 1, GCG_F16 = 2, GCG_BF16_F32 = 3, GCG_F16_F32 = 4 };
