@@ -153,20 +153,25 @@ template <> struct MT<f16_t> : MT16<f16x8> {
 // fp32 matrix path.  Operand tiles in LDS hold the planes of a row side by side (plane m at byte offset
 // m * plane(urow)), each laid out like a 16-bit tile, so operands come from the same transposing reads.
 //
-// NPA = planes of an activation operand.  fp32 tensors: 3.  bf16 tensors computed in fp32 (the pre-gate product
-// of two bf16 values has 16 significant bits): 2 exactly, and 4 terms, all exact, in the filter-gradient product of
-// two activation operands.
+// NPA = planes of an activation operand.  fp32 tensors: 3.  bf16 tensors computed in fp32: 2, exactly (the pre-gate
+// product of two bf16 values has 16 significant bits).  f16 tensors computed in fp32: 3 (22 significant bits).
 // NPW = planes of a filter operand.  fp32 tensors: 3 (results to fp32 accuracy).  16-bit tensors with an fp32
 // filter: 2 -- the taps enter the products rounded to 16 significant bits (2^-17 relative), 256 times below the
 // resolution of the 16-bit outputs they are rounded to (over 99 % of the outputs still equal the exact result
-// rounded once); the filter gradient does not involve the filter and stays exact.  4 terms (5 for f16 tensors)
-// instead of 5 (6): these kernels run at the board's power limit, and a fifth fewer matrix instructions is 8 - 9 %
-// of their time (7B layer shape: forward 109 -> 99 us, backward 282 -> 261 us).
+// rounded once).
+// SUM = the largest m + n of the plane products a_m b_n that are formed.  2 for fp32 and f16 tensors (6 and 5
+// terms).  1 for bf16 tensors: the term left out, low plane times low plane, is at most 2^-18 of |a b|, which is
+// 2^-9 of an output's last bit and, in the filter gradient, four orders of magnitude below what adding bs L dg
+// products in fp32 leaves.  3 terms instead of 4: a single wave issues matrix and vector instructions strictly one
+// after the other, so with one wave per SIMD every matrix instruction left out is time saved (7B layer shape, bf16
+// tensors in fp32 arithmetic: forward 109 -> 99 -> 95.5 us, backward 282 -> 257 -> 232 us for 3 -> 2 filter
+// planes -> 3 terms).
 template <int NPA> struct SplitOp { bf16x8 p[NPA]; };
-template <int NPA_, int NPW_> struct MTSplit {
+template <int NPA_, int NPW_, int SUM_> struct MTSplit {
     static constexpr int LES = 2;
     static constexpr bool SPLIT = true;
     static constexpr int NPA = NPA_, NPW = NPW_;
+    static constexpr int SUM = SUM_;             // plane products a_m b_n with m + n <= SUM are formed
     static constexpr int RPAD = 32;              // with it consecutive rows start an odd multiple of 8 banks apart
     static constexpr int urow(int cb) { return NPA * cb * 2 + RPAD; }
     static __device__ __forceinline__ int plane(int urow) { return (urow - RPAD) / NPA; }   // bytes between planes
@@ -236,7 +241,7 @@ template <int NPA_, int NPW_> struct MTSplit {
     static __device__ __forceinline__ f32x4 mfma_terms(const SplitOp<NA> &a, const SplitOp<NB> &b, f32x4 c)
     {
 #pragma unroll
-        for (int sum = 2; sum >= 0; --sum)
+        for (int sum = SUM; sum >= 0; --sum)
 #pragma unroll
             for (int m = 0; m <= sum; ++m)
                 if (m < NA && sum - m < NB)
@@ -270,19 +275,19 @@ template <int NPA_, int NPW_> struct MTSplit {
         }
     }
 };
-template <> struct MT<float> : MTSplit<3, 3> {
+template <> struct MT<float> : MTSplit<3, 3, 2> {
     static constexpr int ES = 4;                 // bytes per element in memory
     static constexpr int RW = 2;                 // 16-byte words per 8-channel row vector
 };
 // bf16 / f16 tensors, fp32 filter, fp32 arithmetic: what a 16-bit model gets from the operator run "in fp32"
 // (every tensor cast up before it and the result cast down after), without the casts.
-template <> struct MT<bf16w_t> : MTSplit<2, 2> {
+template <> struct MT<bf16w_t> : MTSplit<2, 2, 1> {
     static constexpr int ES = 2;
     static constexpr int RW = 1;
     static __device__ __forceinline__ void unpack2(uint32_t p, float &lo, float &hi) { MT<bf16_t>::unpack2(p, lo, hi); }
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_bf16x2(lo, hi); }
 };
-template <> struct MT<f16w_t> : MTSplit<3, 2> {
+template <> struct MT<f16w_t> : MTSplit<3, 2, 2> {
     static constexpr int ES = 2;
     static constexpr int RW = 1;
     static __device__ __forceinline__ void unpack2(uint32_t p, float &lo, float &hi) { MT<f16_t>::unpack2(p, lo, hi); }
