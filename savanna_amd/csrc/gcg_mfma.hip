@@ -505,6 +505,297 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     TR(7);
 }
 
+// Which element types take the two-kinds-of-waves backward below: bf16 tensors in fp32 arithmetic.  Plain 16-bit tensors
+// wait for memory, not for instructions (bf16: 181 us against 173 with mfma_bwd_kernel); three-plane operands (f16
+// tensors in fp32 arithmetic, fp32 tensors) need 171 KB of LDS for its tiles.
+template <typename T> constexpr bool duo_type() { return std::is_same<T, bf16w_t>::value; }
+
+// --------------------------------------------------------------------------- backward, product waves and row waves
+// The split-arithmetic backward is bound by instruction issue, not by memory (its 87 matrix instructions per step
+// alone are 1600 cycles), and a SIMD runs matrix and vector instructions one after the other whether they come from
+// one wave or from two (16 v_mfma_f32_16x16x32_bf16 take 312 cycles, 128 v_fma_f32 from a second wave 380, both 707).
+// What a second wave per SIMD can hide is the waiting: LDS round trips, barriers, rows in flight.  The register state of
+// mfma_bwd_kernel allows one wave per SIMD, so this kernel splits it over two kinds of waves in one workgroup of 512
+// threads, one of each kind per SIMD, for the same 16 x 4 channels:
+//   product waves (0..3): the Toeplitz operands, the u and g2 operand rings and the y2 / du products of a step;
+//   row waves (4..7): global loads and stores, the gates before and after the products, and the filter-gradient
+//     products (their operands are rows in natural order, which the row waves have just written).
+// They meet at one barrier per step.  Iteration sigma: the product waves work on step sigma (operands written to LDS
+// during iteration sigma-1, results to the y2 / du tiles of sigma's parity); the row waves finish step sigma-1 from
+// the tiles of the other parity, prepare step sigma+1 (u, g2 of step sigma+NK into the tiles of the other parity and
+// into a ring of NK+1 steps of g2) and accumulate the filter-gradient tiles of step sigma from the ring.
+// Five-slice filters only (the rings' periods fix the unrolling: 2 NK for the product waves, NK+1 for the row waves).
+template <typename T, bool PL = false>
+__global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__ dy, const T *__restrict__ x,
+                                                       const T *__restrict__ B, const T *__restrict__ C,
+                                                       const T *__restrict__ h, T *__restrict__ dx,
+                                                       T *__restrict__ dB, T *__restrict__ dC,
+                                                       T *__restrict__ dh, float *__restrict__ ws, Dims dm,
+                                                       MfmaPlan pl)
+{
+    constexpr int NK = 5, NW = 4;
+    typedef MT<T> M;
+    typedef typename M::op_t op_t;
+    typedef typename M::hraw_t hraw_t;
+    typedef Geo<T, NW> G;
+    constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW, ES = M::ES;
+    constexpr int ND = 2 * NK - 1, RSLOTS = NK + 1;
+    constexpr int USZ = STEP * UROW, YSZ = STEP * YROW, RING_ROWS = STEP * RSLOTS;
+    constexpr int OFF_U = 0;                                // u of a step: even steps, odd steps
+    constexpr int OFF_GN = OFF_U + 2 * USZ;                 // g2 of the newest step, for the product waves
+    constexpr int OFF_R = OFF_GN + 2 * USZ;                 // g2 ring of NK+1 steps, for the filter gradient
+    constexpr int OFF_Y = OFF_R + RSLOTS * USZ;             // y2 tiles, fp32
+    constexpr int OFF_D = OFF_Y + 2 * YSZ;                  // du tiles, fp32
+    constexpr int OFF_H = OFF_D + 2 * YSZ;                  // filter tables
+    constexpr int LDS_MAIN = OFF_H + NW * HTAB * (int)sizeof(hraw_t);
+    constexpr int LDS_TAIL = NW * (16 * ND + 16) * 17 * 4;  // P tiles at the end (dh_finish)
+    constexpr int LDS_BYTES = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
+    static_assert(LDS_BYTES <= 160 * 1024, "tiles do not fit the CU's LDS");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
+    hraw_t *htab = (hraw_t *)(smem + OFF_H);
+    unsigned char *const ring = smem + OFF_R;
+    TR_INIT;
+    TR(0);
+
+    const uint32_t wg_id = xcd_contiguous_u32(blockIdx.x, gridDim.x);
+    int cb, seg, bi;
+    wg_place(wg_id, pl, cb, seg, bi);
+    const int64_t b = bi;
+
+    const int tid = threadIdx.x, wv = tid >> 6, l = tid & 63;
+    const bool row_wave = wv >= NW;
+    const int w = wv & (NW - 1);                    // the wave's 16-channel block (either kind)
+    const int vt = tid & (64 * NW - 1);             // row layout of the row waves: row r of the step, channels 8a..8a+7
+    const int r = vt / G::LPR, a = vt % G::LPR;
+    const int j = l & 15, q = l >> 4;               // matrix layout
+    const int64_t d = dm.d, L = dm.L;
+    const int64_t c0 = (int64_t)cb * CB;
+    const bool wave_valid = c0 + 16 * w < d;
+
+    const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
+    const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
+
+    f32x4 P[ND];
+#pragma unroll
+    for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if (!row_wave) {
+        // ------------------------------------------------------------------ product waves
+        hraw_t hv[HTAB / 64];
+        load_taps<T>(dm, h, wave_valid ? fdiv((uint32_t)(cb * NW + w), pl.q_dg16) : 0, l, hv);
+        op_t Au[NK], Ag[NK];
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            Au[i] = M::zero_op();
+            Ag[i] = M::zero_op();
+        }
+        const int y_wr = j * YROW + (16 * w + 4 * q) * 4;
+        const int d_wr = (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
+        store_taps(htab + w * HTAB, l, hv);
+        __syncthreads();                                              // (A)
+        typename M::wop_t W0[NK], W1[NK];
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
+            W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
+        }
+#pragma unroll
+        for (int i = 1; i < NK; ++i) {
+            __syncthreads();                                          // (B_i) lead-in tiles written
+            Au[NK - i] = M::load_operand(smem + OFF_U, UROW, w, j, q, false);
+            Ag[NK - 1 - i] = M::load_operand(smem + OFF_GN, UROW, w, j, q, true);
+            __syncthreads();                                          // (C_i) and read
+        }
+        __syncthreads();                                              // (D) step s_lo prepared
+        TR(5);
+        int64_t s = s_lo;
+        auto product_step = [&](int pu) __attribute__((always_inline)) {
+                    const int ph = pu % NK, par = pu & 1;
+                    const int slot_new = (ph + NK - 1) % NK;
+                    Au[ph] = M::load_operand(smem + OFF_U + par * USZ, UROW, w, j, q, false);
+                    Ag[slot_new] = M::load_operand(smem + OFF_GN + par * USZ, UROW, w, j, q, true);
+                    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+                    f32x4 dac0 = {0.f, 0.f, 0.f, 0.f}, dac1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                    for (int i = 0; i < NK; ++i) {
+                        acc0 = M::mfma(Au[(ph - i + NK) % NK], W0[i], acc0);
+                        acc1 = M::mfma(Au[(ph - i + NK) % NK], W1[i], acc1);
+                        dac0 = M::mfma(Ag[(ph + i) % NK], W1[i], dac0);   // output rows 0..15
+                        dac1 = M::mfma(Ag[(ph + i) % NK], W0[i], dac1);   // output rows 16..31
+                    }
+                    unsigned char *const y_cur = smem + OFF_Y + par * YSZ, *const d_cur = smem + OFF_D + par * YSZ;
+                    *(f32x4 *)(y_cur + y_wr) = acc0;
+                    *(f32x4 *)(y_cur + y_wr + 16 * YROW) = acc1;
+                    *(f32x4 *)(d_cur + d_wr) = dac0;
+                    *(f32x4 *)(d_cur + d_wr + 16 * YROW) = dac1;
+                    __syncthreads();
+                    ++s;
+        };
+        while (s < s_hi) {
+#pragma unroll
+            for (int pu = 0; pu < 2 * NK; ++pu)
+                if (s < s_hi) product_step(pu);
+        }
+    } else {
+        // ------------------------------------------------------------------ row waves
+        // windows as in mfma_bwd_kernel: x, B and the outputs over rows [t0, t1), dy and C over [t0, t2)
+        const int64_t t0 = (s_lo - (NK - 1)) * STEP > 0 ? (s_lo - (NK - 1)) * STEP : 0;
+        const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
+        const int64_t t2 = (s_hi + NK - 1) * STEP < L ? (s_hi + NK - 1) * STEP : L;
+        const int64_t row_bytes = d * ES, origin = (b * L + t0) * d;
+        const int64_t near_bytes = (t1 - t0) * row_bytes, far_bytes = (t2 - t0) * row_bytes;
+        constexpr int IM = PL ? 3 : 1;                  // row stride of x, B, C, dx, dB, dC in rows of dy
+        const win_t wx = make_window(x + IM * origin, IM * near_bytes), wB = make_window(B + IM * origin, IM * near_bytes);
+        const win_t wdy = make_window(dy + origin, far_bytes), wC = make_window(C + IM * origin, IM * far_bytes);
+        const win_t wdx = make_window(dx + IM * origin, IM * near_bytes), wdB = make_window(dB + IM * origin, IM * near_bytes);
+        const win_t wdC = make_window(dC + IM * origin, IM * near_bytes);
+        const uint32_t lane_off = (uint32_t)(r * row_bytes + (c0 + 8 * a) * ES) + (c0 + 8 * a < d ? 0u : WIN_OFF);
+        const uint32_t lane_in = PL ? (uint32_t)(r * IM * row_bytes + (c0 + 8 * a) * ES) + (c0 + 8 * a < d ? 0u : WIN_OFF) : lane_off;
+        auto step_off = [&](int64_t sg) { return (uint32_t)((sg * STEP - t0) * row_bytes); };
+        const int rm_off = r * UROW + 8 * M::LES * a;
+        const int yd_rd = r * YROW + 32 * a;
+
+        // rows of iteration sg: x, B of step sg and dy, C of step sg+NK-1 (zero outside the windows)
+        auto fetch = [&](int64_t sg, Row<T> &xo, Row<T> &Bo, Row<T> &dyo, Row<T> &Co) {
+            const uint32_t o = lane_in + IM * step_off(sg), o2 = lane_off + step_off(sg + NK - 1);
+            xo = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wx, o);
+            Bo = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wB, o);
+            dyo = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wdy, o2);
+            Co = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wC, PL ? lane_in + IM * step_off(sg + NK - 1) : o2);
+        };
+        // u = x * B into a u tile; g2 = dy * C into a newest-step tile and into a slot of the ring
+        auto gate_rows = [&](const Row<T> &xo, const Row<T> &Bo, const Row<T> &dyo, const Row<T> &Co, unsigned char *u_t,
+                             unsigned char *g_t, unsigned char *g_ring) {
+            float f0[8], f1[8], pf[8];
+            unpack8<T>(xo, f0);
+            unpack8<T>(Bo, f1);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
+            store_operand<T>(u_t + rm_off, UROW, pf);
+            unpack8<T>(dyo, f0);
+            unpack8<T>(Co, f1);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
+            store_operand<T>(g_t + rm_off, UROW, pf);
+            store_operand<T>(g_ring + rm_off, UROW, pf);
+        };
+        // dC, dx, dB of step sg from its y2 / du tiles
+        auto finish_step = [&](int64_t sg, bool live, const unsigned char *y_t, const unsigned char *d_t,
+                               const Row<T> &dyo, const Row<T> &xo, const Row<T> &Bo) {
+            const uint32_t o = live ? lane_in + IM * step_off(sg) : WIN_OFF;
+            {
+                const f32x4 p0 = *(const f32x4 *)(y_t + yd_rd);
+                const f32x4 p1 = *(const f32x4 *)(y_t + yd_rd + 16);
+                const float y2f[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
+                float dyf[8], of[8];
+                unpack8<T>(dyo, dyf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) of[e] = dyf[e] * y2f[e];
+                stw_row_policy<T, GCG_MFMA_BWD_ST_DC>(wdC, o, pack8<T>(of));
+            }
+            {
+                const f32x4 p0 = *(const f32x4 *)(d_t + yd_rd);
+                const f32x4 p1 = *(const f32x4 *)(d_t + yd_rd + 16);
+                const float duf[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
+                float xf[8], Bf[8], of[8];
+                unpack8<T>(xo, xf);
+                unpack8<T>(Bo, Bf);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) of[e] = duf[e] * Bf[e];
+                stw_row_policy<T, GCG_MFMA_BWD_ST>(wdx, o, pack8<T>(of));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) of[e] = duf[e] * xf[e];
+                stw_row_policy<T, GCG_MFMA_BWD_ST>(wdB, o, pack8<T>(of));
+            }
+        };
+
+        // Rings of the row waves, indexed by step - s_lo: x, B of three steps (the one being finished, the one in the
+        // matrix cores, the one being prepared, whose slot the rows in flight take over once it is finished);
+        // dy of NK+1 steps; dy, C of the rows in flight in one of two staging sets.
+        Row<T> xh[3], Bh[3], dyq[RSLOTS], dy_st[2], C_st[2];
+        Row<T> xp = zero_row<T>(), Bp = zero_row<T>(), dyp = zero_row<T>();   // x, B, dy of the step being finished
+#pragma unroll
+        for (int i = 0; i < 3; ++i) xh[i] = Bh[i] = zero_row<T>();
+#pragma unroll
+        for (int i = 0; i < RSLOTS; ++i) dyq[i] = zero_row<T>();
+        Row<T> wx_[NK - 1], wB_[NK - 1], wdy_[NK - 1], wC_[NK - 1];
+#pragma unroll
+        for (int i = 1; i < NK; ++i) fetch(s_lo - i, wx_[i - 1], wB_[i - 1], wdy_[i - 1], wC_[i - 1]);
+        fetch(s_lo, xh[0], Bh[0], dy_st[0], C_st[0]);
+        fetch(s_lo + 1, xh[1], Bh[1], dy_st[1], C_st[1]);
+        TR(1);
+        __syncthreads();                                              // (A)
+#pragma unroll
+        for (int i = 1; i < NK; ++i) {
+            // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
+            gate_rows(wx_[i - 1], wB_[i - 1], wdy_[i - 1], wC_[i - 1], smem + OFF_U, smem + OFF_GN,
+                      ring + (NK - 1 - i) * USZ);
+            dyq[NK - 1 - i] = wdy_[i - 1];
+            __syncthreads();                                          // (B_i)
+            __syncthreads();                                          // (C_i)
+        }
+        // step s_lo is prepared here, as an iteration s_lo-1 would have
+        gate_rows(xh[0], Bh[0], dy_st[0], C_st[0], smem + OFF_U, smem + OFF_GN, ring + (NK - 1) * USZ);
+        dyq[NK - 1] = dy_st[0];
+        __syncthreads();                                              // (D)
+
+        int64_t s = s_lo;
+        auto row_step = [&](int pu) __attribute__((always_inline)) {
+                    const int par = pu & 1;
+                    const unsigned char *const u_cur = smem + OFF_U + par * USZ;
+                    unsigned char *const u_nx = smem + OFF_U + (par ^ 1) * USZ, *const g_nx = smem + OFF_GN + (par ^ 1) * USZ;
+                    const unsigned char *const y_old = smem + OFF_Y + (par ^ 1) * YSZ, *const d_old = smem + OFF_D + (par ^ 1) * YSZ;
+                    // Order: the request for rows first, then the stores, then what needs the previous request's rows, the
+                    // filter-gradient products last.  Measured at the 7B shape: products first 240 us, stores before the
+                    // request 218, this order 203 - 205, the gating after the products 221.
+                    // rows of iteration s+2 into the slots that step s-1 has left (past the segment: outside the windows)
+                    fetch(s + 2, xh[(pu + 2) % 3], Bh[(pu + 2) % 3], dy_st[par], C_st[par]);
+                    // step s-1: gate its tiles and store
+                    finish_step(s - 1, s > s_lo, y_old, d_old, dyp, xp, Bp);
+                    // step s+1: its rows arrived during the last iteration
+                    dyq[(pu + RSLOTS - 1) % RSLOTS] = dy_st[par ^ 1];          // dy of step s+NK
+                    gate_rows(xh[(pu + 1) % 3], Bh[(pu + 1) % 3], dy_st[par ^ 1], C_st[par ^ 1], u_nx, g_nx,
+                              ring + ((pu + RSLOTS - 1) % RSLOTS) * USZ);
+                    // filter-gradient tiles of step s: natural-layout operands (rows j and 16+j of a 32-row window)
+                    {
+                        const op_t un = M::load_natural(u_cur + j * UROW, u_cur + (16 + j) * UROW, UROW, w, q);
+#pragma unroll
+                        for (int dl = 0; dl < ND; ++dl) {
+                            int row0 = STEP * pu + 16 * dl + j;              // ring rows of the window's two halves
+                            int row1 = row0 + 16;
+                            row0 = (row0 >= RING_ROWS) ? row0 - RING_ROWS : row0;
+                            row1 = (row1 >= RING_ROWS) ? row1 - RING_ROWS : row1;
+                            const op_t gn = M::load_natural(ring + row0 * UROW, ring + row1 * UROW, UROW, w, q);
+                            P[dl] = M::mfma_aa(gn, un, P[dl]);
+                        }
+                    }
+                    dyp = dyq[pu];                 // step s is finished during the next iteration
+                    xp = xh[pu % 3];
+                    Bp = Bh[pu % 3];
+                    __syncthreads();
+                    ++s;
+        };
+        // Every step can be the run's last, so the compiler's wait counts restart at each: a step's request for rows
+        // then goes out once the previous request has been answered.  With the steps in straight-line groups the
+        // counts are exact, two requests are in flight, and the kernel is 9 % slower (222 against 203 us at the 7B
+        // shape): the memory system delivers less with more on the way, as in the other backward kernels.
+        while (s < s_hi) {
+#pragma unroll
+            for (int pu = 0; pu < RSLOTS; ++pu)
+                if (s < s_hi) row_step(pu);
+        }
+        // the last step of the segment: its tiles are those of parity (s_hi - 1 - s_lo) & 1
+        {
+            const int par = (int)((s_hi - 1 - s_lo) & 1);
+            finish_step(s_hi - 1, true, smem + OFF_Y + par * YSZ, smem + OFF_D + par * YSZ, dyp, xp, Bp);
+        }
+    }
+
+    TR(6);
+    dh_finish<T, NW, ND, 512>(P, smem, ws, dh, dm, pl, wg_id, cb, wave_valid, row_wave, w);
+    TR(7);
+}
+
 template <typename T, int NK, int NW>
 int fwd_launch(const void *x, const void *B, const void *C, const void *h, void *y, void *y2, void *bx,
                const Dims &dm, hipStream_t st)
@@ -608,7 +899,15 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (p.fuse_dh && (p.slot = dh_slot_for_stream(st)) < 0) p.fuse_dh = p.slot = 0;   // no ticket set: second launch
     bool launched = false;
-    if constexpr (NK == 5) {
+    if constexpr (NK == 5 && duo_type<T>()) {
+        // product waves and row waves in one workgroup: the types whose backward is bound by instruction issue
+        auto duo = [&](auto kernel) {
+            return launch_main(kernel, dim3((unsigned)p.nwg), dim3(512), st, (const T *)dy, (const T *)x, (const T *)B,
+                               (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC, (T *)dh, (float *)ws, dm, p);
+        };
+        e = dm.planar ? duo(mfma_bwd_duo_kernel<T, true>) : duo(mfma_bwd_duo_kernel<T, false>);
+        launched = true;
+    } else if constexpr (NK == 5) {
         if (dm.planar) {        // instantiated for the five-slice walk only (bwd_t sends every filter length there)
             e = launch_main((mfma_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
                             (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,

@@ -8,6 +8,7 @@
 #include <atomic>
 #include <cstdlib>
 #include <mutex>
+#include <type_traits>
 
 namespace gcg {
 namespace {
@@ -599,26 +600,30 @@ __device__ __forceinline__ void dh_sum_partials2(const float *pa, const float *p
 
 // Tail of both backward kernels.  P: the wave's ND accumulator tiles, P[dl][v] = element
 // (row 4q+v, column j) of tile dl; smem: at least NW*(16*ND+16)*17*4 bytes of LDS that is no longer in use.
-template <typename T, int NW, int ND>
+// NT: threads of the workgroup.  holds_tiles: whether this wave holds accumulator tiles (its channel block is w);
+// workgroups with more waves than channel blocks pass false in the others, which then only help with the sums.
+template <typename T, int NW, int ND, int NT = 64 * NW>
 __device__ __forceinline__ void dh_finish(const f32x4 (&P)[ND], unsigned char *smem, float *__restrict__ ws,
                                           T *__restrict__ dh, const Dims &dm, const MfmaPlan &pl, int64_t wg_id,
-                                          int cb, bool wave_valid)
+                                          int cb, bool wave_valid, bool holds_tiles = true, int w = (int)(threadIdx.x >> 6))
 {
-    const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, j = l & 15, q = l >> 4;
+    const int tid = threadIdx.x, l = tid & 63, j = l & 15, q = l >> 4;
     // The tiles go to LDS one below the other, as one matrix of 16*ND rows (17 floats apart: the diagonal walks
     // below then touch every bank once) followed by 16 rows of zeros.  lag = (row of the matrix) - column, so the
     // partial for a lag is the sum over columns c of element (lag + c, c).
     constexpr int RS = 17, ROWS = 16 * ND + 16;
     __syncthreads();
     float *pt = (float *)smem + w * ROWS * RS;
+    if (holds_tiles) {
 #pragma unroll
-    for (int dl = 0; dl < ND; ++dl)
+        for (int dl = 0; dl < ND; ++dl)
 #pragma unroll
-        for (int v = 0; v < 4; ++v) pt[(16 * dl + 4 * q + v) * RS + j] = P[dl][v];
+            for (int v = 0; v < 4; ++v) pt[(16 * dl + 4 * q + v) * RS + j] = P[dl][v];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) pt[(16 * ND + 4 * q + v) * RS + j] = 0.f;
+        for (int v = 0; v < 4; ++v) pt[(16 * ND + 4 * q + v) * RS + j] = 0.f;
+    }
     __syncthreads();
-    if (wave_valid) {
+    if (holds_tiles && wave_valid) {
         float *out = ws + ((size_t)wg_id * NW + w) * 128;
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
@@ -634,7 +639,7 @@ __device__ __forceinline__ void dh_finish(const f32x4 (&P)[ND], unsigned char *s
 
     const int64_t np = dm.bs * pl.nseg;
     if (!dh_arrive_last(pl, cb, (unsigned int)np)) return;
-    constexpr int CB = 16 * NW, NT = 64 * NW;
+    constexpr int CB = 16 * NW;
     const int gpc = CB / dm.dg, bpg = dm.dg / 16;      // filter groups per channel block, 16-channel blocks per group
     const int row = dm.fw ? dm.lc : dm.hl;              // taps per group in the output
     // a thread takes outputs idx and idx + NT of the block's gpc * row together (one memory latency for both)
