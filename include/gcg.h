@@ -149,6 +149,18 @@ GCG_API size_t gcg_bwd_workspace_bytes(int64_t bs, int64_t L, int32_t g, int32_t
  *   dh           out, (g, 1, hl), element type `dtype`, overwritten (not accumulated)
  *   workspace    device scratch of at least gcg_bwd_workspace_bytes(...) bytes,
  *                256-byte aligned; contents on entry are ignored
+ *
+ * Streams (this and every other backward entry point of the matrix-core kernels): the last
+ * workgroup of a channel block to finish adds the block's filter-gradient partials, and
+ * which one that is is decided with arrival tickets kept inside the library.  A stream
+ * owns one set of tickets from its first such launch until the process ends; launches on
+ * one stream run in order and share the set, launches on different streams never share
+ * one.  Up to 64 streams hold sets; a launch on a further stream, or on a stream that is
+ * being captured into a graph, takes none and adds the partials with a second small kernel
+ * on the same stream instead (same order of summation, same bits).  The rule for callers:
+ * give concurrent launches their own workspace and outputs, as for any kernel; nothing
+ * else.  (A launch that does not run to its end -- a device fault -- leaves its stream's
+ * tickets mid-count; the process's device context does not survive that either.)
  */
 GCG_API int gcg_bwd(const void *dy, const void *x, const void *B, const void *C, const void *h,
             void *dx, void *dB, void *dC, void *dh,
