@@ -769,7 +769,8 @@ def main():
                      "featurizer_fwdbwd_7b", "mixer_fwdbwd_7b",
                      "mixer_fwdbwd_7b_fused", "mixer_fwdbwd_7b_fused_planar", "mixer_fwd_7b", "mixer_fwd_7b_fused",
                      "mixer_se_fwdbwd_40b", "mixer_se_fwdbwd_40b_fused", "mixer_se_fwdbwd_40b_fused_planar",
-                     "mixer_se_fwdbwd_40b_fp32_arith", "mixer_se_fwdbwd_40b_fused_fp32_arith"):
+                     "mixer_se_fwdbwd_40b_fp32_arith", "mixer_se_fwdbwd_40b_fused_fp32_arith",
+                     "mixer_fwdbwd_7b_fp32_arith", "mixer_fwdbwd_7b_fused_fp32_arith"):
             r = time_workload(WORKLOADS[name], device, max(10, args.steps // 2), 4)
             extra[name] = {k: r[k] for k in ("ms_per_step", "tokens_per_s", "step_gbs", "step_hbm_frac")}
         line["next_rows"] = extra

@@ -92,6 +92,31 @@ def test_bwd(gcg_lib, bs, L, g, dg, hl, dtype, algo):
     assert_close(got[3], ref[3], TOL_DH[torch.float32], "dh")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("bs,L", [(2, 8192), (1, 8192 + 77)], ids=["7b", "ragged"])
+def test_full_size_runs(gcg_lib, bs, L, dtype):
+    """fp32 arithmetic at the Evo2-7B layer shape (runs of 128 steps: every phase of the kernels' rings, the
+    lead-in of a run that starts mid-sequence, the ragged last step), four filter groups against the oracle."""
+    g, dg, hl = 256, 16, 128
+    gen = torch.Generator(device=DEV).manual_seed(17)
+    x, B, C = (torch.randn(bs, L, g, dg, generator=gen, device=DEV).to(dtype) for _ in range(3))
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen, device=DEV)).to(dtype)
+    h = torch.randn(g, 1, hl, generator=gen, device=DEV) / hl ** 0.5
+    _, _, y = _lib.fwd(x, B, C, h)
+    dx, dB, dC, dh = _lib.bwd(dy, x, B, C, h)
+    torch.cuda.synchronize()
+    assert _lib.select_algo(bs, L, g, dg, hl, dtype, True) == "mfma"
+    idx = torch.tensor([0, 3, 130, 255], device=DEV)
+    xs, Bs, Cs, dys = (t.index_select(2, idx).float().cpu() for t in (x, B, C, dy))
+    hs = h.index_select(0, idx).cpu()
+    y_ref = oracle.gcg_fwd_oracle(xs, Bs, Cs, hs)
+    ref = oracle.gcg_bwd_oracle(dys, xs, Bs, Cs, hs)
+    check_rounded_once(y.index_select(2, idx), y_ref, dtype, "y")
+    for o, r, n in zip((dx, dB, dC), ref[:3], ("dx", "dB", "dC")):
+        check_rounded_once(o.index_select(2, idx), r, dtype, n)
+    assert_close(dh.index_select(0, idx), ref[3], TOL_DH[torch.float32], "dh")
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("hl", [7, 128])
 def test_interleaved(gcg_lib, dtype, hl):
