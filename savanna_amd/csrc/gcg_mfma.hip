@@ -533,27 +533,17 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
                                                        T *__restrict__ dh, float *__restrict__ ws, Dims dm,
                                                        MfmaPlan pl)
 {
-    constexpr int NK = 5, NW = 4;
-    typedef MT<T> M;
-    typedef typename M::op_t op_t;
-    typedef typename M::hraw_t hraw_t;
-    typedef Geo<T, NW> G;
-    constexpr int CB = G::CB, UROW = G::UROW, YROW = G::YROW, ES = M::ES;
-    constexpr int ND = 2 * NK - 1, RSLOTS = NK + 1;
-    constexpr int USZ = STEP * UROW, YSZ = STEP * YROW, RING_ROWS = STEP * RSLOTS;
-    constexpr int OFF_U = 0;                                // u of a step: even steps, odd steps
-    constexpr int OFF_GN = OFF_U + 2 * USZ;                 // g2 of the newest step, for the product waves
-    constexpr int OFF_R = OFF_GN + 2 * USZ;                 // g2 ring of NK+1 steps, for the filter gradient
-    constexpr int OFF_Y = OFF_R + RSLOTS * USZ;             // y2 tiles, fp32
-    constexpr int OFF_D = OFF_Y + 2 * YSZ;                  // du tiles, fp32
-    constexpr int OFF_H = OFF_D + 2 * YSZ;                  // filter tables
-    constexpr int LDS_MAIN = OFF_H + NW * HTAB * (int)sizeof(hraw_t);
-    constexpr int LDS_TAIL = NW * (16 * ND + 16) * 17 * 4;  // P tiles at the end (dh_finish)
-    constexpr int LDS_BYTES = LDS_MAIN > LDS_TAIL ? LDS_MAIN : LDS_TAIL;
+    typedef DuoGeo<T> D;
+    typedef typename D::M M;
+    typedef typename D::G G;
+    constexpr int NK = D::NK, NW = D::NW, ND = D::ND, RSLOTS = D::RSLOTS;
+    constexpr int CB = G::CB, UROW = D::UROW, YROW = D::YROW, ES = M::ES, USZ = D::USZ, YSZ = D::YSZ;
+    constexpr int OFF_U = D::OFF_U, OFF_GN = D::OFF_GN, OFF_Y = D::OFF_Y, OFF_D = D::OFF_D;
+    constexpr int LDS_MAIN = D::OFF_H + D::H_BYTES;
+    constexpr int LDS_BYTES = LDS_MAIN > D::LDS_TAIL ? LDS_MAIN : D::LDS_TAIL;
     static_assert(LDS_BYTES <= 160 * 1024, "tiles do not fit the CU's LDS");
     __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
-    hraw_t *htab = (hraw_t *)(smem + OFF_H);
-    unsigned char *const ring = smem + OFF_R;
+    unsigned char *const ring = smem + D::OFF_R;
     TR_INIT;
     TR(0);
 
@@ -580,62 +570,7 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
     for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     if (!row_wave) {
-        // ------------------------------------------------------------------ product waves
-        hraw_t hv[HTAB / 64];
-        load_taps<T>(dm, h, wave_valid ? fdiv((uint32_t)(cb * NW + w), pl.q_dg16) : 0, l, hv);
-        op_t Au[NK], Ag[NK];
-#pragma unroll
-        for (int i = 0; i < NK; ++i) {
-            Au[i] = M::zero_op();
-            Ag[i] = M::zero_op();
-        }
-        const int y_wr = j * YROW + (16 * w + 4 * q) * 4;
-        const int d_wr = (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
-        store_taps(htab + w * HTAB, l, hv);
-        __syncthreads();                                              // (A)
-        typename M::wop_t W0[NK], W1[NK];
-#pragma unroll
-        for (int i = 0; i < NK; ++i) {
-            W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
-            W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
-        }
-#pragma unroll
-        for (int i = 1; i < NK; ++i) {
-            __syncthreads();                                          // (B_i) lead-in tiles written
-            Au[NK - i] = M::load_operand(smem + OFF_U, UROW, w, j, q, false);
-            Ag[NK - 1 - i] = M::load_operand(smem + OFF_GN, UROW, w, j, q, true);
-            __syncthreads();                                          // (C_i) and read
-        }
-        __syncthreads();                                              // (D) step s_lo prepared
-        TR(5);
-        int64_t s = s_lo;
-        auto product_step = [&](int pu) __attribute__((always_inline)) {
-                    const int ph = pu % NK, par = pu & 1;
-                    const int slot_new = (ph + NK - 1) % NK;
-                    Au[ph] = M::load_operand(smem + OFF_U + par * USZ, UROW, w, j, q, false);
-                    Ag[slot_new] = M::load_operand(smem + OFF_GN + par * USZ, UROW, w, j, q, true);
-                    f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
-                    f32x4 dac0 = {0.f, 0.f, 0.f, 0.f}, dac1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                    for (int i = 0; i < NK; ++i) {
-                        acc0 = M::mfma(Au[(ph - i + NK) % NK], W0[i], acc0);
-                        acc1 = M::mfma(Au[(ph - i + NK) % NK], W1[i], acc1);
-                        dac0 = M::mfma(Ag[(ph + i) % NK], W1[i], dac0);   // output rows 0..15
-                        dac1 = M::mfma(Ag[(ph + i) % NK], W0[i], dac1);   // output rows 16..31
-                    }
-                    unsigned char *const y_cur = smem + OFF_Y + par * YSZ, *const d_cur = smem + OFF_D + par * YSZ;
-                    *(f32x4 *)(y_cur + y_wr) = acc0;
-                    *(f32x4 *)(y_cur + y_wr + 16 * YROW) = acc1;
-                    *(f32x4 *)(d_cur + d_wr) = dac0;
-                    *(f32x4 *)(d_cur + d_wr + 16 * YROW) = dac1;
-                    __syncthreads();
-                    ++s;
-        };
-        while (s < s_hi) {
-#pragma unroll
-            for (int pu = 0; pu < 2 * NK; ++pu)
-                if (s < s_hi) product_step(pu);
-        }
+        duo_product_waves<T>(smem, h, dm, pl, cb, w, l, wave_valid, s_lo, s_hi);
     } else {
         // ------------------------------------------------------------------ row waves
         // windows as in mfma_bwd_kernel: x, B and the outputs over rows [t0, t1), dy and C over [t0, t2)
@@ -725,6 +660,7 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
         fetch(s_lo + 1, xh[1], Bh[1], dy_st[1], C_st[1]);
         TR(1);
         __syncthreads();                                              // (A)
+        __syncthreads();                                              // (A2)
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
             // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
@@ -756,19 +692,7 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
                     dyq[(pu + RSLOTS - 1) % RSLOTS] = dy_st[par ^ 1];          // dy of step s+NK
                     gate_rows(xh[(pu + 1) % 3], Bh[(pu + 1) % 3], dy_st[par ^ 1], C_st[par ^ 1], u_nx, g_nx,
                               ring + ((pu + RSLOTS - 1) % RSLOTS) * USZ);
-                    // filter-gradient tiles of step s: natural-layout operands (rows j and 16+j of a 32-row window)
-                    {
-                        const op_t un = M::load_natural(u_cur + j * UROW, u_cur + (16 + j) * UROW, UROW, w, q);
-#pragma unroll
-                        for (int dl = 0; dl < ND; ++dl) {
-                            int row0 = STEP * pu + 16 * dl + j;              // ring rows of the window's two halves
-                            int row1 = row0 + 16;
-                            row0 = (row0 >= RING_ROWS) ? row0 - RING_ROWS : row0;
-                            row1 = (row1 >= RING_ROWS) ? row1 - RING_ROWS : row1;
-                            const op_t gn = M::load_natural(ring + row0 * UROW, ring + row1 * UROW, UROW, w, q);
-                            P[dl] = M::mfma_aa(gn, un, P[dl]);
-                        }
-                    }
+                    duo_filter_gradient<T>(P, u_cur, ring, pu, w, l);    // filter-gradient tiles of step s
                     dyp = dyq[pu];                 // step s is finished during the next iteration
                     xp = xh[pu % 3];
                     Bp = Bh[pu % 3];

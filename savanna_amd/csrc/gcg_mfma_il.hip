@@ -475,6 +475,262 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     dh_finish<T, NW, ND>(P, smem, ws, dh, dm, pl, wg_id, cb, wave_valid);
 }
 
+template <typename T> constexpr bool il_duo_type() { return std::is_same<T, bf16w_t>::value; }
+
+// --------------------------------------------------------------------------- backward, product waves and row waves
+// The interleaved-features form of mfma_bwd_duo_kernel (gcg_mfma.hip) for the element types whose backward is bound
+// by instruction issue: four product waves (duo_product_waves) and four row waves in one workgroup, one barrier per
+// step.  The rows of a step arrive as one interleaved piece per lane and row: C of step s+NK goes into g2 at once,
+// x and B of that step wait in a lane-private ring in LDS until step s+NK is the one being prepared.  Iteration s of
+// the row waves: request the rows of step s+NK+1; finish step s-1 (gate its y2 / du tiles, store its interleaved
+// gradient rows); prepare step s+1 (u from the ring, g2 of step s+NK from the rows that arrived); the filter-gradient
+// products of step s.
+template <typename T, bool KEEP, int KF>
+__global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restrict__ dy, const T *__restrict__ feat,
+                                                          const T *__restrict__ h, const T *__restrict__ wfeat,
+                                                          int kf, T *__restrict__ dfeat, T *__restrict__ dh,
+                                                          float *__restrict__ ws, Dims dm, MfmaPlan pl)
+{
+    typedef DuoGeo<T> D;
+    typedef typename D::M M;
+    typedef typename D::G G;
+    typedef GeoIL<T, D::NW> I;
+    constexpr int NK = D::NK, NW = D::NW, ND = D::ND, RSLOTS = D::RSLOTS;
+    constexpr int CB = G::CB, UROW = D::UROW, YROW = D::YROW, USZ = D::USZ, YSZ = D::YSZ;
+    constexpr int CH = I::CH, LPR = I::LPR, RP = I::RP, NR = I::NR;
+    constexpr bool FEAT = KF > 0;
+    constexpr int NH = FEAT ? KF - 1 : 0;           // rows fetched before the lane's own
+    constexpr int KS = FEAT ? 1 : RP;               // rows between a lane's consecutive rows
+    constexpr int NV = 3 * CH;                      // feature values of a lane's row piece
+    // the waiting x, B values take the place of the filter tables, which are dead after barrier (A2)
+    constexpr int OFF_XB = D::OFF_H;
+    constexpr int XB_VEC = 64 * NW * 16 * M::RW;    // one row vector of every lane of the row waves
+    constexpr int XB_BYTES = (NK - 1) * 2 * XB_VEC;
+    constexpr int LDS_MAIN = OFF_XB + (XB_BYTES > D::H_BYTES ? XB_BYTES : D::H_BYTES);
+    constexpr int LDS_BYTES = LDS_MAIN > D::LDS_TAIL ? LDS_MAIN : D::LDS_TAIL;
+    static_assert(LDS_BYTES <= 160 * 1024, "tiles do not fit the CU's LDS");
+    __shared__ __attribute__((aligned(16))) unsigned char smem[LDS_BYTES];
+    unsigned char *const ring = smem + D::OFF_R;
+
+    const uint32_t wg_id = xcd_contiguous_u32(blockIdx.x, gridDim.x);
+    int cb, seg, bi;
+    wg_place(wg_id, pl, cb, seg, bi);
+    const int64_t b = bi;
+
+    const int tid = threadIdx.x, wv = tid >> 6, l = tid & 63;
+    const bool row_wave = wv >= NW;
+    const int w = wv & (NW - 1);                    // the wave's 16-channel block (either kind)
+    const int64_t d = dm.d, L = dm.L;
+    const int64_t c0 = (int64_t)cb * CB;
+    const bool wave_valid = c0 + 16 * w < d;
+    const int64_t s_lo = (int64_t)seg * pl.steps_per_seg;
+    const int64_t s_hi = (s_lo + pl.steps_per_seg < pl.nsteps) ? s_lo + pl.steps_per_seg : pl.nsteps;
+
+    f32x4 P[ND];
+#pragma unroll
+    for (int i = 0; i < ND; ++i) P[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    if (!row_wave) {
+        duo_product_waves<T>(smem, h, dm, pl, cb, w, l, wave_valid, s_lo, s_hi);
+    } else {
+        const int vt = tid & (64 * NW - 1);
+        const int rr = vt / LPR, a = vt % LPR;      // memory layout: rows row0 + KS*k, channels CH*a ..
+        const int row0 = FEAT ? NR * rr : rr;
+        // windows of this batch row: the outputs over rows [t0, t1), the features and dy over [t0, t2)
+        const int64_t t0 = (s_lo - (NK - 1)) * STEP > 0 ? (s_lo - (NK - 1)) * STEP : 0;
+        const int64_t t1 = s_hi * STEP < L ? s_hi * STEP : L;
+        const int64_t t2 = (s_hi + NK - 1) * STEP < L ? (s_hi + NK - 1) * STEP : L;
+        const int64_t tf = t0 - NH > 0 ? t0 - NH : 0;        // the featurizer looks NH rows further back
+        const int64_t row_bytes = d * M::ES, origin = (b * L + t0) * d;
+        const win_t wf = make_window(feat + 3 * (b * L + tf) * d, 3 * (t2 - tf) * row_bytes);
+        const win_t wdyw = make_window(dy + origin, (t2 - t0) * row_bytes);
+        const win_t wdf = make_window(dfeat + 3 * origin, 3 * (t1 - t0) * row_bytes);
+        const bool cvalid = c0 + CH * a < d;
+        const uint32_t lane_off = (uint32_t)(row0 * row_bytes + (c0 + CH * a) * M::ES);
+        const uint32_t feat_off = lane_off + (uint32_t)((t0 - tf) * row_bytes);
+        const uint32_t pass_off = (uint32_t)(KS * row_bytes), bad = cvalid ? 0u : WIN_OFF;
+        auto step_off = [&](int64_t sg) { return (uint32_t)((sg * STEP - t0) * row_bytes); };
+        const int rm_off = row0 * UROW + M::LES * CH * a;
+        const int yd_rd = row0 * YROW + 4 * CH * a;
+        unsigned char *const xb_own = smem + OFF_XB + vt * 16 * M::RW;           // slot k at + k * 2 * XB_VEC
+
+        // the interleaved rows and dy of one step (zero outside the sequence); with the featurizer the NH rows
+        // before the lane's own come first
+        struct Rows { u32x3 p[NH + NR]; Row<T> dy; };
+        auto fetch_feat = [&](int64_t step, u32x3 (&p)[NH + NR]) {
+            const uint32_t o = feat_off + step_off(step);
+#pragma unroll
+            for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, 3 * (o + (k - NH) * pass_off) + bad);
+        };
+        auto fetch = [&](int64_t step, Rows &r) {
+            fetch_feat(step, r.p);
+            const uint32_t o = lane_off + step_off(step) + bad;
+            uint32_t u[NR];
+#pragma unroll
+            for (int k = 0; k < NR; ++k) u[k] = ldw4(wdyw, o + k * pass_off);
+            r.dy = units_row<T, NR>(u);
+        };
+        float tap[FEAT ? KF : 1][NV];
+        if constexpr (FEAT) load_feat_taps<T, KF, NV>(wfeat, cvalid ? 3 * (c0 + CH * a) : 0, kf, tap);
+        auto rows_of = [&](const u32x3 (&p)[NH + NR], float (&xo)[8], float (&Bo)[8], float (&Co)[8]) {
+            if constexpr (FEAT) featurized_rows<T, NR, KF>(p, tap, xo, Bo, Co);
+            else il_split<T, NR>(p, xo, Bo, Co);
+        };
+        auto store_rows = [&](unsigned char *tile, const float (&f)[8]) {
+#pragma unroll
+            for (int k = 0; k < NR; ++k) store_operand_unit<T>(tile + rm_off + KS * k * UROW, UROW, &f[CH * k]);
+        };
+        // g2 = dy * C of a step into a newest-step tile and into a slot of the ring
+        auto store_g2 = [&](const Row<T> &dyo, const float (&Cf)[8], unsigned char *g_t, unsigned char *g_ring) {
+            float tf8[8], pf[8];
+            unpack8<T>(dyo, tf8);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = tf8[e] * Cf[e];
+            store_rows(g_t, pf);
+            store_rows(g_ring, pf);
+        };
+        auto store_u = [&](const float (&xf)[8], const float (&Bf)[8], unsigned char *u_t) {
+            float pf[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = xf[e] * Bf[e];
+            store_rows(u_t, pf);
+        };
+        // the interleaved gradient rows of step sg from its y2 / du tiles
+        auto finish_step = [&](int64_t sg, bool live, const unsigned char *y_t, const unsigned char *d_t,
+                               const Row<T> &dyo, const Row<T> &xo, const Row<T> &Bo) {
+            float dyf[8], xf[8], Bf[8], oC[8], ox[8], oB[8];
+            unpack8<T>(dyo, dyf);
+            unpack8<T>(xo, xf);
+            unpack8<T>(Bo, Bf);
+#pragma unroll
+            for (int k = 0; k < NR; ++k)
+#pragma unroll
+                for (int c = 0; c < CH; ++c) {
+                    const int e = CH * k + c;
+                    const float y2v = *(const float *)(y_t + yd_rd + KS * k * YROW + 4 * c);
+                    const float duv = *(const float *)(d_t + yd_rd + KS * k * YROW + 4 * c);
+                    oC[e] = dyf[e] * y2v;
+                    ox[e] = duv * Bf[e];
+                    oB[e] = duv * xf[e];
+                }
+            u32x3 po[NR];
+            il_join<T, NR>(ox, oB, oC, po);
+            const uint32_t o3 = live ? 3 * (lane_off + step_off(sg)) + bad : WIN_OFF;
+#pragma unroll
+            for (int k = 0; k < NR; ++k) win_store_as<KEEP>(wdf, o3 + 3 * k * pass_off, po[k]);
+        };
+
+        // Rings of the row waves, indexed by step - s_lo: x, B (as row vectors of the tensors' type) of the step being
+        // finished, the one in the matrix cores and the one being prepared; dy of NK+1 steps; two sets of rows in
+        // turn for the request on its way.
+        Row<T> xh[3], Bh[3], dyq[RSLOTS];
+        Row<T> xp = zero_row<T>(), Bp = zero_row<T>(), dyp = zero_row<T>();   // x, B, dy of the step being finished
+#pragma unroll
+        for (int i = 0; i < 3; ++i) xh[i] = Bh[i] = zero_row<T>();
+#pragma unroll
+        for (int i = 0; i < RSLOTS; ++i) dyq[i] = zero_row<T>();
+        Rows st[2];
+        {
+            // Lead-in: the rows of the NK-1 steps before the run (for u) and of its first NK steps (g2; x, B to wait in
+            // the ring), requested together; the rows of step s_lo+NK follow them.
+            u32x3 past[NK - 1][NH + NR];
+            Rows lead[NK];
+#pragma unroll
+            for (int i = 1; i < NK; ++i) fetch_feat(s_lo - i, past[i - 1]);
+#pragma unroll
+            for (int jj = NK - 2; jj >= 0; --jj) fetch(s_lo + jj, lead[jj]);
+            fetch(s_lo + NK - 1, lead[NK - 1]);
+            fetch(s_lo + NK, st[1]);
+            __syncthreads();                                          // (A)
+            __syncthreads();                                          // (A2): the filter tables' place is free
+            float f0[8], f1[8], f2[8];
+#pragma unroll
+            for (int i = 1; i < NK; ++i) {
+                // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
+                rows_of(past[i - 1], f0, f1, f2);
+                store_u(f0, f1, smem + D::OFF_U);
+                const int jj = NK - 1 - i;
+                rows_of(lead[jj].p, f0, f1, f2);
+                if (jj >= 1) {           // x, B of step s_lo+jj wait in ring slot jj % (NK-1)
+                    unsigned char *slot = xb_own + (jj % (NK - 1)) * 2 * XB_VEC;
+                    lds_store_row<T>(slot, pack8<T>(f0));
+                    lds_store_row<T>(slot + XB_VEC, pack8<T>(f1));
+                } else {                 // step s_lo itself is prepared below
+                    xh[0] = pack8<T>(f0);
+                    Bh[0] = pack8<T>(f1);
+                }
+                store_g2(lead[jj].dy, f2, smem + D::OFF_GN, ring + jj * USZ);
+                dyq[jj] = lead[jj].dy;
+                __syncthreads();                                      // (B_i)
+                __syncthreads();                                      // (C_i)
+            }
+            // step s_lo is prepared here, as an iteration s_lo-1 would have: u of step s_lo, g2 of step s_lo+NK-1
+            {
+                float xf[8], Bf[8];
+                unpack8<T>(xh[0], xf);
+                unpack8<T>(Bh[0], Bf);
+                store_u(xf, Bf, smem + D::OFF_U);
+                rows_of(lead[NK - 1].p, f0, f1, f2);
+                unsigned char *slot = xb_own + ((NK - 1) % (NK - 1)) * 2 * XB_VEC;
+                lds_store_row<T>(slot, pack8<T>(f0));
+                lds_store_row<T>(slot + XB_VEC, pack8<T>(f1));
+                store_g2(lead[NK - 1].dy, f2, smem + D::OFF_GN, ring + (NK - 1) * USZ);
+                dyq[NK - 1] = lead[NK - 1].dy;
+            }
+            __syncthreads();                                          // (D)
+        }
+
+        int xb_slot = 1 % (NK - 1);          // ring slot of step s+1
+        int64_t s = s_lo;
+        auto row_step = [&](int pu) __attribute__((always_inline)) {
+            const int par = pu & 1;
+            const unsigned char *const u_cur = smem + D::OFF_U + par * USZ;
+            unsigned char *const u_nx = smem + D::OFF_U + (par ^ 1) * USZ, *const g_nx = smem + D::OFF_GN + (par ^ 1) * USZ;
+            const unsigned char *const y_old = smem + D::OFF_Y + (par ^ 1) * YSZ, *const d_old = smem + D::OFF_D + (par ^ 1) * YSZ;
+            // Order as in mfma_bwd_duo_kernel: the request for rows first, then the stores, then what needs the previous
+            // request's rows, the filter-gradient products last.
+            fetch(s + NK + 1, st[par]);
+            finish_step(s - 1, s > s_lo, y_old, d_old, dyp, xp, Bp);
+            {
+                // step s+1: x, B from the ring; C and dy of step s+NK from the rows that arrived, whose x, B take the slot
+                float xa[8], Ba[8], cf[8], xf[8], Bf[8];
+                rows_of(st[par ^ 1].p, xa, Ba, cf);
+                unsigned char *slot = xb_own + xb_slot * 2 * XB_VEC;
+                const Row<T> xw = lds_load_row<T>(slot), Bw = lds_load_row<T>(slot + XB_VEC);
+                lds_store_row<T>(slot, pack8<T>(xa));
+                lds_store_row<T>(slot + XB_VEC, pack8<T>(Ba));
+                xb_slot = (xb_slot + 1 == NK - 1) ? 0 : xb_slot + 1;
+                unpack8<T>(xw, xf);
+                unpack8<T>(Bw, Bf);
+                store_u(xf, Bf, u_nx);
+                store_g2(st[par ^ 1].dy, cf, g_nx, ring + ((pu + RSLOTS - 1) % RSLOTS) * USZ);
+                dyq[(pu + RSLOTS - 1) % RSLOTS] = st[par ^ 1].dy;               // dy of step s+NK
+                xh[(pu + 1) % 3] = xw;
+                Bh[(pu + 1) % 3] = Bw;
+            }
+            duo_filter_gradient<T>(P, u_cur, ring, pu, w, l);    // filter-gradient tiles of step s
+            dyp = dyq[pu];                 // step s is finished during the next iteration
+            xp = xh[pu % 3];
+            Bp = Bh[pu % 3];
+            __syncthreads();
+            ++s;
+        };
+        // (every step can be the run's last: see mfma_bwd_duo_kernel for why the steps are not grouped)
+        while (s < s_hi) {
+#pragma unroll
+            for (int pu = 0; pu < RSLOTS; ++pu)
+                if (s < s_hi) row_step(pu);
+        }
+        // the last step of the run: its tiles are those of parity (s_hi - 1 - s_lo) & 1
+        {
+            const int par = (int)((s_hi - 1 - s_lo) & 1);
+            finish_step(s_hi - 1, true, smem + D::OFF_Y + par * YSZ, smem + D::OFF_D + par * YSZ, dyp, xp, Bp);
+        }
+    }
+
+    dh_finish<T, NW, ND, 512>(P, smem, ws, dh, dm, pl, wg_id, cb, wave_valid, row_wave, w);
+}
+
 // ---------------------------------------------------------------------------- launch
 template <typename T, int NK, int NW>
 int fwd_launch(const void *feat, const void *h, void *y, const Dims &dm, hipStream_t st)
@@ -549,7 +805,14 @@ int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, voi
     MfmaPlan p = plan_bwd(dm, MT<T>::SPLIT, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (p.fuse_dh && (p.slot = dh_slot_for_stream(st)) < 0) p.fuse_dh = p.slot = 0;   // no ticket set: second launch
-    if (dm.keep_out)
+    if constexpr (NK == 5 && il_duo_type<T>()) {
+        // product waves and row waves in one workgroup: the types whose backward is bound by instruction issue
+        auto duo = [&](auto kernel) {
+            return launch_main(kernel, dim3((unsigned)p.nwg), dim3(512), st, (const T *)dy, (const T *)feat, (const T *)h,
+                               (const T *)nullptr, 0, (T *)dfeat, (T *)dh, (float *)ws, dm, p);
+        };
+        e = dm.keep_out ? duo(mfma_il_bwd_duo_kernel<T, true, 0>) : duo(mfma_il_bwd_duo_kernel<T, false, 0>);
+    } else if (dm.keep_out)
         e = launch_main((mfma_il_bwd_kernel<T, NK, NW, true, 0>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                            (const T *)dy, (const T *)feat, (const T *)h, (const T *)nullptr, 0, (T *)dfeat, (T *)dh,
                            (float *)ws, dm, p);
@@ -570,7 +833,13 @@ template <typename T, int NW>
 int bwd_feat_launch(const void *dy, const void *raw, const void *wfeat, int kf, const void *h, void *dfeat, void *dh,
                     void *ws, const Dims &dm, MfmaPlan p, hipStream_t st)
 {
-    int e = launch_main((mfma_il_bwd_kernel<T, 5, NW, true, FEAT_KF>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
+    int e;
+    if constexpr (NW == 4 && il_duo_type<T>())
+        e = launch_main((mfma_il_bwd_duo_kernel<T, true, FEAT_KF>), dim3((unsigned)p.nwg), dim3(512), st,
+                        (const T *)dy, (const T *)raw, (const T *)h, (const T *)wfeat, kf, (T *)dfeat, (T *)dh,
+                        (float *)ws, dm, p);
+    else
+        e = launch_main((mfma_il_bwd_kernel<T, 5, NW, true, FEAT_KF>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
                         (const T *)dy, (const T *)raw, (const T *)h, (const T *)wfeat, kf, (T *)dfeat, (T *)dh,
                         (float *)ws, dm, p);
     if (e || p.fuse_dh) return e;

@@ -677,6 +677,122 @@ __device__ __forceinline__ void dh_finish(const f32x4 (&P)[ND], unsigned char *s
     }
 }
 
+// ---- backward kernels with product waves and row waves (gcg_mfma.hip, gcg_mfma_il.hip) ---------------------------
+// LDS of such a workgroup: five-slice filters, four channel blocks of 16, 512 threads.  Every tile of a step
+// exists twice (even and odd steps); g2 is kept once more in a ring of NK+1 steps for the filter gradient.
+template <typename T> struct DuoGeo {
+    typedef MT<T> M;
+    typedef Geo<T, 4> G;
+    static constexpr int NK = 5, NW = 4, ND = 2 * NK - 1, RSLOTS = NK + 1;
+    static constexpr int UROW = G::UROW, YROW = G::YROW;
+    static constexpr int USZ = STEP * UROW, YSZ = STEP * YROW, RING_ROWS = STEP * RSLOTS;
+    static constexpr int OFF_U = 0;                         // u of a step: even steps, odd steps
+    static constexpr int OFF_GN = OFF_U + 2 * USZ;          // g2 of the newest step, for the product waves
+    static constexpr int OFF_R = OFF_GN + 2 * USZ;          // g2 ring of NK+1 steps, for the filter gradient
+    static constexpr int OFF_Y = OFF_R + RSLOTS * USZ;      // y2 tiles, fp32
+    static constexpr int OFF_D = OFF_Y + 2 * YSZ;           // du tiles, fp32
+    static constexpr int OFF_H = OFF_D + 2 * YSZ;           // filter tables (dead after the barrier that follows the Toeplitz tiles)
+    static constexpr int H_BYTES = NW * HTAB * (int)sizeof(typename M::hraw_t);
+    static constexpr int LDS_TAIL = NW * (16 * ND + 16) * 17 * 4;   // P tiles at the end (dh_finish)
+};
+
+// The product waves' whole run: Toeplitz operands from the filter, the operand rings of the lead-in, then per step
+// the operands of step s from the tiles of its parity, the y2 / du products and their tiles.  Barriers: (A) taps in
+// LDS, (A2) Toeplitz tiles built, NK-1 pairs (B_i), (C_i) for the lead-in tiles, (D) step s_lo prepared, then one per
+// step; the row waves make the same calls.
+template <typename T>
+__device__ __forceinline__ void duo_product_waves(unsigned char *smem, const T *__restrict__ h, const Dims &dm,
+                                                  const MfmaPlan &pl, int cb, int w, int l, bool wave_valid, int64_t s_lo,
+                                                  int64_t s_hi)
+{
+    typedef DuoGeo<T> D;
+    typedef typename D::M M;
+    typedef typename M::op_t op_t;
+    typedef typename M::hraw_t hraw_t;
+    constexpr int NK = D::NK, NW = D::NW, UROW = D::UROW, YROW = D::YROW, USZ = D::USZ, YSZ = D::YSZ;
+    const int j = l & 15, q = l >> 4;
+    hraw_t *htab = (hraw_t *)(smem + D::OFF_H);
+    hraw_t hv[HTAB / 64];
+    load_taps<T>(dm, h, wave_valid ? fdiv((uint32_t)(cb * NW + w), pl.q_dg16) : 0, l, hv);
+    op_t Au[NK], Ag[NK];
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+        Au[i] = M::zero_op();
+        Ag[i] = M::zero_op();
+    }
+    const int y_wr = j * YROW + (16 * w + 4 * q) * 4;
+    const int d_wr = (15 - j) * YROW + (16 * w + 4 * q) * 4;      // columns come out reversed
+    store_taps(htab + w * HTAB, l, hv);
+    __syncthreads();                                              // (A)
+    typename M::wop_t W0[NK], W1[NK];
+#pragma unroll
+    for (int i = 0; i < NK; ++i) {
+        W0[i] = M::toeplitz(htab + w * HTAB, 32 * i, j, q);
+        W1[i] = M::toeplitz(htab + w * HTAB, 32 * i + 16, j, q);
+    }
+    __syncthreads();                                              // (A2)
+#pragma unroll
+    for (int i = 1; i < NK; ++i) {
+        __syncthreads();                                          // (B_i) lead-in tiles written
+        Au[NK - i] = M::load_operand(smem + D::OFF_U, UROW, w, j, q, false);
+        Ag[NK - 1 - i] = M::load_operand(smem + D::OFF_GN, UROW, w, j, q, true);
+        __syncthreads();                                          // (C_i) and read
+    }
+    __syncthreads();                                              // (D) step s_lo prepared
+    int64_t s = s_lo;
+    auto product_step = [&](int pu) __attribute__((always_inline)) {
+        const int ph = pu % NK, par = pu & 1;
+        const int slot_new = (ph + NK - 1) % NK;
+        Au[ph] = M::load_operand(smem + D::OFF_U + par * USZ, UROW, w, j, q, false);
+        Ag[slot_new] = M::load_operand(smem + D::OFF_GN + par * USZ, UROW, w, j, q, true);
+        f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+        f32x4 dac0 = {0.f, 0.f, 0.f, 0.f}, dac1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            acc0 = M::mfma(Au[(ph - i + NK) % NK], W0[i], acc0);
+            acc1 = M::mfma(Au[(ph - i + NK) % NK], W1[i], acc1);
+            dac0 = M::mfma(Ag[(ph + i) % NK], W1[i], dac0);   // output rows 0..15
+            dac1 = M::mfma(Ag[(ph + i) % NK], W0[i], dac1);   // output rows 16..31
+        }
+        unsigned char *const y_cur = smem + D::OFF_Y + par * YSZ, *const d_cur = smem + D::OFF_D + par * YSZ;
+        *(f32x4 *)(y_cur + y_wr) = acc0;
+        *(f32x4 *)(y_cur + y_wr + 16 * YROW) = acc1;
+        *(f32x4 *)(d_cur + d_wr) = dac0;
+        *(f32x4 *)(d_cur + d_wr + 16 * YROW) = dac1;
+        __syncthreads();
+        ++s;
+    };
+    while (s < s_hi) {
+#pragma unroll
+        for (int pu = 0; pu < 2 * NK; ++pu)
+            if (s < s_hi) product_step(pu);
+    }
+}
+
+// The row waves' filter-gradient products of the step in ring phase pu (step - s_lo modulo NK+1): u of the step
+// against the 2 NK - 1 windows of 32 rows of g2 that start 16 rows apart at the step's first row; natural-layout
+// operands (rows j and 16+j of a window), wave w's 16 channels.
+template <typename T>
+__device__ __forceinline__ void duo_filter_gradient(f32x4 (&P)[DuoGeo<T>::ND], const unsigned char *u_cur,
+                                                    const unsigned char *ring, int pu, int w, int l)
+{
+    typedef DuoGeo<T> D;
+    typedef typename D::M M;
+    typedef typename M::op_t op_t;
+    constexpr int UROW = D::UROW;
+    const int j = l & 15, q = l >> 4;
+    const op_t un = M::load_natural(u_cur + j * UROW, u_cur + (16 + j) * UROW, UROW, w, q);
+#pragma unroll
+    for (int dl = 0; dl < D::ND; ++dl) {
+        int row0 = STEP * pu + 16 * dl + j;              // ring rows of the window's two halves
+        int row1 = row0 + 16;
+        row0 = (row0 >= D::RING_ROWS) ? row0 - D::RING_ROWS : row0;
+        row1 = (row1 >= D::RING_ROWS) ? row1 - D::RING_ROWS : row1;
+        const op_t gn = M::load_natural(ring + row0 * UROW, ring + row1 * UROW, UROW, w, q);
+        P[dl] = M::mfma_aa(gn, un, P[dl]);
+    }
+}
+
 int cu_count()
 {
     static int n = 0;
