@@ -822,27 +822,19 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
     MfmaPlan p = plan_bwd(dm, MT<T>::SPLIT, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (p.fuse_dh && (p.slot = dh_slot_for_stream(st)) < 0) p.fuse_dh = p.slot = 0;   // no ticket set: second launch
-    bool launched = false;
+    auto launch = [&](auto kernel, int threads) {
+        return launch_main(kernel, dim3((unsigned)p.nwg), dim3(threads), st, (const T *)dy, (const T *)x, (const T *)B,
+                           (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC, (T *)dh, (float *)ws, dm, p);
+    };
     if constexpr (NK == 5 && duo_type<T>()) {
         // product waves and row waves in one workgroup: the types whose backward is bound by instruction issue
-        auto duo = [&](auto kernel) {
-            return launch_main(kernel, dim3((unsigned)p.nwg), dim3(512), st, (const T *)dy, (const T *)x, (const T *)B,
-                               (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC, (T *)dh, (float *)ws, dm, p);
-        };
-        e = dm.planar ? duo(mfma_bwd_duo_kernel<T, true>) : duo(mfma_bwd_duo_kernel<T, false>);
-        launched = true;
+        e = dm.planar ? launch(mfma_bwd_duo_kernel<T, true>, 512) : launch(mfma_bwd_duo_kernel<T, false>, 512);
     } else if constexpr (NK == 5) {
-        if (dm.planar) {        // instantiated for the five-slice walk only (bwd_t sends every filter length there)
-            e = launch_main((mfma_bwd_kernel<T, NK, NW, true>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
-                            (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
-                            (T *)dh, (float *)ws, dm, p);
-            launched = true;
-        }
+        // planar operands: instantiated for the five-slice walk only (bwd_t sends every filter length there)
+        e = dm.planar ? launch(mfma_bwd_kernel<T, NK, NW, true>, 64 * NW) : launch(mfma_bwd_kernel<T, NK, NW>, 64 * NW);
+    } else {
+        e = launch(mfma_bwd_kernel<T, NK, NW>, 64 * NW);
     }
-    if (!launched)
-        e = launch_main((mfma_bwd_kernel<T, NK, NW>), dim3((unsigned)p.nwg), dim3(64 * NW), st, (const T *)dy,
-                        (const T *)x, (const T *)B, (const T *)C, (const T *)h, (T *)dx, (T *)dB, (T *)dC,
-                        (T *)dh, (float *)ws, dm, p);
     if (e || p.fuse_dh) return e;
     const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,

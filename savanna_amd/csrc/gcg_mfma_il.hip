@@ -805,21 +805,17 @@ int bwd_launch(const void *dy, const void *feat, const void *h, void *dfeat, voi
     MfmaPlan p = plan_bwd(dm, MT<T>::SPLIT, MT<T>::ES);
     if (p.nwg > 0x7fffffffLL) return (int)hipErrorInvalidConfiguration;
     if (p.fuse_dh && (p.slot = dh_slot_for_stream(st)) < 0) p.fuse_dh = p.slot = 0;   // no ticket set: second launch
+    auto launch = [&](auto kernel, int threads) {
+        return launch_main(kernel, dim3((unsigned)p.nwg), dim3(threads), st, (const T *)dy, (const T *)feat, (const T *)h,
+                           (const T *)nullptr, 0, (T *)dfeat, (T *)dh, (float *)ws, dm, p);
+    };
     if constexpr (NK == 5 && il_duo_type<T>()) {
         // product waves and row waves in one workgroup: the types whose backward is bound by instruction issue
-        auto duo = [&](auto kernel) {
-            return launch_main(kernel, dim3((unsigned)p.nwg), dim3(512), st, (const T *)dy, (const T *)feat, (const T *)h,
-                               (const T *)nullptr, 0, (T *)dfeat, (T *)dh, (float *)ws, dm, p);
-        };
-        e = dm.keep_out ? duo(mfma_il_bwd_duo_kernel<T, true, 0>) : duo(mfma_il_bwd_duo_kernel<T, false, 0>);
-    } else if (dm.keep_out)
-        e = launch_main((mfma_il_bwd_kernel<T, NK, NW, true, 0>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
-                           (const T *)dy, (const T *)feat, (const T *)h, (const T *)nullptr, 0, (T *)dfeat, (T *)dh,
-                           (float *)ws, dm, p);
-    else
-        e = launch_main((mfma_il_bwd_kernel<T, NK, NW, false, 0>), dim3((unsigned)p.nwg), dim3(64 * NW), st,
-                           (const T *)dy, (const T *)feat, (const T *)h, (const T *)nullptr, 0, (T *)dfeat, (T *)dh,
-                           (float *)ws, dm, p);
+        e = dm.keep_out ? launch(mfma_il_bwd_duo_kernel<T, true, 0>, 512) : launch(mfma_il_bwd_duo_kernel<T, false, 0>, 512);
+    } else {
+        e = dm.keep_out ? launch(mfma_il_bwd_kernel<T, NK, NW, true, 0>, 64 * NW)
+                        : launch(mfma_il_bwd_kernel<T, NK, NW, false, 0>, 64 * NW);
+    }
     if (e || p.fuse_dh) return e;
     const int64_t n = (int64_t)dm.g * (dm.fw ? dm.lc : dm.hl);
     e = launch_plain(mfma_dh_reduce_kernel<T>, dim3((unsigned)((n + 255) / 256)), dim3(256), st,
