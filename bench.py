@@ -284,10 +284,10 @@ def time_workload(wl, device, steps, warmup, graph=False):
     torch.cuda.synchronize()
     # Instrumented steps cost time themselves: a launch that carries a pair of kernel events about 5 us, a bracket
     # of torch events around the call about 9 us more (measured at the headline shape).  So inside the timed region
-    # two steps carry kernel events only (workloads whose dominant call is one library launch), or the bracket where
+    # one or two steps carry kernel events only (workloads whose dominant call is one library launch), or the bracket where
     # the bracket is the measurement (whole-op workloads); the instrumented step is then repeated after the timed
     # region, with both kinds of events, for a steadier mean.  Both sample sets are reported.
-    n_in = min(2, steps)
+    n_in = min(2, max(1, steps // 25))      # one instrumented step in a region of fewer than 50 steps, else two
     marks = {(steps * (2 * j + 1)) // (2 * n_in): j for j in range(n_in)}       # spread over the region, not step 0
     n_after = min(16, max(4, steps))
     nsamp = n_in + n_after
