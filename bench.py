@@ -123,6 +123,8 @@ class Op:
             elif wl.layout != "separate":
                 # kernel names: C = v, B = q, x = k
                 t["feat"] = torch.stack([t.pop("v"), t.pop("q"), t.pop("k")], dim=-1).contiguous()
+            if wl.filt_dtype and not wl.layout.startswith("mixer"):
+                t["h"] = t["h"].to(wl.filt_dtype)
             self.sets.append(t)
         self.layout = wl.layout
         self.wl = wl
@@ -770,7 +772,8 @@ def main():
                      "mixer_fwdbwd_7b_fused", "mixer_fwdbwd_7b_fused_planar", "mixer_fwd_7b", "mixer_fwd_7b_fused",
                      "mixer_se_fwdbwd_40b", "mixer_se_fwdbwd_40b_fused", "mixer_se_fwdbwd_40b_fused_planar",
                      "mixer_se_fwdbwd_40b_fp32_arith", "mixer_se_fwdbwd_40b_fused_fp32_arith",
-                     "mixer_fwdbwd_7b_fp32_arith", "mixer_fwdbwd_7b_fused_fp32_arith"):
+                     "mixer_fwdbwd_7b_fp32_arith", "mixer_fwdbwd_7b_fused_fp32_arith",
+                     "mr_fwdbwd_7b_fp32_arith", "mr_fwdbwd_7b_interleaved_fp32_arith"):
             r = time_workload(WORKLOADS[name], device, max(10, args.steps // 2), 4)
             extra[name] = {k: r[k] for k in ("ms_per_step", "tokens_per_s", "step_gbs", "step_hbm_frac")}
         line["next_rows"] = extra

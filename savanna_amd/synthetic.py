@@ -126,6 +126,13 @@ WORKLOADS = {
     "mixer_fwdbwd_7b_fused_planar": Workload("mixer_fwdbwd_7b_fused_planar", 2, 8192, 256, 16, (128,), torch.bfloat16,
                                              True, "the same on planar features (interleave_projections = false): "
                                              "gcg_mixer_mr_fwd_planar / _bwd_planar", layout="mixer_fused_planar"),
+    "mr_fwdbwd_7b_fp32_arith": Workload("mr_fwdbwd_7b_fp32_arith", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
+                                        "Hyena-MR forward+backward with cgcg_dtype float32 on bf16 tensors (fp32 filter and "
+                                        "arithmetic, dtype code GCG_BF16_F32), B=2 L=8192 D=4096 G=256 hl=128",
+                                        filt_dtype=torch.float32),
+    "mr_fwdbwd_7b_interleaved_fp32_arith": Workload("mr_fwdbwd_7b_interleaved_fp32_arith", 2, 8192, 256, 16, (128,),
+                                                    torch.bfloat16, True, "the same on interleaved features",
+                                                    layout="interleaved", filt_dtype=torch.float32),
     "mixer_fwdbwd_7b_fp32_arith": Workload("mixer_fwdbwd_7b_fp32_arith", 2, 8192, 256, 16, (128,), torch.bfloat16, True,
                                            "featurizer conv + Hyena-MR with cgcg_dtype float32 on the bf16 features (the "
                                            "reference's default precision): two kernels each way", layout="mixer",
