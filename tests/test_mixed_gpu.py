@@ -143,6 +143,43 @@ def test_interleaved(gcg_lib, dtype, hl):
     assert_close(dh, ref[3], TOL_DH[torch.float32], "dh")
 
 
+def _random_shapes(n=24, seed=5):
+    """Shapes around the limits of the five-slice kernels: filter lengths 97..128, ragged lengths from less than one
+    step to several runs, channel counts that leave waves or lanes of a workgroup without work."""
+    import random
+    rnd = random.Random(seed)
+    out = []
+    for _ in range(n):
+        dg = rnd.choice([16, 16, 32, 48])
+        g = rnd.choice([1, 2, 3, 5, 8, 20])
+        L = rnd.choice([rnd.randint(1, 40), rnd.randint(41, 400), rnd.randint(401, 3000)])
+        out.append((rnd.choice([1, 2, 3]), L, g, dg, rnd.randint(97, 128)))
+    return out
+
+
+@pytest.mark.parametrize("bs,L,g,dg,hl", _random_shapes(), ids=lambda v: str(v))
+def test_random_shapes_fp32_arithmetic(gcg_lib, bs, L, g, dg, hl):
+    """bf16 tensors in fp32 arithmetic on separate and on interleaved tensors against the oracle, and against
+    each other bit for bit (the two layouts share the product side)."""
+    dtype = torch.bfloat16
+    x, B, C, h, dy = mixed_inputs(bs, L, g, dg, hl, dtype, seed=bs * 1000 + L)
+    xd, Bd, Cd, hd, dyd = (t.to(DEV) for t in (x, B, C, h, dy))
+    _, _, y = _lib.fwd(xd, Bd, Cd, hd, algo="mfma")
+    dx, dB, dC, dh = _lib.bwd(dyd, xd, Bd, Cd, hd, algo="mfma")
+    feat = torch.stack([Cd, Bd, xd], dim=-1).contiguous()
+    y_i = _lib.fwd_interleaved(feat, hd)
+    dfeat, dh_i = _lib.bwd_interleaved(dyd, feat, hd)
+    torch.cuda.synchronize()
+    ref = oracle.gcg_bwd_oracle(dy.float(), x.float(), B.float(), C.float(), h)
+    check_rounded_once(y, oracle.gcg_fwd_oracle(x.float(), B.float(), C.float(), h), dtype, "y", min_equal=0.97)
+    for o, r, n in zip((dx, dB, dC), ref[:3], ("dx", "dB", "dC")):
+        check_rounded_once(o, r, dtype, n, min_equal=0.97)
+    assert_close(dh, ref[3], TOL_DH[torch.float32], "dh")
+    assert torch.equal(y_i, y)
+    assert torch.equal(dfeat[..., 0], dC) and torch.equal(dfeat[..., 1], dB) and torch.equal(dfeat[..., 2], dx)
+    assert_close(dh_i, dh, 1e-6, "dh interleaved against separate")
+
+
 def test_fp32_filter_needs_16_bit_tensors(gcg_lib):
     x, B, C, h, _ = mixed_inputs(1, 64, 2, 16, 7, torch.bfloat16)
     with pytest.raises((TypeError, RuntimeError), match="filter"):
