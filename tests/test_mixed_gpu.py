@@ -143,6 +143,31 @@ def test_interleaved(gcg_lib, dtype, hl):
     assert_close(dh, ref[3], TOL_DH[torch.float32], "dh")
 
 
+def test_long_sequence_fp32_arithmetic(gcg_lib):
+    """A quarter of a million tokens: long runs (256 steps and more per workgroup), window offsets in the hundreds of
+    megabytes; two filter groups against the oracle, interleaved against separate."""
+    bs, L, g, dg, hl, dtype = 1, 262144 + 19, 32, 16, 128, torch.bfloat16
+    gen = torch.Generator(device=DEV).manual_seed(23)
+    x, B, C = (torch.randn(bs, L, g, dg, generator=gen, device=DEV).to(dtype) for _ in range(3))
+    dy = (0.1 * torch.randn(bs, L, g, dg, generator=gen, device=DEV)).to(dtype)
+    h = torch.randn(g, 1, hl, generator=gen, device=DEV) / hl ** 0.5
+    _, _, y = _lib.fwd(x, B, C, h)
+    dx, dB, dC, dh = _lib.bwd(dy, x, B, C, h)
+    feat = torch.stack([C, B, x], dim=-1).contiguous()
+    dfeat, dh_i = _lib.bwd_interleaved(dy, feat, h)
+    torch.cuda.synchronize()
+    assert torch.equal(dfeat[..., 0], dC) and torch.equal(dfeat[..., 1], dB) and torch.equal(dfeat[..., 2], dx)
+    assert_close(dh_i, dh, 1e-6, "dh interleaved against separate")
+    idx = torch.tensor([0, 31], device=DEV)
+    xs, Bs, Cs, dys = (t.index_select(2, idx).float().cpu() for t in (x, B, C, dy))
+    hs = h.index_select(0, idx).cpu()
+    ref = oracle.gcg_bwd_oracle(dys, xs, Bs, Cs, hs)
+    check_rounded_once(y.index_select(2, idx), oracle.gcg_fwd_oracle(xs, Bs, Cs, hs), dtype, "y")
+    for o, r, n in zip((dx, dB, dC), ref[:3], ("dx", "dB", "dC")):
+        check_rounded_once(o.index_select(2, idx), r, dtype, n)
+    assert_close(dh.index_select(0, idx), ref[3], TOL_DH[torch.float32], "dh")
+
+
 def _random_shapes(n=24, seed=5):
     """Shapes around the limits of the five-slice kernels: filter lengths 97..128, ragged lengths from less than one
     step to several runs, channel counts that leave waves or lanes of a workgroup without work."""
