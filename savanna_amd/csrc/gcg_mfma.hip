@@ -505,10 +505,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
     TR(7);
 }
 
-// Which element types take the two-kinds-of-waves backward below: bf16 tensors in fp32 arithmetic.  Plain 16-bit tensors
-// wait for memory, not for instructions (bf16: 181 us against 173 with mfma_bwd_kernel); three-plane operands (f16
-// tensors in fp32 arithmetic, fp32 tensors) need 171 KB of LDS for its tiles.
-template <typename T> constexpr bool duo_type() { return std::is_same<T, bf16w_t>::value; }
+// Which element types take the two-kinds-of-waves backward below: 16-bit tensors in fp32 arithmetic (7B layer shape:
+// bf16 232 -> 203 us, f16 311 -> 283 us).  Plain 16-bit tensors wait for memory, not for instructions (bf16: 181 us
+// against 173 with mfma_bwd_kernel), and so do fp32 tensors, whose rows are twice as long (492 us against 460).
+template <typename T> constexpr bool duo_type() { return std::is_same<T, bf16w_t>::value || std::is_same<T, f16w_t>::value; }
 
 // --------------------------------------------------------------------------- backward, product waves and row waves
 // The split-arithmetic backward is bound by instruction issue, not by memory (its 87 matrix instructions per step
@@ -538,7 +538,7 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
     typedef typename D::G G;
     constexpr int NK = D::NK, NW = D::NW, ND = D::ND, RSLOTS = D::RSLOTS;
     constexpr int CB = G::CB, UROW = D::UROW, YROW = D::YROW, ES = M::ES, USZ = D::USZ, YSZ = D::YSZ;
-    constexpr int OFF_U = D::OFF_U, OFF_GN = D::OFF_GN, OFF_Y = D::OFF_Y, OFF_D = D::OFF_D;
+    constexpr int OFF_U = D::OFF_U, OFF_Y = D::OFF_Y, OFF_D = D::OFF_D;
     constexpr int LDS_MAIN = D::OFF_H + D::H_BYTES;
     constexpr int LDS_BYTES = LDS_MAIN > D::LDS_TAIL ? LDS_MAIN : D::LDS_TAIL;
     static_assert(LDS_BYTES <= 160 * 1024, "tiles do not fit the CU's LDS");
@@ -598,9 +598,9 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
             dyo = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wdy, o2);
             Co = ldw_row_policy<T, GCG_MFMA_BWD_LD>(wC, PL ? lane_in + IM * step_off(sg + NK - 1) : o2);
         };
-        // u = x * B into a u tile; g2 = dy * C into a newest-step tile and into a slot of the ring
+        // u = x * B into a u tile; g2 = dy * C into a slot of the ring
         auto gate_rows = [&](const Row<T> &xo, const Row<T> &Bo, const Row<T> &dyo, const Row<T> &Co, unsigned char *u_t,
-                             unsigned char *g_t, unsigned char *g_ring) {
+                             unsigned char *g_ring) {
             float f0[8], f1[8], pf[8];
             unpack8<T>(xo, f0);
             unpack8<T>(Bo, f1);
@@ -611,7 +611,6 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
             unpack8<T>(Co, f1);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = f0[e] * f1[e];
-            store_operand<T>(g_t + rm_off, UROW, pf);
             store_operand<T>(g_ring + rm_off, UROW, pf);
         };
         // dC, dx, dB of step sg from its y2 / du tiles
@@ -664,14 +663,14 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
             // iteration s_lo-i carries u of step s_lo-i and g2 / dy of step s_lo+NK-1-i
-            gate_rows(wx_[i - 1], wB_[i - 1], wdy_[i - 1], wC_[i - 1], smem + OFF_U, smem + OFF_GN,
+            gate_rows(wx_[i - 1], wB_[i - 1], wdy_[i - 1], wC_[i - 1], smem + OFF_U,
                       ring + (NK - 1 - i) * USZ);
             dyq[NK - 1 - i] = wdy_[i - 1];
             __syncthreads();                                          // (B_i)
             __syncthreads();                                          // (C_i)
         }
         // step s_lo is prepared here, as an iteration s_lo-1 would have
-        gate_rows(xh[0], Bh[0], dy_st[0], C_st[0], smem + OFF_U, smem + OFF_GN, ring + (NK - 1) * USZ);
+        gate_rows(xh[0], Bh[0], dy_st[0], C_st[0], smem + OFF_U, ring + (NK - 1) * USZ);
         dyq[NK - 1] = dy_st[0];
         __syncthreads();                                              // (D)
 
@@ -679,7 +678,7 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
         auto row_step = [&](int pu) __attribute__((always_inline)) {
                     const int par = pu & 1;
                     const unsigned char *const u_cur = smem + OFF_U + par * USZ;
-                    unsigned char *const u_nx = smem + OFF_U + (par ^ 1) * USZ, *const g_nx = smem + OFF_GN + (par ^ 1) * USZ;
+                    unsigned char *const u_nx = smem + OFF_U + (par ^ 1) * USZ;
                     const unsigned char *const y_old = smem + OFF_Y + (par ^ 1) * YSZ, *const d_old = smem + OFF_D + (par ^ 1) * YSZ;
                     // Order: the request for rows first, then the stores, then what needs the previous request's rows, the
                     // filter-gradient products last.  Measured at the 7B shape: products first 240 us, stores before the
@@ -690,7 +689,7 @@ __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__
                     finish_step(s - 1, s > s_lo, y_old, d_old, dyp, xp, Bp);
                     // step s+1: its rows arrived during the last iteration
                     dyq[(pu + RSLOTS - 1) % RSLOTS] = dy_st[par ^ 1];          // dy of step s+NK
-                    gate_rows(xh[(pu + 1) % 3], Bh[(pu + 1) % 3], dy_st[par ^ 1], C_st[par ^ 1], u_nx, g_nx,
+                    gate_rows(xh[(pu + 1) % 3], Bh[(pu + 1) % 3], dy_st[par ^ 1], C_st[par ^ 1], u_nx,
                               ring + ((pu + RSLOTS - 1) % RSLOTS) * USZ);
                     duo_filter_gradient<T>(P, u_cur, ring, pu, w, l);    // filter-gradient tiles of step s
                     dyp = dyq[pu];                 // step s is finished during the next iteration

@@ -475,6 +475,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     dh_finish<T, NW, ND>(P, smem, ws, dh, dm, pl, wg_id, cb, wave_valid);
 }
 
+// bf16 tensors in fp32 arithmetic only: with f16's three-plane operand tiles the waiting x, B values no longer fit
+// beside them (174 KB of LDS)
 template <typename T> constexpr bool il_duo_type() { return std::is_same<T, bf16w_t>::value; }
 
 // --------------------------------------------------------------------------- backward, product waves and row waves
@@ -580,13 +582,12 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
 #pragma unroll
             for (int k = 0; k < NR; ++k) store_operand_unit<T>(tile + rm_off + KS * k * UROW, UROW, &f[CH * k]);
         };
-        // g2 = dy * C of a step into a newest-step tile and into a slot of the ring
-        auto store_g2 = [&](const Row<T> &dyo, const float (&Cf)[8], unsigned char *g_t, unsigned char *g_ring) {
+        // g2 = dy * C of a step into its slot of the ring
+        auto store_g2 = [&](const Row<T> &dyo, const float (&Cf)[8], unsigned char *g_ring) {
             float tf8[8], pf[8];
             unpack8<T>(dyo, tf8);
 #pragma unroll
             for (int e = 0; e < 8; ++e) pf[e] = tf8[e] * Cf[e];
-            store_rows(g_t, pf);
             store_rows(g_ring, pf);
         };
         auto store_u = [&](const float (&xf)[8], const float (&Bf)[8], unsigned char *u_t) {
@@ -659,7 +660,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
                     xh[0] = pack8<T>(f0);
                     Bh[0] = pack8<T>(f1);
                 }
-                store_g2(lead[jj].dy, f2, smem + D::OFF_GN, ring + jj * USZ);
+                store_g2(lead[jj].dy, f2, ring + jj * USZ);
                 dyq[jj] = lead[jj].dy;
                 __syncthreads();                                      // (B_i)
                 __syncthreads();                                      // (C_i)
@@ -674,7 +675,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
                 unsigned char *slot = xb_own + ((NK - 1) % (NK - 1)) * 2 * XB_VEC;
                 lds_store_row<T>(slot, pack8<T>(f0));
                 lds_store_row<T>(slot + XB_VEC, pack8<T>(f1));
-                store_g2(lead[NK - 1].dy, f2, smem + D::OFF_GN, ring + (NK - 1) * USZ);
+                store_g2(lead[NK - 1].dy, f2, ring + (NK - 1) * USZ);
                 dyq[NK - 1] = lead[NK - 1].dy;
             }
             __syncthreads();                                          // (D)
@@ -685,7 +686,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
         auto row_step = [&](int pu) __attribute__((always_inline)) {
             const int par = pu & 1;
             const unsigned char *const u_cur = smem + D::OFF_U + par * USZ;
-            unsigned char *const u_nx = smem + D::OFF_U + (par ^ 1) * USZ, *const g_nx = smem + D::OFF_GN + (par ^ 1) * USZ;
+            unsigned char *const u_nx = smem + D::OFF_U + (par ^ 1) * USZ;
             const unsigned char *const y_old = smem + D::OFF_Y + (par ^ 1) * YSZ, *const d_old = smem + D::OFF_D + (par ^ 1) * YSZ;
             // Order as in mfma_bwd_duo_kernel: the request for rows first, then the stores, then what needs the previous
             // request's rows, the filter-gradient products last.
@@ -703,7 +704,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
                 unpack8<T>(xw, xf);
                 unpack8<T>(Bw, Bf);
                 store_u(xf, Bf, u_nx);
-                store_g2(st[par ^ 1].dy, cf, g_nx, ring + ((pu + RSLOTS - 1) % RSLOTS) * USZ);
+                store_g2(st[par ^ 1].dy, cf, ring + ((pu + RSLOTS - 1) % RSLOTS) * USZ);
                 dyq[(pu + RSLOTS - 1) % RSLOTS] = st[par ^ 1].dy;               // dy of step s+NK
                 xh[(pu + 1) % 3] = xw;
                 Bh[(pu + 1) % 3] = Bw;

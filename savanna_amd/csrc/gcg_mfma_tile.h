@@ -679,7 +679,8 @@ __device__ __forceinline__ void dh_finish(const f32x4 (&P)[ND], unsigned char *s
 
 // ---- backward kernels with product waves and row waves (gcg_mfma.hip, gcg_mfma_il.hip) ---------------------------
 // LDS of such a workgroup: five-slice filters, four channel blocks of 16, 512 threads.  Every tile of a step
-// exists twice (even and odd steps); g2 is kept once more in a ring of NK+1 steps for the filter gradient.
+// but g2 exists twice (even and odd steps); g2 is kept in a ring of NK+1 steps, read by the product waves (the
+// newest step) and by the filter-gradient products (NK steps) while the row waves write the one after.
 template <typename T> struct DuoGeo {
     typedef MT<T> M;
     typedef Geo<T, 4> G;
@@ -687,8 +688,7 @@ template <typename T> struct DuoGeo {
     static constexpr int UROW = G::UROW, YROW = G::YROW;
     static constexpr int USZ = STEP * UROW, YSZ = STEP * YROW, RING_ROWS = STEP * RSLOTS;
     static constexpr int OFF_U = 0;                         // u of a step: even steps, odd steps
-    static constexpr int OFF_GN = OFF_U + 2 * USZ;          // g2 of the newest step, for the product waves
-    static constexpr int OFF_R = OFF_GN + 2 * USZ;          // g2 ring of NK+1 steps, for the filter gradient
+    static constexpr int OFF_R = OFF_U + 2 * USZ;           // g2 ring of NK+1 steps: slot (step - s_lo) % (NK+1)
     static constexpr int OFF_Y = OFF_R + RSLOTS * USZ;      // y2 tiles, fp32
     static constexpr int OFF_D = OFF_Y + 2 * YSZ;           // du tiles, fp32
     static constexpr int OFF_H = OFF_D + 2 * YSZ;           // filter tables (dead after the barrier that follows the Toeplitz tiles)
@@ -735,16 +735,18 @@ __device__ __forceinline__ void duo_product_waves(unsigned char *smem, const T *
     for (int i = 1; i < NK; ++i) {
         __syncthreads();                                          // (B_i) lead-in tiles written
         Au[NK - i] = M::load_operand(smem + D::OFF_U, UROW, w, j, q, false);
-        Ag[NK - 1 - i] = M::load_operand(smem + D::OFF_GN, UROW, w, j, q, true);
+        Ag[NK - 1 - i] = M::load_operand(smem + D::OFF_R + (NK - 1 - i) * USZ, UROW, w, j, q, true);
         __syncthreads();                                          // (C_i) and read
     }
     __syncthreads();                                              // (D) step s_lo prepared
     int64_t s = s_lo;
+    int gnew = NK - 1;                    // ring slot of step s+NK-1, the newest g2 (the ring's period is not the operand rings')
     auto product_step = [&](int pu) __attribute__((always_inline)) {
         const int ph = pu % NK, par = pu & 1;
         const int slot_new = (ph + NK - 1) % NK;
         Au[ph] = M::load_operand(smem + D::OFF_U + par * USZ, UROW, w, j, q, false);
-        Ag[slot_new] = M::load_operand(smem + D::OFF_GN + par * USZ, UROW, w, j, q, true);
+        Ag[slot_new] = M::load_operand(smem + D::OFF_R + gnew * USZ, UROW, w, j, q, true);
+        gnew = (gnew + 1 == D::RSLOTS) ? 0 : gnew + 1;
         f32x4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
         f32x4 dac0 = {0.f, 0.f, 0.f, 0.f}, dac1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
