@@ -522,8 +522,9 @@ template <typename T> constexpr bool duo_type() { return std::is_same<T, bf16w_t
 //     products (their operands are rows in natural order, which the row waves have just written).
 // They meet at one barrier per step.  Iteration sigma: the product waves work on step sigma (operands written to LDS
 // during iteration sigma-1, results to the y2 / du tiles of sigma's parity); the row waves finish step sigma-1 from
-// the tiles of the other parity, prepare step sigma+1 (u, g2 of step sigma+NK into the tiles of the other parity and
-// into a ring of NK+1 steps of g2) and accumulate the filter-gradient tiles of step sigma from the ring.
+// the tiles of the other parity, prepare step sigma+1 (u into the tile of the other parity, g2 of step sigma+NK into
+// a ring of NK+1 steps of g2, which both kinds of waves read) and accumulate the filter-gradient tiles of step sigma
+// from the ring.
 // Five-slice filters only (the rings' periods fix the unrolling: 2 NK for the product waves, NK+1 for the row waves).
 template <typename T, bool PL = false>
 __global__ __launch_bounds__(512) void mfma_bwd_duo_kernel(const T *__restrict__ dy, const T *__restrict__ x,

@@ -182,11 +182,13 @@ def _random_shapes(n=24, seed=5):
     return out
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
 @pytest.mark.parametrize("bs,L,g,dg,hl", _random_shapes(), ids=lambda v: str(v))
-def test_random_shapes_fp32_arithmetic(gcg_lib, bs, L, g, dg, hl):
-    """bf16 tensors in fp32 arithmetic on separate and on interleaved tensors against the oracle, and against
-    each other bit for bit (the two layouts share the product side)."""
-    dtype = torch.bfloat16
+def test_random_shapes_fp32_arithmetic(gcg_lib, bs, L, g, dg, hl, dtype):
+    """16-bit tensors in fp32 arithmetic on separate and on interleaved tensors against the oracle, and against
+    each other bit for bit (the two layouts add the same plane products in the same order, whichever kernel
+    runs them: for f16 the separate tensors take the kernel with product waves and row waves, the interleaved
+    ones the 4-wave kernel)."""
     x, B, C, h, dy = mixed_inputs(bs, L, g, dg, hl, dtype, seed=bs * 1000 + L)
     xd, Bd, Cd, hd, dyd = (t.to(DEV) for t in (x, B, C, h, dy))
     _, _, y = _lib.fwd(xd, Bd, Cd, hd, algo="mfma")
