@@ -33,6 +33,24 @@ __device__ __forceinline__ void il_split(const u32x3 (&p)[NR], float (&xf)[8], f
         }
     }
 }
+// 16-bit pieces of NR = 4 rows -> the row vectors of x and B as they are (element e = 2 k + c, no conversion) and C
+// as fp32
+template <typename T>
+__device__ __forceinline__ void il_split_rows(const u32x3 (&p)[4], Row<T> &xr, Row<T> &Br, float (&Cf)[8])
+{
+    static_assert(MT<T>::ES == 2, "16-bit pieces");
+    uint32_t xw[4], Bw[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float skip;
+        MT<T>::unpack2(p[k][0], Cf[2 * k], skip);
+        MT<T>::unpack2(p[k][1], skip, Cf[2 * k + 1]);
+        xw[k] = (p[k][1] & 0xffffu) | (p[k][2] & 0xffff0000u);          // x0 | x1
+        Bw[k] = __builtin_amdgcn_alignbit(p[k][2], p[k][0], 16);        // B0 | B1
+    }
+    xr.w[0] = make_uint4(xw[0], xw[1], xw[2], xw[3]);
+    Br.w[0] = make_uint4(Bw[0], Bw[1], Bw[2], Bw[3]);
+}
 template <typename T, int NR>
 __device__ __forceinline__ void il_join(const float (&xf)[8], const float (&Bf)[8], const float (&Cf)[8],
                                         u32x3 (&p)[NR])
@@ -60,15 +78,22 @@ template <typename T> __device__ __forceinline__ uint32_t pack_unit(const float 
 template <typename T> __device__ __forceinline__ void store_operand_unit(unsigned char *p, int urow, const float *f)
 {
     typedef MT<T> M;
-    if constexpr (M::SPLIT) {
-        constexpr int CH = 4 / M::ES;
-        uint16_t v[CH][M::NPA];
+    if constexpr (M::SPLIT && M::ES == 4) {
+        uint16_t v[M::NPA];
+        M::template split<M::NPA>(f[0], v);
 #pragma unroll
-        for (int c = 0; c < CH; ++c) M::template split<M::NPA>(f[c], v[c]);
+        for (int m = 0; m < M::NPA; ++m) *(uint16_t *)(p + m * M::plane(urow)) = v[m];
+    } else if constexpr (M::SPLIT) {
+        // the two channels plane by plane as pairs (MTSplit::split on each, with one packed conversion per plane)
+        float r0 = f[0], r1 = f[1];
 #pragma unroll
         for (int m = 0; m < M::NPA; ++m) {
-            if constexpr (CH == 1) *(uint16_t *)(p + m * M::plane(urow)) = v[0][m];
-            else *(uint32_t *)(p + m * M::plane(urow)) = (uint32_t)v[0][m] | ((uint32_t)v[1][m] << 16);
+            const uint32_t pk = pack_bf16x2(r0, r1);
+            *(uint32_t *)(p + m * M::plane(urow)) = pk;
+            if (m + 1 < M::NPA) {
+                r0 -= __uint_as_float(pk << 16);
+                r1 -= __uint_as_float(pk & 0xffff0000u);
+            }
         }
     } else {
         *(uint32_t *)p = M::pack2(f[0], f[1]);

@@ -559,14 +559,16 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
         // the interleaved rows and dy of one step (zero outside the sequence); with the featurizer the NH rows
         // before the lane's own come first
         struct Rows { u32x3 p[NH + NR]; Row<T> dy; };
-        auto fetch_feat = [&](int64_t step, u32x3 (&p)[NH + NR]) {
-            const uint32_t o = feat_off + step_off(step);
+        // (so: the step's offset, step_off(step); inside the loop a running 32-bit value, advanced by step_b per step)
+        // (the lane's part and the uniform part are multiplied separately: the uniform one on the scalar unit)
+        const uint32_t feat_off3 = 3 * feat_off + bad, lane_off3 = 3 * lane_off + bad;
+        auto fetch_feat = [&](uint32_t so, u32x3 (&p)[NH + NR]) {
 #pragma unroll
-            for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, 3 * (o + (k - NH) * pass_off) + bad);
+            for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, feat_off3 + 3 * (so + (k - NH) * pass_off));
         };
-        auto fetch = [&](int64_t step, Rows &r) {
-            fetch_feat(step, r.p);
-            const uint32_t o = lane_off + step_off(step) + bad;
+        auto fetch = [&](uint32_t so, Rows &r) {
+            fetch_feat(so, r.p);
+            const uint32_t o = lane_off + so + bad;
             uint32_t u[NR];
 #pragma unroll
             for (int k = 0; k < NR; ++k) u[k] = ldw4(wdyw, o + k * pass_off);
@@ -597,7 +599,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
             store_rows(u_t, pf);
         };
         // the interleaved gradient rows of step sg from its y2 / du tiles
-        auto finish_step = [&](int64_t sg, bool live, const unsigned char *y_t, const unsigned char *d_t,
+        auto finish_step = [&](uint32_t so, bool live, const unsigned char *y_t, const unsigned char *d_t,
                                const Row<T> &dyo, const Row<T> &xo, const Row<T> &Bo) {
             float dyf[8], xf[8], Bf[8], oC[8], ox[8], oB[8];
             unpack8<T>(dyo, dyf);
@@ -616,7 +618,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
                 }
             u32x3 po[NR];
             il_join<T, NR>(ox, oB, oC, po);
-            const uint32_t o3 = live ? 3 * (lane_off + step_off(sg)) + bad : WIN_OFF;
+            const uint32_t o3 = live ? lane_off3 + 3 * so : WIN_OFF;
 #pragma unroll
             for (int k = 0; k < NR; ++k) win_store_as<KEEP>(wdf, o3 + 3 * k * pass_off, po[k]);
         };
@@ -625,7 +627,6 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
         // finished, the one in the matrix cores and the one being prepared; dy of NK+1 steps; two sets of rows in
         // turn for the request on its way.
         Row<T> xh[3], Bh[3], dyq[RSLOTS];
-        Row<T> xp = zero_row<T>(), Bp = zero_row<T>(), dyp = zero_row<T>();   // x, B, dy of the step being finished
 #pragma unroll
         for (int i = 0; i < 3; ++i) xh[i] = Bh[i] = zero_row<T>();
 #pragma unroll
@@ -637,11 +638,11 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
             u32x3 past[NK - 1][NH + NR];
             Rows lead[NK];
 #pragma unroll
-            for (int i = 1; i < NK; ++i) fetch_feat(s_lo - i, past[i - 1]);
+            for (int i = 1; i < NK; ++i) fetch_feat(step_off(s_lo - i), past[i - 1]);
 #pragma unroll
-            for (int jj = NK - 2; jj >= 0; --jj) fetch(s_lo + jj, lead[jj]);
-            fetch(s_lo + NK - 1, lead[NK - 1]);
-            fetch(s_lo + NK, st[1]);
+            for (int jj = NK - 2; jj >= 0; --jj) fetch(step_off(s_lo + jj), lead[jj]);
+            fetch(step_off(s_lo + NK - 1), lead[NK - 1]);
+            fetch(step_off(s_lo + NK), st[1]);
             __syncthreads();                                          // (A)
             __syncthreads();                                          // (A2): the filter tables' place is free
             float f0[8], f1[8], f2[8];
@@ -682,7 +683,12 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
         }
 
         int xb_slot = 1 % (NK - 1);          // ring slot of step s+1
-        int64_t s = s_lo;
+        // the run's steps are counted from 0 in 32 bits, and so are their offsets (the same values modulo 2^32 as
+        // step_off gives): 64-bit multiplications per step are a tenth of the row waves' vector cycles otherwise
+        const int n_steps = (int)(s_hi - s_lo);
+        const uint32_t step_b = (uint32_t)(STEP * row_bytes);
+        uint32_t so = step_off(s_lo);        // of step s
+        int s = 0;
         auto row_step = [&](int pu) __attribute__((always_inline)) {
             const int par = pu & 1;
             const unsigned char *const u_cur = smem + D::OFF_U + par * USZ;
@@ -690,16 +696,24 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
             const unsigned char *const y_old = smem + D::OFF_Y + (par ^ 1) * YSZ, *const d_old = smem + D::OFF_D + (par ^ 1) * YSZ;
             // Order as in mfma_bwd_duo_kernel: the request for rows first, then the stores, then what needs the previous
             // request's rows, the filter-gradient products last.
-            fetch(s + NK + 1, st[par]);
-            finish_step(s - 1, s > s_lo, y_old, d_old, dyp, xp, Bp);
+            fetch(so + (uint32_t)(NK + 1) * step_b, st[par]);
+            finish_step(so - step_b, s > 0, y_old, d_old, dyq[(pu + RSLOTS - 1) % RSLOTS], xh[(pu + 2) % 3], Bh[(pu + 2) % 3]);
             {
                 // step s+1: x, B from the ring; C and dy of step s+NK from the rows that arrived, whose x, B take the slot
-                float xa[8], Ba[8], cf[8], xf[8], Bf[8];
-                rows_of(st[par ^ 1].p, xa, Ba, cf);
+                float cf[8], xf[8], Bf[8];
+                Row<T> xa, Ba;
+                if constexpr (FEAT || M::ES == 4) {
+                    float xv[8], Bv[8];
+                    rows_of(st[par ^ 1].p, xv, Bv, cf);
+                    xa = pack8<T>(xv);
+                    Ba = pack8<T>(Bv);
+                } else {
+                    il_split_rows<T>(st[par ^ 1].p, xa, Ba, cf);
+                }
                 unsigned char *slot = xb_own + xb_slot * 2 * XB_VEC;
                 const Row<T> xw = lds_load_row<T>(slot), Bw = lds_load_row<T>(slot + XB_VEC);
-                lds_store_row<T>(slot, pack8<T>(xa));
-                lds_store_row<T>(slot + XB_VEC, pack8<T>(Ba));
+                lds_store_row<T>(slot, xa);
+                lds_store_row<T>(slot + XB_VEC, Ba);
                 xb_slot = (xb_slot + 1 == NK - 1) ? 0 : xb_slot + 1;
                 unpack8<T>(xw, xf);
                 unpack8<T>(Bw, Bf);
@@ -710,22 +724,27 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
                 Bh[(pu + 1) % 3] = Bw;
             }
             duo_filter_gradient<T>(P, u_cur, ring, pu, w, l);    // filter-gradient tiles of step s
-            dyp = dyq[pu];                 // step s is finished during the next iteration
-            xp = xh[pu % 3];
-            Bp = Bh[pu % 3];
             __syncthreads();
             ++s;
+            so += step_b;
         };
-        // (every step can be the run's last: see mfma_bwd_duo_kernel for why the steps are not grouped)
-        while (s < s_hi) {
+        // Every step can be the run's last (see mfma_bwd_duo_kernel for why the steps are not grouped); the run's
+        // last step is finished where the loop leaves, so that the rings keep compile-time indices.
+        bool done = false;
+        while (!done) {
 #pragma unroll
-            for (int pu = 0; pu < RSLOTS; ++pu)
-                if (s < s_hi) row_step(pu);
-        }
-        // the last step of the run: its tiles are those of parity (s_hi - 1 - s_lo) & 1
-        {
-            const int par = (int)((s_hi - 1 - s_lo) & 1);
-            finish_step(s_hi - 1, true, smem + D::OFF_Y + par * YSZ, smem + D::OFF_D + par * YSZ, dyp, xp, Bp);
+            for (int pu = 0; pu < RSLOTS; ++pu) {
+                if (!done) {
+                    if (s < n_steps) {
+                        row_step(pu);
+                    } else {
+                        const int par = (pu & 1) ^ 1;         // of step n_steps-1
+                        finish_step(so - step_b, true, smem + D::OFF_Y + par * YSZ, smem + D::OFF_D + par * YSZ,
+                                    dyq[(pu + RSLOTS - 1) % RSLOTS], xh[(pu + 2) % 3], Bh[(pu + 2) % 3]);
+                        done = true;
+                    }
+                }
+            }
         }
     }
 
