@@ -68,6 +68,14 @@ __device__ unsigned long long g_trace[(size_t)TRACE_WGS * TRACE_SLOTS];
 #ifndef GCG_MFMA_FWD_LEAD_LD
 #define GCG_MFMA_FWD_LEAD_LD WIN_NT
 #endif
+// Idle cycles in front of each output store of the backward's long runs (tuning builds may override).  Measured
+// at the 7B layer shape (2 x 8192 x 4096, bf16): 0 cycles 172.3 - 173.8 us, 16: 171.0, 24: 169.5, 32: 167.3 - 170.4,
+// 36 - 40: 165.5 - 169.8 (by the box), 48: 168.5 - 171.1, 64: 178; at 1 x 32768 x 8192 24 - 32 cycles gain 1 %, more
+// gains nothing; runs of 16 steps lose 2 % with any.  The stores of a step leave while its workgroup's next rows are
+// still on their way, and a little later is better for those.
+#ifndef GCG_MFMA_BWD_ST_GAP
+#define GCG_MFMA_BWD_ST_GAP 36
+#endif
 #ifndef GCG_MFMA_BWD_LD
 #define GCG_MFMA_BWD_LD WIN_NT
 #endif
@@ -264,7 +272,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_fwd_kernel(const T *__restrict__
 // end the diagonals of the P tiles are summed in a fixed order into per-wave partials in
 // the workspace, and a second kernel adds the partials in a fixed order.
 // PL: x, B, C and dx, dB, dC are thirds of the rows of (bs, L, 3 d) tensors (Dims::planar).
-template <typename T, int NK, int NW, bool PL = false>
+// GAP: idle cycles in front of the output stores (GCG_MFMA_BWD_ST_GAP), for long runs.
+template <typename T, int NK, int NW, bool PL = false, bool GAP = false>
 __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__ dy, const T *__restrict__ x,
                                                        const T *__restrict__ B, const T *__restrict__ C,
                                                        const T *__restrict__ h, T *__restrict__ dx,
@@ -479,6 +488,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         unpack8<T>(dyq[ph], dyf);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = dyf[e] * y2f[e];
+                        if constexpr (GAP) idle_cycles<GCG_MFMA_BWD_ST_GAP>();
                         stw_row_policy<T, GCG_MFMA_BWD_ST_DC>(wdC, o, pack8<T>(of));
                     }
                     {
@@ -488,9 +498,11 @@ __global__ __launch_bounds__(64 * NW) void mfma_bwd_kernel(const T *__restrict__
                         float of[8];
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * Bf[e];
+                        if constexpr (GAP) idle_cycles<GCG_MFMA_BWD_ST_GAP>();
                         stw_row_policy<T, GCG_MFMA_BWD_ST>(wdx, o, pack8<T>(of));
 #pragma unroll
                         for (int e = 0; e < 8; ++e) of[e] = duf[e] * xf[e];
+                        if constexpr (GAP) idle_cycles<GCG_MFMA_BWD_ST_GAP>();
                         stw_row_policy<T, GCG_MFMA_BWD_ST>(wdB, o, pack8<T>(of));
                     }
                 }
@@ -830,8 +842,11 @@ int bwd_launch(const void *dy, const void *x, const void *B, const void *C, cons
         // product waves and row waves in one workgroup: the types whose backward is bound by instruction issue
         e = dm.planar ? launch(mfma_bwd_duo_kernel<T, true>, 512) : launch(mfma_bwd_duo_kernel<T, false>, 512);
     } else if constexpr (NK == 5) {
-        // planar operands: instantiated for the five-slice walk only (bwd_t sends every filter length there)
-        e = dm.planar ? launch(mfma_bwd_kernel<T, NK, NW, true>, 64 * NW) : launch(mfma_bwd_kernel<T, NK, NW>, 64 * NW);
+        // planar operands: instantiated for the five-slice walk only (bwd_t sends every filter length there);
+        // plain 16-bit tensors in runs of 32 steps and more: with the idle cycles in front of the stores
+        if (dm.planar) e = launch(mfma_bwd_kernel<T, NK, NW, true>, 64 * NW);
+        else if (!MT<T>::SPLIT && p.steps_per_seg >= 32) e = launch(mfma_bwd_kernel<T, NK, NW, false, !MT<T>::SPLIT>, 64 * NW);
+        else e = launch(mfma_bwd_kernel<T, NK, NW>, 64 * NW);
     } else {
         e = launch(mfma_bwd_kernel<T, NK, NW>, 64 * NW);
     }

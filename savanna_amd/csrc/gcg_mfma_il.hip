@@ -20,6 +20,13 @@
 #define GCG_MFMA_IL_FWD_ST 16
 #endif
 
+// Idle cycles in front of each output store of the 4-wave backward (tuning builds may override).  Measured at the
+// 7B layer shape: bf16 174.0 us without, 170.4 - 170.9 with 8 - 12 cycles, 171.9 with 16, 178.7 with 24; f16 171.9,
+// 168.4 - 169.1, 166.1, 167.3; 1 x 32768 x 8192 bf16: 663, 655 - 657, 665, 670.  (The kernel with product waves and
+// row waves is bound by instruction issue and loses with any.)
+#ifndef GCG_MFMA_IL_BWD_ST_GAP
+#define GCG_MFMA_IL_BWD_ST_GAP 12
+#endif
 namespace gcg {
 namespace {
 
@@ -72,8 +79,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     const bool cvalid = c0 + CH * a < d;
     const uint32_t lane_off = (uint32_t)(row0 * row_bytes + (c0 + CH * a) * M::ES);
     const uint32_t feat_off = lane_off + (uint32_t)((t0 - tf) * row_bytes);
-    const uint32_t pass_off = (uint32_t)(KS * row_bytes), bad = cvalid ? 0u : WIN_OFF;
+    const uint32_t pass_off = __builtin_amdgcn_readfirstlane((uint32_t)(KS * row_bytes)), bad = cvalid ? 0u : WIN_OFF;
     auto step_off = [&](int64_t s) { return (uint32_t)((s * STEP - t0) * row_bytes); };
+    // The lane's part and the uniform part of a feature offset are tripled separately, and inside the loop the uniform
+    // part is a running value (so3): written as 3 * (lane + uniform) each access costs a 64-bit multiply-add on the
+    // vector unit.
+    const uint32_t feat_off3 = 3 * feat_off + bad;
+    const uint32_t pass_off3 = __builtin_amdgcn_readfirstlane(3 * pass_off);
 
     op_t A[NK];            // A[(ph - i + NK) % NK]: operand of step s-i while step s runs in phase ph
 #pragma unroll
@@ -84,10 +96,9 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     const unsigned char *y_rd = y_st + row0 * YROW + 4 * CH * a;
 
     // rows of step s: the NH rows before the lane's own first, then its NR rows
-    auto fetch = [&](int64_t s, u32x3 (&p)[NH + NR]) {
-        const uint32_t o = feat_off + step_off(s);
+    auto fetch = [&](uint32_t so3, u32x3 (&p)[NH + NR]) {
 #pragma unroll
-        for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, 3 * (o + (k - NH) * pass_off) + bad);
+        for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, feat_off3 + (so3 + (uint32_t)(k - NH) * pass_off3));
     };
     auto store_u = [&](const float (&uf)[8]) {
 #pragma unroll
@@ -113,10 +124,10 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
     u32x3 lead[NLEAD][NH + NR];
     if constexpr (NK > 1) {
 #pragma unroll
-        for (int i = 1; i < NK; ++i) fetch(s_lo - i, lead[i - 1]);
+        for (int i = 1; i < NK; ++i) fetch(3 * step_off(s_lo - i), lead[i - 1]);
     }
     u32x3 in[NH + NR];
-    fetch(s_lo, in);
+    fetch(3 * step_off(s_lo), in);
 
     store_taps(htab[w], l, hv);
     __syncthreads();
@@ -141,13 +152,19 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
         }
     }
 
-    int64_t s = s_lo;
-    while (s < s_hi) {
+    // the run's steps are counted from 0 in 32 bits, and so are their offsets (the values of step_off modulo 2^32)
+    const int n_steps = (int)(s_hi - s_lo);
+    const uint32_t step_b = __builtin_amdgcn_readfirstlane((uint32_t)(STEP * row_bytes));
+    const uint32_t step_b3 = __builtin_amdgcn_readfirstlane(3 * step_b);
+    uint32_t so = __builtin_amdgcn_readfirstlane(step_off(s_lo));            // of step s
+    uint32_t so3 = __builtin_amdgcn_readfirstlane(3 * step_off(s_lo));
+    int s = 0;
+    while (s < n_steps) {
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
-            if (s < s_hi) {
+            if (s < n_steps) {
                 u32x3 nx[NH + NR];   // rows of the next step; past the segment they fall outside the window
-                fetch(s + 1, nx);
+                fetch(so3 + step_b3, nx);
 
                 float xf[8], Bf[8], Cf[8], uf[8];
                 rows_of(in, xf, Bf, Cf);
@@ -167,7 +184,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
                     *(f32x4 *)(y_wr + 16 * YROW) = acc1;
                 }
                 __syncthreads();
-                const uint32_t o = lane_off + step_off(s) + bad;
+                const uint32_t o = lane_off + so + bad;
 #pragma unroll
                 for (int k = 0; k < NR; ++k) {
                     float yf[CH];
@@ -180,6 +197,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_fwd_kernel(const T *__restric
 #pragma unroll
                 for (int k = 0; k < NH + NR; ++k) in[k] = nx[k];
                 ++s;
+                so += step_b;
+                so3 += step_b3;
             }
         }
     }
@@ -263,7 +282,7 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     const bool cvalid = c0 + CH * a < d;
     const uint32_t lane_off = (uint32_t)(row0 * row_bytes + (c0 + CH * a) * M::ES);
     const uint32_t feat_off = lane_off + (uint32_t)((t0 - tf) * row_bytes);
-    const uint32_t pass_off = (uint32_t)(KS * row_bytes), bad = cvalid ? 0u : WIN_OFF;
+    const uint32_t pass_off = __builtin_amdgcn_readfirstlane((uint32_t)(KS * row_bytes)), bad = cvalid ? 0u : WIN_OFF;
     auto step_off = [&](int64_t sg) { return (uint32_t)((sg * STEP - t0) * row_bytes); };
 
     // While step s runs in phase ph:  Au[(ph - i + NK) % NK] is the u operand of step s-i,
@@ -290,10 +309,17 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
 
     // interleaved rows and dy of one step (zero outside the sequence)
     // (with the featurizer: the NH rows before the lane's own first, then its NR rows)
-    auto fetch_feat = [&](int64_t step, u32x3 (&p)[NH + NR]) {
-        const uint32_t o = feat_off + step_off(step);
+    // (so3: three times the step's offset step_off(step).  The lane's part and the uniform part of an offset are
+    // tripled separately and the uniform one is a running value inside the loop: written as 3 * (lane + uniform)
+    // each access costs a 64-bit multiply-add on the vector unit.)
+    const uint32_t feat_off3 = 3 * feat_off + bad, lane_off3 = 3 * lane_off + bad;
+    const uint32_t pass_off3 = __builtin_amdgcn_readfirstlane(3 * pass_off);
+    // x, B rows straight from the pieces (il_split_rows): not for plain f16, whose conversions through fp32 the compiler
+    // removes by itself, and whose backward measures 10 us slower with the explicit form (7B layer shape)
+    constexpr bool SPLIT_ROWS = !std::is_same<T, f16_t>::value;
+    auto fetch_feat = [&](uint32_t so3, u32x3 (&p)[NH + NR]) {
 #pragma unroll
-        for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, 3 * (o + (k - NH) * pass_off) + bad);
+        for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, feat_off3 + (so3 + (uint32_t)(k - NH) * pass_off3));
     };
     float tap[FEAT ? KF : 1][NV];
     if constexpr (FEAT) load_feat_taps<T, KF, NV>(wfeat, cvalid ? 3 * (c0 + CH * a) : 0, kf, tap);
@@ -302,8 +328,8 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
         if constexpr (FEAT) featurized_rows<T, NR, KF>(p, tap, xo, Bo, Co);
         else il_split<T, NR>(p, xo, Bo, Co);
     };
-    auto fetch_dy = [&](int64_t step, Row<T> &out) {
-        const uint32_t o = lane_off + step_off(step) + bad;
+    auto fetch_dy = [&](uint32_t so, Row<T> &out) {
+        const uint32_t o = lane_off + so + bad;
         uint32_t u[NR];
 #pragma unroll
         for (int k = 0; k < NR; ++k) u[k] = ldw4(wdyw, o + k * pass_off);
@@ -331,13 +357,13 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     if constexpr (NK > 1) {
 #pragma unroll
         for (int i = 1; i < NK; ++i) {
-            fetch_feat(s_lo - i, past[i - 1]);
-            fetch_feat(s_lo + NK - 1 - i, lead[i - 1]);
-            fetch_dy(s_lo + NK - 1 - i, wdy[i - 1]);
+            fetch_feat(3 * step_off(s_lo - i), past[i - 1]);
+            fetch_feat(3 * step_off(s_lo + NK - 1 - i), lead[i - 1]);
+            fetch_dy(step_off(s_lo + NK - 1 - i), wdy[i - 1]);
         }
     }
-    fetch_feat(s_lo + NK - 1, in);
-    fetch_dy(s_lo + NK - 1, dyr);
+    fetch_feat(3 * step_off(s_lo + NK - 1), in);
+    fetch_dy(step_off(s_lo + NK - 1), dyr);
 
     store_taps(htab + w * HTAB, l, hv);
     __syncthreads();
@@ -377,19 +403,36 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
     }
 
     int xb_slot = 0;      // ring slot of step s (step s_lo+k sits in slot k % (NK-1))
-    int64_t s = s_lo;
-    while (s < s_hi) {
+    // the run's steps are counted from 0 in 32 bits, and so are their offsets (the values of step_off modulo 2^32)
+    const int n_steps = (int)(s_hi - s_lo);
+    const uint32_t step_b = __builtin_amdgcn_readfirstlane((uint32_t)(STEP * row_bytes));
+    uint32_t so = __builtin_amdgcn_readfirstlane(step_off(s_lo));        // of step s
+    uint32_t so3 = __builtin_amdgcn_readfirstlane(3 * step_off(s_lo));
+    const uint32_t step_b3 = __builtin_amdgcn_readfirstlane(3 * step_b);
+    int s = 0;
+    while (s < n_steps) {
 #pragma unroll
         for (int ph = 0; ph < NK; ++ph) {
-            if (s < s_hi) {
+            if (s < n_steps) {
                 const int slot_new = (ph + NK - 1) % NK;     // ring slot of step s+NK-1
                 u32x3 nx[NH + NR];   // rows of the next iteration; past the segment's reach they are
                 Row<T> dyn;          // outside the windows
-                fetch_feat(s + NK, nx);
-                fetch_dy(s + NK, dyn);
+                fetch_feat(so3 + (uint32_t)NK * step_b3, nx);
+                fetch_dy(so + (uint32_t)NK * step_b, dyn);
 
                 float xf[8], Bf[8], tf[8], cf[8], pf[8];
-                {
+                if constexpr (SPLIT_ROWS && NK > 1 && !FEAT && M::ES == 2) {
+                    // x, B of step s+NK-1 go to the ring as they are; C as fp32
+                    Row<T> xa, Ba;
+                    il_split_rows<T>(in, xa, Ba, cf);
+                    unsigned char *slot = xb_own + xb_slot * 2 * XB_VEC;
+                    const Row<T> xw = lds_load_row<T>(slot), Bw = lds_load_row<T>(slot + XB_VEC);
+                    lds_store_row<T>(slot, xa);
+                    lds_store_row<T>(slot + XB_VEC, Ba);
+                    xb_slot = (xb_slot + 1 == NK - 1) ? 0 : xb_slot + 1;
+                    unpack8<T>(xw, xf);
+                    unpack8<T>(Bw, Bf);
+                } else {
                     float xa[8], Ba[8];
                     rows_of(in, xa, Ba, cf);                  // x, B, C of step s+NK-1
                     if constexpr (NK > 1) {
@@ -460,14 +503,18 @@ __global__ __launch_bounds__(64 * NW) void mfma_il_bwd_kernel(const T *__restric
                         }
                     u32x3 po[NR];
                     il_join<T, NR>(ox, oB, oC, po);
-                    const uint32_t o = lane_off + step_off(s);
 #pragma unroll
-                    for (int k = 0; k < NR; ++k) win_store_as<KEEP>(wdf, 3 * (o + k * pass_off) + bad, po[k]);
+                    for (int k = 0; k < NR; ++k) {
+                        if constexpr (GCG_MFMA_IL_BWD_ST_GAP > 0 && M::ES == 2 && !M::SPLIT) idle_cycles<GCG_MFMA_IL_BWD_ST_GAP>();
+                        win_store_as<KEEP>(wdf, lane_off3 + (so3 + (uint32_t)k * pass_off3), po[k]);
+                    }
                 }
 #pragma unroll
                 for (int k = 0; k < NH + NR; ++k) in[k] = nx[k];
                 dyr = dyn;
                 ++s;
+                so += step_b;
+                so3 += step_b3;
             }
         }
     }
@@ -550,7 +597,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
         const bool cvalid = c0 + CH * a < d;
         const uint32_t lane_off = (uint32_t)(row0 * row_bytes + (c0 + CH * a) * M::ES);
         const uint32_t feat_off = lane_off + (uint32_t)((t0 - tf) * row_bytes);
-        const uint32_t pass_off = (uint32_t)(KS * row_bytes), bad = cvalid ? 0u : WIN_OFF;
+        const uint32_t pass_off = __builtin_amdgcn_readfirstlane((uint32_t)(KS * row_bytes)), bad = cvalid ? 0u : WIN_OFF;
         auto step_off = [&](int64_t sg) { return (uint32_t)((sg * STEP - t0) * row_bytes); };
         const int rm_off = row0 * UROW + M::LES * CH * a;
         const int yd_rd = row0 * YROW + 4 * CH * a;
@@ -559,15 +606,17 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
         // the interleaved rows and dy of one step (zero outside the sequence); with the featurizer the NH rows
         // before the lane's own come first
         struct Rows { u32x3 p[NH + NR]; Row<T> dy; };
-        // (so: the step's offset, step_off(step); inside the loop a running 32-bit value, advanced by step_b per step)
-        // (the lane's part and the uniform part are multiplied separately: the uniform one on the scalar unit)
+        // (so: the step's offset, step_off(step), and so3 three times that; inside the loop running 32-bit values.  The
+        // lane's part and the uniform part of an offset are tripled separately: written as 3 * (lane + uniform) each
+        // access costs a 64-bit multiply-add on the vector unit.)
         const uint32_t feat_off3 = 3 * feat_off + bad, lane_off3 = 3 * lane_off + bad;
-        auto fetch_feat = [&](uint32_t so, u32x3 (&p)[NH + NR]) {
+        const uint32_t pass_off3 = __builtin_amdgcn_readfirstlane(3 * pass_off);
+        auto fetch_feat = [&](uint32_t so3, u32x3 (&p)[NH + NR]) {
 #pragma unroll
-            for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, feat_off3 + 3 * (so + (k - NH) * pass_off));
+            for (int k = 0; k < NH + NR; ++k) p[k] = ldw12(wf, feat_off3 + (so3 + (uint32_t)(k - NH) * pass_off3));
         };
-        auto fetch = [&](uint32_t so, Rows &r) {
-            fetch_feat(so, r.p);
+        auto fetch = [&](uint32_t so, uint32_t so3, Rows &r) {
+            fetch_feat(so3, r.p);
             const uint32_t o = lane_off + so + bad;
             uint32_t u[NR];
 #pragma unroll
@@ -599,7 +648,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
             store_rows(u_t, pf);
         };
         // the interleaved gradient rows of step sg from its y2 / du tiles
-        auto finish_step = [&](uint32_t so, bool live, const unsigned char *y_t, const unsigned char *d_t,
+        auto finish_step = [&](uint32_t so3, bool live, const unsigned char *y_t, const unsigned char *d_t,
                                const Row<T> &dyo, const Row<T> &xo, const Row<T> &Bo) {
             float dyf[8], xf[8], Bf[8], oC[8], ox[8], oB[8];
             unpack8<T>(dyo, dyf);
@@ -618,9 +667,9 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
                 }
             u32x3 po[NR];
             il_join<T, NR>(ox, oB, oC, po);
-            const uint32_t o3 = live ? lane_off3 + 3 * so : WIN_OFF;
+            const uint32_t o3 = live ? lane_off3 + so3 : WIN_OFF;
 #pragma unroll
-            for (int k = 0; k < NR; ++k) win_store_as<KEEP>(wdf, o3 + 3 * k * pass_off, po[k]);
+            for (int k = 0; k < NR; ++k) win_store_as<KEEP>(wdf, o3 + (uint32_t)k * pass_off3, po[k]);
         };
 
         // Rings of the row waves, indexed by step - s_lo: x, B (as row vectors of the tensors' type) of the step being
@@ -638,11 +687,11 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
             u32x3 past[NK - 1][NH + NR];
             Rows lead[NK];
 #pragma unroll
-            for (int i = 1; i < NK; ++i) fetch_feat(step_off(s_lo - i), past[i - 1]);
+            for (int i = 1; i < NK; ++i) fetch_feat(3 * step_off(s_lo - i), past[i - 1]);
 #pragma unroll
-            for (int jj = NK - 2; jj >= 0; --jj) fetch(step_off(s_lo + jj), lead[jj]);
-            fetch(step_off(s_lo + NK - 1), lead[NK - 1]);
-            fetch(step_off(s_lo + NK), st[1]);
+            for (int jj = NK - 2; jj >= 0; --jj) fetch(step_off(s_lo + jj), 3 * step_off(s_lo + jj), lead[jj]);
+            fetch(step_off(s_lo + NK - 1), 3 * step_off(s_lo + NK - 1), lead[NK - 1]);
+            fetch(step_off(s_lo + NK), 3 * step_off(s_lo + NK), st[1]);
             __syncthreads();                                          // (A)
             __syncthreads();                                          // (A2): the filter tables' place is free
             float f0[8], f1[8], f2[8];
@@ -686,8 +735,10 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
         // the run's steps are counted from 0 in 32 bits, and so are their offsets (the same values modulo 2^32 as
         // step_off gives): 64-bit multiplications per step are a tenth of the row waves' vector cycles otherwise
         const int n_steps = (int)(s_hi - s_lo);
-        const uint32_t step_b = (uint32_t)(STEP * row_bytes);
-        uint32_t so = step_off(s_lo);        // of step s
+        const uint32_t step_b = __builtin_amdgcn_readfirstlane((uint32_t)(STEP * row_bytes));
+        const uint32_t step_b3 = __builtin_amdgcn_readfirstlane(3 * step_b);
+        uint32_t so = __builtin_amdgcn_readfirstlane(step_off(s_lo));        // of step s
+        uint32_t so3 = __builtin_amdgcn_readfirstlane(3 * step_off(s_lo));
         int s = 0;
         auto row_step = [&](int pu) __attribute__((always_inline)) {
             const int par = pu & 1;
@@ -696,8 +747,8 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
             const unsigned char *const y_old = smem + D::OFF_Y + (par ^ 1) * YSZ, *const d_old = smem + D::OFF_D + (par ^ 1) * YSZ;
             // Order as in mfma_bwd_duo_kernel: the request for rows first, then the stores, then what needs the previous
             // request's rows, the filter-gradient products last.
-            fetch(so + (uint32_t)(NK + 1) * step_b, st[par]);
-            finish_step(so - step_b, s > 0, y_old, d_old, dyq[(pu + RSLOTS - 1) % RSLOTS], xh[(pu + 2) % 3], Bh[(pu + 2) % 3]);
+            fetch(so + (uint32_t)(NK + 1) * step_b, so3 + (uint32_t)(NK + 1) * step_b3, st[par]);
+            finish_step(so3 - step_b3, s > 0, y_old, d_old, dyq[(pu + RSLOTS - 1) % RSLOTS], xh[(pu + 2) % 3], Bh[(pu + 2) % 3]);
             {
                 // step s+1: x, B from the ring; C and dy of step s+NK from the rows that arrived, whose x, B take the slot
                 float cf[8], xf[8], Bf[8];
@@ -727,6 +778,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
             __syncthreads();
             ++s;
             so += step_b;
+            so3 += step_b3;
         };
         // Every step can be the run's last (see mfma_bwd_duo_kernel for why the steps are not grouped); the run's
         // last step is finished where the loop leaves, so that the rings keep compile-time indices.
@@ -739,7 +791,7 @@ __global__ __launch_bounds__(512) void mfma_il_bwd_duo_kernel(const T *__restric
                         row_step(pu);
                     } else {
                         const int par = (pu & 1) ^ 1;         // of step n_steps-1
-                        finish_step(so - step_b, true, smem + D::OFF_Y + par * YSZ, smem + D::OFF_D + par * YSZ,
+                        finish_step(so3 - step_b3, true, smem + D::OFF_Y + par * YSZ, smem + D::OFF_D + par * YSZ,
                                     dyq[(pu + RSLOTS - 1) % RSLOTS], xh[(pu + 2) % 3], Bh[(pu + 2) % 3]);
                         done = true;
                     }

@@ -295,6 +295,15 @@ template <> struct MT<f16w_t> : MTSplit<3, 2, 2> {
     static __device__ __forceinline__ uint32_t pack2(float lo, float hi) { return pack_f16x2(lo, hi); }
 };
 
+// CYCLES idle cycles of the wave, and nothing scheduled across them
+template <int CYCLES> __device__ __forceinline__ void idle_cycles()
+{
+#pragma unroll
+    for (int i = 0; i < CYCLES / 16; ++i) asm volatile("s_nop 15");
+    if constexpr (CYCLES % 16 != 0) asm volatile("s_nop %0" ::"n"(CYCLES % 16 - 1));
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // A workgroup of NW waves owns CB = 16*NW adjacent channels; LDS rows are padded (see MT<T>::urow;
 // the fp32 result tile: consecutive rows start 4 banks apart).
 template <typename T, int NW> struct Geo {
