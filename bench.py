@@ -412,6 +412,10 @@ KERNEL_TABLE = (
     ("window bf16 hl=7, 7B", "sep", 2, 8192, 256, 16, 7, torch.bfloat16, torch.bfloat16),
     ("window fp32 hl=7, 7B", "sep", 2, 8192, 256, 16, 7, torch.float32, torch.float32),
     ("window interleaved fp32 hl=7, 7B", "il", 2, 8192, 256, 16, 7, torch.float32, torch.float32),
+    # a tensor-parallel rank's share of the 40B layer at TP = 8 (get_groups_and_group_sizes: g = 64, d = 1024)
+    ("mfma bf16 hl=128, 40B / 8 ranks, L=8192", "sep", 1, 8192, 64, 16, 128, torch.bfloat16, torch.bfloat16),
+    ("mfma interleaved bf16 hl=128, 40B / 8 ranks, L=8192", "il", 1, 8192, 64, 16, 128, torch.bfloat16, torch.bfloat16),
+    ("window bf16 hl=7, 40B / 8 ranks, L=8192", "sep", 1, 8192, 64, 16, 7, torch.bfloat16, torch.bfloat16),
 )
 
 
